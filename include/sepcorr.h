@@ -1,0 +1,114 @@
+/*
+ * sepcorr.h - C ABI of libsepcorr.so: memory-saving separation of the 4D correlation volume
+ * for AMD gfx950 (MI355X).  The 4D volume S[b,i,j,u,v] = <f1[b,i,j,:], f2[b,u,v,:]> is formed tile
+ * by tile in registers with fp32 MFMA and reduced on the fly; it is never written to memory.
+ *
+ * Every entry point replaces one function of the reference's native module `MemorySaver`
+ * (libs/MemorySaver/src/MemorySaver_cuda.cpp:105-112) with plain pointers and sizes in place of
+ * at::Tensor.  Conventions shared by all of them:
+ *
+ *  - All pointers are DEVICE pointers on the current HIP device.  Inputs are borrowed and never
+ *    written; outputs are fully overwritten (no pre-initialisation needed, unlike the reference
+ *    kernels which accumulate into buffers the host pre-fills, MemorySaver_kernel_forward.cu:916-927).
+ *  - All tensors are contiguous fp32 except the argmax tensors (int32):
+ *      f1      (B, H1, W1, C)   image-1 features at pyramid level 0, pre-scaled by the caller
+ *      f2      (B, H2, W2, C)   image-2 features at pyramid level k
+ *      *_u     (B, H1, W1, ch, H2)   keeps u (fmap2 row), was reduced over v (fmap2 column)
+ *      *_v     (B, H1, W1, ch, W2)   keeps v, was reduced over u
+ *    ch = 2 (max, avg) for the max/avg tensors, 1 for argmax, K for the attention tensors.
+ *  - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Calls are asynchronous:
+ *    they enqueue kernels and return.
+ *  - Return value: 0 on success, a negative SEPCORR_E* code otherwise; sepcorr_last_error() then
+ *    returns a message for the calling thread.  Nothing is launched when a check fails.
+ *  - Limits of this build: 1 <= W2 <= 256, 1 <= C <= 1024, 1 <= K <= 8, all sizes >= 1 and small
+ *    enough that every tensor has fewer than 2^31 elements.
+ *  - Backward entry points need scratch memory: query sepcorr_backward_workspace_bytes() and pass a
+ *    device buffer of at least that size (256-byte aligned).  Its contents on entry are ignored.
+ */
+#ifndef SEPCORR_H
+#define SEPCORR_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SEPCORR_OK 0
+#define SEPCORR_EINVAL (-1)   /* null pointer, non-positive or unsupported size */
+#define SEPCORR_ELAUNCH (-2)  /* HIP reported an error at launch */
+#define SEPCORR_EWORKSPACE (-3) /* workspace missing or too small */
+
+/* Message describing the last failure on this thread ("" if none). */
+const char *sepcorr_last_error(void);
+
+/* ABI version of this library (bumped on incompatible change). */
+int sepcorr_abi_version(void);
+
+/*
+ * Replaces MemorySaver.max_avg_forward (MemorySaver_cuda.cpp:10-21 -> max_avg_cuda_forward,
+ * MemorySaver_kernel_forward.cu:901-949).
+ *   out_u[b,i,j,0,u] = max_v S   out_u[b,i,j,1,u] = (sum_v S) / W2      (B,H1,W1,2,H2)
+ *   out_v[b,i,j,0,v] = max_u S   out_v[b,i,j,1,v] = (sum_u S) / H2      (B,H1,W1,2,W2)
+ */
+int sepcorr_max_avg_forward(const float *f1, const float *f2, float *out_u, float *out_v,
+                            int B, int H1, int W1, int H2, int W2, int C, void *stream);
+
+/*
+ * Replaces MemorySaver.max_argmax_avg_forward (MemorySaver_cuda.cpp:23-34 ->
+ * MemorySaver_kernel_forward.cu:962-1016).  As above plus
+ *   argmax_u[b,i,j,0,u] = the v attaining max_v S,  argmax_v[b,i,j,0,v] = the u attaining max_u S,
+ * lowest index on exact ties (MemorySaver_kernel_forward.cu:498-507).
+ */
+int sepcorr_max_argmax_avg_forward(const float *f1, const float *f2, float *out_u, float *out_v,
+                                   int32_t *argmax_u, int32_t *argmax_v,
+                                   int B, int H1, int W1, int H2, int W2, int C, void *stream);
+
+/*
+ * Replaces MemorySaver.compression_forward (MemorySaver_cuda.cpp:36-53 ->
+ * MemorySaver_kernel_forward.cu:1029-1074), for any K (the reference kernel is fixed to K=2).
+ *   comp_u[b,i,j,k,u] = sum_v S * a_u[b,i,j,k,v]      a_u (B,H1,W1,K,W2) -> comp_u (B,H1,W1,K,H2)
+ *   comp_v[b,i,j,k,v] = sum_u S * a_v[b,i,j,k,u]      a_v (B,H1,W1,K,H2) -> comp_v (B,H1,W1,K,W2)
+ * Weights are used as given (the caller applies the softmax, core/corr.py:441-442).
+ */
+int sepcorr_compression_forward(const float *f1, const float *f2, const float *a_u, const float *a_v,
+                                float *comp_u, float *comp_v,
+                                int B, int H1, int W1, int H2, int W2, int C, int K, void *stream);
+
+/* Scratch bytes needed by either backward entry point for these sizes (0 is possible). */
+size_t sepcorr_backward_workspace_bytes(int B, int H1, int W1, int H2, int W2, int C);
+
+/*
+ * Replaces MemorySaver.max_argmax_avg_backward (MemorySaver_cuda.cpp:55-78 ->
+ * MemorySaver_kernel_max_avg_argmax_backward.cu:1198-1221).  With
+ *   G = g_u[..,0,u]*[v==argmax_u[..,u]] + g_u[..,1,u]/W2 + g_v[..,0,v]*[u==argmax_v[..,v]] + g_v[..,1,v]/H2
+ *   d_f1[b,i,j,:] = sum_{u,v} G f2[b,u,v,:]     d_f2[b,u,v,:] = sum_{i,j} G f1[b,i,j,:]
+ * d_f2 is accumulated by the owner of each (u,v) in a fixed order: no atomics, run-to-run identical
+ * (the reference uses atomicAdd, MemorySaver_kernel_max_avg_argmax_backward.cu:305-310).
+ * Argmax entries are data: a value outside its axis selects nothing.
+ */
+int sepcorr_max_argmax_avg_backward(const float *f1, const float *f2,
+                                    const int32_t *argmax_u, const int32_t *argmax_v,
+                                    const float *grad_u, const float *grad_v,
+                                    float *d_f1, float *d_f2,
+                                    int B, int H1, int W1, int H2, int W2, int C,
+                                    void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Replaces MemorySaver.compression_backward (MemorySaver_cuda.cpp:80-103 ->
+ * MemorySaver_kernel_compression_backward.cu:651-666).  With
+ *   G = sum_k a_u[..,k,v]*g_cu[..,k,u] + a_v[..,k,u]*g_cv[..,k,v]
+ *   d_f1 = sum_{u,v} G f2      d_f2 = sum_{i,j} G f1
+ *   d_a_u[b,i,j,k,v] = sum_u S * g_cu[b,i,j,k,u]      d_a_v[b,i,j,k,u] = sum_v S * g_cv[b,i,j,k,v]
+ */
+int sepcorr_compression_backward(const float *f1, const float *f2, const float *a_u, const float *a_v,
+                                 const float *g_cu, const float *g_cv,
+                                 float *d_f1, float *d_f2, float *d_a_u, float *d_a_v,
+                                 int B, int H1, int W1, int H2, int W2, int C, int K,
+                                 void *workspace, size_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SEPCORR_H */

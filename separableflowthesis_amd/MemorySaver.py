@@ -1,0 +1,151 @@
+"""Python face of the native module the reference calls `MemorySaver`.
+
+Same five functions, argument order and return lists as the reference's pybind module
+(libs/MemorySaver/src/MemorySaver_cuda.cpp:105-112), taking torch tensors.  torch is used for
+device memory and the current stream only; the arithmetic happens in libsepcorr.so.
+
+Checks mirror CHECK_CUDA / CHECK_CONTIGUOUS (MemorySaver_cuda.cpp:6-8) and add the dtype and
+shape agreement the reference leaves unchecked; every violation raises RuntimeError.
+"""
+import torch
+
+from . import _lib
+
+
+def _check(name, t, dtype=torch.float32, ndim=None):
+    if not isinstance(t, torch.Tensor):
+        raise RuntimeError(f"{name} must be a torch.Tensor")
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+    if t.dtype != dtype:
+        raise RuntimeError(f"{name} must have dtype {dtype}, got {t.dtype}")
+    if ndim is not None and t.dim() != ndim:
+        raise RuntimeError(f"{name} must have {ndim} dimensions, got {t.dim()}")
+
+
+def _dims(f1, f2):
+    _check("img1_features_l0", f1, ndim=4)
+    _check("img2_features_lk", f2, ndim=4)
+    if f1.device != f2.device:
+        raise RuntimeError("img1_features_l0 and img2_features_lk must be on the same device")
+    B, H1, W1, C = f1.shape
+    B2, H2, W2, C2 = f2.shape
+    if B != B2 or C != C2:
+        raise RuntimeError(f"batch/feature sizes differ: {tuple(f1.shape)} vs {tuple(f2.shape)}")
+    return B, H1, W1, H2, W2, C
+
+
+def _expect(name, t, shape, device, dtype=torch.float32):
+    _check(name, t, dtype=dtype, ndim=len(shape))
+    if tuple(t.shape) != tuple(shape):
+        raise RuntimeError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
+    if t.device != device:
+        raise RuntimeError(f"{name} must be on {device}")
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _workspace(lib, dims, device):
+    n = lib.sepcorr_backward_workspace_bytes(*dims)
+    ws = torch.empty(max(n, 1), dtype=torch.uint8, device=device)
+    return ws, n
+
+
+def max_avg_forward(img1_features_l0, img2_features_lk):
+    """-> [max_avg_output_u (B,H1,W1,2,H2), max_avg_output_v (B,H1,W1,2,W2)]"""
+    f1, f2 = img1_features_l0, img2_features_lk
+    B, H1, W1, H2, W2, C = _dims(f1, f2)
+    lib = _lib.load()
+    with torch.cuda.device(f1.device):
+        out_u = torch.empty((B, H1, W1, 2, H2), dtype=f1.dtype, device=f1.device)
+        out_v = torch.empty((B, H1, W1, 2, W2), dtype=f1.dtype, device=f1.device)
+        _lib.check(lib.sepcorr_max_avg_forward(f1.data_ptr(), f2.data_ptr(), out_u.data_ptr(), out_v.data_ptr(),
+                                               B, H1, W1, H2, W2, C, _stream()))
+    return [out_u, out_v]
+
+
+def max_argmax_avg_forward(img1_features_l0, img2_features_lk):
+    """-> [max_avg_output_u, max_avg_output_v, argmax_output_u (B,H1,W1,1,H2) i32, argmax_output_v (B,H1,W1,1,W2) i32]"""
+    f1, f2 = img1_features_l0, img2_features_lk
+    B, H1, W1, H2, W2, C = _dims(f1, f2)
+    lib = _lib.load()
+    with torch.cuda.device(f1.device):
+        out_u = torch.empty((B, H1, W1, 2, H2), dtype=f1.dtype, device=f1.device)
+        out_v = torch.empty((B, H1, W1, 2, W2), dtype=f1.dtype, device=f1.device)
+        am_u = torch.empty((B, H1, W1, 1, H2), dtype=torch.int32, device=f1.device)
+        am_v = torch.empty((B, H1, W1, 1, W2), dtype=torch.int32, device=f1.device)
+        _lib.check(lib.sepcorr_max_argmax_avg_forward(f1.data_ptr(), f2.data_ptr(), out_u.data_ptr(), out_v.data_ptr(),
+                                                      am_u.data_ptr(), am_v.data_ptr(), B, H1, W1, H2, W2, C, _stream()))
+    return [out_u, out_v, am_u, am_v]
+
+
+def max_argmax_avg_backward(img1_features_l0, img2_features_lk, argmax_output_u, argmax_output_v,
+                            grad_MaxAvg_u, grad_MaxAvg_v):
+    """-> [grad_fmap1_l0 (B,H1,W1,C), grad_fmap2_lk (B,H2,W2,C)]"""
+    f1, f2 = img1_features_l0, img2_features_lk
+    B, H1, W1, H2, W2, C = _dims(f1, f2)
+    dev = f1.device
+    _expect("argmax_output_u", argmax_output_u, (B, H1, W1, 1, H2), dev, torch.int32)
+    _expect("argmax_output_v", argmax_output_v, (B, H1, W1, 1, W2), dev, torch.int32)
+    _expect("grad_MaxAvg_u", grad_MaxAvg_u, (B, H1, W1, 2, H2), dev)
+    _expect("grad_MaxAvg_v", grad_MaxAvg_v, (B, H1, W1, 2, W2), dev)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        d1 = torch.empty_like(f1)
+        d2 = torch.empty_like(f2)
+        ws, n = _workspace(lib, (B, H1, W1, H2, W2, C), dev)
+        _lib.check(lib.sepcorr_max_argmax_avg_backward(
+            f1.data_ptr(), f2.data_ptr(), argmax_output_u.data_ptr(), argmax_output_v.data_ptr(),
+            grad_MaxAvg_u.data_ptr(), grad_MaxAvg_v.data_ptr(), d1.data_ptr(), d2.data_ptr(),
+            B, H1, W1, H2, W2, C, ws.data_ptr(), n, _stream()))
+    return [d1, d2]
+
+
+def compression_forward(img1_features_l0, img2_features_lk, attention_weights_u, attention_weights_v):
+    """-> [compression_output_u (B,H1,W1,K,H2), compression_output_v (B,H1,W1,K,W2)]"""
+    f1, f2 = img1_features_l0, img2_features_lk
+    B, H1, W1, H2, W2, C = _dims(f1, f2)
+    dev = f1.device
+    _check("attention_weights_u", attention_weights_u, ndim=5)
+    K = attention_weights_u.shape[3]
+    _expect("attention_weights_u", attention_weights_u, (B, H1, W1, K, W2), dev)
+    _expect("attention_weights_v", attention_weights_v, (B, H1, W1, K, H2), dev)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        cu = torch.empty((B, H1, W1, K, H2), dtype=f1.dtype, device=dev)
+        cv = torch.empty((B, H1, W1, K, W2), dtype=f1.dtype, device=dev)
+        _lib.check(lib.sepcorr_compression_forward(
+            f1.data_ptr(), f2.data_ptr(), attention_weights_u.data_ptr(), attention_weights_v.data_ptr(),
+            cu.data_ptr(), cv.data_ptr(), B, H1, W1, H2, W2, C, K, _stream()))
+    return [cu, cv]
+
+
+def compression_backward(img1_features_l0, img2_features_lk, attention_weights_u, attention_weights_v,
+                         grad_compressed_output_u, grad_compressed_output_v):
+    """-> [grad_fmap1_l0, grad_fmap2_lk, grad_attention_u (B,H1,W1,K,W2), grad_attention_v (B,H1,W1,K,H2)]"""
+    f1, f2 = img1_features_l0, img2_features_lk
+    B, H1, W1, H2, W2, C = _dims(f1, f2)
+    dev = f1.device
+    _check("attention_weights_u", attention_weights_u, ndim=5)
+    K = attention_weights_u.shape[3]
+    _expect("attention_weights_u", attention_weights_u, (B, H1, W1, K, W2), dev)
+    _expect("attention_weights_v", attention_weights_v, (B, H1, W1, K, H2), dev)
+    _expect("grad_compressed_output_u", grad_compressed_output_u, (B, H1, W1, K, H2), dev)
+    _expect("grad_compressed_output_v", grad_compressed_output_v, (B, H1, W1, K, W2), dev)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        d1 = torch.empty_like(f1)
+        d2 = torch.empty_like(f2)
+        da_u = torch.empty_like(attention_weights_u)
+        da_v = torch.empty_like(attention_weights_v)
+        ws, n = _workspace(lib, (B, H1, W1, H2, W2, C), dev)
+        _lib.check(lib.sepcorr_compression_backward(
+            f1.data_ptr(), f2.data_ptr(), attention_weights_u.data_ptr(), attention_weights_v.data_ptr(),
+            grad_compressed_output_u.data_ptr(), grad_compressed_output_v.data_ptr(),
+            d1.data_ptr(), d2.data_ptr(), da_u.data_ptr(), da_v.data_ptr(),
+            B, H1, W1, H2, W2, C, K, ws.data_ptr(), n, _stream()))
+    return [d1, d2, da_u, da_v]

@@ -1,0 +1,57 @@
+"""Host-side caller of the op: the reference's AlternateCorrBlockSepflow (core/corr.py:335-510).
+
+Builds the two separated 3D correlation volumes over a 4-level fmap2 pyramid without ever
+holding the 4D volume.  Behaviour kept from the reference: NLF guidance is refused, the
+function class is picked by `support_backward`, outputs are
+  corr1 (B, K*levels, W, H1, W1)  and  corr2 (B, K*levels, H, H1, W1),
+channel order [max, avg, att_0..] per level, levels concatenated on dim 1, every level
+trilinearly upsampled (align_corners=True) to the level-0 displacement length.
+"""
+import torch
+import torch.nn.functional as F
+
+from .functions import ComputeMaxArgmaxAvgFunction, ComputeMaxAvgFunction, ComputeSelfCompressionFunction
+
+
+class AlternateCorrBlockSepflow:
+    def __init__(self, fmap1, fmap2, guid, num_levels=4, radius=4, support_backward=False):
+        if guid is not None:
+            # core/corr.py:356-358: NLF couples entries of the 4D volume, which is never stored here
+            raise Exception("Cannot use NLF while not storing the 4d correlation volume")
+        self.max_avg_function = ComputeMaxArgmaxAvgFunction if support_backward else ComputeMaxAvgFunction
+        self.num_levels = num_levels
+        self.radius = radius
+        self.fmap1_l0 = fmap1
+        self.pyramid = [fmap2]
+        for _ in range(self.num_levels - 1):
+            fmap2 = F.avg_pool2d(fmap2, 2, stride=2)
+            self.pyramid.append(fmap2)
+
+    def separate(self, attention_weights):
+        batch, fdim, h1, w1 = self.fmap1_l0.shape
+        h2, w2 = h1, w1
+        sep_u_lvls, sep_v_lvls = [], []
+        # the scaled NHWC copy of fmap1 is level independent; made once (the reference redoes it per level)
+        fmap1 = self.fmap1_l0.permute(0, 2, 3, 1).contiguous() / torch.sqrt(torch.tensor(fdim).float())
+        for i in range(self.num_levels):
+            fmap2 = self.pyramid[i].permute(0, 2, 3, 1).contiguous()
+            maxavg_u, maxavg_v = self.max_avg_function.apply(fmap1, fmap2)
+            sep_v = maxavg_u.permute(0, 3, 4, 1, 2).contiguous()   # (B,2,H2_i,h1,w1)
+            sep_u = maxavg_v.permute(0, 3, 4, 1, 2).contiguous()   # (B,2,W2_i,h1,w1)
+            if attention_weights is not None:
+                attention1, attention2 = attention_weights
+                a_u = attention1(sep_u).softmax(dim=2).permute(0, 3, 4, 1, 2).contiguous()
+                a_v = attention2(sep_v).softmax(dim=2).permute(0, 3, 4, 1, 2).contiguous()
+                adaptive_corr_u, adaptive_corr_v = ComputeSelfCompressionFunction.apply(fmap1, fmap2, a_u, a_v)
+                sep_v = torch.cat((sep_v, adaptive_corr_u.permute(0, 3, 4, 1, 2)), dim=1)
+                sep_u = torch.cat((sep_u, adaptive_corr_v.permute(0, 3, 4, 1, 2)), dim=1)
+            sep_u_lvls.append(F.interpolate(sep_u, [w2, h1, w1], mode='trilinear', align_corners=True))
+            sep_v_lvls.append(F.interpolate(sep_v, [h2, h1, w1], mode='trilinear', align_corners=True))
+        return torch.cat(sep_u_lvls, dim=1), torch.cat(sep_v_lvls, dim=1)
+
+    def __call__(self, coords, sep=False, attention_weights=None):
+        if sep:
+            return self.separate(attention_weights)
+        # core/corr.py:491-492
+        raise NotImplementedError("Missing the cpp/cuda part for lookup"
+                                  "of the 4d correlation volume without storing it")

@@ -1,0 +1,877 @@
+// libsepcorr: memory-saving separation of the 4D correlation volume, hand-written for gfx950.
+//
+// S[p,q] = <f1[p,:], f2[q,:]> with p = image-1 pixel (i,j), q = image-2 pixel (u,v) is produced
+// 32x32 tiles at a time by v_mfma_f32_32x32x2_f32 and consumed in registers; it never reaches
+// memory.  Three kernels cover the five entry points of include/sepcorr.h:
+//
+//   fwd_kernel  workgroup owns 32 pixels p and sweeps every fmap2 row u.  Wave w owns the column
+//               chunk v in [32w, 32w+32).  MFMA rows are v (A operand = f2, loaded straight from
+//               global memory in operand layout), MFMA columns are p (B operand = f1 tile in LDS).
+//               One lane therefore holds one p and 16 v's: reductions over v are in-lane plus one
+//               cross-half shuffle plus a cross-wave combine through LDS; reductions over u are
+//               element-wise running state in registers in the accumulator layout.
+//               Epilogues: max/avg(/argmax), or K weighted sums (attention compression; also the
+//               d_a_u/d_a_v pass of the compression backward, which has the same form).
+//   df1_kernel  same ownership.  G[p,q] is synthesised in registers directly in MFMA B-operand
+//               layout from the saved argmax / upstream grads (or attention weights), A = f2^T
+//               from global memory, D = d_f1^T partial per wave, summed across waves in LDS.
+//   df2_kernel  wave owns 32 pixels q = (u, 32 consecutive v) and sweeps p; G^T synthesised in
+//               registers, A = f1^T from global.  The p range can be split over workgroups; the
+//               partial sums are written to scratch and added in a fixed order (no atomics).
+//
+// The contraction index of an MFMA may be permuted freely as long as A and B agree, and so may the
+// row index of D as long as the store agrees; both freedoms are used so that every lane loads 16
+// contiguous bytes.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "sepcorr.h"
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+namespace {
+
+constexpr int TP = 32;        // pixels per MFMA column block
+constexpr int MAX_W2 = 256;   // 8 waves x 32 columns
+constexpr int MAX_C = 1024;
+constexpr int MAX_K = 8;
+constexpr int KCH = 4;        // attention channels handled per launch
+
+thread_local char g_err[256] = "";
+
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+// Row of the 32x32 accumulator held in register r of a lane in half h (lane / 32).
+__device__ __forceinline__ int vmap(int r, int h) { return 8 * (r >> 2) + 4 * h + (r & 3); }
+
+// 4 consecutive floats base[c..c+3], zero where out of range or !ok.
+template <bool CVEC>
+__device__ __forceinline__ v4f load4(const float *base, int c, int C, bool ok) {
+    v4f x = {0.f, 0.f, 0.f, 0.f};
+    if (ok) {
+        if constexpr (CVEC) {
+            if (c < C) x = *reinterpret_cast<const v4f *>(base + c);
+        } else {
+            if (c + 0 < C) x[0] = base[c + 0];
+            if (c + 1 < C) x[1] = base[c + 1];
+            if (c + 2 < C) x[2] = base[c + 2];
+            if (c + 3 < C) x[3] = base[c + 3];
+        }
+    }
+    return x;
+}
+
+template <bool CVEC>
+__device__ __forceinline__ void store4(float *base, int c, int C, v4f x, bool accumulate) {
+    if constexpr (CVEC) {
+        if (c < C) {
+            v4f *d = reinterpret_cast<v4f *>(base + c);
+            if (accumulate) x += *d;
+            *d = x;
+        }
+    } else {
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            if (c + t < C) base[c + t] = accumulate ? base[c + t] + x[t] : x[t];
+    }
+}
+
+__device__ __forceinline__ v16f mfma(float a, float b, v16f c) {
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+
+// ------------------------------------------------------------------------------------------
+// forward
+// ------------------------------------------------------------------------------------------
+enum { MODE_MAXAVG = 0, MODE_ARGMAX = 1, MODE_WEIGHTED = 2 };
+
+struct FwdArgs {
+    const float *f1, *f2;
+    const float *wv;   // MODE_WEIGHTED: weights indexed by v, (B,N1,KT,W2)
+    const float *wu;   // MODE_WEIGHTED: weights indexed by u, (B,N1,KT,H2)
+    float *out_u;      // (B,N1,CH,H2)
+    float *out_v;      // (B,N1,CH,W2)
+    int *am_u, *am_v;  // MODE_ARGMAX
+    int N1, H2, W2, C, CP;
+    int KT, k0;        // total weight channels and first channel of this launch
+    int tiles_per_batch;
+};
+
+template <int MODE, int KC, int UR, bool CVEC, int MAXT>
+__global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
+    constexpr int GJ = 2;  // 8-channel slices per prefetch group
+    constexpr int NPART = (MODE == MODE_WEIGHTED) ? KC : 3;
+    extern __shared__ float smem[];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, pl = lane & 31, h = lane >> 5;
+    const int nW = blockDim.x >> 6;
+    const int b = blockIdx.x / a.tiles_per_batch;
+    const int p0 = (blockIdx.x % a.tiles_per_batch) * TP;
+    const int N1 = a.N1, H2 = a.H2, W2 = a.W2, C = a.C;
+    const int LS = a.CP + 4;
+    float *f1s = smem;
+    float *part = smem + TP * LS;
+
+    {   // stage the f1 tile [TP][CP] (zero padded) into LDS
+        const int c4n = a.CP >> 2;
+        for (int idx = tid; idx < TP * c4n; idx += blockDim.x) {
+            const int row = idx / c4n, c = (idx - row * c4n) * 4;
+            const bool ok = p0 + row < N1;
+            const float *src = a.f1 + ((size_t)b * N1 + (ok ? p0 + row : 0)) * C;
+            *reinterpret_cast<v4f *>(f1s + row * LS + c) = load4<CVEC>(src, c, C, ok);
+        }
+    }
+    __syncthreads();
+
+    const int pix = p0 + pl;           // this lane's image-1 pixel
+    const bool pok = pix < N1;
+    const size_t bp = (size_t)b * N1 + (pok ? pix : 0);
+    const int vrow = 32 * wave + pl;   // the fmap2 column this lane feeds to the A operand
+    const bool vrow_ok = vrow < W2;
+    const float *f2lane = a.f2 + ((size_t)b * H2 * W2 + (vrow_ok ? vrow : 0)) * C;
+    const size_t rowstride = (size_t)W2 * C;
+
+    unsigned vmask = 0;  // bit r: accumulator register r maps to a real column
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+        if (32 * wave + vmap(r, h) < W2) vmask |= 1u << r;
+
+    // running state over u, accumulator layout
+    float vmax[16], vsum[16];
+    int vidx[16];
+    float wvr[KC][16], rv[KC][16];
+    if constexpr (MODE == MODE_WEIGHTED) {
+#pragma unroll
+        for (int k = 0; k < KC; ++k)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int v = 32 * wave + vmap(r, h);
+                rv[k][r] = 0.f;
+                wvr[k][r] = (pok && v < W2) ? a.wv[(bp * a.KT + a.k0 + k) * W2 + v] : 0.f;
+            }
+    } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            vmax[r] = -INFINITY;
+            vsum[r] = 0.f;
+            vidx[r] = 0;
+        }
+    }
+
+    const int NJ = a.CP >> 3;
+    const int NG = (NJ + GJ - 1) / GJ;
+    const int nsteps = (H2 + UR - 1) / UR;
+    const int T = nsteps * NG;
+
+    v16f acc[UR];
+#pragma unroll
+    for (int r = 0; r < UR; ++r)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[r][e] = 0.f;
+
+    float wur[UR][KC];  // MODE_WEIGHTED: u-indexed weights of the rows of the current step
+
+    auto issue = [&](int step, int g, v4f(&buf)[UR][GJ]) {
+#pragma unroll
+        for (int r = 0; r < UR; ++r) {
+            const int u = step * UR + r;
+#pragma unroll
+            for (int jj = 0; jj < GJ; ++jj) {
+                const int j = g * GJ + jj;
+                buf[r][jj] = load4<CVEC>(f2lane + (size_t)(u < H2 ? u : 0) * rowstride, 8 * j + 4 * h, C,
+                                         vrow_ok && u < H2 && j < NJ);
+            }
+        }
+    };
+
+    auto epilogue = [&](int step) {
+        float *pb = part + (step & 1) * (UR * NPART * nW * 32);
+#pragma unroll
+        for (int ru = 0; ru < UR; ++ru) {
+            const int u = step * UR + ru;
+            if (u < H2) {
+                if constexpr (MODE == MODE_WEIGHTED) {
+#pragma unroll
+                    for (int k = 0; k < KC; ++k) {
+                        float s = 0.f;
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) s += acc[ru][r] * wvr[k][r];
+                        s += __shfl_xor(s, 32);
+                        if (h == 0) pb[((ru * NPART + k) * nW + wave) * 32 + pl] = s;
+                        const float w = wur[ru][k];
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) rv[k][r] += acc[ru][r] * w;
+                    }
+                } else {
+                    float m = -INFINITY, s = 0.f;
+                    int mi = 0x7fffffff;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const float x = acc[ru][r];
+                        const bool ok = (vmask >> r) & 1u;
+                        const float xm = ok ? x : -INFINITY;
+                        if (xm > m) { m = xm; mi = 32 * wave + vmap(r, h); }
+                        s += x;  // columns outside the image hold exact zeros
+                        if (x > vmax[r]) { vmax[r] = x; vidx[r] = u; }
+                        vsum[r] += x;
+                    }
+                    const float m2 = __shfl_xor(m, 32);
+                    const int mi2 = __shfl_xor(mi, 32);
+                    s += __shfl_xor(s, 32);
+                    if (m2 > m || (m2 == m && mi2 < mi)) { m = m2; mi = mi2; }
+                    if (h == 0) {
+                        pb[((ru * NPART + 0) * nW + wave) * 32 + pl] = m;
+                        pb[((ru * NPART + 1) * nW + wave) * 32 + pl] = __int_as_float(mi);
+                        pb[((ru * NPART + 2) * nW + wave) * 32 + pl] = s;
+                    }
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[ru][e] = 0.f;
+        }
+        __syncthreads();
+        // combine the per-wave partials in wave order and store the finished rows
+        if constexpr (MODE == MODE_WEIGHTED) {
+            for (int idx = tid; idx < UR * KC * 32; idx += blockDim.x) {
+                const int p = idx & 31, k = (idx >> 5) % KC, ru = idx / (32 * KC);
+                const int u = step * UR + ru;
+                if (u < H2 && p0 + p < N1) {
+                    float s = 0.f;
+                    for (int w = 0; w < nW; ++w) s += pb[((ru * NPART + k) * nW + w) * 32 + p];
+                    a.out_u[(((size_t)b * N1 + p0 + p) * a.KT + a.k0 + k) * H2 + u] = s;
+                }
+            }
+        } else {
+            for (int idx = tid; idx < UR * 32; idx += blockDim.x) {
+                const int p = idx & 31, ru = idx >> 5;
+                const int u = step * UR + ru;
+                if (u < H2 && p0 + p < N1) {
+                    float m = pb[((ru * NPART + 0) * nW + 0) * 32 + p];
+                    int mi = __float_as_int(pb[((ru * NPART + 1) * nW + 0) * 32 + p]);
+                    float s = pb[((ru * NPART + 2) * nW + 0) * 32 + p];
+                    for (int w = 1; w < nW; ++w) {
+                        const float m2 = pb[((ru * NPART + 0) * nW + w) * 32 + p];
+                        if (m2 > m) { m = m2; mi = __float_as_int(pb[((ru * NPART + 1) * nW + w) * 32 + p]); }
+                        s += pb[((ru * NPART + 2) * nW + w) * 32 + p];
+                    }
+                    const size_t o = ((size_t)b * N1 + p0 + p);
+                    a.out_u[(o * 2 + 0) * H2 + u] = m;
+                    a.out_u[(o * 2 + 1) * H2 + u] = s / (float)W2;
+                    if constexpr (MODE == MODE_ARGMAX) a.am_u[o * H2 + u] = mi;
+                }
+            }
+        }
+    };
+
+    auto compute = [&](int step, int g, v4f(&buf)[UR][GJ]) {
+        if constexpr (MODE == MODE_WEIGHTED) {
+            if (g == 0) {
+#pragma unroll
+                for (int r = 0; r < UR; ++r) {
+                    const int u = step * UR + r;
+#pragma unroll
+                    for (int k = 0; k < KC; ++k)
+                        wur[r][k] = (pok && u < H2) ? a.wu[(bp * a.KT + a.k0 + k) * H2 + u] : 0.f;
+                }
+            }
+        }
+#pragma unroll
+        for (int jj = 0; jj < GJ; ++jj) {
+            const int j = g * GJ + jj;
+            if (j < NJ) {
+                const v4f bv = *reinterpret_cast<const v4f *>(f1s + pl * LS + 8 * j + 4 * h);
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int r = 0; r < UR; ++r) acc[r] = mfma(buf[r][jj][t], bv[t], acc[r]);
+            }
+        }
+        if (g == NG - 1) epilogue(step);
+    };
+
+    v4f bufA[UR][GJ], bufB[UR][GJ];
+    int step = 0, g = 0;  // position of iteration `it`
+    issue(0, 0, bufA);
+    for (int it = 0; it < T; it += 2) {
+        int g1 = g + 1, s1 = step;
+        if (g1 == NG) { g1 = 0; ++s1; }
+        int g2 = g1 + 1, s2 = s1;
+        if (g2 == NG) { g2 = 0; ++s2; }
+        if (it + 1 < T) issue(s1, g1, bufB);
+        compute(step, g, bufA);
+        if (it + 2 < T) issue(s2, g2, bufA);
+        if (it + 1 < T) compute(s1, g1, bufB);
+        step = s2;
+        g = g2;
+    }
+
+    // store the state that was reduced over u
+    if (pok) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int v = 32 * wave + vmap(r, h);
+            if (v < W2) {
+                if constexpr (MODE == MODE_WEIGHTED) {
+#pragma unroll
+                    for (int k = 0; k < KC; ++k) a.out_v[(bp * a.KT + a.k0 + k) * W2 + v] = rv[k][r];
+                } else {
+                    a.out_v[(bp * 2 + 0) * W2 + v] = vmax[r];
+                    a.out_v[(bp * 2 + 1) * W2 + v] = vsum[r] / (float)H2;
+                    if constexpr (MODE == MODE_ARGMAX) a.am_v[bp * W2 + v] = vidx[r];
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// backward: G synthesis shared by df1 / df2
+// ------------------------------------------------------------------------------------------
+enum { GMODE_MAXAVG = 0, GMODE_COMP = 1 };
+
+struct BwdArgs {
+    const float *f1, *f2;
+    const int *am_u, *am_v;          // GMODE_MAXAVG
+    const float *g_u, *g_v;          // GMODE_MAXAVG: (B,N1,2,H2), (B,N1,2,W2)
+    const float *a_u, *a_v;          // GMODE_COMP:   (B,N1,KT,W2), (B,N1,KT,H2)
+    const float *g_cu, *g_cv;        // GMODE_COMP:   (B,N1,KT,H2), (B,N1,KT,W2)
+    float *d1;                       // (B,N1,C)
+    float *d2;                       // (B,N2,C) or scratch [nsplit][B,N2,C]
+    int B, N1, H2, W2, C;
+    int KT, k0;
+    int tiles_per_batch;             // df1: p tiles per batch
+    int nsplit, tiles_per_split;     // df2: split of the p range
+    int accumulate;                  // add to the destination instead of overwriting
+};
+
+// Weights of one lane that depend on (p, v) and on (p, u).
+template <int GMODE, int KC>
+struct VW {
+    float a[GMODE == GMODE_COMP ? KC : 1];   // maxavg: g_v[max];        comp: a_u[k]
+    float g[GMODE == GMODE_COMP ? KC : 1];   // maxavg: g_v[avg] / H2;   comp: g_cv[k]
+    int am;                                  // maxavg: argmax_v
+};
+template <int GMODE, int KC>
+struct UW {
+    float a[GMODE == GMODE_COMP ? KC : 1];   // maxavg: g_u[max];        comp: a_v[k]
+    float g[GMODE == GMODE_COMP ? KC : 1];   // maxavg: g_u[avg] / W2;   comp: g_cu[k]
+    int am;                                  // maxavg: argmax_u
+};
+
+template <int GMODE, int KC>
+__device__ __forceinline__ VW<GMODE, KC> load_vw(const BwdArgs &a, size_t bp, int v, bool ok) {
+    VW<GMODE, KC> w;
+    if constexpr (GMODE == GMODE_COMP) {
+#pragma unroll
+        for (int k = 0; k < KC; ++k) {
+            const size_t o = (bp * a.KT + a.k0 + k) * a.W2 + v;
+            w.a[k] = ok ? a.a_u[o] : 0.f;
+            w.g[k] = ok ? a.g_cv[o] : 0.f;
+        }
+        w.am = 0;
+    } else {
+        w.a[0] = ok ? a.g_v[(bp * 2 + 0) * a.W2 + v] : 0.f;
+        w.g[0] = ok ? a.g_v[(bp * 2 + 1) * a.W2 + v] / (float)a.H2 : 0.f;
+        w.am = ok ? a.am_v[bp * a.W2 + v] : -1;
+    }
+    return w;
+}
+template <int GMODE, int KC>
+__device__ __forceinline__ UW<GMODE, KC> load_uw(const BwdArgs &a, size_t bp, int u, bool ok) {
+    UW<GMODE, KC> w;
+    if constexpr (GMODE == GMODE_COMP) {
+#pragma unroll
+        for (int k = 0; k < KC; ++k) {
+            const size_t o = (bp * a.KT + a.k0 + k) * a.H2 + u;
+            w.a[k] = ok ? a.a_v[o] : 0.f;
+            w.g[k] = ok ? a.g_cu[o] : 0.f;
+        }
+        w.am = 0;
+    } else {
+        w.a[0] = ok ? a.g_u[(bp * 2 + 0) * a.H2 + u] : 0.f;
+        w.g[0] = ok ? a.g_u[(bp * 2 + 1) * a.H2 + u] / (float)a.W2 : 0.f;
+        w.am = ok ? a.am_u[bp * a.H2 + u] : -1;
+    }
+    return w;
+}
+// dL/dS at (p, u, v); `ok` false gives exactly 0.
+template <int GMODE, int KC>
+__device__ __forceinline__ float gval(const VW<GMODE, KC> &wv, const UW<GMODE, KC> &wu, int u, int v, bool ok) {
+    float g = 0.f;
+    if constexpr (GMODE == GMODE_COMP) {
+#pragma unroll
+        for (int k = 0; k < KC; ++k) g += wv.a[k] * wu.g[k] + wu.a[k] * wv.g[k];
+    } else {
+        g = wu.g[0] + wv.g[0];
+        if (wu.am == v) g += wu.a[0];
+        if (wv.am == u) g += wv.a[0];
+    }
+    return ok ? g : 0.f;
+}
+
+// d_f1[p, c] = sum_q G[p,q] f2[q,c].  Grid: (B * tiles_per_batch, channel blocks of 128*NCB).
+template <int GMODE, int KC, int NCB, bool CVEC, int MAXT>
+__global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
+    constexpr int GS = 2;            // MFMA k-steps (pairs of v) per prefetch group
+    constexpr int NG = 16 / GS;
+    constexpr int CB = 128 * NCB;
+    constexpr int RS = CB + 4;
+    extern __shared__ float smem[];  // [TP][RS] cross-wave sum
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, pl = lane & 31, h = lane >> 5;
+    const int nW = blockDim.x >> 6;
+    const int b = blockIdx.x / a.tiles_per_batch;
+    const int p0 = (blockIdx.x % a.tiles_per_batch) * TP;
+    const int cb0 = blockIdx.y * CB;
+    const int N1 = a.N1, H2 = a.H2, W2 = a.W2, C = a.C;
+    const int pix = p0 + pl;
+    const bool pok = pix < N1;
+    const size_t bp = (size_t)b * N1 + (pok ? pix : 0);
+
+    VW<GMODE, KC> wv[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int v = 32 * wave + vmap(r, h);
+        wv[r] = load_vw<GMODE, KC>(a, bp, v < W2 ? v : 0, pok && v < W2);
+    }
+
+    v16f acc[NCB][4];
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[cb][t][e] = 0.f;
+
+    const float *f2b = a.f2 + (size_t)b * H2 * W2 * C;
+    auto issue = [&](int u, int g, v4f(&buf)[GS][NCB]) {
+#pragma unroll
+        for (int ss = 0; ss < GS; ++ss) {
+            const int v = 32 * wave + vmap(g * GS + ss, h);
+            const bool ok = v < W2;
+            const float *src = f2b + ((size_t)u * W2 + (ok ? v : 0)) * C;
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) buf[ss][cb] = load4<CVEC>(src, cb0 + 128 * cb + 4 * pl, C, ok);
+        }
+    };
+
+    float G[16];
+    UW<GMODE, KC> wu_next = load_uw<GMODE, KC>(a, bp, 0, pok);
+    auto compute = [&](int u, int g, v4f(&buf)[GS][NCB]) {
+        if (g == 0) {
+            const UW<GMODE, KC> wu = wu_next;
+            if (u + 1 < H2) wu_next = load_uw<GMODE, KC>(a, bp, u + 1, pok);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int v = 32 * wave + vmap(r, h);
+                G[r] = gval<GMODE, KC>(wv[r], wu, u, v, pok && v < W2);
+            }
+        }
+#pragma unroll
+        for (int ss = 0; ss < GS; ++ss)
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) acc[cb][t] = mfma(buf[ss][cb][t], G[g * GS + ss], acc[cb][t]);
+    };
+
+    // G is indexed with a value known after unrolling only if the group index is static: unroll rows by hand
+    v4f bufA[GS][NCB], bufB[GS][NCB];
+    issue(0, 0, bufA);
+    for (int u = 0; u < H2; ++u) {
+#pragma unroll
+        for (int g = 0; g < NG; g += 2) {
+            issue(u, g + 1, bufB);
+            compute(u, g, bufA);
+            if (g + 2 < NG) issue(u, g + 2, bufA);
+            else if (u + 1 < H2) issue(u + 1, 0, bufA);
+            compute(u, g + 1, bufB);
+        }
+    }
+
+    // sum the per-wave partials in wave order through LDS, then store coalesced
+    for (int w = 0; w < nW; ++w) {
+        if (wave == w) {
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    v4f x = {acc[cb][0][r], acc[cb][1][r], acc[cb][2][r], acc[cb][3][r]};
+                    v4f *d = reinterpret_cast<v4f *>(smem + pl * RS + 128 * cb + 4 * vmap(r, h));
+                    if (w > 0) x += *d;
+                    *d = x;
+                }
+        }
+        __syncthreads();
+    }
+    for (int idx = tid; idx < TP * (CB / 4); idx += blockDim.x) {
+        const int row = idx / (CB / 4), c = (idx - row * (CB / 4)) * 4;
+        if (p0 + row < N1) {
+            const v4f x = *reinterpret_cast<const v4f *>(smem + row * RS + c);
+            store4<CVEC>(a.d1 + ((size_t)b * N1 + p0 + row) * C, cb0 + c, C, x, a.accumulate != 0);
+        }
+    }
+}
+
+// d_f2[q, c] = sum_p G[p,q] f1[p,c].  Each wave is an independent task (b, split, u, v chunk);
+// grid: (ceil(tasks / 4), channel blocks of 128*NCB), 256 threads.
+template <int GMODE, int KC, int NCB, bool CVEC>
+__global__ void __launch_bounds__(256) df2_kernel(const BwdArgs a, int ntasks, int nvc) {
+    constexpr int GS = 2;
+    constexpr int NG = 16 / GS;
+    constexpr int CB = 128 * NCB;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, pl = lane & 31, h = lane >> 5;
+    int task = blockIdx.x * 4 + wave;
+    if (task >= ntasks) return;
+    const int N1 = a.N1, H2 = a.H2, W2 = a.W2, C = a.C;
+    const int vc = task % nvc; task /= nvc;
+    const int u = task % H2; task /= H2;
+    const int split = task % a.nsplit;
+    const int b = task / a.nsplit;
+    const int cb0 = blockIdx.y * CB;
+    const int v = 32 * vc + pl;
+    const bool vok = v < W2;
+    const int vs = vok ? v : 0;
+    const int pbeg = split * a.tiles_per_split * TP;
+    const int pend = min(N1, pbeg + a.tiles_per_split * TP);
+    const int ntiles = (pend - pbeg + TP - 1) / TP;
+
+    v16f acc[NCB][4];
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[cb][t][e] = 0.f;
+
+    struct Buf {
+        v4f f[GS][NCB];
+        VW<GMODE, KC> wv[GS];
+        UW<GMODE, KC> wu[GS];
+    };
+    auto issue = [&](int tile, int g, Buf &buf) {
+#pragma unroll
+        for (int ss = 0; ss < GS; ++ss) {
+            const int p = pbeg + tile * TP + 2 * (g * GS + ss) + h;
+            const bool ok = p < pend;
+            const size_t bp = (size_t)b * N1 + (ok ? p : 0);
+            buf.wv[ss] = load_vw<GMODE, KC>(a, bp, vs, ok && vok);
+            buf.wu[ss] = load_uw<GMODE, KC>(a, bp, u, ok);
+            const float *src = a.f1 + bp * C;
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) buf.f[ss][cb] = load4<CVEC>(src, cb0 + 128 * cb + 4 * pl, C, ok);
+        }
+    };
+    auto compute = [&](int tile, int g, const Buf &buf) {
+#pragma unroll
+        for (int ss = 0; ss < GS; ++ss) {
+            const int p = pbeg + tile * TP + 2 * (g * GS + ss) + h;
+            const float G = gval<GMODE, KC>(buf.wv[ss], buf.wu[ss], u, v, p < pend && vok);
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) acc[cb][t] = mfma(buf.f[ss][cb][t], G, acc[cb][t]);
+        }
+    };
+
+    Buf bufA, bufB;
+    if (ntiles > 0) issue(0, 0, bufA);
+    for (int tile = 0; tile < ntiles; ++tile) {
+#pragma unroll
+        for (int g = 0; g < NG; g += 2) {
+            issue(tile, g + 1, bufB);
+            compute(tile, g, bufA);
+            if (g + 2 < NG) issue(tile, g + 2, bufA);
+            else if (tile + 1 < ntiles) issue(tile + 1, 0, bufA);
+            compute(tile, g + 1, bufB);
+        }
+    }
+
+    if (vok) {
+        float *dst = a.d2 + ((size_t)split * a.B + b) * H2 * W2 * C + ((size_t)u * W2 + v) * C;
+        const bool accum = a.accumulate != 0 && a.nsplit == 1;
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const v4f x = {acc[cb][0][r], acc[cb][1][r], acc[cb][2][r], acc[cb][3][r]};
+                store4<CVEC>(dst, cb0 + 128 * cb + 4 * vmap(r, h), C, x, accum);
+            }
+    }
+}
+
+// out[i] (+)= sum_s part[s*n + i], in split order.
+__global__ void __launch_bounds__(256) reduce_splits_kernel(const float *part, float *out, size_t n, int nsplit,
+                                                            int accumulate) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        float s = accumulate ? out[i] : 0.f;
+        for (int k = 0; k < nsplit; ++k) s += part[(size_t)k * n + i];
+        out[i] = s;
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------------------------
+struct Dims {
+    int B, H1, W1, H2, W2, C;
+};
+
+int check_dims(const Dims &d, int K) {
+    if (d.B < 1 || d.H1 < 1 || d.W1 < 1 || d.H2 < 1 || d.W2 < 1 || d.C < 1)
+        return fail(SEPCORR_EINVAL, "sepcorr: all sizes must be >= 1 (B=%d H1=%d W1=%d H2=%d W2=%d C=%d)", d.B, d.H1,
+                    d.W1, d.H2, d.W2, d.C);
+    if (d.W2 > MAX_W2) return fail(SEPCORR_EINVAL, "sepcorr: W2=%d exceeds the supported maximum %d", d.W2, MAX_W2);
+    if (d.C > MAX_C) return fail(SEPCORR_EINVAL, "sepcorr: C=%d exceeds the supported maximum %d", d.C, MAX_C);
+    if (K < 1 || K > MAX_K) return fail(SEPCORR_EINVAL, "sepcorr: K=%d outside 1..%d", K, MAX_K);
+    const double lim = 2147483647.0;
+    const double n1 = (double)d.B * d.H1 * d.W1, n2 = (double)d.B * d.H2 * d.W2;
+    const int ch = K > 2 ? K : 2;
+    if (n1 * d.C > lim || n2 * d.C > lim || n1 * ch * d.H2 > lim || n1 * ch * d.W2 > lim)
+        return fail(SEPCORR_EINVAL, "sepcorr: a tensor would have 2^31 or more elements");
+    return SEPCORR_OK;
+}
+
+int check_launch(const char *what) {
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(SEPCORR_ELAUNCH, "sepcorr: %s: %s", what, hipGetErrorString(e));
+    return SEPCORR_OK;
+}
+
+template <typename KernelT>
+int set_lds(KernelT kernel, size_t bytes) {
+    if (bytes > 64 * 1024) {
+        const hipError_t e =
+            hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+        if (e != hipSuccess) return fail(SEPCORR_ELAUNCH, "sepcorr: cannot reserve %zu bytes of LDS: %s", bytes, hipGetErrorString(e));
+    }
+    return SEPCORR_OK;
+}
+
+template <int MODE, int KC, int UR>
+int launch_fwd(const FwdArgs &a, int B, hipStream_t s) {
+    const int nW = (a.W2 + 31) / 32;
+    constexpr int NPART = (MODE == MODE_WEIGHTED) ? KC : 3;
+    const size_t lds = ((size_t)TP * (a.CP + 4) + 2 * UR * NPART * nW * 32) * sizeof(float);
+    const dim3 grid(B * a.tiles_per_batch), block(64 * nW);
+    const bool cvec = (a.C % 4) == 0;
+#define SEPCORR_FWD(CV, MT)                                                      \
+    do {                                                                         \
+        auto k = fwd_kernel<MODE, KC, UR, CV, MT>;                               \
+        if (int rc = set_lds(k, lds)) return rc;                                 \
+        hipLaunchKernelGGL(k, grid, block, lds, s, a);                           \
+    } while (0)
+    if (nW <= 4) {
+        if (cvec) SEPCORR_FWD(true, 256); else SEPCORR_FWD(false, 256);
+    } else {
+        if (cvec) SEPCORR_FWD(true, 512); else SEPCORR_FWD(false, 512);
+    }
+#undef SEPCORR_FWD
+    return check_launch("forward kernel");
+}
+
+template <int MODE>
+int launch_fwd_weighted_k(const FwdArgs &a, int kc, int B, hipStream_t s) {
+    switch (kc) {
+        case 1: return launch_fwd<MODE, 1, 2>(a, B, s);
+        case 2: return launch_fwd<MODE, 2, 2>(a, B, s);
+        case 3: return launch_fwd<MODE, 3, 1>(a, B, s);
+        default: return launch_fwd<MODE, 4, 1>(a, B, s);
+    }
+}
+
+FwdArgs fwd_args(const Dims &d) {
+    FwdArgs a;
+    memset(&a, 0, sizeof(a));
+    a.N1 = d.H1 * d.W1;
+    a.H2 = d.H2;
+    a.W2 = d.W2;
+    a.C = d.C;
+    a.CP = (d.C + 7) & ~7;
+    a.tiles_per_batch = (a.N1 + TP - 1) / TP;
+    return a;
+}
+
+// sum_v S wv[k,v] -> out_u[k,u];  sum_u S wu[k,u] -> out_v[k,v]  for K channels, KCH per launch
+int weighted_forward(const Dims &d, const float *f1, const float *f2, const float *wv, const float *wu, float *out_u,
+                     float *out_v, int K, hipStream_t s) {
+    FwdArgs a = fwd_args(d);
+    a.f1 = f1; a.f2 = f2; a.wv = wv; a.wu = wu; a.out_u = out_u; a.out_v = out_v;
+    a.KT = K;
+    for (int k0 = 0; k0 < K; k0 += KCH) {
+        a.k0 = k0;
+        const int kc = K - k0 < KCH ? K - k0 : KCH;
+        if (int rc = launch_fwd_weighted_k<MODE_WEIGHTED>(a, kc, d.B, s)) return rc;
+    }
+    return SEPCORR_OK;
+}
+
+int df2_nsplit(const Dims &d) {
+    const long tasks = (long)d.B * d.H2 * ((d.W2 + 31) / 32);
+    const int tiles = (d.H1 * d.W1 + TP - 1) / TP;
+    long n = (2048 + tasks - 1) / tasks;  // aim at two waves per SIMD on 256 CUs
+    if (n > 8) n = 8;
+    if (n > tiles) n = tiles;
+    if (n < 1) n = 1;
+    return (int)n;
+}
+
+template <int GMODE, int KC>
+int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s) {
+    const bool cvec = (d.C % 4) == 0;
+    const int nW = (d.W2 + 31) / 32;
+    a.tiles_per_batch = (a.N1 + TP - 1) / TP;
+    {
+        // more than 4 waves share the register file two to a SIMD: halve the channel block
+        const int ncb = (d.C <= 128 || nW > 4) ? 1 : 2;
+        const int cblocks = (d.C + 128 * ncb - 1) / (128 * ncb);
+        const dim3 grid(d.B * a.tiles_per_batch, cblocks), block(64 * nW);
+        const size_t lds = (size_t)TP * (128 * ncb + 4) * sizeof(float);
+#define SEPCORR_DF1(NCB, CV, MT) hipLaunchKernelGGL((df1_kernel<GMODE, KC, NCB, CV, MT>), grid, block, lds, s, a)
+        if (nW > 4) { if (cvec) SEPCORR_DF1(1, true, 512); else SEPCORR_DF1(1, false, 512); }
+        else if (ncb == 1) { if (cvec) SEPCORR_DF1(1, true, 256); else SEPCORR_DF1(1, false, 256); }
+        else { if (cvec) SEPCORR_DF1(2, true, 256); else SEPCORR_DF1(2, false, 256); }
+#undef SEPCORR_DF1
+        if (int rc = check_launch("d_f1 kernel")) return rc;
+    }
+    {
+        const int ncb = d.C <= 128 ? 1 : 2;
+        const int cblocks = (d.C + 128 * ncb - 1) / (128 * ncb);
+        const int tiles = a.tiles_per_batch;
+        a.nsplit = df2_nsplit(d);
+        a.tiles_per_split = (tiles + a.nsplit - 1) / a.nsplit;
+        const int nvc = nW;
+        const int ntasks = d.B * a.nsplit * d.H2 * nvc;
+        float *d2 = a.d2;
+        if (a.nsplit > 1) a.d2 = static_cast<float *>(ws);
+        const dim3 grid((ntasks + 3) / 4, cblocks), block(256);
+#define SEPCORR_DF2(NCB, CV) hipLaunchKernelGGL((df2_kernel<GMODE, KC, NCB, CV>), grid, block, 0, s, a, ntasks, nvc)
+        if (ncb == 1) { if (cvec) SEPCORR_DF2(1, true); else SEPCORR_DF2(1, false); }
+        else          { if (cvec) SEPCORR_DF2(2, true); else SEPCORR_DF2(2, false); }
+#undef SEPCORR_DF2
+        if (int rc = check_launch("d_f2 kernel")) return rc;
+        if (a.nsplit > 1) {
+            const size_t n = (size_t)d.B * d.H2 * d.W2 * d.C;
+            const int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+            hipLaunchKernelGGL(reduce_splits_kernel, dim3(blocks), dim3(256), 0, s, static_cast<const float *>(ws), d2, n,
+                               a.nsplit, a.accumulate);
+            if (int rc = check_launch("d_f2 split reduction")) return rc;
+        }
+    }
+    return SEPCORR_OK;
+}
+
+int check_workspace(const Dims &d, void *ws, size_t ws_bytes) {
+    const size_t need = sepcorr_backward_workspace_bytes(d.B, d.H1, d.W1, d.H2, d.W2, d.C);
+    if (need > 0 && (ws == nullptr || ws_bytes < need))
+        return fail(SEPCORR_EWORKSPACE, "sepcorr: backward needs %zu bytes of workspace, got %zu", need, ws ? ws_bytes : (size_t)0);
+    if (need > 0 && (reinterpret_cast<uintptr_t>(ws) & 15))
+        return fail(SEPCORR_EWORKSPACE, "sepcorr: workspace must be 16-byte aligned");
+    return SEPCORR_OK;
+}
+
+#define REQUIRE_PTR(p) \
+    if ((p) == nullptr) return fail(SEPCORR_EINVAL, "sepcorr: argument %s is NULL", #p)
+
+}  // namespace
+
+extern "C" {
+
+const char *sepcorr_last_error(void) { return g_err; }
+int sepcorr_abi_version(void) { return 1; }
+
+int sepcorr_max_avg_forward(const float *f1, const float *f2, float *out_u, float *out_v, int B, int H1, int W1, int H2,
+                            int W2, int C, void *stream) {
+    REQUIRE_PTR(f1); REQUIRE_PTR(f2); REQUIRE_PTR(out_u); REQUIRE_PTR(out_v);
+    const Dims d = {B, H1, W1, H2, W2, C};
+    if (int rc = check_dims(d, 2)) return rc;
+    FwdArgs a = fwd_args(d);
+    a.f1 = f1; a.f2 = f2; a.out_u = out_u; a.out_v = out_v;
+    return launch_fwd<MODE_MAXAVG, 1, 2>(a, B, static_cast<hipStream_t>(stream));
+}
+
+int sepcorr_max_argmax_avg_forward(const float *f1, const float *f2, float *out_u, float *out_v, int32_t *argmax_u,
+                                   int32_t *argmax_v, int B, int H1, int W1, int H2, int W2, int C, void *stream) {
+    REQUIRE_PTR(f1); REQUIRE_PTR(f2); REQUIRE_PTR(out_u); REQUIRE_PTR(out_v); REQUIRE_PTR(argmax_u); REQUIRE_PTR(argmax_v);
+    const Dims d = {B, H1, W1, H2, W2, C};
+    if (int rc = check_dims(d, 2)) return rc;
+    FwdArgs a = fwd_args(d);
+    a.f1 = f1; a.f2 = f2; a.out_u = out_u; a.out_v = out_v; a.am_u = argmax_u; a.am_v = argmax_v;
+    return launch_fwd<MODE_ARGMAX, 1, 2>(a, B, static_cast<hipStream_t>(stream));
+}
+
+int sepcorr_compression_forward(const float *f1, const float *f2, const float *a_u, const float *a_v, float *comp_u,
+                                float *comp_v, int B, int H1, int W1, int H2, int W2, int C, int K, void *stream) {
+    REQUIRE_PTR(f1); REQUIRE_PTR(f2); REQUIRE_PTR(a_u); REQUIRE_PTR(a_v); REQUIRE_PTR(comp_u); REQUIRE_PTR(comp_v);
+    const Dims d = {B, H1, W1, H2, W2, C};
+    if (int rc = check_dims(d, K)) return rc;
+    return weighted_forward(d, f1, f2, a_u, a_v, comp_u, comp_v, K, static_cast<hipStream_t>(stream));
+}
+
+size_t sepcorr_backward_workspace_bytes(int B, int H1, int W1, int H2, int W2, int C) {
+    if (B < 1 || H1 < 1 || W1 < 1 || H2 < 1 || W2 < 1 || C < 1) return 0;
+    const Dims d = {B, H1, W1, H2, W2, C};
+    const int ns = df2_nsplit(d);
+    return ns > 1 ? (size_t)ns * B * H2 * W2 * C * sizeof(float) : 0;
+}
+
+int sepcorr_max_argmax_avg_backward(const float *f1, const float *f2, const int32_t *argmax_u, const int32_t *argmax_v,
+                                    const float *grad_u, const float *grad_v, float *d_f1, float *d_f2, int B, int H1,
+                                    int W1, int H2, int W2, int C, void *workspace, size_t workspace_bytes, void *stream) {
+    REQUIRE_PTR(f1); REQUIRE_PTR(f2); REQUIRE_PTR(argmax_u); REQUIRE_PTR(argmax_v); REQUIRE_PTR(grad_u); REQUIRE_PTR(grad_v);
+    REQUIRE_PTR(d_f1); REQUIRE_PTR(d_f2);
+    const Dims d = {B, H1, W1, H2, W2, C};
+    if (int rc = check_dims(d, 2)) return rc;
+    if (int rc = check_workspace(d, workspace, workspace_bytes)) return rc;
+    BwdArgs a;
+    memset(&a, 0, sizeof(a));
+    a.f1 = f1; a.f2 = f2; a.am_u = argmax_u; a.am_v = argmax_v; a.g_u = grad_u; a.g_v = grad_v;
+    a.d1 = d_f1; a.d2 = d_f2;
+    a.B = B; a.N1 = H1 * W1; a.H2 = H2; a.W2 = W2; a.C = C; a.KT = 1;
+    return launch_bwd<GMODE_MAXAVG, 1>(a, d, workspace, static_cast<hipStream_t>(stream));
+}
+
+int sepcorr_compression_backward(const float *f1, const float *f2, const float *a_u, const float *a_v, const float *g_cu,
+                                 const float *g_cv, float *d_f1, float *d_f2, float *d_a_u, float *d_a_v, int B, int H1,
+                                 int W1, int H2, int W2, int C, int K, void *workspace, size_t workspace_bytes,
+                                 void *stream) {
+    REQUIRE_PTR(f1); REQUIRE_PTR(f2); REQUIRE_PTR(a_u); REQUIRE_PTR(a_v); REQUIRE_PTR(g_cu); REQUIRE_PTR(g_cv);
+    REQUIRE_PTR(d_f1); REQUIRE_PTR(d_f2); REQUIRE_PTR(d_a_u); REQUIRE_PTR(d_a_v);
+    const Dims d = {B, H1, W1, H2, W2, C};
+    if (int rc = check_dims(d, K)) return rc;
+    if (int rc = check_workspace(d, workspace, workspace_bytes)) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // d_a_v[k,u] = sum_v S g_cv[k,v];  d_a_u[k,v] = sum_u S g_cu[k,u]: the forward's weighted sums
+    if (int rc = weighted_forward(d, f1, f2, g_cv, g_cu, d_a_v, d_a_u, K, s)) return rc;
+    BwdArgs a;
+    memset(&a, 0, sizeof(a));
+    a.f1 = f1; a.f2 = f2; a.a_u = a_u; a.a_v = a_v; a.g_cu = g_cu; a.g_cv = g_cv;
+    a.d1 = d_f1; a.d2 = d_f2;
+    a.B = B; a.N1 = H1 * W1; a.H2 = H2; a.W2 = W2; a.C = C; a.KT = K;
+    const int kch = W2 > 128 ? 2 : KCH;  // wide workgroups have half the registers per lane
+    for (int k0 = 0; k0 < K; k0 += kch) {
+        a.k0 = k0;
+        a.accumulate = k0 > 0;
+        const int kc = K - k0 < kch ? K - k0 : kch;
+        int rc;
+        switch (kc) {
+            case 1: rc = launch_bwd<GMODE_COMP, 1>(a, d, workspace, s); break;
+            case 2: rc = launch_bwd<GMODE_COMP, 2>(a, d, workspace, s); break;
+            case 3: rc = launch_bwd<GMODE_COMP, 3>(a, d, workspace, s); break;
+            default: rc = launch_bwd<GMODE_COMP, 4>(a, d, workspace, s); break;
+        }
+        if (rc) return rc;
+    }
+    return SEPCORR_OK;
+}
+
+}  // extern "C"

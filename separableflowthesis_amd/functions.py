@@ -1,0 +1,79 @@
+"""The three autograd Functions of the reference's libs/MemorySaver/functions/MemorySaver.py.
+
+Same class names, argument order, outputs, layouts and saved-tensor order, so that
+core/corr.py:425 (`.apply(fmap1, fmap2)`) and :448 (`.apply(fmap1, fmap2, a_u, a_v)`) work
+unchanged.  `backward` may also be called directly with an object exposing `saved_tensors`,
+as the reference's debug helpers do (scripts/test_maxavg_autograd.py:560-562).
+"""
+import torch
+from torch.autograd import Function
+
+from . import MemorySaver
+
+
+def _contig(*ts):
+    assert all(bool(t.is_contiguous()) for t in ts), "inputs must be contiguous"
+
+
+class ComputeMaxAvgFunction(Function):
+    """Max and mean of the 4D correlation volume over each displacement axis; forward only.
+
+    Mirrors functions/MemorySaver.py:6-38.
+    """
+
+    @staticmethod
+    def forward(ctx, img1_features_l0, img2_features_lk):
+        _contig(img1_features_l0, img2_features_lk)
+        with torch.cuda.device_of(img1_features_l0):
+            out_u, out_v = MemorySaver.max_avg_forward(img1_features_l0, img2_features_lk)
+        return out_u.contiguous(), out_v.contiguous()
+
+    @staticmethod
+    def backward(ctx, gradOutput_u, gradOutput_v):
+        raise NotImplementedError("max avg backward pass is not implemented: use max argmax avg")
+
+
+class ComputeMaxArgmaxAvgFunction(Function):
+    """As above, with argmax saved so that the backward pass exists (functions/MemorySaver.py:40-105)."""
+
+    @staticmethod
+    def forward(ctx, img1_features_l0, img2_features_lk):
+        _contig(img1_features_l0, img2_features_lk)
+        with torch.cuda.device_of(img1_features_l0):
+            out_u, out_v, am_u, am_v = MemorySaver.max_argmax_avg_forward(img1_features_l0, img2_features_lk)
+        ctx.save_for_backward(img1_features_l0, img2_features_lk, am_u, am_v)
+        return out_u.contiguous(), out_v.contiguous()
+
+    @staticmethod
+    def backward(ctx, grad_MaxAvg_u, grad_MaxAvg_v):
+        f1, f2, am_u, am_v = ctx.saved_tensors
+        grad_MaxAvg_u = grad_MaxAvg_u.contiguous()
+        grad_MaxAvg_v = grad_MaxAvg_v.contiguous()
+        _contig(f1, f2, am_u, am_v)
+        with torch.cuda.device_of(grad_MaxAvg_u):
+            d1, d2 = MemorySaver.max_argmax_avg_backward(f1, f2, am_u, am_v, grad_MaxAvg_u, grad_MaxAvg_v)
+        return d1.contiguous(), d2.contiguous()
+
+
+class ComputeSelfCompressionFunction(Function):
+    """Attention-weighted sums of the 4D volume (functions/MemorySaver.py:107-177), any K."""
+
+    @staticmethod
+    def forward(ctx, img1_features_l0, img2_features_lk, attention_weights_u, attention_weights_v):
+        _contig(img1_features_l0, img2_features_lk, attention_weights_u, attention_weights_v)
+        with torch.cuda.device_of(img1_features_l0):
+            cu, cv = MemorySaver.compression_forward(img1_features_l0, img2_features_lk,
+                                                     attention_weights_u, attention_weights_v)
+        ctx.save_for_backward(img1_features_l0, img2_features_lk, attention_weights_u, attention_weights_v)
+        return cu.contiguous(), cv.contiguous()
+
+    @staticmethod
+    def backward(ctx, grad_compressed_output_u, grad_compressed_output_v):
+        f1, f2, a_u, a_v = ctx.saved_tensors
+        grad_compressed_output_u = grad_compressed_output_u.contiguous()
+        grad_compressed_output_v = grad_compressed_output_v.contiguous()
+        _contig(f1, f2, a_u, a_v)
+        with torch.cuda.device_of(grad_compressed_output_u):
+            d1, d2, da_u, da_v = MemorySaver.compression_backward(
+                f1, f2, a_u, a_v, grad_compressed_output_u, grad_compressed_output_v)
+        return d1.contiguous(), d2.contiguous(), da_u.contiguous(), da_v.contiguous()
