@@ -1,0 +1,224 @@
+#!/usr/bin/env python3
+"""Benchmark of the memory-saving correlation separation on one MI355X.
+
+A step is one pass of the hot path over one synthetic batch, called through the C ABI with every
+input already resident in HBM: max/argmax/avg forward, attention-compression forward, compression
+backward, max/avg backward (the default workload, BASELINE config 4: B=2, C=256, 55x128, K'=4).
+Prints ONE JSON line.  `value` is algorithmic TFLOP/s: (contraction passes x 2*B*N1*N2*C) / time,
+with passes = 7 for forward+backward with attention; epilogue flops are not counted.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3   # 256 CU x 256 flop/clk x 2.4 GHz
+METRIC = "fused corr-separation fwd+bwd ms and MFMA TFLOP/s at B=2, C=256, 55×128"
+
+# name -> (B, H, W, K', ops).  ops: f = max/avg(+argmax) fwd, c = compression fwd, C = compression bwd, F = max/avg bwd
+WORKLOADS = {
+    "cfg1": (1, 48, 64, 0, "f"),
+    "cfg2": (4, 48, 64, 0, "fF"),
+    "cfg3": (1, 55, 128, 4, "fc"),
+    "cfg4": (2, 55, 128, 4, "fcCF"),
+    "cfg5": (1, 136, 240, 4, "fc"),
+}
+PASSES = {"f": 1, "c": 1, "C": 3, "F": 2}
+# contraction passes (units of W = 2*B*N1*N2*C flops) executed by one launch of each kernel
+KERNEL_PASSES = {"fwd_maxavg": 1, "fwd_weighted": 1, "df1_comp": 1, "df2_comp": 1, "df1_maxavg": 1, "df2_maxavg": 1}
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (see profiles/); None = not measured
+TRAFFIC_BYTES = {}
+
+
+def make_inputs(B, H, W, C, Kp, torch):
+    """Seeded CPU tensors exactly as the caller builds them (core/corr.py:419-422)."""
+    g = torch.Generator().manual_seed(1234)
+    fmap1 = torch.randn(B, C, H, W, generator=g)
+    fmap2 = torch.randn(B, C, H, W, generator=g)
+    f1 = fmap1.permute(0, 2, 3, 1).contiguous() / torch.sqrt(torch.tensor(C).float())
+    f2 = fmap2.permute(0, 2, 3, 1).contiguous()
+    grads = dict(g_u=torch.randn(B, H, W, 2, H, generator=g), g_v=torch.randn(B, H, W, 2, W, generator=g))
+    if Kp:
+        grads.update(g_cu=torch.randn(B, H, W, Kp, H, generator=g), g_cv=torch.randn(B, H, W, Kp, W, generator=g))
+    torch.manual_seed(1234)
+    att = (torch.nn.Conv3d(2, Kp, 3, padding=1), torch.nn.Conv3d(2, Kp, 3, padding=1)) if Kp else None
+    return f1, f2, grads, att
+
+
+def cpu_baseline(B, H, W, C, Kp, ops, torch, budget_s=20.0):
+    """The full-4D PyTorch path (oracle restatement of core/corr.py) timed on the host cores.
+
+    Bounded sample: batch 1 of the workload, repeated until ~budget_s of CPU time is spent.
+    """
+    from oracle import oracle as O
+    f1, f2, grads, att = make_inputs(1, H, W, C, Kp, torch)
+    backward = "C" in ops or "F" in ops
+    threads = torch.get_num_threads()
+
+    def once():
+        x1 = f1.clone().requires_grad_(backward)
+        x2 = f2.clone().requires_grad_(backward)
+        with torch.set_grad_enabled(backward):
+            s = O.corr_volume(x1, x2)
+            out_u = torch.stack((s.max(dim=4)[0], s.mean(dim=4)), dim=3)
+            out_v = torch.stack((s.max(dim=3)[0], s.mean(dim=3)), dim=3)
+            loss = (out_u * grads["g_u"]).sum() + (out_v * grads["g_v"]).sum() if backward else None
+            if Kp:
+                a_u = att[0](out_v.permute(0, 3, 4, 1, 2)).softmax(dim=2).permute(0, 3, 4, 1, 2)
+                a_v = att[1](out_u.permute(0, 3, 4, 1, 2)).softmax(dim=2).permute(0, 3, 4, 1, 2)
+                cu, cv = O.compression_from_volume(s, a_u, a_v)
+                if backward:
+                    loss = loss + (cu * grads["g_cu"]).sum() + (cv * grads["g_cv"]).sum()
+            if backward:
+                loss.backward()
+
+    once()  # warm-up (allocator, thread pool)
+    n, t0 = 0, time.perf_counter()
+    while True:
+        once()
+        n += 1
+        dt = time.perf_counter() - t0
+        if dt >= budget_s or n >= 20:
+            break
+    ms = dt / n * 1e3
+    passes = sum(PASSES[o] for o in ops)
+    flops = passes * 2.0 * 1 * (H * W) ** 2 * C
+    return {
+        "value": round(flops / (ms * 1e-3) / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+        "ms_per_step": round(ms, 1),
+        "sample": f"batch 1 of the workload (B=1, {H}x{W}, C={C}, K'={Kp}), full-4D torch path "
+                  f"{'fwd+bwd via autograd' if backward else 'fwd'}, {n} repeats after 1 warm-up, same algorithmic flop count",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="cfg4", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--profile-steps", type=int, default=5)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
+
+    import torch
+    from separableflowthesis_amd import _lib
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    B, H, W, Kp, ops = WORKLOADS[args.workload]
+    C = 256
+    N = H * W
+    f1c, f2c, gr, att = make_inputs(B, H, W, C, Kp, torch)
+    f1, f2 = f1c.to(dev), f2c.to(dev)
+    gr = {k: v.to(dev) for k, v in gr.items()}
+    E = lambda *s, dt=torch.float32: torch.empty(*s, dtype=dt, device=dev)
+    out_u, out_v = E(B, H, W, 2, H), E(B, H, W, 2, W)
+    am_u, am_v = E(B, H, W, 1, H, dt=torch.int32), E(B, H, W, 1, W, dt=torch.int32)
+    d1, d2, d1b, d2b = E(B, H, W, C), E(B, H, W, C), E(B, H, W, C), E(B, H, W, C)
+    nws = lib.sepcorr_backward_workspace_bytes(B, H, W, H, W, C)
+    ws = torch.empty(max(nws, 256), dtype=torch.uint8, device=dev)
+    dims = (B, H, W, H, W, C)
+    stream = torch.cuda.current_stream().cuda_stream
+    P = lambda t: t.data_ptr()
+
+    def op_f():
+        _lib.check(lib.sepcorr_max_argmax_avg_forward(P(f1), P(f2), P(out_u), P(out_v), P(am_u), P(am_v), *dims, stream))
+
+    op_f()
+    if Kp:
+        # attention weights as the caller produces them: Conv3d on the (max,avg) volumes, softmax over the
+        # kept axis, back to (B,H1,W1,K',L) (core/corr.py:437-446)
+        with torch.no_grad():
+            a_u = att[0].to(dev)(out_v.permute(0, 3, 4, 1, 2)).softmax(dim=2).permute(0, 3, 4, 1, 2).contiguous()
+            a_v = att[1].to(dev)(out_u.permute(0, 3, 4, 1, 2)).softmax(dim=2).permute(0, 3, 4, 1, 2).contiguous()
+        cu, cv = E(B, H, W, Kp, H), E(B, H, W, Kp, W)
+        da_u, da_v = torch.empty_like(a_u), torch.empty_like(a_v)
+
+    def op_c():
+        _lib.check(lib.sepcorr_compression_forward(P(f1), P(f2), P(a_u), P(a_v), P(cu), P(cv), *dims, Kp, stream))
+
+    def op_C():
+        _lib.check(lib.sepcorr_compression_backward(P(f1), P(f2), P(a_u), P(a_v), P(gr["g_cu"]), P(gr["g_cv"]),
+                                                    P(d1), P(d2), P(da_u), P(da_v), *dims, Kp, P(ws), nws, stream))
+
+    def op_F():
+        _lib.check(lib.sepcorr_max_argmax_avg_backward(P(f1), P(f2), P(am_u), P(am_v), P(gr["g_u"]), P(gr["g_v"]),
+                                                       P(d1b), P(d2b), *dims, P(ws), nws, stream))
+
+    table = {"f": op_f, "c": op_c, "C": op_C, "F": op_F}
+    seq = [table[o] for o in ops]
+
+    def step():
+        for fn in seq:
+            fn()
+
+    torch.cuda.reset_peak_memory_stats()
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+
+    # per-kernel durations: HIP events recorded by the library on the launch stream
+    lib.sepcorr_profile_enable(1)
+    for _ in range(max(1, args.profile_steps)):
+        step()
+    torch.cuda.synchronize()
+    cap = 4096
+    names = ctypes.create_string_buffer(1 << 16)
+    tms = (ctypes.c_float * cap)()
+    n = lib.sepcorr_profile_collect(names, len(names), tms, cap)
+    lib.sepcorr_profile_enable(0)
+    per = {}
+    for nm, t in zip(names.value.decode().split("\n")[:n], list(tms)[:n]):
+        per.setdefault(nm, []).append(t)
+    Wf = 2.0 * B * N * N * C
+    kernels = {}
+    for nm, ts in per.items():
+        avg = sum(ts) / len(ts)
+        calls = len(ts) / max(1, args.profile_steps)
+        ent = {"avg_ms": round(avg, 4), "launches_per_step": round(calls, 2)}
+        if nm in KERNEL_PASSES:
+            ent["tflops"] = round(KERNEL_PASSES[nm] * Wf / (avg * 1e-3) / 1e12, 2)
+        kernels[nm] = ent
+    dom = max((k for k in kernels if k in KERNEL_PASSES),
+              key=lambda k: kernels[k]["avg_ms"] * kernels[k]["launches_per_step"])
+    ach = kernels[dom]["tflops"]
+    passes = sum(PASSES[o] for o in ops)
+    value = passes * Wf / (ms * 1e-3) / 1e12
+
+    out = {
+        "metric": METRIC, "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: B={B}, C={C}, {H}x{W}, K'={Kp}, ops={ops} "
+                               "(f=max/argmax/avg fwd, c=compression fwd, C=compression bwd, F=max/avg bwd)",
+                   "contraction_passes": passes, "gflop_per_step": round(passes * Wf / 1e9, 2),
+                   "frac_of_fp32_mfma_peak": round(value / PEAK_FP32_MFMA_TFLOPS, 4),
+                   "peak_hbm_allocated_mib": round(torch.cuda.max_memory_allocated() / 2**20, 1),
+                   "volume_4d_never_allocated_mib": round(B * N * N * 4 / 2**20, 1)},
+        "roofline": {"bound": "mfma", "kernel": dom, "achieved": ach, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(ach / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": TRAFFIC_BYTES.get(dom)},
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(B, H, W, C, Kp, ops, torch)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

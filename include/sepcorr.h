@@ -47,6 +47,15 @@ const char *sepcorr_last_error(void);
 int sepcorr_abi_version(void);
 
 /*
+ * Measurement aid; no counterpart in the reference.  While enabled, every kernel launched by this
+ * library is bracketed by HIP events on its launch stream.  sepcorr_profile_collect() waits for the
+ * recorded kernels, writes up to `cap` durations (milliseconds, launch order) to `ms` and the kernel
+ * labels joined by '\n' to `names`, forgets them, and returns how many it wrote.
+ */
+int sepcorr_profile_enable(int on);
+int sepcorr_profile_collect(char *names, size_t names_cap, float *ms, int cap);
+
+/*
  * Replaces MemorySaver.max_avg_forward (MemorySaver_cuda.cpp:10-21 -> max_avg_cuda_forward,
  * MemorySaver_kernel_forward.cu:901-949).
  *   out_u[b,i,j,0,u] = max_v S   out_u[b,i,j,1,u] = (sum_v S) / W2      (B,H1,W1,2,H2)

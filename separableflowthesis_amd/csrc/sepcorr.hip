@@ -28,6 +28,10 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
+#include <string>
+#include <vector>
+
 #include "sepcorr.h"
 
 typedef float v16f __attribute__((ext_vector_type(16)));
@@ -641,6 +645,34 @@ int check_dims(const Dims &d, int K) {
     return SEPCORR_OK;
 }
 
+// Optional per-kernel timing: when enabled, every kernel launch is bracketed by HIP events recorded
+// on the stream it is launched on.  Off by default (zero cost: one branch per launch).
+struct ProfRec {
+    const char *name;
+    hipEvent_t e0, e1;
+};
+bool g_prof_on = false;
+std::mutex g_prof_mu;
+std::vector<ProfRec> g_prof_recs;
+
+struct ProfScope {
+    ProfRec rec;
+    hipStream_t s;
+    bool on;
+    ProfScope(const char *name, hipStream_t stream) : s(stream), on(g_prof_on) {
+        if (!on) return;
+        rec.name = name;
+        if (hipEventCreate(&rec.e0) != hipSuccess || hipEventCreate(&rec.e1) != hipSuccess) { on = false; return; }
+        (void)hipEventRecord(rec.e0, s);
+    }
+    ~ProfScope() {
+        if (!on) return;
+        (void)hipEventRecord(rec.e1, s);
+        std::lock_guard<std::mutex> lk(g_prof_mu);
+        g_prof_recs.push_back(rec);
+    }
+};
+
 int check_launch(const char *what) {
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(SEPCORR_ELAUNCH, "sepcorr: %s: %s", what, hipGetErrorString(e));
@@ -668,6 +700,7 @@ int launch_fwd(const FwdArgs &a, int B, hipStream_t s) {
     do {                                                                         \
         auto k = fwd_kernel<MODE, KC, UR, CV, MT>;                               \
         if (int rc = set_lds(k, lds)) return rc;                                 \
+        ProfScope ps(MODE == MODE_WEIGHTED ? "fwd_weighted" : "fwd_maxavg", s);  \
         hipLaunchKernelGGL(k, grid, block, lds, s, a);                           \
     } while (0)
     if (nW <= 4) {
@@ -736,7 +769,11 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s) {
         const int cblocks = (d.C + 128 * ncb - 1) / (128 * ncb);
         const dim3 grid(d.B * a.tiles_per_batch, cblocks), block(64 * nW);
         const size_t lds = (size_t)TP * (128 * ncb + 4) * sizeof(float);
-#define SEPCORR_DF1(NCB, CV, MT) hipLaunchKernelGGL((df1_kernel<GMODE, KC, NCB, CV, MT>), grid, block, lds, s, a)
+#define SEPCORR_DF1(NCB, CV, MT)                                                                   \
+    do {                                                                                           \
+        ProfScope ps(GMODE == GMODE_COMP ? "df1_comp" : "df1_maxavg", s);                          \
+        hipLaunchKernelGGL((df1_kernel<GMODE, KC, NCB, CV, MT>), grid, block, lds, s, a);          \
+    } while (0)
         if (nW > 4) { if (cvec) SEPCORR_DF1(1, true, 512); else SEPCORR_DF1(1, false, 512); }
         else if (ncb == 1) { if (cvec) SEPCORR_DF1(1, true, 256); else SEPCORR_DF1(1, false, 256); }
         else { if (cvec) SEPCORR_DF1(2, true, 256); else SEPCORR_DF1(2, false, 256); }
@@ -754,7 +791,11 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s) {
         float *d2 = a.d2;
         if (a.nsplit > 1) a.d2 = static_cast<float *>(ws);
         const dim3 grid((ntasks + 3) / 4, cblocks), block(256);
-#define SEPCORR_DF2(NCB, CV) hipLaunchKernelGGL((df2_kernel<GMODE, KC, NCB, CV>), grid, block, 0, s, a, ntasks, nvc)
+#define SEPCORR_DF2(NCB, CV)                                                                       \
+    do {                                                                                           \
+        ProfScope ps(GMODE == GMODE_COMP ? "df2_comp" : "df2_maxavg", s);                          \
+        hipLaunchKernelGGL((df2_kernel<GMODE, KC, NCB, CV>), grid, block, 0, s, a, ntasks, nvc);   \
+    } while (0)
         if (ncb == 1) { if (cvec) SEPCORR_DF2(1, true); else SEPCORR_DF2(1, false); }
         else          { if (cvec) SEPCORR_DF2(2, true); else SEPCORR_DF2(2, false); }
 #undef SEPCORR_DF2
@@ -762,6 +803,7 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s) {
         if (a.nsplit > 1) {
             const size_t n = (size_t)d.B * d.H2 * d.W2 * d.C;
             const int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+            ProfScope ps("df2_reduce_splits", s);
             hipLaunchKernelGGL(reduce_splits_kernel, dim3(blocks), dim3(256), 0, s, static_cast<const float *>(ws), d2, n,
                                a.nsplit, a.accumulate);
             if (int rc = check_launch("d_f2 split reduction")) return rc;
@@ -788,6 +830,33 @@ extern "C" {
 
 const char *sepcorr_last_error(void) { return g_err; }
 int sepcorr_abi_version(void) { return 1; }
+
+int sepcorr_profile_enable(int on) {
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    g_prof_on = on != 0;
+    return SEPCORR_OK;
+}
+
+int sepcorr_profile_collect(char *names, size_t names_cap, float *ms, int cap) {
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    std::string joined;
+    int n = 0;
+    for (const ProfRec &r : g_prof_recs) {
+        float t = 0.f;
+        (void)hipEventSynchronize(r.e1);
+        const hipError_t e = hipEventElapsedTime(&t, r.e0, r.e1);
+        (void)hipEventDestroy(r.e0);
+        (void)hipEventDestroy(r.e1);
+        if (e != hipSuccess || n >= cap) continue;
+        if (joined.size() + strlen(r.name) + 2 > names_cap) continue;
+        if (n) joined += '\n';
+        joined += r.name;
+        ms[n++] = t;
+    }
+    g_prof_recs.clear();
+    if (names && names_cap) snprintf(names, names_cap, "%s", joined.c_str());
+    return n;
+}
 
 int sepcorr_max_avg_forward(const float *f1, const float *f2, float *out_u, float *out_v, int B, int H1, int W1, int H2,
                             int W2, int C, void *stream) {
