@@ -91,6 +91,16 @@ __device__ __forceinline__ void store4(float *base, int c, int C, v4f x, bool ac
     }
 }
 
+// Raw buffer resource over `bytes` bytes at p: loads whose byte offset (voffset) is >= bytes return 0,
+// which replaces every bounds branch in the fast paths.
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, bytes, 0x00020000);
+}
+__device__ __forceinline__ v4f buf_load4(__amdgpu_buffer_rsrc_t r, unsigned byte_off) {
+    return __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 0));
+}
+
 __device__ __forceinline__ v16f mfma(float a, float b, v16f c) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
 }
@@ -112,8 +122,10 @@ struct FwdArgs {
     int tiles_per_batch;
 };
 
-template <int MODE, int KC, int UR, bool CVEC, int MAXT>
+// CMODE: 0 = any C (scalar loads), 1 = C % 4 == 0 (16-byte loads), 2 = C % 32 == 0 (branch-free fast path)
+template <int MODE, int KC, int UR, int CMODE, int MAXT>
 __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
+    constexpr bool CVEC = CMODE >= 1;
     constexpr int GJ = 2;  // 8-channel slices per prefetch group
     constexpr int NPART = (MODE == MODE_WEIGHTED) ? KC : 3;
     extern __shared__ float smem[];
@@ -303,6 +315,62 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
         if (g == NG - 1) epilogue(step);
     };
 
+    if constexpr (CMODE == 2) {
+        // Fast path.  Contraction index permuted so that a lane reads 64 contiguous bytes of its fmap2
+        // pixel per 32-channel block J: MFMA step (tq,t) of block J contracts channels 32J+4tq+t (lanes
+        // 0..31) and 32J+16+4tq+t (lanes 32..63); the f1 tile in LDS is read with the same mapping.
+        const unsigned rowbytes = (unsigned)W2 * C * 4u;
+        const unsigned nbytes = (unsigned)H2 * rowbytes;
+        const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(a.f2 + (size_t)b * H2 * W2 * C, nbytes);
+        const unsigned lane_off = vrow_ok ? ((unsigned)vrow * C + 16u * h) * 4u : nbytes;
+        const int NJB = C >> 5;
+        auto issueF = [&](int step, int J, v4f(&buf)[UR][4]) {
+#pragma unroll
+            for (int r = 0; r < UR; ++r) {
+                const unsigned off = lane_off + (unsigned)(step * UR + r) * rowbytes + (unsigned)J * 128u;
+#pragma unroll
+                for (int tq = 0; tq < 4; ++tq) buf[r][tq] = buf_load4(rsrc, off + 16u * tq);
+            }
+        };
+        auto computeF = [&](int step, int J, v4f(&buf)[UR][4]) {
+            if constexpr (MODE == MODE_WEIGHTED) {
+                if (J == 0) {
+#pragma unroll
+                    for (int r = 0; r < UR; ++r) {
+                        const int u = min(step * UR + r, H2 - 1);
+#pragma unroll
+                        for (int k = 0; k < KC; ++k) wur[r][k] = a.wu[(bp * a.KT + a.k0 + k) * H2 + u];
+                    }
+                }
+            }
+            const float *brow = f1s + pl * LS + 32 * J + 16 * h;
+#pragma unroll
+            for (int tq = 0; tq < 4; ++tq) {
+                const v4f bv = *reinterpret_cast<const v4f *>(brow + 4 * tq);
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int r = 0; r < UR; ++r) acc[r] = mfma(buf[r][tq][t], bv[t], acc[r]);
+            }
+            if (J == NJB - 1) epilogue(step);
+        };
+        const int TF = nsteps * NJB;
+        v4f bufA[UR][4], bufB[UR][4];
+        int step = 0, J = 0;
+        issueF(0, 0, bufA);
+        for (int it = 0; it < TF; it += 2) {
+            int J1 = J + 1, s1 = step;
+            if (J1 == NJB) { J1 = 0; ++s1; }
+            int J2 = J1 + 1, s2 = s1;
+            if (J2 == NJB) { J2 = 0; ++s2; }
+            if (it + 1 < TF) issueF(s1, J1, bufB);
+            computeF(step, J, bufA);
+            if (it + 2 < TF) issueF(s2, J2, bufA);
+            if (it + 1 < TF) computeF(s1, J1, bufB);
+            step = s2;
+            J = J2;
+        }
+    } else {
     v4f bufA[UR][GJ], bufB[UR][GJ];
     int step = 0, g = 0;  // position of iteration `it`
     issue(0, 0, bufA);
@@ -317,6 +385,7 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
         if (it + 1 < T) compute(s1, g1, bufB);
         step = s2;
         g = g2;
+    }
     }
 
     // store the state that was reduced over u
@@ -457,23 +526,38 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
             for (int e = 0; e < 16; ++e) acc[cb][t][e] = 0.f;
 
     const float *f2b = a.f2 + (size_t)b * H2 * W2 * C;
+    // CVEC: raw buffer loads, out-of-image columns and channels read as zero without a branch
+    const unsigned nbytes = (unsigned)H2 * W2 * C * 4u;
+    const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(f2b, nbytes);
+    unsigned coff[NCB];
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb) {
+        const int c = cb0 + 128 * cb + 4 * pl;
+        coff[cb] = c < C ? (unsigned)c * 4u : nbytes;
+    }
     auto issue = [&](int u, int g, v4f(&buf)[GS][NCB]) {
 #pragma unroll
         for (int ss = 0; ss < GS; ++ss) {
             const int v = 32 * wave + vmap(g * GS + ss, h);
             const bool ok = v < W2;
-            const float *src = f2b + ((size_t)u * W2 + (ok ? v : 0)) * C;
+            if constexpr (CVEC) {
+                const unsigned voff = ok ? ((unsigned)(u * W2 + v) * C) * 4u : nbytes;
 #pragma unroll
-            for (int cb = 0; cb < NCB; ++cb) buf[ss][cb] = load4<CVEC>(src, cb0 + 128 * cb + 4 * pl, C, ok);
+                for (int cb = 0; cb < NCB; ++cb) buf[ss][cb] = buf_load4(rsrc, voff + coff[cb]);
+            } else {
+                const float *src = f2b + ((size_t)u * W2 + (ok ? v : 0)) * C;
+#pragma unroll
+                for (int cb = 0; cb < NCB; ++cb) buf[ss][cb] = load4<false>(src, cb0 + 128 * cb + 4 * pl, C, ok);
+            }
         }
     };
 
     float G[16];
-    UW<GMODE, KC> wu_next = load_uw<GMODE, KC>(a, bp, 0, pok);
+    UW<GMODE, KC> wu_next = load_uw<GMODE, KC>(a, bp, 0, true);  // bp is clamped: always a valid pixel
     auto compute = [&](int u, int g, v4f(&buf)[GS][NCB]) {
         if (g == 0) {
             const UW<GMODE, KC> wu = wu_next;
-            if (u + 1 < H2) wu_next = load_uw<GMODE, KC>(a, bp, u + 1, pok);
+            wu_next = load_uw<GMODE, KC>(a, bp, min(u + 1, H2 - 1), true);
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int v = 32 * wave + vmap(r, h);
@@ -562,17 +646,31 @@ __global__ void __launch_bounds__(256) df2_kernel(const BwdArgs a, int ntasks, i
         VW<GMODE, KC> wv[GS];
         UW<GMODE, KC> wu[GS];
     };
+    const unsigned nbytes1 = (unsigned)max(pend, 0) * C * 4u;   // pixels >= pend read as zero
+    const __amdgpu_buffer_rsrc_t rsrc1 = make_rsrc(a.f1 + (size_t)b * N1 * C, nbytes1);
+    unsigned coff[NCB];
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb) {
+        const int c = cb0 + 128 * cb + 4 * pl;
+        coff[cb] = c < C ? (unsigned)c * 4u : nbytes1;
+    }
     auto issue = [&](int tile, int g, Buf &buf) {
 #pragma unroll
         for (int ss = 0; ss < GS; ++ss) {
             const int p = pbeg + tile * TP + 2 * (g * GS + ss) + h;
             const bool ok = p < pend;
-            const size_t bp = (size_t)b * N1 + (ok ? p : 0);
-            buf.wv[ss] = load_vw<GMODE, KC>(a, bp, vs, ok && vok);
-            buf.wu[ss] = load_uw<GMODE, KC>(a, bp, u, ok);
-            const float *src = a.f1 + bp * C;
+            const size_t bp = (size_t)b * N1 + min(p, pend - 1);   // clamped: weights of a real pixel, masked in gval
+            buf.wv[ss] = load_vw<GMODE, KC>(a, bp, vs, true);
+            buf.wu[ss] = load_uw<GMODE, KC>(a, bp, u, true);
+            if constexpr (CVEC) {
+                const unsigned poff = ok ? (unsigned)p * C * 4u : nbytes1;
 #pragma unroll
-            for (int cb = 0; cb < NCB; ++cb) buf.f[ss][cb] = load4<CVEC>(src, cb0 + 128 * cb + 4 * pl, C, ok);
+                for (int cb = 0; cb < NCB; ++cb) buf.f[ss][cb] = buf_load4(rsrc1, poff + coff[cb]);
+            } else {
+                const float *src = a.f1 + bp * C;
+#pragma unroll
+                for (int cb = 0; cb < NCB; ++cb) buf.f[ss][cb] = load4<false>(src, cb0 + 128 * cb + 4 * pl, C, ok);
+            }
         }
     };
     auto compute = [&](int tile, int g, const Buf &buf) {
@@ -695,7 +793,8 @@ int launch_fwd(const FwdArgs &a, int B, hipStream_t s) {
     constexpr int NPART = (MODE == MODE_WEIGHTED) ? KC : 3;
     const size_t lds = ((size_t)TP * (a.CP + 4) + 2 * UR * NPART * nW * 32) * sizeof(float);
     const dim3 grid(B * a.tiles_per_batch), block(64 * nW);
-    const bool cvec = (a.C % 4) == 0;
+    const size_t f2_batch_bytes = (size_t)a.H2 * a.W2 * a.C * sizeof(float);
+    const int cmode = (a.C % 32 == 0 && f2_batch_bytes <= (1u << 30)) ? 2 : (a.C % 4 == 0 ? 1 : 0);
 #define SEPCORR_FWD(CV, MT)                                                      \
     do {                                                                         \
         auto k = fwd_kernel<MODE, KC, UR, CV, MT>;                               \
@@ -704,9 +803,9 @@ int launch_fwd(const FwdArgs &a, int B, hipStream_t s) {
         hipLaunchKernelGGL(k, grid, block, lds, s, a);                           \
     } while (0)
     if (nW <= 4) {
-        if (cvec) SEPCORR_FWD(true, 256); else SEPCORR_FWD(false, 256);
+        if (cmode == 2) SEPCORR_FWD(2, 256); else if (cmode == 1) SEPCORR_FWD(1, 256); else SEPCORR_FWD(0, 256);
     } else {
-        if (cvec) SEPCORR_FWD(true, 512); else SEPCORR_FWD(false, 512);
+        if (cmode == 2) SEPCORR_FWD(2, 512); else if (cmode == 1) SEPCORR_FWD(1, 512); else SEPCORR_FWD(0, 512);
     }
 #undef SEPCORR_FWD
     return check_launch("forward kernel");
@@ -760,7 +859,8 @@ int df2_nsplit(const Dims &d) {
 
 template <int GMODE, int KC>
 int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s) {
-    const bool cvec = (d.C % 4) == 0;
+    const size_t big = (size_t)1 << 30;
+    const bool cvec = (d.C % 4) == 0 && (size_t)d.H2 * d.W2 * d.C * 4 <= big && (size_t)d.H1 * d.W1 * d.C * 4 <= big;
     const int nW = (d.W2 + 31) / 32;
     a.tiles_per_batch = (a.N1 + TP - 1) / TP;
     {
