@@ -711,6 +711,191 @@ __global__ void __launch_bounds__(256) df2_kernel(const BwdArgs a, int ntasks, i
     }
 }
 
+
+// Tiled d_f2: workgroup = 4 waves = 4 consecutive fmap2 rows u of one 32-column chunk; it sweeps the
+// pixels p of its split in tiles of 32.  Per tile the f1 rows (A operand) and every weight indexed by
+// (p, v) are DMA'd straight into LDS (buffer_load ... lds, double buffered, one barrier per tile) and
+// shared by the four rows; the weights indexed by (p, u) are wave private.  G^T is synthesised from
+// LDS into the B operand.  Requires C % 4 == 0 and W2 % 4 == 0.
+__device__ __forceinline__ void dma16(__amdgpu_buffer_rsrc_t r, float *lds_chunk, unsigned voff) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void *)lds_chunk, 16, voff, 0, 0, 0);
+}
+constexpr unsigned DMA_OOB = 0x80000000u;   // above every buffer size used here: reads as zero
+
+template <int GMODE, int KC, int NCB>
+__global__ void __launch_bounds__(256) df2_tiled_kernel(const BwdArgs a, int nvc, int nug) {
+    constexpr int NWV = 4;
+    constexpr int NV = GMODE == GMODE_COMP ? 2 * KC : 3;
+    constexpr int NUP = (NV + 3) & ~3;
+    constexpr int CB = 128 * NCB;
+    extern __shared__ float smem[];
+    float *F1s = smem;                         // [2][32][CB]
+    float *VWs = F1s + 2 * 32 * CB;            // [2][NV][32 p][32 v]
+    float *UWs = VWs + 2 * NV * 1024;          // [NWV][2][32 p][NUP]
+    const int tid = threadIdx.x, lane = tid & 63, pl = lane & 31, h = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int N1 = a.N1, H2 = a.H2, W2 = a.W2, C = a.C;
+    int task = blockIdx.x;
+    const int vc = task % nvc; task /= nvc;
+    const int ug = task % nug; task /= nug;
+    const int split = task % a.nsplit;
+    const int b = task / a.nsplit;
+    const int cb0 = blockIdx.y * CB;
+    const int u_raw = ug * NWV + wave;
+    const int u = min(u_raw, H2 - 1);
+    const int v0 = 32 * vc, v = v0 + pl;
+    const bool vok = v < W2;
+    const int pbeg = split * a.tiles_per_split * TP;
+    const int pend = min(N1, pbeg + a.tiles_per_split * TP);
+    const int ntiles = (pend - pbeg + TP - 1) / TP;
+    const float inv_h2 = 1.f / (float)H2, inv_w2 = 1.f / (float)W2;
+
+    v16f acc[NCB][4];
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[cb][t][e] = 0.f;
+
+    if (ntiles > 0) {
+        // buffer resources end at pixel `pend`: rows of later pixels read as zero
+        const unsigned up = (unsigned)pend;
+        const __amdgpu_buffer_rsrc_t rs_f1 = make_rsrc(a.f1 + (size_t)b * N1 * C, up * C * 4u);
+        __amdgpu_buffer_rsrc_t rs_va, rs_vb;   // the two (p,v)-indexed tensors
+        unsigned pstride_v;                    // floats per pixel in them
+        if constexpr (GMODE == GMODE_COMP) {
+            pstride_v = (unsigned)a.KT * W2;
+            rs_va = make_rsrc(a.a_u + (size_t)b * N1 * pstride_v, up * pstride_v * 4u);
+            rs_vb = make_rsrc(a.g_cv + (size_t)b * N1 * pstride_v, up * pstride_v * 4u);
+        } else {
+            pstride_v = 2u * W2;
+            rs_va = make_rsrc(a.g_v + (size_t)b * N1 * pstride_v, up * pstride_v * 4u);
+            rs_vb = make_rsrc(a.am_v + (size_t)b * N1 * W2, up * W2 * 4u);
+        }
+        // lane-constant parts of the DMA offsets
+        const int frow = (lane * 4) / CB, fcol = (lane * 4) % CB;        // within a 256-float chunk of the f1 tile
+        const unsigned fcoff = (cb0 + fcol < C) ? (unsigned)(cb0 + fcol) * 4u : DMA_OOB;
+        const int vrow = 8 * wave + (lane >> 3);                          // pixel row of this lane in the weight tile
+        const unsigned vcol = (unsigned)(v0 + 4 * (lane & 7)) * 4u;
+
+        auto issue_tile = [&](int tile, int bi) {
+            const int pt0 = pbeg + tile * TP;
+            float *fdst = F1s + bi * 32 * CB;
+            constexpr int FCH = CB / 32;   // 256-float chunks per wave
+#pragma unroll
+            for (int i = 0; i < FCH; ++i) {
+                const int ch = wave * FCH + i;
+                const int row = ch * (256 / CB) + frow;
+                dma16(rs_f1, fdst + ch * 256, (unsigned)(pt0 + row) * C * 4u + fcoff);
+            }
+            float *vdst = VWs + bi * NV * 1024;
+            const unsigned p = (unsigned)(pt0 + vrow);
+#pragma unroll
+            for (int kk = 0; kk < NV; ++kk) {
+                float *dst = vdst + kk * 1024 + wave * 256;
+                if constexpr (GMODE == GMODE_COMP) {
+                    const unsigned off = (p * pstride_v + (unsigned)(a.k0 + (kk % KC)) * W2) * 4u + vcol;
+                    dma16(kk < KC ? rs_va : rs_vb, dst, off);
+                } else {
+                    if (kk < 2) dma16(rs_va, dst, (p * pstride_v + (unsigned)kk * W2) * 4u + vcol);
+                    else dma16(rs_vb, dst, p * W2 * 4u + vcol);
+                }
+            }
+        };
+        // (p,u)-indexed weights of this wave's row: lane pl fetches pixel pt0+pl (both halves the same)
+        auto load_uw_tile = [&](int tile, float(&r)[NUP]) {
+            const int p = min(pbeg + tile * TP + pl, pend - 1);
+            const size_t bp = (size_t)b * N1 + p;
+#pragma unroll
+            for (int i = 0; i < NUP; ++i) r[i] = 0.f;
+            if constexpr (GMODE == GMODE_COMP) {
+#pragma unroll
+                for (int k = 0; k < KC; ++k) {
+                    const size_t o = (bp * a.KT + a.k0 + k) * H2 + u;
+                    r[k] = a.a_v[o];
+                    r[KC + k] = a.g_cu[o];
+                }
+            } else {
+                r[0] = a.g_u[(bp * 2 + 0) * H2 + u];
+                r[1] = a.g_u[(bp * 2 + 1) * H2 + u];
+                r[2] = __int_as_float(a.am_u[bp * H2 + u]);
+            }
+        };
+        auto store_uw_tile = [&](int bi, const float(&r)[NUP]) {
+            float *dst = UWs + ((wave * 2 + bi) * 32 + pl) * NUP;
+#pragma unroll
+            for (int i = 0; i < NUP; i += 4) {
+                const v4f x = {r[i], r[i + 1], r[i + 2], r[i + 3]};
+                *reinterpret_cast<v4f *>(dst + i) = x;
+            }
+        };
+
+        float uwr[NUP];
+        issue_tile(0, 0);
+        load_uw_tile(0, uwr);
+        store_uw_tile(0, uwr);
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's DMA has landed
+        __syncthreads();
+
+        for (int tile = 0; tile < ntiles; ++tile) {
+            const int bi = tile & 1;
+            const bool more = tile + 1 < ntiles;
+            if (more) {
+                issue_tile(tile + 1, bi ^ 1);
+                load_uw_tile(tile + 1, uwr);
+            }
+            const float *fs = F1s + bi * 32 * CB;
+            const float *vs = VWs + bi * NV * 1024;
+            const float *us = UWs + (wave * 2 + bi) * 32 * NUP;
+            const int pt0 = pbeg + tile * TP;
+#pragma unroll
+            for (int s = 0; s < 16; ++s) {
+                const int row = 2 * s + h;
+                float uw[NUP], vw[NV];
+#pragma unroll
+                for (int i = 0; i < NUP; i += 4) {
+                    const v4f x = *reinterpret_cast<const v4f *>(us + row * NUP + i);
+                    uw[i] = x[0]; uw[i + 1] = x[1]; uw[i + 2] = x[2]; uw[i + 3] = x[3];
+                }
+#pragma unroll
+                for (int kk = 0; kk < NV; ++kk) vw[kk] = vs[kk * 1024 + row * 32 + pl];
+                float G = 0.f;
+                if constexpr (GMODE == GMODE_COMP) {
+#pragma unroll
+                    for (int k = 0; k < KC; ++k) G += vw[k] * uw[KC + k] + uw[k] * vw[KC + k];
+                } else {
+                    G = uw[1] * inv_w2 + vw[1] * inv_h2;
+                    if (__float_as_int(uw[2]) == v) G += uw[0];
+                    if (__float_as_int(vw[2]) == u) G += vw[0];
+                }
+                if (!(pt0 + row < pend && vok)) G = 0.f;
+#pragma unroll
+                for (int cb = 0; cb < NCB; ++cb) {
+                    const v4f fa = *reinterpret_cast<const v4f *>(fs + row * CB + 128 * cb + 4 * pl);
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) acc[cb][t] = mfma(fa[t], G, acc[cb][t]);
+                }
+            }
+            if (more) store_uw_tile(bi ^ 1, uwr);
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+            __syncthreads();
+        }
+    }
+
+    if (vok && u_raw < H2) {
+        float *dst = a.d2 + ((size_t)split * a.B + b) * H2 * W2 * C + ((size_t)u * W2 + v) * C;
+        const bool accum = a.accumulate != 0 && a.nsplit == 1;
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const v4f x = {acc[cb][0][r], acc[cb][1][r], acc[cb][2][r], acc[cb][3][r]};
+                store4<true>(dst, cb0 + 128 * cb + 4 * vmap(r, h), C, x, accum);
+            }
+    }
+}
+
 // out[i] (+)= sum_s part[s*n + i], in split order.
 __global__ void __launch_bounds__(256) reduce_splits_kernel(const float *part, float *out, size_t n, int nsplit,
                                                             int accumulate) {
@@ -847,14 +1032,39 @@ int weighted_forward(const Dims &d, const float *f1, const float *f2, const floa
     return SEPCORR_OK;
 }
 
-int df2_nsplit(const Dims &d) {
-    const long tasks = (long)d.B * d.H2 * ((d.W2 + 31) / 32);
-    const int tiles = (d.H1 * d.W1 + TP - 1) / TP;
-    long n = (2048 + tasks - 1) / tasks;  // aim at two waves per SIMD on 256 CUs
-    if (n > 8) n = 8;
-    if (n > tiles) n = tiles;
-    if (n < 1) n = 1;
-    return (int)n;
+struct Df2Plan {
+    bool tiled;
+    int nsplit;
+};
+
+// How d_f2 is computed for these sizes.  The p range is split over workgroups so that the grid fills
+// the 256 CUs evenly; each split writes a partial d_f2 to scratch, summed in split order afterwards.
+Df2Plan df2_plan(const Dims &d) {
+    Df2Plan pl;
+    const size_t big = (size_t)1 << 30;
+    const size_t n1 = (size_t)d.H1 * d.W1;
+    pl.tiled = d.C % 4 == 0 && d.W2 % 4 == 0 && n1 * d.C * 4 <= big && n1 * MAX_K * d.W2 * 4 <= big;
+    const int tiles = (int)((n1 + TP - 1) / TP);
+    const int nvc = (d.W2 + 31) / 32;
+    const int cblocks = (d.C + 255) / 256;
+    if (pl.tiled) {
+        const long base = (long)d.B * ((d.H2 + 3) / 4) * nvc * (d.C <= 128 ? 1 : cblocks);
+        double best = -1.0;
+        pl.nsplit = 1;
+        for (int ns = 1; ns <= 16 && ns <= tiles; ++ns) {
+            const long wgs = base * ns;
+            const double eff = (double)wgs / (double)(((wgs + 255) / 256) * 256) - 0.004 * ns;
+            if (eff > best) { best = eff; pl.nsplit = ns; }
+        }
+    } else {
+        const long tasks = (long)d.B * d.H2 * nvc;
+        long n = (2048 + tasks - 1) / tasks;  // aim at two waves per SIMD on 256 CUs
+        if (n > 8) n = 8;
+        if (n > tiles) n = tiles;
+        if (n < 1) n = 1;
+        pl.nsplit = (int)n;
+    }
+    return pl;
 }
 
 template <int GMODE, int KC>
@@ -884,12 +1094,29 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s) {
         const int ncb = d.C <= 128 ? 1 : 2;
         const int cblocks = (d.C + 128 * ncb - 1) / (128 * ncb);
         const int tiles = a.tiles_per_batch;
-        a.nsplit = df2_nsplit(d);
+        const Df2Plan plan = df2_plan(d);
+        a.nsplit = plan.nsplit;
         a.tiles_per_split = (tiles + a.nsplit - 1) / a.nsplit;
         const int nvc = nW;
-        const int ntasks = d.B * a.nsplit * d.H2 * nvc;
         float *d2 = a.d2;
         if (a.nsplit > 1) a.d2 = static_cast<float *>(ws);
+        if (plan.tiled) {
+            constexpr int NV = GMODE == GMODE_COMP ? 2 * KC : 3;
+            constexpr int NUP = (NV + 3) & ~3;
+            const int nug = (d.H2 + 3) / 4;
+            const dim3 grid(d.B * a.nsplit * nug * nvc, cblocks), block(256);
+            const size_t lds = ((size_t)2 * 32 * 128 * ncb + 2 * NV * 1024 + 4 * 2 * 32 * NUP) * sizeof(float);
+#define SEPCORR_DF2T(NCB)                                                                          \
+    do {                                                                                           \
+        auto k = df2_tiled_kernel<GMODE, KC, NCB>;                                                 \
+        if (int rc = set_lds(k, lds)) return rc;                                                   \
+        ProfScope ps(GMODE == GMODE_COMP ? "df2_comp" : "df2_maxavg", s);                          \
+        hipLaunchKernelGGL(k, grid, block, lds, s, a, nvc, nug);                                   \
+    } while (0)
+            if (ncb == 1) SEPCORR_DF2T(1); else SEPCORR_DF2T(2);
+#undef SEPCORR_DF2T
+        } else {
+        const int ntasks = d.B * a.nsplit * d.H2 * nvc;
         const dim3 grid((ntasks + 3) / 4, cblocks), block(256);
 #define SEPCORR_DF2(NCB, CV)                                                                       \
     do {                                                                                           \
@@ -899,6 +1126,7 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s) {
         if (ncb == 1) { if (cvec) SEPCORR_DF2(1, true); else SEPCORR_DF2(1, false); }
         else          { if (cvec) SEPCORR_DF2(2, true); else SEPCORR_DF2(2, false); }
 #undef SEPCORR_DF2
+        }
         if (int rc = check_launch("d_f2 kernel")) return rc;
         if (a.nsplit > 1) {
             const size_t n = (size_t)d.B * d.H2 * d.W2 * d.C;
@@ -989,7 +1217,7 @@ int sepcorr_compression_forward(const float *f1, const float *f2, const float *a
 size_t sepcorr_backward_workspace_bytes(int B, int H1, int W1, int H2, int W2, int C) {
     if (B < 1 || H1 < 1 || W1 < 1 || H2 < 1 || W2 < 1 || C < 1) return 0;
     const Dims d = {B, H1, W1, H2, W2, C};
-    const int ns = df2_nsplit(d);
+    const int ns = df2_plan(d).nsplit;
     return ns > 1 ? (size_t)ns * B * H2 * W2 * C * sizeof(float) : 0;
 }
 

@@ -20,6 +20,9 @@ SHAPES = [
     (1, 6, 250, 3, 125, 36),    # 8-wave f1 side irrelevant; W2=125 -> 4 waves, ragged
     (1, 4, 256, 4, 256, 32),    # widest supported row: 8 waves
     (2, 24, 32, 24, 32, 256),
+    (2, 9, 20, 9, 20, 64),      # W2 % 4 == 0 and C % 4 == 0: tiled d_f2 path, row count not a multiple of 4
+    (1, 30, 36, 15, 20, 100),   # tiled d_f2 with a ragged 128-channel block and pooled fmap2
+    (1, 16, 48, 16, 48, 300),   # two channel blocks, the second ragged
 ]
 
 
@@ -81,7 +84,7 @@ def test_forward_ties_lowest_index(device):
     assert torch.all(au == 0) and torch.all(av == 0) and torch.all(ou == 4) and torch.all(ov == 4)
 
 
-@pytest.mark.parametrize("shape", SHAPES[:8])
+@pytest.mark.parametrize("shape", SHAPES)
 def test_max_argmax_avg_backward(device, shape):
     B, H1, W1, H2, W2, C = shape
     f1, f2, g = op_inputs(B, H1, W1, H2, W2, C, seed=21)
@@ -124,7 +127,7 @@ def test_backward_out_of_range_argmax_is_harmless(device):
     assert torch.all(d1 == 0) and torch.all(d2 == 0)
 
 
-@pytest.mark.parametrize("shape", SHAPES[1:7])
+@pytest.mark.parametrize("shape", SHAPES[1:7] + SHAPES[9:])
 @pytest.mark.parametrize("K", [1, 2, 4, 5])
 def test_compression_backward(device, shape, K):
     B, H1, W1, H2, W2, C = shape
