@@ -324,6 +324,9 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
         const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(a.f2 + (size_t)b * H2 * W2 * C, nbytes);
         const unsigned lane_off = vrow_ok ? ((unsigned)vrow * C + 16u * h) * 4u : nbytes;
         const int NJB = C >> 5;
+        v16f acc_alt;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc_alt[e] = 0.f;
         auto issueF = [&](int step, int J, v4f(&buf)[UR][4]) {
 #pragma unroll
             for (int r = 0; r < UR; ++r) {
@@ -348,11 +351,26 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
             for (int tq = 0; tq < 4; ++tq) {
                 const v4f bv = *reinterpret_cast<const v4f *>(brow + 4 * tq);
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
+                for (int t = 0; t < 4; ++t) {
+                    if constexpr (UR == 1) {
+                        // one row per step: split the contraction over two accumulators so that
+                        // consecutive MFMAs are independent
+                        if (t & 1) acc_alt = mfma(buf[0][tq][t], bv[t], acc_alt);
+                        else acc[0] = mfma(buf[0][tq][t], bv[t], acc[0]);
+                    } else {
 #pragma unroll
-                    for (int r = 0; r < UR; ++r) acc[r] = mfma(buf[r][tq][t], bv[t], acc[r]);
+                        for (int r = 0; r < UR; ++r) acc[r] = mfma(buf[r][tq][t], bv[t], acc[r]);
+                    }
+                }
             }
-            if (J == NJB - 1) epilogue(step);
+            if (J == NJB - 1) {
+                if constexpr (UR == 1) {
+                    acc[0] += acc_alt;
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) acc_alt[e] = 0.f;
+                }
+                epilogue(step);
+            }
         };
         const int TF = nsteps * NJB;
         v4f bufA[UR][4], bufB[UR][4];
@@ -987,11 +1005,9 @@ int launch_fwd(const FwdArgs &a, int B, hipStream_t s) {
         ProfScope ps(MODE == MODE_WEIGHTED ? "fwd_weighted" : "fwd_maxavg", s);  \
         hipLaunchKernelGGL(k, grid, block, lds, s, a);                           \
     } while (0)
-    if (nW <= 4) {
-        if (cmode == 2) SEPCORR_FWD(2, 256); else if (cmode == 1) SEPCORR_FWD(1, 256); else SEPCORR_FWD(0, 256);
-    } else {
-        if (cmode == 2) SEPCORR_FWD(2, 512); else if (cmode == 1) SEPCORR_FWD(1, 512); else SEPCORR_FWD(0, 512);
-    }
+    // Always built for two waves per SIMD (256 registers): the accumulators then stay in ordinary
+    // VGPRs, where the epilogue reads them without accumulator-register copies.
+    if (cmode == 2) SEPCORR_FWD(2, 512); else if (cmode == 1) SEPCORR_FWD(1, 512); else SEPCORR_FWD(0, 512);
 #undef SEPCORR_FWD
     return check_launch("forward kernel");
 }
