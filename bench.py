@@ -31,8 +31,11 @@ WORKLOADS = {
 PASSES = {"f": 1, "c": 1, "C": 3, "F": 2}
 # contraction passes (units of W = 2*B*N1*N2*C flops) executed by one launch of each kernel
 KERNEL_PASSES = {"fwd_maxavg": 1, "fwd_weighted": 1, "df1_comp": 1, "df2_comp": 1, "df1_maxavg": 1, "df2_maxavg": 1}
-# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (see profiles/); None = not measured
-TRAFFIC_BYTES = {}
+# HBM bytes per launch at cfg4 from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by the factors a
+# 256 MiB device copy gives in the same run (profiles/cfg4_fwd_bwd_kernels.txt); None = not measured
+_MIB = 2 ** 20
+TRAFFIC_BYTES_CFG4 = {"fwd_maxavg": 266.4 * _MIB, "fwd_weighted": 546.9 * _MIB, "df1_comp": 546.7 * _MIB,
+                      "df2_comp": 611.1 * _MIB, "df1_maxavg": 211.6 * _MIB, "df2_maxavg": 384.8 * _MIB}
 
 
 def make_inputs(B, H, W, C, Kp, torch):
@@ -104,6 +107,8 @@ def main():
     ap.add_argument("--workload", default="cfg4", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--profile-steps", type=int, default=5)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run three 256 MiB device copies (known traffic) for scaling rocprofv3 FETCH_SIZE/WRITE_SIZE")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
@@ -163,6 +168,14 @@ def main():
         for fn in seq:
             fn()
 
+    if args.calibrate_copy:
+        src = torch.empty(64 * 2**20, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     torch.cuda.reset_peak_memory_stats()
     for _ in range(args.warmup):
         step()
@@ -212,7 +225,7 @@ def main():
                    "peak_hbm_allocated_mib": round(torch.cuda.max_memory_allocated() / 2**20, 1),
                    "volume_4d_never_allocated_mib": round(B * N * N * 4 / 2**20, 1)},
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": ach, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(ach / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": TRAFFIC_BYTES.get(dom)},
+                     "frac": round(ach / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": TRAFFIC_BYTES_CFG4.get(dom) if args.workload == "cfg4" else None},
         "kernels": kernels,
     }
     if not args.no_cpu_baseline:

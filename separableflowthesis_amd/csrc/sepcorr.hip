@@ -94,8 +94,14 @@ __device__ __forceinline__ void store4(float *base, int c, int C, v4f x, bool ac
 // Raw buffer resource over `bytes` bytes at p: loads whose byte offset (voffset) is >= bytes return 0,
 // which replaces every bounds branch in the fast paths.
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+// The descriptor must live in scalar registers; the pointer and size are wave-uniform by construction,
+// and saying so explicitly keeps the compiler from emitting a per-lane search loop around every load.
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p, unsigned bytes) {
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, bytes, 0x00020000);
+    const uint64_t addr = reinterpret_cast<uint64_t>(p);
+    const uint64_t lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)addr);
+    const uint64_t hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(addr >> 32));
+    const int n = __builtin_amdgcn_readfirstlane((int)bytes);
+    return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void *>((hi << 32) | lo), 0, n, 0x00020000);
 }
 __device__ __forceinline__ v4f buf_load4(__amdgpu_buffer_rsrc_t r, unsigned byte_off) {
     return __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 0));
