@@ -128,7 +128,8 @@ struct FwdArgs {
     int tiles_per_batch;
 };
 
-// CMODE: 0 = any C (scalar loads), 1 = C % 4 == 0 (16-byte loads), 2 = C % 32 == 0 (branch-free fast path)
+// CMODE: 0 = any C (scalar loads), 1 = C % 4 == 0 (16-byte loads), 2 = C % 32 == 0 (branch-free fast path),
+//        3 = C == 256 (fast path with the channel loop unrolled: every load offset is an immediate)
 template <int MODE, int KC, int UR, int CMODE, int MAXT>
 __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
     constexpr bool CVEC = CMODE >= 1;
@@ -163,6 +164,7 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
     const float *f2lane = a.f2 + ((size_t)b * H2 * W2 + (vrow_ok ? vrow : 0)) * C;
     const size_t rowstride = (size_t)W2 * C;
 
+    const bool ragged = 32 * wave + 32 > W2;
     unsigned vmask = 0;  // bit r: accumulator register r maps to a real column
 #pragma unroll
     for (int r = 0; r < 16; ++r)
@@ -237,12 +239,22 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
                 } else {
                     float m = -INFINITY, s = 0.f;
                     int mi = 0x7fffffff;
+                    if (ragged) {   // wave-uniform: only the last column chunk of a row can be partial
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            const float xm = ((vmask >> r) & 1u) ? acc[ru][r] : -INFINITY;
+                            if (xm > m) { m = xm; mi = 32 * wave + vmap(r, h); }
+                        }
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            const float xm = acc[ru][r];
+                            if (xm > m) { m = xm; mi = 32 * wave + vmap(r, h); }
+                        }
+                    }
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         const float x = acc[ru][r];
-                        const bool ok = (vmask >> r) & 1u;
-                        const float xm = ok ? x : -INFINITY;
-                        if (xm > m) { m = xm; mi = 32 * wave + vmap(r, h); }
                         s += x;  // columns outside the image hold exact zeros
                         if (x > vmax[r]) { vmax[r] = x; vidx[r] = u; }
                         vsum[r] += x;
@@ -321,7 +333,7 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
         if (g == NG - 1) epilogue(step);
     };
 
-    if constexpr (CMODE == 2) {
+    if constexpr (CMODE >= 2) {
         // Fast path.  Contraction index permuted so that a lane reads 64 contiguous bytes of its fmap2
         // pixel per 32-channel block J: MFMA step (tq,t) of block J contracts channels 32J+4tq+t (lanes
         // 0..31) and 32J+16+4tq+t (lanes 32..63); the f1 tile in LDS is read with the same mapping.
@@ -329,7 +341,13 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
         const unsigned nbytes = (unsigned)H2 * rowbytes;
         const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(a.f2 + (size_t)b * H2 * W2 * C, nbytes);
         const unsigned lane_off = vrow_ok ? ((unsigned)vrow * C + 16u * h) * 4u : nbytes;
-        const int NJB = C >> 5;
+        const int NJB = (CMODE == 3) ? 8 : (C >> 5);
+        constexpr bool BPIPE = !(MODE == MODE_WEIGHTED && KC >= 3);   // needs 16 more registers
+        v4f bcur[4];
+        if constexpr (BPIPE) {
+#pragma unroll
+            for (int tq = 0; tq < 4; ++tq) bcur[tq] = *reinterpret_cast<const v4f *>(f1s + pl * LS + 16 * h + 4 * tq);
+        }
         v16f acc_alt;
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc_alt[e] = 0.f;
@@ -338,8 +356,14 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
             for (int r = 0; r < UR; ++r) {
                 const unsigned off = lane_off + (unsigned)(step * UR + r) * rowbytes + (unsigned)J * 128u;
 #pragma unroll
-                for (int tq = 0; tq < 4; ++tq) buf[r][tq] = buf_load4(rsrc, off + 16u * tq);
+                for (int tq = 0; tq < 4; ++tq) {
+#if defined(SEPCORR_EXP) && SEPCORR_EXP == 2
+                    if (step == 0 && J == 0)   // experiment: load only once
+#endif
+                    buf[r][tq] = buf_load4(rsrc, off + 16u * tq);
+                }
             }
+            __builtin_amdgcn_sched_barrier(0);   // keep the loads here: a full block ahead of their use
         };
         auto computeF = [&](int step, int J, v4f(&buf)[UR][4]) {
             if constexpr (MODE == MODE_WEIGHTED) {
@@ -352,10 +376,7 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
                     }
                 }
             }
-            const float *brow = f1s + pl * LS + 32 * J + 16 * h;
-#pragma unroll
-            for (int tq = 0; tq < 4; ++tq) {
-                const v4f bv = *reinterpret_cast<const v4f *>(brow + 4 * tq);
+            auto mfma_tq = [&](int tq, const v4f &bv) {
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
                     if constexpr (UR == 1) {
@@ -368,8 +389,36 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
                         for (int r = 0; r < UR; ++r) acc[r] = mfma(buf[r][tq][t], bv[t], acc[r]);
                     }
                 }
+            };
+            if constexpr (BPIPE) {
+                // the f1 operand of the next block is fetched from LDS in the middle of this block
+                mfma_tq(0, bcur[0]);
+                mfma_tq(1, bcur[1]);
+                __builtin_amdgcn_sched_barrier(0);
+                v4f bnext[4];
+                const float *nrow = f1s + pl * LS + 32 * (J + 1 == NJB ? 0 : J + 1) + 16 * h;
+#pragma unroll
+                for (int tq = 0; tq < 4; ++tq) bnext[tq] = *reinterpret_cast<const v4f *>(nrow + 4 * tq);
+                __builtin_amdgcn_sched_barrier(0);
+                mfma_tq(2, bcur[2]);
+                mfma_tq(3, bcur[3]);
+#pragma unroll
+                for (int tq = 0; tq < 4; ++tq) bcur[tq] = bnext[tq];
+            } else {
+                const float *brow = f1s + pl * LS + 32 * J + 16 * h;
+                v4f bv[4];
+#pragma unroll
+                for (int tq = 0; tq < 4; ++tq) bv[tq] = *reinterpret_cast<const v4f *>(brow + 4 * tq);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int tq = 0; tq < 4; ++tq) mfma_tq(tq, bv[tq]);
             }
+            __builtin_amdgcn_sched_barrier(0);
+#if defined(SEPCORR_EXP) && SEPCORR_EXP == 1
+            if (J == NJB - 1 && step == nsteps - 1) {   // experiment: epilogue only once
+#else
             if (J == NJB - 1) {
+#endif
                 if constexpr (UR == 1) {
                     acc[0] += acc_alt;
 #pragma unroll
@@ -378,21 +427,44 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
                 epilogue(step);
             }
         };
-        const int TF = nsteps * NJB;
-        v4f bufA[UR][4], bufB[UR][4];
-        int step = 0, J = 0;
-        issueF(0, 0, bufA);
-        for (int it = 0; it < TF; it += 2) {
-            int J1 = J + 1, s1 = step;
-            if (J1 == NJB) { J1 = 0; ++s1; }
-            int J2 = J1 + 1, s2 = s1;
-            if (J2 == NJB) { J2 = 0; ++s2; }
-            if (it + 1 < TF) issueF(s1, J1, bufB);
-            computeF(step, J, bufA);
-            if (it + 2 < TF) issueF(s2, J2, bufA);
-            if (it + 1 < TF) computeF(s1, J1, bufB);
-            step = s2;
-            J = J2;
+        // Ring of NB register buffers: the loads of block i+NB-1 are issued before the MFMAs of block i,
+        // so NB-1 blocks of MFMA work cover the latency of an L2 miss.
+        if constexpr (CMODE == 3) {
+            constexpr int NJT = 8;
+            constexpr int NB = (UR == 1) ? 4 : 2;   // divides NJT: ring slots are static across steps
+            v4f ring[NB][UR][4];
+#pragma unroll
+            for (int k = 0; k < NB - 1; ++k) issueF(0, k, ring[k]);
+            for (int step = 0; step < nsteps; ++step) {
+#pragma unroll
+                for (int J = 0; J < NJT; ++J) {
+                    constexpr int AHEAD = NB - 1;
+                    if (J + AHEAD < NJT) issueF(step, J + AHEAD, ring[(J + AHEAD) % NB]);
+                    else if (step + 1 < nsteps) issueF(step + 1, J + AHEAD - NJT, ring[(J + AHEAD) % NB]);
+                    computeF(step, J, ring[J % NB]);
+                }
+            }
+        } else {
+            constexpr int NB = (UR == 1) ? 4 : 3;
+            const int TF = nsteps * NJB;
+            v4f ring[NB][UR][4];
+            int is = 0, iJ = 0;   // position of the next block to issue
+            int cs = 0, cJ = 0;   // position of the next block to compute
+            auto advance = [&](int &st, int &jj) { if (++jj == NJB) { jj = 0; ++st; } };
+#pragma unroll
+            for (int k = 0; k < NB - 1; ++k) {
+                if (k < TF) { issueF(is, iJ, ring[k]); advance(is, iJ); }
+            }
+            for (int it = 0; it < TF; it += NB) {
+#pragma unroll
+                for (int k = 0; k < NB; ++k) {
+                    if (it + k < TF) {
+                        if (it + k + NB - 1 < TF) { issueF(is, iJ, ring[(k + NB - 1) % NB]); advance(is, iJ); }
+                        computeF(cs, cJ, ring[k]);
+                        advance(cs, cJ);
+                    }
+                }
+            }
         }
     } else {
     v4f bufA[UR][GJ], bufB[UR][GJ];
@@ -1003,7 +1075,7 @@ int launch_fwd(const FwdArgs &a, int B, hipStream_t s) {
     const size_t lds = ((size_t)TP * (a.CP + 4) + 2 * UR * NPART * nW * 32) * sizeof(float);
     const dim3 grid(B * a.tiles_per_batch), block(64 * nW);
     const size_t f2_batch_bytes = (size_t)a.H2 * a.W2 * a.C * sizeof(float);
-    const int cmode = (a.C % 32 == 0 && f2_batch_bytes <= (1u << 30)) ? 2 : (a.C % 4 == 0 ? 1 : 0);
+    const int cmode = (a.C % 32 == 0 && f2_batch_bytes <= (1u << 30)) ? (a.C == 256 ? 3 : 2) : (a.C % 4 == 0 ? 1 : 0);
 #define SEPCORR_FWD(CV, MT)                                                      \
     do {                                                                         \
         auto k = fwd_kernel<MODE, KC, UR, CV, MT>;                               \
@@ -1013,7 +1085,8 @@ int launch_fwd(const FwdArgs &a, int B, hipStream_t s) {
     } while (0)
     // Always built for two waves per SIMD (256 registers): the accumulators then stay in ordinary
     // VGPRs, where the epilogue reads them without accumulator-register copies.
-    if (cmode == 2) SEPCORR_FWD(2, 512); else if (cmode == 1) SEPCORR_FWD(1, 512); else SEPCORR_FWD(0, 512);
+    if (cmode == 3) SEPCORR_FWD(3, 512); else if (cmode == 2) SEPCORR_FWD(2, 512);
+    else if (cmode == 1) SEPCORR_FWD(1, 512); else SEPCORR_FWD(0, 512);
 #undef SEPCORR_FWD
     return check_launch("forward kernel");
 }
