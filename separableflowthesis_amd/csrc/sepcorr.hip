@@ -668,17 +668,24 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
                 for (int t = 0; t < 4; ++t) acc[cb][t] = mfma(buf[ss][cb][t], G[g * GS + ss], acc[cb][t]);
     };
 
-    // G is indexed with a value known after unrolling only if the group index is static: unroll rows by hand
-    v4f bufA[GS][NCB], bufB[GS][NCB];
-    issue(0, 0, bufA);
+    // Ring of NB register buffers (NB divides the NG groups of a row, so slots are static): the loads of
+    // group i+NB-1 are issued, and pinned there, before the MFMAs of group i.
+    constexpr int NB = 4;
+    v4f ring[NB][GS][NCB];
+#pragma unroll
+    for (int k = 0; k < NB - 1; ++k) {
+        issue(0, k, ring[k]);
+        __builtin_amdgcn_sched_barrier(0);
+    }
     for (int u = 0; u < H2; ++u) {
 #pragma unroll
-        for (int g = 0; g < NG; g += 2) {
-            issue(u, g + 1, bufB);
-            compute(u, g, bufA);
-            if (g + 2 < NG) issue(u, g + 2, bufA);
-            else if (u + 1 < H2) issue(u + 1, 0, bufA);
-            compute(u, g + 1, bufB);
+        for (int g = 0; g < NG; ++g) {
+            constexpr int AHEAD = NB - 1;
+            if (g + AHEAD < NG) issue(u, g + AHEAD, ring[(g + AHEAD) % NB]);
+            else if (u + 1 < H2) issue(u + 1, g + AHEAD - NG, ring[(g + AHEAD) % NB]);
+            __builtin_amdgcn_sched_barrier(0);
+            compute(u, g, ring[g % NB]);
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 
@@ -945,33 +952,54 @@ __global__ void __launch_bounds__(256) df2_tiled_kernel(const BwdArgs a, int nvc
             const float *vs = VWs + bi * NV * 1024;
             const float *us = UWs + (wave * 2 + bi) * 32 * NUP;
             const int pt0 = pbeg + tile * TP;
-#pragma unroll
-            for (int s = 0; s < 16; ++s) {
-                const int row = 2 * s + h;
+            // Software pipeline over the 16 MFMA steps of the tile: the LDS operands of step s+1 are
+            // fetched before the MFMAs of step s and its G is computed between them, so the matrix
+            // pipe does not wait for LDS latency or for the G arithmetic.
+            struct StepOps {
                 float uw[NUP], vw[NV];
+                v4f fa[NCB];
+            };
+            auto lds_fetch = [&](int s, StepOps &o) {
+                const int row = 2 * s + h;
 #pragma unroll
                 for (int i = 0; i < NUP; i += 4) {
                     const v4f x = *reinterpret_cast<const v4f *>(us + row * NUP + i);
-                    uw[i] = x[0]; uw[i + 1] = x[1]; uw[i + 2] = x[2]; uw[i + 3] = x[3];
+                    o.uw[i] = x[0]; o.uw[i + 1] = x[1]; o.uw[i + 2] = x[2]; o.uw[i + 3] = x[3];
                 }
 #pragma unroll
-                for (int kk = 0; kk < NV; ++kk) vw[kk] = vs[kk * 1024 + row * 32 + pl];
+                for (int kk = 0; kk < NV; ++kk) o.vw[kk] = vs[kk * 1024 + row * 32 + pl];
+#pragma unroll
+                for (int cb = 0; cb < NCB; ++cb) o.fa[cb] = *reinterpret_cast<const v4f *>(fs + row * CB + 128 * cb + 4 * pl);
+            };
+            auto g_of = [&](int s, const StepOps &o) {
                 float G = 0.f;
                 if constexpr (GMODE == GMODE_COMP) {
 #pragma unroll
-                    for (int k = 0; k < KC; ++k) G += vw[k] * uw[KC + k] + uw[k] * vw[KC + k];
+                    for (int k = 0; k < KC; ++k) G += o.vw[k] * o.uw[KC + k] + o.uw[k] * o.vw[KC + k];
                 } else {
-                    G = uw[1] * inv_w2 + vw[1] * inv_h2;
-                    if (__float_as_int(uw[2]) == v) G += uw[0];
-                    if (__float_as_int(vw[2]) == u) G += vw[0];
+                    G = o.uw[1] * inv_w2 + o.vw[1] * inv_h2;
+                    if (__float_as_int(o.uw[2]) == v) G += o.uw[0];
+                    if (__float_as_int(o.vw[2]) == u) G += o.vw[0];
                 }
-                if (!(pt0 + row < pend && vok)) G = 0.f;
+                // No mask needed: pixels at or beyond `pend` have all-zero f1 rows and (p,v) weights (DMA
+                // bounds), so whatever finite G they get multiplies zeros; columns beyond W2 are not stored.
+                return G;
+            };
+            StepOps cur, nxt;
+            lds_fetch(0, cur);
+            float Gc = g_of(0, cur), Gn = 0.f;
 #pragma unroll
-                for (int cb = 0; cb < NCB; ++cb) {
-                    const v4f fa = *reinterpret_cast<const v4f *>(fs + row * CB + 128 * cb + 4 * pl);
+            for (int s = 0; s < 16; ++s) {
+                if (s + 1 < 16) lds_fetch(s + 1, nxt);
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) acc[cb][t] = mfma(fa[t], G, acc[cb][t]);
-                }
+                for (int t = 0; t < 4; ++t) acc[0][t] = mfma(cur.fa[0][t], Gc, acc[0][t]);
+                if (s + 1 < 16) Gn = g_of(s + 1, nxt);
+#pragma unroll
+                for (int cb = 1; cb < NCB; ++cb)
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) acc[cb][t] = mfma(cur.fa[cb][t], Gc, acc[cb][t]);
+                cur = nxt;
+                Gc = Gn;
             }
             if (more) store_uw_tile(bi ^ 1, uwr);
             __builtin_amdgcn_s_waitcnt(0x0F70);
