@@ -126,6 +126,7 @@ struct FwdArgs {
     int N1, H2, W2, C, CP;
     int KT, k0;        // total weight channels and first channel of this launch
     int tiles_per_batch;
+    int stage;         // collect the rows of out_u in LDS and store them coalesced at the end
 };
 
 // CMODE: 0 = any C (scalar loads), 1 = C % 4 == 0 (16-byte loads), 2 = C % 32 == 0 (branch-free fast path),
@@ -144,6 +145,9 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
     const int LS = a.CP + 4;
     float *f1s = smem;
     float *part = smem + TP * LS;
+    constexpr int NCHO = (MODE == MODE_WEIGHTED) ? KC : 2;            // out_u channels of this launch
+    float *ostage = part + 2 * UR * NPART * (blockDim.x >> 6) * 32;   // [32 p][NCHO][H2] when a.stage
+    int *ostage_am = reinterpret_cast<int *>(ostage + TP * NCHO * a.H2);   // [32 p][H2], MODE_ARGMAX
 
     {   // stage the f1 tile [TP][CP] (zero padded) into LDS
         const int c4n = a.CP >> 2;
@@ -282,7 +286,8 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
                 if (u < H2 && p0 + p < N1) {
                     float s = 0.f;
                     for (int w = 0; w < nW; ++w) s += pb[((ru * NPART + k) * nW + w) * 32 + p];
-                    a.out_u[(((size_t)b * N1 + p0 + p) * a.KT + a.k0 + k) * H2 + u] = s;
+                    if (a.stage) ostage[(p * NCHO + k) * H2 + u] = s;
+                    else a.out_u[(((size_t)b * N1 + p0 + p) * a.KT + a.k0 + k) * H2 + u] = s;
                 }
             }
         } else {
@@ -298,10 +303,16 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
                         if (m2 > m) { m = m2; mi = __float_as_int(pb[((ru * NPART + 1) * nW + w) * 32 + p]); }
                         s += pb[((ru * NPART + 2) * nW + w) * 32 + p];
                     }
-                    const size_t o = ((size_t)b * N1 + p0 + p);
-                    a.out_u[(o * 2 + 0) * H2 + u] = m;
-                    a.out_u[(o * 2 + 1) * H2 + u] = s / (float)W2;
-                    if constexpr (MODE == MODE_ARGMAX) a.am_u[o * H2 + u] = mi;
+                    if (a.stage) {
+                        ostage[(p * 2 + 0) * H2 + u] = m;
+                        ostage[(p * 2 + 1) * H2 + u] = s / (float)W2;
+                        if constexpr (MODE == MODE_ARGMAX) ostage_am[p * H2 + u] = mi;
+                    } else {
+                        const size_t o = ((size_t)b * N1 + p0 + p);
+                        a.out_u[(o * 2 + 0) * H2 + u] = m;
+                        a.out_u[(o * 2 + 1) * H2 + u] = s / (float)W2;
+                        if constexpr (MODE == MODE_ARGMAX) a.am_u[o * H2 + u] = mi;
+                    }
                 }
             }
         }
@@ -482,6 +493,23 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
         step = s2;
         g = g2;
     }
+    }
+
+    // flush the staged out_u rows: per pixel a contiguous run of NCHO*H2 floats
+    if (a.stage) {
+        __syncthreads();
+        const int runlen = NCHO * H2;
+        const int cht = (MODE == MODE_WEIGHTED) ? a.KT : 2, ch0 = (MODE == MODE_WEIGHTED) ? a.k0 : 0;
+        for (int idx = tid; idx < TP * runlen; idx += blockDim.x) {
+            const int p = idx / runlen, o = idx - p * runlen;
+            if (p0 + p < N1) a.out_u[(((size_t)b * N1 + p0 + p) * cht + ch0) * H2 + o] = ostage[idx];
+        }
+        if constexpr (MODE == MODE_ARGMAX) {
+            for (int idx = tid; idx < TP * H2; idx += blockDim.x) {
+                const int p = idx / H2;
+                if (p0 + p < N1) a.am_u[((size_t)b * N1 + p0) * H2 + idx] = ostage_am[idx];
+            }
+        }
     }
 
     // store the state that was reduced over u
@@ -1097,10 +1125,16 @@ int set_lds(KernelT kernel, size_t bytes) {
 }
 
 template <int MODE, int KC, int UR>
-int launch_fwd(const FwdArgs &a, int B, hipStream_t s) {
+int launch_fwd(FwdArgs a, int B, hipStream_t s) {
     const int nW = (a.W2 + 31) / 32;
     constexpr int NPART = (MODE == MODE_WEIGHTED) ? KC : 3;
-    const size_t lds = ((size_t)TP * (a.CP + 4) + 2 * UR * NPART * nW * 32) * sizeof(float);
+    size_t lds = ((size_t)TP * (a.CP + 4) + 2 * UR * NPART * nW * 32) * sizeof(float);
+    {   // stage out_u in LDS when two workgroups still fit a CU's 160 KB
+        constexpr int NCHO = (MODE == MODE_WEIGHTED) ? KC : 2;
+        const size_t extra = (size_t)TP * (NCHO + (MODE == MODE_ARGMAX ? 1 : 0)) * a.H2 * sizeof(float);
+        a.stage = lds + extra <= 80 * 1024;
+        if (a.stage) lds += extra;
+    }
     const dim3 grid(B * a.tiles_per_batch), block(64 * nW);
     const size_t f2_batch_bytes = (size_t)a.H2 * a.W2 * a.C * sizeof(float);
     const int cmode = (a.C % 32 == 0 && f2_batch_bytes <= (1u << 30)) ? (a.C == 256 ? 3 : 2) : (a.C % 4 == 0 ? 1 : 0);
