@@ -126,19 +126,26 @@ struct FwdArgs {
     int N1, H2, W2, C, CP;
     int KT, k0;        // total weight channels and first channel of this launch
     int tiles_per_batch;
+    int nvc;           // column chunks of 32 per fmap2 row = ceil(W2 / 32)
     int stage;         // collect the rows of out_u in LDS and store them coalesced at the end
 };
 
 // CMODE: 0 = any C (scalar loads), 1 = C % 4 == 0 (16-byte loads), 2 = C % 32 == 0 (branch-free fast path),
 //        3 = C == 256 (fast path with the channel loop unrolled: every load offset is an immediate)
-template <int MODE, int KC, int UR, int CMODE, int MAXT>
-__global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
+// RG: row groups enabled (narrow rows); without it NUG == 1 is a compile-time constant.
+template <int MODE, int KC, int UR, int CMODE, bool RG>
+__global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     constexpr bool CVEC = CMODE >= 1;
     constexpr int GJ = 2;  // 8-channel slices per prefetch group
     constexpr int NPART = (MODE == MODE_WEIGHTED) ? KC : 3;
     extern __shared__ float smem[];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, pl = lane & 31, h = lane >> 5;
     const int nW = blockDim.x >> 6;
+    // Waves form a grid: nvc column chunks x NUG row groups.  Wave (vcw, ug) owns columns [32 vcw, 32 vcw + 32)
+    // and the steps ug, ug + NUG, ... (narrow fmap2 levels have few column chunks; row groups keep the
+    // workgroup at 4 or 8 waves).  NUG == 1 for rows of 97 or more columns.
+    const int nvc = RG ? a.nvc : nW, NUG = RG ? nW / nvc : 1;
+    const int vcw = RG ? wave % nvc : wave, ug = RG ? wave / nvc : 0;
     const int b = blockIdx.x / a.tiles_per_batch;
     const int p0 = (blockIdx.x % a.tiles_per_batch) * TP;
     const int N1 = a.N1, H2 = a.H2, W2 = a.W2, C = a.C;
@@ -163,16 +170,16 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
     const int pix = p0 + pl;           // this lane's image-1 pixel
     const bool pok = pix < N1;
     const size_t bp = (size_t)b * N1 + (pok ? pix : 0);
-    const int vrow = 32 * wave + pl;   // the fmap2 column this lane feeds to the A operand
+    const int vrow = 32 * vcw + pl;   // the fmap2 column this lane feeds to the A operand
     const bool vrow_ok = vrow < W2;
     const float *f2lane = a.f2 + ((size_t)b * H2 * W2 + (vrow_ok ? vrow : 0)) * C;
     const size_t rowstride = (size_t)W2 * C;
 
-    const bool ragged = 32 * wave + 32 > W2;
+    const bool ragged = 32 * vcw + 32 > W2;
     unsigned vmask = 0;  // bit r: accumulator register r maps to a real column
 #pragma unroll
     for (int r = 0; r < 16; ++r)
-        if (32 * wave + vmap(r, h) < W2) vmask |= 1u << r;
+        if (32 * vcw + vmap(r, h) < W2) vmask |= 1u << r;
 
     // running state over u, accumulator layout
     float vmax[16], vsum[16];
@@ -183,7 +190,7 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
         for (int k = 0; k < KC; ++k)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int v = 32 * wave + vmap(r, h);
+                const int v = 32 * vcw + vmap(r, h);
                 rv[k][r] = 0.f;
                 wvr[k][r] = (pok && v < W2) ? a.wv[(bp * a.KT + a.k0 + k) * W2 + v] : 0.f;
             }
@@ -198,7 +205,7 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
 
     const int NJ = a.CP >> 3;
     const int NG = (NJ + GJ - 1) / GJ;
-    const int nsteps = (H2 + UR - 1) / UR;
+    const int nsteps = ((H2 + UR - 1) / UR + NUG - 1) / NUG;   // steps per wave; rows past H2 are skipped
     const int T = nsteps * NG;
 
     v16f acc[UR];
@@ -212,7 +219,7 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
     auto issue = [&](int step, int g, v4f(&buf)[UR][GJ]) {
 #pragma unroll
         for (int r = 0; r < UR; ++r) {
-            const int u = step * UR + r;
+            const int u = (step * NUG + ug) * UR + r;
 #pragma unroll
             for (int jj = 0; jj < GJ; ++jj) {
                 const int j = g * GJ + jj;
@@ -226,7 +233,7 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
         float *pb = part + (step & 1) * (UR * NPART * nW * 32);
 #pragma unroll
         for (int ru = 0; ru < UR; ++ru) {
-            const int u = step * UR + ru;
+            const int u = (step * NUG + ug) * UR + ru;
             if (u < H2) {
                 if constexpr (MODE == MODE_WEIGHTED) {
 #pragma unroll
@@ -247,13 +254,13 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
 #pragma unroll
                         for (int r = 0; r < 16; ++r) {
                             const float xm = ((vmask >> r) & 1u) ? acc[ru][r] : -INFINITY;
-                            if (xm > m) { m = xm; mi = 32 * wave + vmap(r, h); }
+                            if (xm > m) { m = xm; mi = 32 * vcw + vmap(r, h); }
                         }
                     } else {
 #pragma unroll
                         for (int r = 0; r < 16; ++r) {
                             const float xm = acc[ru][r];
-                            if (xm > m) { m = xm; mi = 32 * wave + vmap(r, h); }
+                            if (xm > m) { m = xm; mi = 32 * vcw + vmap(r, h); }
                         }
                     }
 #pragma unroll
@@ -280,25 +287,26 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
         __syncthreads();
         // combine the per-wave partials in wave order and store the finished rows
         if constexpr (MODE == MODE_WEIGHTED) {
-            for (int idx = tid; idx < UR * KC * 32; idx += blockDim.x) {
-                const int p = idx & 31, k = (idx >> 5) % KC, ru = idx / (32 * KC);
-                const int u = step * UR + ru;
+            for (int idx = tid; idx < NUG * UR * KC * 32; idx += blockDim.x) {
+                const int p = idx & 31, k = (idx >> 5) % KC, ru = (idx / (32 * KC)) % UR, g2 = idx / (32 * KC * UR);
+                const int u = (step * NUG + g2) * UR + ru;
                 if (u < H2 && p0 + p < N1) {
                     float s = 0.f;
-                    for (int w = 0; w < nW; ++w) s += pb[((ru * NPART + k) * nW + w) * 32 + p];
+                    for (int w = g2 * nvc; w < (g2 + 1) * nvc; ++w) s += pb[((ru * NPART + k) * nW + w) * 32 + p];
                     if (a.stage) ostage[(p * NCHO + k) * H2 + u] = s;
                     else a.out_u[(((size_t)b * N1 + p0 + p) * a.KT + a.k0 + k) * H2 + u] = s;
                 }
             }
         } else {
-            for (int idx = tid; idx < UR * 32; idx += blockDim.x) {
-                const int p = idx & 31, ru = idx >> 5;
-                const int u = step * UR + ru;
+            for (int idx = tid; idx < NUG * UR * 32; idx += blockDim.x) {
+                const int p = idx & 31, ru = (idx >> 5) % UR, g2 = idx / (32 * UR);
+                const int u = (step * NUG + g2) * UR + ru;
                 if (u < H2 && p0 + p < N1) {
-                    float m = pb[((ru * NPART + 0) * nW + 0) * 32 + p];
-                    int mi = __float_as_int(pb[((ru * NPART + 1) * nW + 0) * 32 + p]);
-                    float s = pb[((ru * NPART + 2) * nW + 0) * 32 + p];
-                    for (int w = 1; w < nW; ++w) {
+                    const int w0 = g2 * nvc;
+                    float m = pb[((ru * NPART + 0) * nW + w0) * 32 + p];
+                    int mi = __float_as_int(pb[((ru * NPART + 1) * nW + w0) * 32 + p]);
+                    float s = pb[((ru * NPART + 2) * nW + w0) * 32 + p];
+                    for (int w = w0 + 1; w < w0 + nvc; ++w) {
                         const float m2 = pb[((ru * NPART + 0) * nW + w) * 32 + p];
                         if (m2 > m) { m = m2; mi = __float_as_int(pb[((ru * NPART + 1) * nW + w) * 32 + p]); }
                         s += pb[((ru * NPART + 2) * nW + w) * 32 + p];
@@ -323,7 +331,7 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
             if (g == 0) {
 #pragma unroll
                 for (int r = 0; r < UR; ++r) {
-                    const int u = step * UR + r;
+                    const int u = (step * NUG + ug) * UR + r;
 #pragma unroll
                     for (int k = 0; k < KC; ++k)
                         wur[r][k] = (pok && u < H2) ? a.wu[(bp * a.KT + a.k0 + k) * H2 + u] : 0.f;
@@ -365,7 +373,7 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
         auto issueF = [&](int step, int J, v4f(&buf)[UR][4]) {
 #pragma unroll
             for (int r = 0; r < UR; ++r) {
-                const unsigned off = lane_off + (unsigned)(step * UR + r) * rowbytes + (unsigned)J * 128u;
+                const unsigned off = lane_off + (unsigned)((step * NUG + ug) * UR + r) * rowbytes + (unsigned)J * 128u;
 #pragma unroll
                 for (int tq = 0; tq < 4; ++tq) {
 #if defined(SEPCORR_EXP) && SEPCORR_EXP == 2
@@ -381,7 +389,7 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
                 if (J == 0) {
 #pragma unroll
                     for (int r = 0; r < UR; ++r) {
-                        const int u = min(step * UR + r, H2 - 1);
+                        const int u = min((step * NUG + ug) * UR + r, H2 - 1);
 #pragma unroll
                         for (int k = 0; k < KC; ++k) wur[r][k] = a.wu[(bp * a.KT + a.k0 + k) * H2 + u];
                     }
@@ -512,11 +520,49 @@ __global__ void __launch_bounds__(MAXT) fwd_kernel(const FwdArgs a) {
         }
     }
 
+    // merge the running state of the row groups into group 0, one group at a time, through the LDS
+    // region of the f1 tile (no longer needed).  Equal maxima keep the smaller row index.
+    if (NUG > 1) {
+        constexpr int NQ = (MODE == MODE_WEIGHTED) ? KC : 3;
+        float *mst = smem + vcw * (NQ * 16 * 64);   // [vcw][quantity][r][lane]
+        for (int g2 = 1; g2 < NUG; ++g2) {
+            __syncthreads();
+            if (ug == g2) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    if constexpr (MODE == MODE_WEIGHTED) {
+#pragma unroll
+                        for (int k = 0; k < KC; ++k) mst[(k * 16 + r) * 64 + lane] = rv[k][r];
+                    } else {
+                        mst[(0 * 16 + r) * 64 + lane] = vmax[r];
+                        mst[(1 * 16 + r) * 64 + lane] = __int_as_float(vidx[r]);
+                        mst[(2 * 16 + r) * 64 + lane] = vsum[r];
+                    }
+                }
+            }
+            __syncthreads();
+            if (ug == 0) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    if constexpr (MODE == MODE_WEIGHTED) {
+#pragma unroll
+                        for (int k = 0; k < KC; ++k) rv[k][r] += mst[(k * 16 + r) * 64 + lane];
+                    } else {
+                        const float m2 = mst[(0 * 16 + r) * 64 + lane];
+                        const int i2 = __float_as_int(mst[(1 * 16 + r) * 64 + lane]);
+                        if (m2 > vmax[r] || (m2 == vmax[r] && i2 < vidx[r])) { vmax[r] = m2; vidx[r] = i2; }
+                        vsum[r] += mst[(2 * 16 + r) * 64 + lane];
+                    }
+                }
+            }
+        }
+    }
+
     // store the state that was reduced over u
-    if (pok) {
+    if (pok && ug == 0) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const int v = 32 * wave + vmap(r, h);
+            const int v = 32 * vcw + vmap(r, h);
             if (v < W2) {
                 if constexpr (MODE == MODE_WEIGHTED) {
 #pragma unroll
@@ -546,6 +592,7 @@ struct BwdArgs {
     float *d2;                       // (B,N2,C) or scratch [nsplit][B,N2,C]
     int B, N1, H2, W2, C;
     int KT, k0;
+    int nvc;                         // df1: column chunks of 32 per fmap2 row
     int tiles_per_batch;             // df1: p tiles per batch
     int nsplit, tiles_per_split;     // df2: split of the p range
     int accumulate;                  // add to the destination instead of overwriting
@@ -626,6 +673,9 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
     extern __shared__ float smem[];  // [TP][RS] cross-wave sum
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, pl = lane & 31, h = lane >> 5;
     const int nW = blockDim.x >> 6;
+    // wave (vcw, ug): columns [32 vcw, 32 vcw + 32), rows ug, ug + NUG, ... (see fwd_kernel)
+    const int nvc = a.nvc, NUG = nW / nvc;
+    const int vcw = wave % nvc, ug = wave / nvc;
     const int b = blockIdx.x / a.tiles_per_batch;
     const int p0 = (blockIdx.x % a.tiles_per_batch) * TP;
     const int cb0 = blockIdx.y * CB;
@@ -637,7 +687,7 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
     VW<GMODE, KC> wv[16];
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-        const int v = 32 * wave + vmap(r, h);
+        const int v = 32 * vcw + vmap(r, h);
         wv[r] = load_vw<GMODE, KC>(a, bp, v < W2 ? v : 0, pok && v < W2);
     }
 
@@ -662,7 +712,7 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
     auto issue = [&](int u, int g, v4f(&buf)[GS][NCB]) {
 #pragma unroll
         for (int ss = 0; ss < GS; ++ss) {
-            const int v = 32 * wave + vmap(g * GS + ss, h);
+            const int v = 32 * vcw + vmap(g * GS + ss, h);
             const bool ok = v < W2;
             if constexpr (CVEC) {
                 const unsigned voff = ok ? ((unsigned)(u * W2 + v) * C) * 4u : nbytes;
@@ -677,14 +727,14 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
     };
 
     float G[16];
-    UW<GMODE, KC> wu_next = load_uw<GMODE, KC>(a, bp, 0, true);  // bp is clamped: always a valid pixel
+    UW<GMODE, KC> wu_next = load_uw<GMODE, KC>(a, bp, min(ug, H2 - 1), true);  // bp is clamped: always a valid pixel
     auto compute = [&](int u, int g, v4f(&buf)[GS][NCB]) {
         if (g == 0) {
             const UW<GMODE, KC> wu = wu_next;
-            wu_next = load_uw<GMODE, KC>(a, bp, min(u + 1, H2 - 1), true);
+            wu_next = load_uw<GMODE, KC>(a, bp, min(u + NUG, H2 - 1), true);
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int v = 32 * wave + vmap(r, h);
+                const int v = 32 * vcw + vmap(r, h);
                 G[r] = gval<GMODE, KC>(wv[r], wu, u, v, pok && v < W2);
             }
         }
@@ -702,15 +752,15 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
     v4f ring[NB][GS][NCB];
 #pragma unroll
     for (int k = 0; k < NB - 1; ++k) {
-        issue(0, k, ring[k]);
+        issue(min(ug, H2 - 1), k, ring[k]);
         __builtin_amdgcn_sched_barrier(0);
     }
-    for (int u = 0; u < H2; ++u) {
+    for (int u = ug; u < H2; u += NUG) {
 #pragma unroll
         for (int g = 0; g < NG; ++g) {
             constexpr int AHEAD = NB - 1;
             if (g + AHEAD < NG) issue(u, g + AHEAD, ring[(g + AHEAD) % NB]);
-            else if (u + 1 < H2) issue(u + 1, g + AHEAD - NG, ring[(g + AHEAD) % NB]);
+            else if (u + NUG < H2) issue(u + NUG, g + AHEAD - NG, ring[(g + AHEAD) % NB]);
             __builtin_amdgcn_sched_barrier(0);
             compute(u, g, ring[g % NB]);
             __builtin_amdgcn_sched_barrier(0);
@@ -1124,9 +1174,27 @@ int set_lds(KernelT kernel, size_t bytes) {
     return SEPCORR_OK;
 }
 
+// Waves per workgroup of the p-owner kernels: nvc column chunks x NUG row groups.
+struct WaveGrid {
+    int nvc, nug;
+};
+WaveGrid wave_grid(int B, int tiles_per_batch, int W2, int H2) {
+    WaveGrid g;
+    g.nvc = (W2 + 31) / 32;
+    g.nug = 1;
+    if (g.nvc <= 2) {
+        g.nug = 4 / g.nvc;                                        // 4 waves
+        if ((long)B * tiles_per_batch * 4 < 1536) g.nug *= 2;     // small problem: 8 waves fill more SIMDs
+        while (g.nug > 1 && g.nug > H2) g.nug /= 2;
+    }
+    return g;
+}
+
 template <int MODE, int KC, int UR>
 int launch_fwd(FwdArgs a, int B, hipStream_t s) {
-    const int nW = (a.W2 + 31) / 32;
+    const WaveGrid wg = wave_grid(B, a.tiles_per_batch, a.W2, a.H2);
+    a.nvc = wg.nvc;
+    const int nW = wg.nvc * wg.nug;
     constexpr int NPART = (MODE == MODE_WEIGHTED) ? KC : 3;
     size_t lds = ((size_t)TP * (a.CP + 4) + 2 * UR * NPART * nW * 32) * sizeof(float);
     {   // stage out_u in LDS when two workgroups still fit a CU's 160 KB
@@ -1134,21 +1202,29 @@ int launch_fwd(FwdArgs a, int B, hipStream_t s) {
         const size_t extra = (size_t)TP * (NCHO + (MODE == MODE_ARGMAX ? 1 : 0)) * a.H2 * sizeof(float);
         a.stage = lds + extra <= 80 * 1024;
         if (a.stage) lds += extra;
+        // the final merge of the row groups reuses LDS from offset 0
+        const size_t merge = wg.nug > 1 ? (size_t)wg.nvc * NPART * 16 * 64 * sizeof(float) : 0;
+        if (lds < merge) lds = merge;
     }
     const dim3 grid(B * a.tiles_per_batch), block(64 * nW);
     const size_t f2_batch_bytes = (size_t)a.H2 * a.W2 * a.C * sizeof(float);
     const int cmode = (a.C % 32 == 0 && f2_batch_bytes <= (1u << 30)) ? (a.C == 256 ? 3 : 2) : (a.C % 4 == 0 ? 1 : 0);
-#define SEPCORR_FWD(CV, MT)                                                      \
+#define SEPCORR_FWD(CV, RGV)                                                      \
     do {                                                                         \
-        auto k = fwd_kernel<MODE, KC, UR, CV, MT>;                               \
+        auto k = fwd_kernel<MODE, KC, UR, CV, RGV>;                              \
         if (int rc = set_lds(k, lds)) return rc;                                 \
         ProfScope ps(MODE == MODE_WEIGHTED ? "fwd_weighted" : "fwd_maxavg", s);  \
         hipLaunchKernelGGL(k, grid, block, lds, s, a);                           \
     } while (0)
     // Always built for two waves per SIMD (256 registers): the accumulators then stay in ordinary
     // VGPRs, where the epilogue reads them without accumulator-register copies.
-    if (cmode == 3) SEPCORR_FWD(3, 512); else if (cmode == 2) SEPCORR_FWD(2, 512);
-    else if (cmode == 1) SEPCORR_FWD(1, 512); else SEPCORR_FWD(0, 512);
+    if (wg.nug > 1) {
+        if (cmode == 3) SEPCORR_FWD(3, true); else if (cmode == 2) SEPCORR_FWD(2, true);
+        else if (cmode == 1) SEPCORR_FWD(1, true); else SEPCORR_FWD(0, true);
+    } else {
+        if (cmode == 3) SEPCORR_FWD(3, false); else if (cmode == 2) SEPCORR_FWD(2, false);
+        else if (cmode == 1) SEPCORR_FWD(1, false); else SEPCORR_FWD(0, false);
+    }
 #undef SEPCORR_FWD
     return check_launch("forward kernel");
 }
@@ -1228,9 +1304,13 @@ template <int GMODE, int KC>
 int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s) {
     const size_t big = (size_t)1 << 30;
     const bool cvec = (d.C % 4) == 0 && (size_t)d.H2 * d.W2 * d.C * 4 <= big && (size_t)d.H1 * d.W1 * d.C * 4 <= big;
-    const int nW = (d.W2 + 31) / 32;
     a.tiles_per_batch = (a.N1 + TP - 1) / TP;
+    const int nvc_all = (d.W2 + 31) / 32;
     {
+        WaveGrid wg = wave_grid(d.B, a.tiles_per_batch, d.W2, d.H2);
+        if (wg.nvc * wg.nug > 4) wg.nug = 4 / wg.nvc > 0 ? 4 / wg.nvc : 1;   // d_f1 runs one wave per SIMD
+        a.nvc = wg.nvc;
+        const int nW = wg.nvc * wg.nug;
         // more than 4 waves share the register file two to a SIMD: halve the channel block
         const int ncb = (d.C <= 128 || nW > 4) ? 1 : 2;
         const int cblocks = (d.C + 128 * ncb - 1) / (128 * ncb);
@@ -1254,7 +1334,7 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s) {
         const Df2Plan plan = df2_plan(d);
         a.nsplit = plan.nsplit;
         a.tiles_per_split = (tiles + a.nsplit - 1) / a.nsplit;
-        const int nvc = nW;
+        const int nvc = nvc_all;
         float *d2 = a.d2;
         if (a.nsplit > 1) a.d2 = static_cast<float *>(ws);
         if (plan.tiled) {

@@ -23,6 +23,7 @@ SHAPES = [
     (2, 9, 20, 9, 20, 64),      # W2 % 4 == 0 and C % 4 == 0: tiled d_f2 path, row count not a multiple of 4
     (1, 30, 36, 15, 20, 100),   # tiled d_f2 with a ragged 128-channel block and pooled fmap2
     (1, 16, 48, 16, 48, 300),   # two channel blocks, the second ragged
+    (8, 32, 48, 16, 24, 32),    # narrow rows, many workgroups: 1 column chunk x 4 row groups
 ]
 
 
