@@ -726,24 +726,42 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
         }
     };
 
-    float G[16];
-    UW<GMODE, KC> wu_next = load_uw<GMODE, KC>(a, bp, min(ug, H2 - 1), true);  // bp is clamped: always a valid pixel
-    auto compute = [&](int u, int g, v4f(&buf)[GS][NCB]) {
-        if (g == 0) {
-            const UW<GMODE, KC> wu = wu_next;
-            wu_next = load_uw<GMODE, KC>(a, bp, min(u + NUG, H2 - 1), true);
+    // G of the current row lives in G[]; G of this wave's next row (u + NUG) is computed two values per
+    // MFMA group, between the group's MFMAs, so the arithmetic runs in the shadow of the matrix pipe.
+    float G[16], Gn[16];
+    UW<GMODE, KC> wu_n = load_uw<GMODE, KC>(a, bp, min(ug, H2 - 1), true);   // bp is clamped: always a valid pixel
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int v = 32 * vcw + vmap(r, h);
-                G[r] = gval<GMODE, KC>(wv[r], wu, u, v, pok && v < W2);
-            }
+    for (int r = 0; r < 16; ++r) {
+        const int v = 32 * vcw + vmap(r, h);
+        G[r] = gval<GMODE, KC>(wv[r], wu_n, ug, v, pok && v < W2);
+    }
+    UW<GMODE, KC> wu_next = load_uw<GMODE, KC>(a, bp, min(ug + NUG, H2 - 1), true);
+    auto compute = [&](int u, int g, v4f(&buf)[GS][NCB]) {
+        static_assert(GS == 2, "two G values are produced per group");
+        if (g == 0) {
+            wu_n = wu_next;                                                       // weights of row u + NUG
+            wu_next = load_uw<GMODE, KC>(a, bp, min(u + 2 * NUG, H2 - 1), true);  // and of the row after it
         }
 #pragma unroll
-        for (int ss = 0; ss < GS; ++ss)
+        for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
-            for (int cb = 0; cb < NCB; ++cb)
+            for (int t = 0; t < 4; ++t) acc[cb][t] = mfma(buf[0][cb][t], G[g * GS], acc[cb][t]);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int t = 0; t < 4; ++t) acc[cb][t] = mfma(buf[ss][cb][t], G[g * GS + ss], acc[cb][t]);
+        for (int ss = 0; ss < GS; ++ss) {
+            const int r = g * GS + ss;
+            const int v = 32 * vcw + vmap(r, h);
+            Gn[r] = gval<GMODE, KC>(wv[r], wu_n, u + NUG, v, pok && v < W2);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) acc[cb][t] = mfma(buf[1][cb][t], G[g * GS + 1], acc[cb][t]);
+        if (g == NG - 1) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) G[r] = Gn[r];
+        }
     };
 
     // Ring of NB register buffers (NB divides the NG groups of a row, so slots are static): the loads of
@@ -1069,9 +1087,12 @@ __global__ void __launch_bounds__(256) df2_tiled_kernel(const BwdArgs a, int nvc
 #pragma unroll
             for (int s = 0; s < 16; ++s) {
                 if (s + 1 < 16) lds_fetch(s + 1, nxt);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int t = 0; t < 4; ++t) acc[0][t] = mfma(cur.fa[0][t], Gc, acc[0][t]);
+                __builtin_amdgcn_sched_barrier(0);
                 if (s + 1 < 16) Gn = g_of(s + 1, nxt);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int cb = 1; cb < NCB; ++cb)
 #pragma unroll
