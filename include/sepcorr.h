@@ -20,7 +20,7 @@
  *    they enqueue kernels and return.
  *  - Return value: 0 on success, a negative SEPCORR_E* code otherwise; sepcorr_last_error() then
  *    returns a message for the calling thread.  Nothing is launched when a check fails.
- *  - Limits of this build: 1 <= W2 <= 256, 1 <= C <= 1024, 1 <= K <= 8, all sizes >= 1 and small
+ *  - Limits of this build: 1 <= W2 <= 2048, 1 <= C <= 1024, 1 <= K <= 8, all sizes >= 1 and small
  *    enough that every tensor has fewer than 2^31 elements.
  *  - Backward entry points need scratch memory: query sepcorr_backward_workspace_bytes() and pass a
  *    device buffer of at least that size (256-byte aligned).  Its contents on entry are ignored.

@@ -40,7 +40,7 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 namespace {
 
 constexpr int TP = 32;        // pixels per MFMA column block
-constexpr int MAX_W2 = 256;   // 8 waves x 32 columns
+constexpr int MAX_W2 = 2048;  // rows beyond 256 columns are swept in passes of 8 waves x 32 columns
 constexpr int MAX_C = 1024;
 constexpr int MAX_K = 8;
 constexpr int KCH = 4;        // attention channels handled per launch
@@ -126,7 +126,8 @@ struct FwdArgs {
     int N1, H2, W2, C, CP;
     int KT, k0;        // total weight channels and first channel of this launch
     int tiles_per_batch;
-    int nvc;           // column chunks of 32 per fmap2 row = ceil(W2 / 32)
+    int nvc;           // column chunks of 32 handled per pass = min(8, ceil(W2 / 32))
+    int vpasses;       // passes of 256 columns = ceil(W2 / 256)
     int stage;         // collect the rows of out_u in LDS and store them coalesced at the end
 };
 
@@ -170,16 +171,21 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     const int pix = p0 + pl;           // this lane's image-1 pixel
     const bool pok = pix < N1;
     const size_t bp = (size_t)b * N1 + (pok ? pix : 0);
-    const int vrow = 32 * vcw + pl;   // the fmap2 column this lane feeds to the A operand
+    // Rows wider than 256 columns are swept in passes of 256 columns; a pass merges its out_u rows with
+    // what the earlier passes left (same thread, same address), the out_v columns of a pass are its own.
+    for (int vp = 0; vp < a.vpasses; ++vp) {
+    if (vp > 0) __syncthreads();   // the previous pass has finished with the LDS partial buffers
+    const int vbase = vp * 256;
+    const int vrow = vbase + 32 * vcw + pl;   // the fmap2 column this lane feeds to the A operand
     const bool vrow_ok = vrow < W2;
     const float *f2lane = a.f2 + ((size_t)b * H2 * W2 + (vrow_ok ? vrow : 0)) * C;
     const size_t rowstride = (size_t)W2 * C;
 
-    const bool ragged = 32 * vcw + 32 > W2;
+    const bool ragged = vbase + 32 * vcw + 32 > W2;
     unsigned vmask = 0;  // bit r: accumulator register r maps to a real column
 #pragma unroll
     for (int r = 0; r < 16; ++r)
-        if (32 * vcw + vmap(r, h) < W2) vmask |= 1u << r;
+        if (vbase + 32 * vcw + vmap(r, h) < W2) vmask |= 1u << r;
 
     // running state over u, accumulator layout
     float vmax[16], vsum[16];
@@ -190,7 +196,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         for (int k = 0; k < KC; ++k)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int v = 32 * vcw + vmap(r, h);
+                const int v = vbase + 32 * vcw + vmap(r, h);
                 rv[k][r] = 0.f;
                 wvr[k][r] = (pok && v < W2) ? a.wv[(bp * a.KT + a.k0 + k) * W2 + v] : 0.f;
             }
@@ -254,13 +260,13 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
 #pragma unroll
                         for (int r = 0; r < 16; ++r) {
                             const float xm = ((vmask >> r) & 1u) ? acc[ru][r] : -INFINITY;
-                            if (xm > m) { m = xm; mi = 32 * vcw + vmap(r, h); }
+                            if (xm > m) { m = xm; mi = vbase + 32 * vcw + vmap(r, h); }
                         }
                     } else {
 #pragma unroll
                         for (int r = 0; r < 16; ++r) {
                             const float xm = acc[ru][r];
-                            if (xm > m) { m = xm; mi = 32 * vcw + vmap(r, h); }
+                            if (xm > m) { m = xm; mi = vbase + 32 * vcw + vmap(r, h); }
                         }
                     }
 #pragma unroll
@@ -293,8 +299,10 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                 if (u < H2 && p0 + p < N1) {
                     float s = 0.f;
                     for (int w = g2 * nvc; w < (g2 + 1) * nvc; ++w) s += pb[((ru * NPART + k) * nW + w) * 32 + p];
-                    if (a.stage) ostage[(p * NCHO + k) * H2 + u] = s;
-                    else a.out_u[(((size_t)b * N1 + p0 + p) * a.KT + a.k0 + k) * H2 + u] = s;
+                    float *dst = a.stage ? &ostage[(p * NCHO + k) * H2 + u]
+                                         : &a.out_u[(((size_t)b * N1 + p0 + p) * a.KT + a.k0 + k) * H2 + u];
+                    if (vp > 0) s += *dst;   // earlier column passes, written by this same thread
+                    *dst = s;
                 }
             }
         } else {
@@ -311,16 +319,21 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                         if (m2 > m) { m = m2; mi = __float_as_int(pb[((ru * NPART + 1) * nW + w) * 32 + p]); }
                         s += pb[((ru * NPART + 2) * nW + w) * 32 + p];
                     }
-                    if (a.stage) {
-                        ostage[(p * 2 + 0) * H2 + u] = m;
-                        ostage[(p * 2 + 1) * H2 + u] = s / (float)W2;
-                        if constexpr (MODE == MODE_ARGMAX) ostage_am[p * H2 + u] = mi;
-                    } else {
-                        const size_t o = ((size_t)b * N1 + p0 + p);
-                        a.out_u[(o * 2 + 0) * H2 + u] = m;
-                        a.out_u[(o * 2 + 1) * H2 + u] = s / (float)W2;
-                        if constexpr (MODE == MODE_ARGMAX) a.am_u[o * H2 + u] = mi;
+                    const size_t o = ((size_t)b * N1 + p0 + p);
+                    float *dm = a.stage ? &ostage[(p * 2 + 0) * H2 + u] : &a.out_u[(o * 2 + 0) * H2 + u];
+                    float *ds = a.stage ? &ostage[(p * 2 + 1) * H2 + u] : &a.out_u[(o * 2 + 1) * H2 + u];
+                    int *di = a.stage ? &ostage_am[p * H2 + u] : (MODE == MODE_ARGMAX ? &a.am_u[o * H2 + u] : nullptr);
+                    if (vp > 0) {   // merge with the earlier column passes (lower v: they win ties)
+                        const float pm = *dm;
+                        s += *ds;
+                        if (!(m > pm)) {
+                            m = pm;
+                            if constexpr (MODE == MODE_ARGMAX) mi = *di;
+                        }
                     }
+                    *dm = m;
+                    *ds = (vp == a.vpasses - 1) ? s / (float)W2 : s;   // the running sum until the last pass
+                    if constexpr (MODE == MODE_ARGMAX) *di = mi;
                 }
             }
         }
@@ -504,7 +517,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     }
 
     // flush the staged out_u rows: per pixel a contiguous run of NCHO*H2 floats
-    if (a.stage) {
+    if (a.stage && vp == a.vpasses - 1) {
         __syncthreads();
         const int runlen = NCHO * H2;
         const int cht = (MODE == MODE_WEIGHTED) ? a.KT : 2, ch0 = (MODE == MODE_WEIGHTED) ? a.k0 : 0;
@@ -562,7 +575,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     if (pok && ug == 0) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const int v = 32 * vcw + vmap(r, h);
+            const int v = vbase + 32 * vcw + vmap(r, h);
             if (v < W2) {
                 if constexpr (MODE == MODE_WEIGHTED) {
 #pragma unroll
@@ -575,6 +588,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
             }
         }
     }
+    }   // column passes
 }
 
 // ------------------------------------------------------------------------------------------
@@ -592,7 +606,8 @@ struct BwdArgs {
     float *d2;                       // (B,N2,C) or scratch [nsplit][B,N2,C]
     int B, N1, H2, W2, C;
     int KT, k0;
-    int nvc;                         // df1: column chunks of 32 per fmap2 row
+    int nvc;                         // df1: column chunks of 32 per pass = min(8, ceil(W2 / 32))
+    int vpasses;                     // df1: passes of 256 columns
     int tiles_per_batch;             // df1: p tiles per batch
     int nsplit, tiles_per_split;     // df2: split of the p range
     int accumulate;                  // add to the destination instead of overwriting
@@ -684,13 +699,6 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
     const bool pok = pix < N1;
     const size_t bp = (size_t)b * N1 + (pok ? pix : 0);
 
-    VW<GMODE, KC> wv[16];
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const int v = 32 * vcw + vmap(r, h);
-        wv[r] = load_vw<GMODE, KC>(a, bp, v < W2 ? v : 0, pok && v < W2);
-    }
-
     v16f acc[NCB][4];
 #pragma unroll
     for (int cb = 0; cb < NCB; ++cb)
@@ -698,6 +706,16 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
         for (int t = 0; t < 4; ++t)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[cb][t][e] = 0.f;
+
+    // rows wider than 256 columns: passes of 256 columns accumulate into the same registers
+    for (int vp = 0; vp < a.vpasses; ++vp) {
+    const int vbase = vp * 256;
+    VW<GMODE, KC> wv[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int v = vbase + 32 * vcw + vmap(r, h);
+        wv[r] = load_vw<GMODE, KC>(a, bp, v < W2 ? v : 0, pok && v < W2);
+    }
 
     const float *f2b = a.f2 + (size_t)b * H2 * W2 * C;
     // CVEC: raw buffer loads, out-of-image columns and channels read as zero without a branch
@@ -712,7 +730,7 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
     auto issue = [&](int u, int g, v4f(&buf)[GS][NCB]) {
 #pragma unroll
         for (int ss = 0; ss < GS; ++ss) {
-            const int v = 32 * vcw + vmap(g * GS + ss, h);
+            const int v = vbase + 32 * vcw + vmap(g * GS + ss, h);
             const bool ok = v < W2;
             if constexpr (CVEC) {
                 const unsigned voff = ok ? ((unsigned)(u * W2 + v) * C) * 4u : nbytes;
@@ -732,7 +750,7 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
     UW<GMODE, KC> wu_n = load_uw<GMODE, KC>(a, bp, min(ug, H2 - 1), true);   // bp is clamped: always a valid pixel
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-        const int v = 32 * vcw + vmap(r, h);
+        const int v = vbase + 32 * vcw + vmap(r, h);
         G[r] = gval<GMODE, KC>(wv[r], wu_n, ug, v, pok && v < W2);
     }
     UW<GMODE, KC> wu_next = load_uw<GMODE, KC>(a, bp, min(ug + NUG, H2 - 1), true);
@@ -750,7 +768,7 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
 #pragma unroll
         for (int ss = 0; ss < GS; ++ss) {
             const int r = g * GS + ss;
-            const int v = 32 * vcw + vmap(r, h);
+            const int v = vbase + 32 * vcw + vmap(r, h);
             Gn[r] = gval<GMODE, KC>(wv[r], wu_n, u + NUG, v, pok && v < W2);
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -784,6 +802,8 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
             __builtin_amdgcn_sched_barrier(0);
         }
     }
+
+    }   // column passes
 
     // sum the per-wave partials in wave order through LDS, then store coalesced
     for (int w = 0; w < nW; ++w) {
@@ -1197,11 +1217,13 @@ int set_lds(KernelT kernel, size_t bytes) {
 
 // Waves per workgroup of the p-owner kernels: nvc column chunks x NUG row groups.
 struct WaveGrid {
-    int nvc, nug;
+    int nvc, nug, vpasses;
 };
 WaveGrid wave_grid(int B, int tiles_per_batch, int W2, int H2) {
     WaveGrid g;
     g.nvc = (W2 + 31) / 32;
+    g.vpasses = (g.nvc + 7) / 8;
+    if (g.nvc > 8) g.nvc = 8;
     g.nug = 1;
     if (g.nvc <= 2) {
         g.nug = 4 / g.nvc;                                        // 4 waves
@@ -1215,6 +1237,7 @@ template <int MODE, int KC, int UR>
 int launch_fwd(FwdArgs a, int B, hipStream_t s) {
     const WaveGrid wg = wave_grid(B, a.tiles_per_batch, a.W2, a.H2);
     a.nvc = wg.nvc;
+    a.vpasses = wg.vpasses;
     const int nW = wg.nvc * wg.nug;
     constexpr int NPART = (MODE == MODE_WEIGHTED) ? KC : 3;
     size_t lds = ((size_t)TP * (a.CP + 4) + 2 * UR * NPART * nW * 32) * sizeof(float);
@@ -1331,6 +1354,7 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s) {
         WaveGrid wg = wave_grid(d.B, a.tiles_per_batch, d.W2, d.H2);
         if (wg.nvc * wg.nug > 4) wg.nug = 4 / wg.nvc > 0 ? 4 / wg.nvc : 1;   // d_f1 runs one wave per SIMD
         a.nvc = wg.nvc;
+        a.vpasses = wg.vpasses;
         const int nW = wg.nvc * wg.nug;
         // more than 4 waves share the register file two to a SIMD: halve the channel block
         const int ncb = (d.C <= 128 || nW > 4) ? 1 : 2;

@@ -43,8 +43,8 @@ def test_argument_checks_precede_any_launch():
     assert lib.sepcorr_max_avg_forward(None, one, one, one, 1, 1, 1, 1, 1, 1, None) == -1
     assert b"NULL" in lib.sepcorr_last_error()
     assert lib.sepcorr_max_avg_forward(one, one, one, one, 1, 1, 1, 1, 0, 1, None) == -1
-    assert lib.sepcorr_max_avg_forward(one, one, one, one, 1, 1, 1, 1, 257, 1, None) == -1
-    assert b"W2=257" in lib.sepcorr_last_error()
+    assert lib.sepcorr_max_avg_forward(one, one, one, one, 1, 1, 1, 1, 2049, 1, None) == -1
+    assert b"W2=2049" in lib.sepcorr_last_error()
     assert lib.sepcorr_max_argmax_avg_forward(one, one, one, one, one, one, 1, 1, 1, 1, 1, 2000, None) == -1
     assert lib.sepcorr_compression_forward(one, one, one, one, one, one, 1, 1, 1, 1, 1, 1, 9, None) == -1
     assert b"K=9" in lib.sepcorr_last_error()

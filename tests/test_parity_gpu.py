@@ -24,6 +24,9 @@ SHAPES = [
     (1, 30, 36, 15, 20, 100),   # tiled d_f2 with a ragged 128-channel block and pooled fmap2
     (1, 16, 48, 16, 48, 300),   # two channel blocks, the second ragged
     (8, 32, 48, 16, 24, 32),    # narrow rows, many workgroups: 1 column chunk x 4 row groups
+    (1, 4, 40, 3, 300, 32),     # rows wider than 256 columns: two column passes
+    (1, 5, 24, 2, 520, 20),     # three column passes, last one ragged
+    (1, 3, 11, 2, 301, 7),      # wide rows on the generic load paths
 ]
 
 
@@ -51,7 +54,7 @@ def test_max_argmax_avg_forward(device, shape):
     assert torch.equal(ou, ou2) and torch.equal(ov, ov2)
 
 
-@pytest.mark.parametrize("shape", SHAPES[1:7])
+@pytest.mark.parametrize("shape", SHAPES[1:7] + SHAPES[12:])
 @pytest.mark.parametrize("K", [1, 2, 4, 5])
 def test_compression_forward(device, shape, K):
     B, H1, W1, H2, W2, C = shape
@@ -194,6 +197,6 @@ def test_error_conventions_on_device(device):
     with pytest.raises(RuntimeError, match="differ"):
         ms.max_avg_forward(f, torch.randn(1, 4, 4, 9, device=device))
     with pytest.raises(RuntimeError, match="exceeds"):
-        ms.max_avg_forward(torch.randn(1, 1, 2, 4, device=device), torch.randn(1, 1, 300, 4, device=device))
+        ms.max_avg_forward(torch.randn(1, 1, 2, 4, device=device), torch.randn(1, 1, 2100, 4, device=device))
     with pytest.raises(RuntimeError, match="shape"):
         ms.compression_forward(f, f, torch.randn(1, 4, 4, 2, 4, device=device), torch.randn(1, 4, 4, 2, 5, device=device))
