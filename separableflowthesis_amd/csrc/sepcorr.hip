@@ -133,8 +133,9 @@ struct FwdArgs {
 
 // CMODE: 0 = any C (scalar loads), 1 = C % 4 == 0 (16-byte loads), 2 = C % 32 == 0 (branch-free fast path),
 //        3 = C == 256 (fast path with the channel loop unrolled: every load offset is an immediate)
-// RG: row groups enabled (narrow rows); without it NUG == 1 is a compile-time constant.
-template <int MODE, int KC, int UR, int CMODE, bool RG>
+// WM: 0 = one pass, one row group (both compile-time constants: the lean common case),
+//     1 = row groups enabled (narrow rows), 2 = column passes enabled (rows wider than 256).
+template <int MODE, int KC, int UR, int CMODE, int WM>
 __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     constexpr bool CVEC = CMODE >= 1;
     constexpr int GJ = 2;  // 8-channel slices per prefetch group
@@ -145,8 +146,10 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     // Waves form a grid: nvc column chunks x NUG row groups.  Wave (vcw, ug) owns columns [32 vcw, 32 vcw + 32)
     // and the steps ug, ug + NUG, ... (narrow fmap2 levels have few column chunks; row groups keep the
     // workgroup at 4 or 8 waves).  NUG == 1 for rows of 97 or more columns.
+    constexpr bool RG = WM == 1;
     const int nvc = RG ? a.nvc : nW, NUG = RG ? nW / nvc : 1;
     const int vcw = RG ? wave % nvc : wave, ug = RG ? wave / nvc : 0;
+    const int vpasses = (WM == 2) ? a.vpasses : 1;
     const int b = blockIdx.x / a.tiles_per_batch;
     const int p0 = (blockIdx.x % a.tiles_per_batch) * TP;
     const int N1 = a.N1, H2 = a.H2, W2 = a.W2, C = a.C;
@@ -173,9 +176,9 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     const size_t bp = (size_t)b * N1 + (pok ? pix : 0);
     // Rows wider than 256 columns are swept in passes of 256 columns; a pass merges its out_u rows with
     // what the earlier passes left (same thread, same address), the out_v columns of a pass are its own.
-    for (int vp = 0; vp < a.vpasses; ++vp) {
+    for (int vp = 0; vp < vpasses; ++vp) {
     if (vp > 0) __syncthreads();   // the previous pass has finished with the LDS partial buffers
-    const int vbase = vp * 256;
+    const int vbase = (WM == 2) ? vp * 256 : 0;
     const int vrow = vbase + 32 * vcw + pl;   // the fmap2 column this lane feeds to the A operand
     const bool vrow_ok = vrow < W2;
     const float *f2lane = a.f2 + ((size_t)b * H2 * W2 + (vrow_ok ? vrow : 0)) * C;
@@ -299,10 +302,17 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                 if (u < H2 && p0 + p < N1) {
                     float s = 0.f;
                     for (int w = g2 * nvc; w < (g2 + 1) * nvc; ++w) s += pb[((ru * NPART + k) * nW + w) * 32 + p];
-                    float *dst = a.stage ? &ostage[(p * NCHO + k) * H2 + u]
-                                         : &a.out_u[(((size_t)b * N1 + p0 + p) * a.KT + a.k0 + k) * H2 + u];
-                    if (vp > 0) s += *dst;   // earlier column passes, written by this same thread
-                    *dst = s;
+                    // (LDS and global destinations are kept in separate branches: a pointer that may be either
+                    // turns into FLAT accesses, whose counters force every later wait to zero)
+                    if (a.stage) {
+                        float *dst = &ostage[(p * NCHO + k) * H2 + u];
+                        if (vp > 0) s += *dst;   // earlier column passes, written by this same thread
+                        *dst = s;
+                    } else {
+                        float *dst = &a.out_u[(((size_t)b * N1 + p0 + p) * a.KT + a.k0 + k) * H2 + u];
+                        if (vp > 0) s += *dst;
+                        *dst = s;
+                    }
                 }
             }
         } else {
@@ -319,21 +329,30 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                         if (m2 > m) { m = m2; mi = __float_as_int(pb[((ru * NPART + 1) * nW + w) * 32 + p]); }
                         s += pb[((ru * NPART + 2) * nW + w) * 32 + p];
                     }
-                    const size_t o = ((size_t)b * N1 + p0 + p);
-                    float *dm = a.stage ? &ostage[(p * 2 + 0) * H2 + u] : &a.out_u[(o * 2 + 0) * H2 + u];
-                    float *ds = a.stage ? &ostage[(p * 2 + 1) * H2 + u] : &a.out_u[(o * 2 + 1) * H2 + u];
-                    int *di = a.stage ? &ostage_am[p * H2 + u] : (MODE == MODE_ARGMAX ? &a.am_u[o * H2 + u] : nullptr);
-                    if (vp > 0) {   // merge with the earlier column passes (lower v: they win ties)
-                        const float pm = *dm;
-                        s += *ds;
-                        if (!(m > pm)) {
-                            m = pm;
-                            if constexpr (MODE == MODE_ARGMAX) mi = *di;
+                    const bool last = vp == vpasses - 1;   // the running sum is kept until the last pass
+                    if (a.stage) {
+                        float *dm = &ostage[(p * 2 + 0) * H2 + u], *ds = &ostage[(p * 2 + 1) * H2 + u];
+                        int *di = &ostage_am[p * H2 + u];
+                        if (vp > 0) {   // merge with the earlier column passes (lower v: they win ties)
+                            const float pm = *dm;
+                            s += *ds;
+                            if (!(m > pm)) { m = pm; if constexpr (MODE == MODE_ARGMAX) mi = *di; }
                         }
+                        *dm = m;
+                        *ds = last ? s / (float)W2 : s;
+                        if constexpr (MODE == MODE_ARGMAX) *di = mi;
+                    } else {
+                        const size_t o = ((size_t)b * N1 + p0 + p);
+                        float *dm = &a.out_u[(o * 2 + 0) * H2 + u], *ds = &a.out_u[(o * 2 + 1) * H2 + u];
+                        if (vp > 0) {
+                            const float pm = *dm;
+                            s += *ds;
+                            if (!(m > pm)) { m = pm; if constexpr (MODE == MODE_ARGMAX) mi = a.am_u[o * H2 + u]; }
+                        }
+                        *dm = m;
+                        *ds = last ? s / (float)W2 : s;
+                        if constexpr (MODE == MODE_ARGMAX) a.am_u[o * H2 + u] = mi;
                     }
-                    *dm = m;
-                    *ds = (vp == a.vpasses - 1) ? s / (float)W2 : s;   // the running sum until the last pass
-                    if constexpr (MODE == MODE_ARGMAX) *di = mi;
                 }
             }
         }
@@ -375,6 +394,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         const unsigned lane_off = vrow_ok ? ((unsigned)vrow * C + 16u * h) * 4u : nbytes;
         const int NJB = (CMODE == 3) ? 8 : (C >> 5);
         constexpr bool BPIPE = !(MODE == MODE_WEIGHTED && KC >= 3);   // needs 16 more registers
+        constexpr bool DUAL = UR == 1 && !(MODE == MODE_WEIGHTED && KC >= 3);
         v4f bcur[4];
         if constexpr (BPIPE) {
 #pragma unroll
@@ -411,9 +431,10 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
             auto mfma_tq = [&](int tq, const v4f &bv) {
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
-                    if constexpr (UR == 1) {
+                    if constexpr (DUAL) {
                         // one row per step: split the contraction over two accumulators so that
-                        // consecutive MFMAs are independent
+                        // consecutive MFMAs are independent (skipped where registers are short: the
+                        // matrix pipe accepts back-to-back dependent MFMAs without a bubble)
                         if (t & 1) acc_alt = mfma(buf[0][tq][t], bv[t], acc_alt);
                         else acc[0] = mfma(buf[0][tq][t], bv[t], acc[0]);
                     } else {
@@ -451,7 +472,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
 #else
             if (J == NJB - 1) {
 #endif
-                if constexpr (UR == 1) {
+                if constexpr (DUAL) {
                     acc[0] += acc_alt;
 #pragma unroll
                     for (int e = 0; e < 16; ++e) acc_alt[e] = 0.f;
@@ -517,7 +538,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     }
 
     // flush the staged out_u rows: per pixel a contiguous run of NCHO*H2 floats
-    if (a.stage && vp == a.vpasses - 1) {
+    if (a.stage && vp == vpasses - 1) {
         __syncthreads();
         const int runlen = NCHO * H2;
         const int cht = (MODE == MODE_WEIGHTED) ? a.KT : 2, ch0 = (MODE == MODE_WEIGHTED) ? a.k0 : 0;
@@ -1262,12 +1283,14 @@ int launch_fwd(FwdArgs a, int B, hipStream_t s) {
     } while (0)
     // Always built for two waves per SIMD (256 registers): the accumulators then stay in ordinary
     // VGPRs, where the epilogue reads them without accumulator-register copies.
-    if (wg.nug > 1) {
-        if (cmode == 3) SEPCORR_FWD(3, true); else if (cmode == 2) SEPCORR_FWD(2, true);
-        else if (cmode == 1) SEPCORR_FWD(1, true); else SEPCORR_FWD(0, true);
+    if (wg.vpasses > 1) {
+        if (cmode >= 2) SEPCORR_FWD(2, 2); else if (cmode == 1) SEPCORR_FWD(1, 2); else SEPCORR_FWD(0, 2);
+    } else if (wg.nug > 1) {
+        if (cmode == 3) SEPCORR_FWD(3, 1); else if (cmode == 2) SEPCORR_FWD(2, 1);
+        else if (cmode == 1) SEPCORR_FWD(1, 1); else SEPCORR_FWD(0, 1);
     } else {
-        if (cmode == 3) SEPCORR_FWD(3, false); else if (cmode == 2) SEPCORR_FWD(2, false);
-        else if (cmode == 1) SEPCORR_FWD(1, false); else SEPCORR_FWD(0, false);
+        if (cmode == 3) SEPCORR_FWD(3, 0); else if (cmode == 2) SEPCORR_FWD(2, 0);
+        else if (cmode == 1) SEPCORR_FWD(1, 0); else SEPCORR_FWD(0, 0);
     }
 #undef SEPCORR_FWD
     return check_launch("forward kernel");
