@@ -34,8 +34,8 @@ KERNEL_PASSES = {"fwd_maxavg": 1, "fwd_weighted": 1, "df1_comp": 1, "df2_comp": 
 # HBM bytes per launch at cfg4 from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by the factors a
 # 256 MiB device copy gives in the same run (profiles/cfg4_fwd_bwd_kernels.txt); None = not measured
 _MIB = 2 ** 20
-TRAFFIC_BYTES_CFG4 = {"fwd_maxavg": 266.4 * _MIB, "fwd_weighted": 546.9 * _MIB, "df1_comp": 546.7 * _MIB,
-                      "df2_comp": 611.1 * _MIB, "df1_maxavg": 211.6 * _MIB, "df2_maxavg": 384.8 * _MIB}
+TRAFFIC_BYTES_CFG4 = {"fwd_maxavg": 232.1 * _MIB, "fwd_weighted": 299.9 * _MIB, "df1_comp": 524.0 * _MIB,
+                      "df2_comp": 612.1 * _MIB, "df1_maxavg": 211.7 * _MIB, "df2_maxavg": 384.6 * _MIB}
 
 
 def make_inputs(B, H, W, C, Kp, torch):

@@ -592,19 +592,46 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         }
     }
 
-    // store the state that was reduced over u
+    // store the state that was reduced over u: registers 4g..4g+3 hold 4 consecutive columns
     if (pok && ug == 0) {
+        if ((W2 & 3) == 0) {   // 16-byte stores (rows of out_v are then 16-byte aligned)
+            typedef int v4i __attribute__((ext_vector_type(4)));
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int v = vbase + 32 * vcw + vmap(r, h);
-            if (v < W2) {
-                if constexpr (MODE == MODE_WEIGHTED) {
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const int v = vbase + 32 * vcw + vmap(4 * g4, h);
+                if (v < W2) {
+                    if constexpr (MODE == MODE_WEIGHTED) {
 #pragma unroll
-                    for (int k = 0; k < KC; ++k) a.out_v[(bp * a.KT + a.k0 + k) * W2 + v] = rv[k][r];
-                } else {
-                    a.out_v[(bp * 2 + 0) * W2 + v] = vmax[r];
-                    a.out_v[(bp * 2 + 1) * W2 + v] = vsum[r] / (float)H2;
-                    if constexpr (MODE == MODE_ARGMAX) a.am_v[bp * W2 + v] = vidx[r];
+                        for (int k = 0; k < KC; ++k) {
+                            const v4f x = {rv[k][4 * g4], rv[k][4 * g4 + 1], rv[k][4 * g4 + 2], rv[k][4 * g4 + 3]};
+                            *reinterpret_cast<v4f *>(a.out_v + (bp * a.KT + a.k0 + k) * W2 + v) = x;
+                        }
+                    } else {
+                        const v4f xm = {vmax[4 * g4], vmax[4 * g4 + 1], vmax[4 * g4 + 2], vmax[4 * g4 + 3]};
+                        const v4f xs = {vsum[4 * g4] / (float)H2, vsum[4 * g4 + 1] / (float)H2, vsum[4 * g4 + 2] / (float)H2,
+                                        vsum[4 * g4 + 3] / (float)H2};
+                        *reinterpret_cast<v4f *>(a.out_v + (bp * 2 + 0) * W2 + v) = xm;
+                        *reinterpret_cast<v4f *>(a.out_v + (bp * 2 + 1) * W2 + v) = xs;
+                        if constexpr (MODE == MODE_ARGMAX) {
+                            const v4i xi = {vidx[4 * g4], vidx[4 * g4 + 1], vidx[4 * g4 + 2], vidx[4 * g4 + 3]};
+                            *reinterpret_cast<v4i *>(a.am_v + bp * W2 + v) = xi;
+                        }
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int v = vbase + 32 * vcw + vmap(r, h);
+                if (v < W2) {
+                    if constexpr (MODE == MODE_WEIGHTED) {
+#pragma unroll
+                        for (int k = 0; k < KC; ++k) a.out_v[(bp * a.KT + a.k0 + k) * W2 + v] = rv[k][r];
+                    } else {
+                        a.out_v[(bp * 2 + 0) * W2 + v] = vmax[r];
+                        a.out_v[(bp * 2 + 1) * W2 + v] = vsum[r] / (float)H2;
+                        if constexpr (MODE == MODE_ARGMAX) a.am_v[bp * W2 + v] = vidx[r];
+                    }
                 }
             }
         }
