@@ -25,6 +25,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdarg.h>
+#include <stdlib.h>
 #include <stdio.h>
 #include <string.h>
 
@@ -1395,7 +1396,8 @@ Df2Plan df2_plan(const Dims &d) {
 }
 
 template <int GMODE, int KC>
-int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s) {
+int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s) {
+    // s1: stream of the d_f1 kernel; s: stream of the d_f2 kernel and its split reduction
     const size_t big = (size_t)1 << 30;
     const bool cvec = (d.C % 4) == 0 && (size_t)d.H2 * d.W2 * d.C * 4 <= big && (size_t)d.H1 * d.W1 * d.C * 4 <= big;
     a.tiles_per_batch = (a.N1 + TP - 1) / TP;
@@ -1413,8 +1415,8 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s) {
         const size_t lds = (size_t)TP * (128 * ncb + 4) * sizeof(float);
 #define SEPCORR_DF1(NCB, CV, MT)                                                                   \
     do {                                                                                           \
-        ProfScope ps(GMODE == GMODE_COMP ? "df1_comp" : "df1_maxavg", s);                          \
-        hipLaunchKernelGGL((df1_kernel<GMODE, KC, NCB, CV, MT>), grid, block, lds, s, a);          \
+        ProfScope ps(GMODE == GMODE_COMP ? "df1_comp" : "df1_maxavg", s1);                         \
+        hipLaunchKernelGGL((df1_kernel<GMODE, KC, NCB, CV, MT>), grid, block, lds, s1, a);         \
     } while (0)
         if (nW > 4) { if (cvec) SEPCORR_DF1(1, true, 512); else SEPCORR_DF1(1, false, 512); }
         else if (ncb == 1) { if (cvec) SEPCORR_DF1(1, true, 256); else SEPCORR_DF1(1, false, 256); }
@@ -1471,6 +1473,74 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s) {
     }
     return SEPCORR_OK;
 }
+
+// The kernels of one backward call are independent of each other (they only read the inputs), so they
+// are issued on separate streams: the tail of one kernel, where part of the chip would idle, is filled
+// by the next.  Fork: the side streams wait for everything queued on the caller's stream; join: the
+// caller's stream waits for the side streams.  Works under stream capture (ordinary fork/join pattern).
+// Per device: two side streams at default priority and three events, created on first use.
+struct SideStreams {
+    hipStream_t a = nullptr, b = nullptr;
+    hipEvent_t fork = nullptr, ja = nullptr, jb = nullptr;
+    bool ok = false;
+};
+std::mutex g_side_mu;
+SideStreams g_side[64];
+
+bool overlap_enabled() {
+    static const bool on = [] {
+        const char *e = getenv("SEPCORR_SINGLE_STREAM");
+        return !(e && e[0] == '1');
+    }();
+    return on && !g_prof_on;   // per-kernel timing wants the kernels one after the other
+}
+
+SideStreams *side_streams() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+    SideStreams &ss = g_side[dev];
+    if (!ss.ok) {
+        if (hipStreamCreateWithFlags(&ss.a, hipStreamNonBlocking) != hipSuccess) return nullptr;
+        if (hipStreamCreateWithFlags(&ss.b, hipStreamNonBlocking) != hipSuccess) return nullptr;
+        if (hipEventCreateWithFlags(&ss.fork, hipEventDisableTiming) != hipSuccess) return nullptr;
+        if (hipEventCreateWithFlags(&ss.ja, hipEventDisableTiming) != hipSuccess) return nullptr;
+        if (hipEventCreateWithFlags(&ss.jb, hipEventDisableTiming) != hipSuccess) return nullptr;
+        ss.ok = true;
+    }
+    return &ss;
+}
+
+// RAII fork/join around the launches of one backward call.  With overlap off, both side streams are
+// the caller's stream and nothing is recorded.
+struct ForkJoin {
+    std::unique_lock<std::mutex> lk;
+    SideStreams *ss = nullptr;
+    hipStream_t user, sa, sb;
+    bool failed = false;
+    explicit ForkJoin(hipStream_t u) : user(u), sa(u), sb(u) {
+        if (!overlap_enabled()) return;
+        lk = std::unique_lock<std::mutex>(g_side_mu);
+        ss = side_streams();
+        if (!ss) return;
+        if (hipEventRecord(ss->fork, user) != hipSuccess || hipStreamWaitEvent(ss->a, ss->fork, 0) != hipSuccess ||
+            hipStreamWaitEvent(ss->b, ss->fork, 0) != hipSuccess) {
+            ss = nullptr;
+            (void)hipGetLastError();
+            return;
+        }
+        sa = ss->a;
+        sb = ss->b;
+    }
+    // Must be called on every path once the fork has happened, also after a failed launch.
+    int join() {
+        if (!ss) return SEPCORR_OK;
+        const bool bad = hipEventRecord(ss->ja, sa) != hipSuccess || hipEventRecord(ss->jb, sb) != hipSuccess ||
+                         hipStreamWaitEvent(user, ss->ja, 0) != hipSuccess || hipStreamWaitEvent(user, ss->jb, 0) != hipSuccess;
+        ss = nullptr;
+        return bad ? fail(SEPCORR_ELAUNCH, "sepcorr: joining the side streams failed") : SEPCORR_OK;
+    }
+    ~ForkJoin() { (void)join(); }
+};
 
 int check_workspace(const Dims &d, void *ws, size_t ws_bytes) {
     const size_t need = sepcorr_backward_workspace_bytes(d.B, d.H1, d.W1, d.H2, d.W2, d.C);
@@ -1566,7 +1636,10 @@ int sepcorr_max_argmax_avg_backward(const float *f1, const float *f2, const int3
     a.f1 = f1; a.f2 = f2; a.am_u = argmax_u; a.am_v = argmax_v; a.g_u = grad_u; a.g_v = grad_v;
     a.d1 = d_f1; a.d2 = d_f2;
     a.B = B; a.N1 = H1 * W1; a.H2 = H2; a.W2 = W2; a.C = C; a.KT = 1;
-    return launch_bwd<GMODE_MAXAVG, 1>(a, d, workspace, static_cast<hipStream_t>(stream));
+    ForkJoin fj(static_cast<hipStream_t>(stream));
+    const int rc = launch_bwd<GMODE_MAXAVG, 1>(a, d, workspace, fj.sa, fj.user);   // d_f1 aside, d_f2 on the caller's stream
+    const int rj = fj.join();
+    return rc ? rc : rj;
 }
 
 int sepcorr_compression_backward(const float *f1, const float *f2, const float *a_u, const float *a_v, const float *g_cu,
@@ -1578,29 +1651,29 @@ int sepcorr_compression_backward(const float *f1, const float *f2, const float *
     const Dims d = {B, H1, W1, H2, W2, C};
     if (int rc = check_dims(d, K)) return rc;
     if (int rc = check_workspace(d, workspace, workspace_bytes)) return rc;
-    hipStream_t s = static_cast<hipStream_t>(stream);
+    ForkJoin fj(static_cast<hipStream_t>(stream));
     // d_a_v[k,u] = sum_v S g_cv[k,v];  d_a_u[k,v] = sum_u S g_cu[k,u]: the forward's weighted sums
-    if (int rc = weighted_forward(d, f1, f2, g_cv, g_cu, d_a_v, d_a_u, K, s)) return rc;
+    int rc = weighted_forward(d, f1, f2, g_cv, g_cu, d_a_v, d_a_u, K, fj.user);
     BwdArgs a;
     memset(&a, 0, sizeof(a));
     a.f1 = f1; a.f2 = f2; a.a_u = a_u; a.a_v = a_v; a.g_cu = g_cu; a.g_cv = g_cv;
     a.d1 = d_f1; a.d2 = d_f2;
     a.B = B; a.N1 = H1 * W1; a.H2 = H2; a.W2 = W2; a.C = C; a.KT = K;
     const int kch = W2 > 128 ? 2 : KCH;  // wide workgroups have half the registers per lane
-    for (int k0 = 0; k0 < K; k0 += kch) {
+    // channel chunks accumulate into d_f1 / d_f2: each output keeps its own stream, so chunks stay ordered
+    for (int k0 = 0; k0 < K && rc == SEPCORR_OK; k0 += kch) {
         a.k0 = k0;
         a.accumulate = k0 > 0;
         const int kc = K - k0 < kch ? K - k0 : kch;
-        int rc;
         switch (kc) {
-            case 1: rc = launch_bwd<GMODE_COMP, 1>(a, d, workspace, s); break;
-            case 2: rc = launch_bwd<GMODE_COMP, 2>(a, d, workspace, s); break;
-            case 3: rc = launch_bwd<GMODE_COMP, 3>(a, d, workspace, s); break;
-            default: rc = launch_bwd<GMODE_COMP, 4>(a, d, workspace, s); break;
+            case 1: rc = launch_bwd<GMODE_COMP, 1>(a, d, workspace, fj.sa, fj.sb); break;
+            case 2: rc = launch_bwd<GMODE_COMP, 2>(a, d, workspace, fj.sa, fj.sb); break;
+            case 3: rc = launch_bwd<GMODE_COMP, 3>(a, d, workspace, fj.sa, fj.sb); break;
+            default: rc = launch_bwd<GMODE_COMP, 4>(a, d, workspace, fj.sa, fj.sb); break;
         }
-        if (rc) return rc;
     }
-    return SEPCORR_OK;
+    const int rj = fj.join();
+    return rc ? rc : rj;
 }
 
 }  // extern "C"
