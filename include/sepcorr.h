@@ -117,6 +117,32 @@ int sepcorr_compression_backward(const float *f1, const float *f2, const float *
                                  int B, int H1, int W1, int H2, int W2, int C, int K,
                                  void *workspace, size_t workspace_bytes, void *stream);
 
+/*
+ * Attention-weight producer in the operator's layout.  Replaces, for one of the two volumes, the caller's
+ *   a = attention(sep.permute(0,3,4,1,2)).softmax(dim=2).permute(0,3,4,1,2).contiguous()
+ * (core/corr.py:428-429, 437-446) where `attention` is the reference's torch.nn.Conv3d(2, K, 3, padding=1)
+ * (core/sepflow.py:59-60):
+ *   sep    (B,H1,W1,2,L)   the max/avg output of sepcorr_max_*_forward (either one)
+ *   weight (K,2,3,3,3)     Conv3d weight; kernel axes are (L, H1, W1)        bias (K) or NULL
+ *   a      (B,H1,W1,K,L)   softmax over L of the convolution: the weights sepcorr_compression_forward takes
+ */
+int sepcorr_attention_forward(const float *sep, const float *weight, const float *bias, float *a,
+                              int B, int H1, int W1, int L, int K, void *stream);
+
+/* Scratch bytes needed by sepcorr_attention_backward. */
+size_t sepcorr_attention_workspace_bytes(int B, int H1, int W1, int L, int K);
+
+/*
+ * Gradients of the above (what torch autograd computes through softmax and Conv3d in the reference,
+ * core/corr.py:437-446): given grad_a = dLoss/da and the saved output a,
+ *   d_sep (B,H1,W1,2,L), d_weight (K,2,3,3,3), d_bias (K) or NULL.
+ * Sums run in a fixed order: results are run-to-run identical.
+ */
+int sepcorr_attention_backward(const float *sep, const float *weight, const float *a, const float *grad_a,
+                               float *d_sep, float *d_weight, float *d_bias,
+                               int B, int H1, int W1, int L, int K,
+                               void *workspace, size_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -164,6 +164,17 @@ def compression_backward(f1, f2, a_u, a_v, g_cu, g_cv):
     return d1, d2, da_u, da_v
 
 
+def attention_weights(sep, weight, bias):
+    """The caller's attention-weight producer, op-level layout in and out.
+
+    Follows core/corr.py:428-429 and 437-446 with core/sepflow.py:59-60: the (B,H1,W1,2,L) max/avg output is
+    permuted to (B,2,L,H1,W1), passed through Conv3d(2,K,3,padding=1), softmax over dim 2 (L), and permuted
+    back to (B,H1,W1,K,L).  Library routines only (conv3d is a cross-correlation).
+    """
+    vol = sep.permute(0, 3, 4, 1, 2)
+    return F.conv3d(vol, weight, bias, padding=1).softmax(dim=2).permute(0, 3, 4, 1, 2).contiguous()
+
+
 # --------------------------------------------------------------------------
 # autograd through the stored 4D volume (what the reference's tests compare with)
 # --------------------------------------------------------------------------

@@ -149,3 +149,46 @@ def compression_backward(img1_features_l0, img2_features_lk, attention_weights_u
             d1.data_ptr(), d2.data_ptr(), da_u.data_ptr(), da_v.data_ptr(),
             B, H1, W1, H2, W2, C, K, ws.data_ptr(), n, _stream()))
     return [d1, d2, da_u, da_v]
+
+
+# --- not part of the reference's native module: the attention-weight producer the caller runs between
+# --- the two operators (core/corr.py:437-446), fused and in the operator's layout
+
+def attention_forward(sep, weight, bias):
+    """sep (B,H1,W1,2,L), Conv3d weight (K,2,3,3,3), bias (K) or None -> softmax_L(conv3d) as (B,H1,W1,K,L)."""
+    _check("sep", sep, ndim=5)
+    B, H1, W1, ch, L = sep.shape
+    if ch != 2:
+        raise RuntimeError(f"sep must have 2 channels (max, avg), got {ch}")
+    _check("weight", weight, ndim=5)
+    K = weight.shape[0]
+    _expect("weight", weight, (K, 2, 3, 3, 3), sep.device)
+    if bias is not None:
+        _expect("bias", bias, (K,), sep.device)
+    lib = _lib.load()
+    with torch.cuda.device(sep.device):
+        a = torch.empty((B, H1, W1, K, L), dtype=sep.dtype, device=sep.device)
+        _lib.check(lib.sepcorr_attention_forward(sep.data_ptr(), weight.data_ptr(), bias.data_ptr() if bias is not None else None,
+                                                 a.data_ptr(), B, H1, W1, L, K, _stream()))
+    return a
+
+
+def attention_backward(sep, weight, a, grad_a, need_bias=True):
+    """-> [d_sep (B,H1,W1,2,L), d_weight (K,2,3,3,3), d_bias (K) or None]"""
+    _check("sep", sep, ndim=5)
+    B, H1, W1, _, L = sep.shape
+    K = weight.shape[0]
+    _expect("weight", weight, (K, 2, 3, 3, 3), sep.device)
+    _expect("a", a, (B, H1, W1, K, L), sep.device)
+    _expect("grad_a", grad_a, (B, H1, W1, K, L), sep.device)
+    lib = _lib.load()
+    with torch.cuda.device(sep.device):
+        d_sep = torch.empty_like(sep)
+        d_w = torch.empty_like(weight)
+        d_b = torch.empty(K, dtype=sep.dtype, device=sep.device) if need_bias else None
+        n = lib.sepcorr_attention_workspace_bytes(B, H1, W1, L, K)
+        ws = torch.empty(max(n, 1), dtype=torch.uint8, device=sep.device)
+        _lib.check(lib.sepcorr_attention_backward(sep.data_ptr(), weight.data_ptr(), a.data_ptr(), grad_a.data_ptr(),
+                                                  d_sep.data_ptr(), d_w.data_ptr(), d_b.data_ptr() if need_bias else None,
+                                                  B, H1, W1, L, K, ws.data_ptr(), n, _stream()))
+    return [d_sep, d_w, d_b]

@@ -10,7 +10,23 @@ trilinearly upsampled (align_corners=True) to the level-0 displacement length.
 import torch
 import torch.nn.functional as F
 
-from .functions import ComputeMaxArgmaxAvgFunction, ComputeMaxAvgFunction, ComputeSelfCompressionFunction
+from .functions import (AttentionWeightsFunction, ComputeMaxArgmaxAvgFunction, ComputeMaxAvgFunction,
+                        ComputeSelfCompressionFunction)
+
+
+def _is_reference_attention(m):
+    """True for the module the reference builds: Conv3d(2, K, 3, padding=1) (core/sepflow.py:59-60)."""
+    return (isinstance(m, torch.nn.Conv3d) and m.in_channels == 2 and m.out_channels <= 8
+            and tuple(m.kernel_size) == (3, 3, 3) and tuple(m.padding) == (1, 1, 1) and tuple(m.stride) == (1, 1, 1)
+            and tuple(m.dilation) == (1, 1, 1) and m.groups == 1 and m.padding_mode == 'zeros'
+            and m.weight.dtype == torch.float32)
+
+
+def produce_attention(sep_oplevel, sep_modlevel, module):
+    """a = softmax_L(module(volume)) as (B,H1,W1,K,L): fused kernel for the reference's Conv3d, torch otherwise."""
+    if _is_reference_attention(module) and sep_oplevel.is_cuda:
+        return AttentionWeightsFunction.apply(sep_oplevel, module.weight.contiguous(), module.bias)
+    return module(sep_modlevel).softmax(dim=2).permute(0, 3, 4, 1, 2).contiguous()
 
 
 class AlternateCorrBlockSepflow:
@@ -40,8 +56,9 @@ class AlternateCorrBlockSepflow:
             sep_u = maxavg_v.permute(0, 3, 4, 1, 2).contiguous()   # (B,2,W2_i,h1,w1)
             if attention_weights is not None:
                 attention1, attention2 = attention_weights
-                a_u = attention1(sep_u).softmax(dim=2).permute(0, 3, 4, 1, 2).contiguous()
-                a_v = attention2(sep_v).softmax(dim=2).permute(0, 3, 4, 1, 2).contiguous()
+                # core/corr.py:437-446; sep_u is the permuted maxavg_v, sep_v the permuted maxavg_u
+                a_u = produce_attention(maxavg_v, sep_u, attention1)
+                a_v = produce_attention(maxavg_u, sep_v, attention2)
                 adaptive_corr_u, adaptive_corr_v = ComputeSelfCompressionFunction.apply(fmap1, fmap2, a_u, a_v)
                 sep_v = torch.cat((sep_v, adaptive_corr_u.permute(0, 3, 4, 1, 2)), dim=1)
                 sep_u = torch.cat((sep_u, adaptive_corr_v.permute(0, 3, 4, 1, 2)), dim=1)

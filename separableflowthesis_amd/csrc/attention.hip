@@ -1,0 +1,374 @@
+// Attention-weight producer of the separated correlation volumes, fused for gfx950:
+//   a = softmax_L( Conv3d(2 -> K, kernel 3, padding 1)(sep) )
+// taken and returned in the operator's own layout, sep (B,H1,W1,2,L) -> a (B,H1,W1,K,L), so the
+// permutes around it disappear.  In the reference this is attention1(sep_u) / attention2(sep_v), a
+// torch Conv3d over the volume (B,2,L,H1,W1), followed by softmax(dim=2) and permute(0,3,4,1,2)
+// (core/sepflow.py:59-60, core/corr.py:437-446).  The convolution's depth axis is L, its height and
+// width are H1 and W1: weight[k][c][dl][di][dj].
+//
+// HBM-bound element-wise work (54 K multiply-adds per output): one wave per image-1 pixel, lanes along
+// L (rows of L contiguous floats: every access is coalesced), softmax statistics by wave reduction.
+// The backward pass is three kernels: softmax backward -> dlogits (scratch), the transposed
+// convolution for d_sep, and the weight gradient as per-workgroup partial sums that a last kernel
+// adds in a fixed order (deterministic, no atomics).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "sepcorr.h"
+#include "sepcorr_internal.h"
+
+namespace {
+
+constexpr int MAXK = 8;
+constexpr int WPB = 4;          // waves (pixels) per workgroup
+constexpr int DW_PIX = 64;      // pixels per workgroup in the weight-gradient kernel
+
+__device__ __forceinline__ float wave_max(float x) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) x = fmaxf(x, __shfl_xor(x, o));
+    return x;
+}
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o);
+    return x;
+}
+
+struct AttArgs {
+    const float *sep, *weight, *bias, *a, *grad_a;
+    float *out;        // forward: a; softmax backward: dlogits; conv backward: d_sep
+    float *dlogits;    // scratch (B,H1,W1,K,L)
+    float *partial;    // scratch [nwg][K*54 + K]
+    int B, H1, W1, L, K;
+};
+
+// Forward.  NCH = ceil(L / 64) chunks per row held in registers.
+template <int NCH>
+__global__ void __launch_bounds__(64 * WPB) att_forward_kernel(const AttArgs a) {
+    __shared__ float ws[MAXK * 54 + MAXK];
+    const int K = a.K, L = a.L, H1 = a.H1, W1 = a.W1;
+    for (int t = threadIdx.x; t < K * 54; t += blockDim.x) ws[t] = a.weight[t];
+    for (int t = threadIdx.x; t < K; t += blockDim.x) ws[MAXK * 54 + t] = a.bias ? a.bias[t] : 0.f;
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const long pix = (long)blockIdx.x * WPB + wave;       // flattened (b,i,j)
+    const long npix = (long)a.B * H1 * W1;
+    if (pix >= npix) return;
+    const int j = (int)(pix % W1), i = (int)((pix / W1) % H1);
+
+    for (int k = 0; k < K; ++k) {
+        float logit[NCH];
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) logit[c] = ws[MAXK * 54 + k];
+        for (int di = 0; di < 3; ++di) {
+            const int ii = i + di - 1;
+            if (ii < 0 || ii >= H1) continue;
+            for (int dj = 0; dj < 3; ++dj) {
+                const int jj = j + dj - 1;
+                if (jj < 0 || jj >= W1) continue;
+                const float *row = a.sep + (pix + (long)(di - 1) * W1 + (dj - 1)) * 2 * L;
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    const float w0 = ws[((k * 2 + c) * 3 + 0) * 9 + di * 3 + dj];
+                    const float w1 = ws[((k * 2 + c) * 3 + 1) * 9 + di * 3 + dj];
+                    const float w2 = ws[((k * 2 + c) * 3 + 2) * 9 + di * 3 + dj];
+#pragma unroll
+                    for (int ch = 0; ch < NCH; ++ch) {
+                        const int l = ch * 64 + lane;
+                        const float x0 = (l - 1 >= 0 && l - 1 < L) ? row[c * L + l - 1] : 0.f;
+                        const float x1 = (l < L) ? row[c * L + l] : 0.f;
+                        const float x2 = (l + 1 < L) ? row[c * L + l + 1] : 0.f;
+                        logit[ch] += w0 * x0 + w1 * x1 + w2 * x2;
+                    }
+                }
+            }
+        }
+        float m = -INFINITY;
+#pragma unroll
+        for (int ch = 0; ch < NCH; ++ch)
+            if (ch * 64 + lane < L) m = fmaxf(m, logit[ch]);
+        m = wave_max(m);
+        float s = 0.f;
+#pragma unroll
+        for (int ch = 0; ch < NCH; ++ch) {
+            logit[ch] = (ch * 64 + lane < L) ? __expf(logit[ch] - m) : 0.f;
+            s += logit[ch];
+        }
+        s = wave_sum(s);
+        const float inv = 1.f / s;
+        float *dst = a.out + (pix * K + k) * L;
+#pragma unroll
+        for (int ch = 0; ch < NCH; ++ch)
+            if (ch * 64 + lane < L) dst[ch * 64 + lane] = logit[ch] * inv;
+    }
+}
+
+// Forward for long rows: logits go to the output buffer first, then are normalised in place.
+__global__ void __launch_bounds__(64 * WPB) att_forward_long_kernel(const AttArgs a) {
+    __shared__ float ws[MAXK * 54 + MAXK];
+    const int K = a.K, L = a.L, H1 = a.H1, W1 = a.W1;
+    for (int t = threadIdx.x; t < K * 54; t += blockDim.x) ws[t] = a.weight[t];
+    for (int t = threadIdx.x; t < K; t += blockDim.x) ws[MAXK * 54 + t] = a.bias ? a.bias[t] : 0.f;
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const long pix = (long)blockIdx.x * WPB + wave;
+    const long npix = (long)a.B * H1 * W1;
+    if (pix >= npix) return;
+    const int j = (int)(pix % W1), i = (int)((pix / W1) % H1);
+    for (int k = 0; k < K; ++k) {
+        float *dst = a.out + (pix * K + k) * L;
+        float m = -INFINITY;
+        for (int l = lane; l < L; l += 64) {
+            float x = ws[MAXK * 54 + k];
+            for (int di = 0; di < 3; ++di) {
+                const int ii = i + di - 1;
+                if (ii < 0 || ii >= H1) continue;
+                for (int dj = 0; dj < 3; ++dj) {
+                    const int jj = j + dj - 1;
+                    if (jj < 0 || jj >= W1) continue;
+                    const float *row = a.sep + (pix + (long)(di - 1) * W1 + (dj - 1)) * 2 * L;
+                    for (int c = 0; c < 2; ++c)
+                        for (int dl = 0; dl < 3; ++dl) {
+                            const int ll = l + dl - 1;
+                            if (ll >= 0 && ll < L) x += ws[((k * 2 + c) * 3 + dl) * 9 + di * 3 + dj] * row[c * L + ll];
+                        }
+                }
+            }
+            dst[l] = x;
+            m = fmaxf(m, x);
+        }
+        m = wave_max(m);
+        float s = 0.f;
+        for (int l = lane; l < L; l += 64) {
+            const float e = __expf(dst[l] - m);   // written by this same lane
+            dst[l] = e;
+            s += e;
+        }
+        s = wave_sum(s);
+        const float inv = 1.f / s;
+        for (int l = lane; l < L; l += 64) dst[l] *= inv;
+    }
+}
+
+// dlogits = a * (grad_a - sum_l a * grad_a), one wave per pixel.
+__global__ void __launch_bounds__(64 * WPB) att_softmax_backward_kernel(const AttArgs a) {
+    const int K = a.K, L = a.L;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const long pix = (long)blockIdx.x * WPB + wave;
+    if (pix >= (long)a.B * a.H1 * a.W1) return;
+    for (int k = 0; k < K; ++k) {
+        const float *pa = a.a + (pix * K + k) * L, *pg = a.grad_a + (pix * K + k) * L;
+        float dot = 0.f;
+        for (int l = lane; l < L; l += 64) dot += pa[l] * pg[l];
+        dot = wave_sum(dot);
+        float *dst = a.dlogits + (pix * K + k) * L;
+        for (int l = lane; l < L; l += 64) dst[l] = pa[l] * (pg[l] - dot);
+    }
+}
+
+// d_sep[(i,j),c,l] = sum_{k,dl,di,dj} w[k][c][dl][di][dj] * dlogits[(i-di+1, j-dj+1), k, l-dl+1]
+__global__ void __launch_bounds__(64 * WPB) att_input_backward_kernel(const AttArgs a) {
+    __shared__ float ws[MAXK * 54];
+    const int K = a.K, L = a.L, H1 = a.H1, W1 = a.W1;
+    for (int t = threadIdx.x; t < K * 54; t += blockDim.x) ws[t] = a.weight[t];
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const long pix = (long)blockIdx.x * WPB + wave;
+    if (pix >= (long)a.B * H1 * W1) return;
+    const int j = (int)(pix % W1), i = (int)((pix / W1) % H1);
+    for (int l = lane; l < L; l += 64) {
+        float d0 = 0.f, d1 = 0.f;
+        for (int di = 0; di < 3; ++di) {
+            const int ii = i - di + 1;
+            if (ii < 0 || ii >= H1) continue;
+            for (int dj = 0; dj < 3; ++dj) {
+                const int jj = j - dj + 1;
+                if (jj < 0 || jj >= W1) continue;
+                const float *g = a.dlogits + (pix + (long)(1 - di) * W1 + (1 - dj)) * K * L;
+                for (int k = 0; k < K; ++k)
+                    for (int dl = 0; dl < 3; ++dl) {
+                        const int ll = l - dl + 1;
+                        if (ll >= 0 && ll < L) {
+                            const float gv = g[k * L + ll];
+                            d0 += ws[((k * 2 + 0) * 3 + dl) * 9 + di * 3 + dj] * gv;
+                            d1 += ws[((k * 2 + 1) * 3 + dl) * 9 + di * 3 + dj] * gv;
+                        }
+                    }
+            }
+        }
+        a.out[(pix * 2 + 0) * L + l] = d0;
+        a.out[(pix * 2 + 1) * L + l] = d1;
+    }
+}
+
+// Weight and bias gradient, stage 1.  Workgroup (x, y): pixels [x*DW_PIX, ...), neighbour y = di*3+dj.
+// Wave w of the 4 handles every 4th pixel; per lane 6*K accumulators (c, dl, k); reduced over lanes and
+// waves, written as partial[x][...].
+__global__ void __launch_bounds__(256) att_weight_backward_kernel(const AttArgs a) {
+    __shared__ float red[4][6 * MAXK + MAXK];
+    const int K = a.K, L = a.L, H1 = a.H1, W1 = a.W1;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int di = blockIdx.y / 3, dj = blockIdx.y % 3;
+    const long npix = (long)a.B * H1 * W1;
+    const long p0 = (long)blockIdx.x * DW_PIX;
+    float acc[6 * MAXK], accb[MAXK];
+#pragma unroll
+    for (int t = 0; t < 6 * MAXK; ++t) acc[t] = 0.f;
+#pragma unroll
+    for (int t = 0; t < MAXK; ++t) accb[t] = 0.f;
+    for (int q = wave; q < DW_PIX; q += 4) {
+        const long pix = p0 + q;
+        if (pix >= npix) break;
+        const int j = (int)(pix % W1), i = (int)((pix / W1) % H1);
+        const int ii = i + di - 1, jj = j + dj - 1;
+        const bool inb = ii >= 0 && ii < H1 && jj >= 0 && jj < W1;
+        const float *g = a.dlogits + pix * K * L;
+        const float *row = a.sep + (pix + (long)(di - 1) * W1 + (dj - 1)) * 2 * L;
+        for (int l = lane; l < L; l += 64) {
+            float x[2][3];
+#pragma unroll
+            for (int c = 0; c < 2; ++c)
+#pragma unroll
+                for (int dl = 0; dl < 3; ++dl) {
+                    const int ll = l + dl - 1;
+                    x[c][dl] = (inb && ll >= 0 && ll < L) ? row[c * L + ll] : 0.f;
+                }
+#pragma unroll
+            for (int k = 0; k < MAXK; ++k) {
+                if (k < K) {
+                    const float gv = g[k * L + l];
+                    if (blockIdx.y == 4) accb[k] += gv;   // bias: counted once, by the centre tap
+#pragma unroll
+                    for (int c = 0; c < 2; ++c)
+#pragma unroll
+                        for (int dl = 0; dl < 3; ++dl) acc[(k * 2 + c) * 3 + dl] += gv * x[c][dl];
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < 6 * MAXK; ++t) {
+        const float r = wave_sum(acc[t]);
+        if (lane == 0) red[wave][t] = r;
+    }
+#pragma unroll
+    for (int t = 0; t < MAXK; ++t) {
+        const float r = wave_sum(accb[t]);
+        if (lane == 0) red[wave][6 * MAXK + t] = r;
+    }
+    __syncthreads();
+    // partial layout per workgroup x: [K*54 weights in weight order][K biases]
+    float *dst = a.partial + (long)blockIdx.x * (K * 54 + K);
+    for (int t = threadIdx.x; t < 6 * K; t += blockDim.x) {
+        const int k = t / 6, c = (t / 3) % 2, dl = t % 3;
+        dst[((k * 2 + c) * 3 + dl) * 9 + di * 3 + dj] = red[0][t] + red[1][t] + red[2][t] + red[3][t];
+    }
+    if (blockIdx.y == 4)
+        for (int t = threadIdx.x; t < K; t += blockDim.x)
+            dst[K * 54 + t] = red[0][6 * MAXK + t] + red[1][6 * MAXK + t] + red[2][6 * MAXK + t] + red[3][6 * MAXK + t];
+}
+
+// Stage 2: out[t] = sum over workgroups of partial[x][t], in order.  One workgroup per 256 outputs.
+__global__ void __launch_bounds__(256) att_weight_reduce_kernel(const float *partial, float *d_weight, float *d_bias, int nwg,
+                                                                int K) {
+    const int n = K * 54 + K;
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n) return;
+    float s = 0.f;
+    for (int x = 0; x < nwg; ++x) s += partial[(long)x * n + t];
+    if (t < K * 54) d_weight[t] = s;
+    else if (d_bias) d_bias[t - K * 54] = s;
+}
+
+int check(const void *p, const char *name) {
+    if (p) return 0;
+    char msg[128];
+    snprintf(msg, sizeof(msg), "sepcorr: argument %s is NULL", name);
+    return sepcorr_set_error(SEPCORR_EINVAL, msg);
+}
+#define REQ(p) if (int rc = check(p, #p)) return rc
+
+int check_sizes(int B, int H1, int W1, int L, int K) {
+    char msg[160];
+    if (B < 1 || H1 < 1 || W1 < 1 || L < 1 || K < 1 || K > MAXK) {
+        snprintf(msg, sizeof(msg), "sepcorr: attention sizes out of range (B=%d H1=%d W1=%d L=%d K=%d, K <= %d)", B, H1, W1, L, K, MAXK);
+        return sepcorr_set_error(SEPCORR_EINVAL, msg);
+    }
+    if ((double)B * H1 * W1 * K * L > 2147483647.0 || (double)B * H1 * W1 * 2 * L > 2147483647.0)
+        return sepcorr_set_error(SEPCORR_EINVAL, "sepcorr: a tensor would have 2^31 or more elements");
+    return 0;
+}
+
+int launched(const char *what) {
+    const hipError_t e = hipGetLastError();
+    if (e == hipSuccess) return 0;
+    char msg[200];
+    snprintf(msg, sizeof(msg), "sepcorr: %s: %s", what, hipGetErrorString(e));
+    return sepcorr_set_error(SEPCORR_ELAUNCH, msg);
+}
+
+size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+}  // namespace
+
+extern "C" {
+
+int sepcorr_attention_forward(const float *sep, const float *weight, const float *bias, float *a, int B, int H1, int W1, int L,
+                              int K, void *stream) {
+    REQ(sep); REQ(weight); REQ(a);
+    if (int rc = check_sizes(B, H1, W1, L, K)) return rc;
+    AttArgs args = {};
+    args.sep = sep; args.weight = weight; args.bias = bias; args.out = a;
+    args.B = B; args.H1 = H1; args.W1 = W1; args.L = L; args.K = K;
+    const long npix = (long)B * H1 * W1;
+    const dim3 grid((unsigned)((npix + WPB - 1) / WPB)), block(64 * WPB);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (L <= 64) hipLaunchKernelGGL(att_forward_kernel<1>, grid, block, 0, s, args);
+    else if (L <= 128) hipLaunchKernelGGL(att_forward_kernel<2>, grid, block, 0, s, args);
+    else if (L <= 256) hipLaunchKernelGGL(att_forward_kernel<4>, grid, block, 0, s, args);
+    else hipLaunchKernelGGL(att_forward_long_kernel, grid, block, 0, s, args);
+    return launched("attention forward kernel");
+}
+
+size_t sepcorr_attention_workspace_bytes(int B, int H1, int W1, int L, int K) {
+    if (B < 1 || H1 < 1 || W1 < 1 || L < 1 || K < 1 || K > MAXK) return 0;
+    const size_t npix = (size_t)B * H1 * W1;
+    const size_t nwg = (npix + DW_PIX - 1) / DW_PIX;
+    return align256(npix * K * L * sizeof(float)) + align256(nwg * (K * 54 + K) * sizeof(float));
+}
+
+int sepcorr_attention_backward(const float *sep, const float *weight, const float *a, const float *grad_a, float *d_sep,
+                               float *d_weight, float *d_bias, int B, int H1, int W1, int L, int K, void *workspace,
+                               size_t workspace_bytes, void *stream) {
+    REQ(sep); REQ(weight); REQ(a); REQ(grad_a); REQ(d_sep); REQ(d_weight);
+    if (int rc = check_sizes(B, H1, W1, L, K)) return rc;
+    const size_t need = sepcorr_attention_workspace_bytes(B, H1, W1, L, K);
+    if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15)) {
+        char msg[160];
+        snprintf(msg, sizeof(msg), "sepcorr: attention backward needs %zu bytes of 16-byte aligned workspace, got %zu", need,
+                 workspace ? workspace_bytes : (size_t)0);
+        return sepcorr_set_error(SEPCORR_EWORKSPACE, msg);
+    }
+    const long npix = (long)B * H1 * W1;
+    const int nwg = (int)((npix + DW_PIX - 1) / DW_PIX);
+    AttArgs args = {};
+    args.sep = sep; args.weight = weight; args.a = a; args.grad_a = grad_a;
+    args.dlogits = static_cast<float *>(workspace);
+    args.partial = reinterpret_cast<float *>(static_cast<char *>(workspace) + align256((size_t)npix * K * L * sizeof(float)));
+    args.B = B; args.H1 = H1; args.W1 = W1; args.L = L; args.K = K;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dim3 grid((unsigned)((npix + WPB - 1) / WPB)), block(64 * WPB);
+    hipLaunchKernelGGL(att_softmax_backward_kernel, grid, block, 0, s, args);
+    if (int rc = launched("attention softmax backward kernel")) return rc;
+    args.out = d_sep;
+    hipLaunchKernelGGL(att_input_backward_kernel, grid, block, 0, s, args);
+    if (int rc = launched("attention input gradient kernel")) return rc;
+    hipLaunchKernelGGL(att_weight_backward_kernel, dim3(nwg, 9), dim3(256), 0, s, args);
+    if (int rc = launched("attention weight gradient kernel")) return rc;
+    const int n = K * 54 + K;
+    hipLaunchKernelGGL(att_weight_reduce_kernel, dim3((n + 255) / 256), dim3(256), 0, s, args.partial, d_weight, d_bias, nwg, K);
+    return launched("attention weight gradient reduction");
+}
+
+}  // extern "C"

@@ -56,6 +56,15 @@ int fail(int code, const char *fmt, ...) {
     va_end(ap);
     return code;
 }
+}  // namespace
+
+// shared with the other translation units of the library (sepcorr_internal.h)
+int sepcorr_set_error(int code, const char *msg) {
+    snprintf(g_err, sizeof(g_err), "%s", msg);
+    return code;
+}
+
+namespace {
 
 // Row of the 32x32 accumulator held in register r of a lane in half h (lane / 32).
 __device__ __forceinline__ int vmap(int r, int h) { return 8 * (r >> 2) + 4 * h + (r & 3); }

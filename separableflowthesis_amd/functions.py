@@ -77,3 +77,25 @@ class ComputeSelfCompressionFunction(Function):
             d1, d2, da_u, da_v = MemorySaver.compression_backward(
                 f1, f2, a_u, a_v, grad_compressed_output_u, grad_compressed_output_v)
         return d1.contiguous(), d2.contiguous(), da_u.contiguous(), da_v.contiguous()
+
+
+class AttentionWeightsFunction(Function):
+    """softmax over L of Conv3d(2 -> K, 3, padding=1) of a max/avg volume, in the operator's layout.
+
+    Not a class of the reference: it stands for the torch ops the caller runs between the two operators
+    (core/corr.py:437-446: attention(sep).softmax(dim=2) wrapped in two permutes), with the same result.
+    """
+
+    @staticmethod
+    def forward(ctx, sep, weight, bias):
+        _contig(sep, weight)
+        a = MemorySaver.attention_forward(sep, weight, bias)
+        ctx.save_for_backward(sep, weight, a)
+        ctx.has_bias = bias is not None
+        return a
+
+    @staticmethod
+    def backward(ctx, grad_a):
+        sep, weight, a = ctx.saved_tensors
+        d_sep, d_w, d_b = MemorySaver.attention_backward(sep, weight, a, grad_a.contiguous(), need_bias=ctx.has_bias)
+        return d_sep, d_w, d_b

@@ -54,6 +54,32 @@ def test_corr_block_matches_full_4d_corr_block(device, B, C, H, W, K, backward):
             assert_close(m.bias.grad, rm.bias.grad, n + ".bias.grad", scale_atol=True)
 
 
+@pytest.mark.parametrize("B,H1,W1,L,K", [(1, 3, 4, 5, 1), (2, 9, 13, 70, 4), (1, 6, 10, 128, 4), (1, 4, 5, 200, 3),
+                                          (1, 3, 6, 300, 2), (1, 2, 3, 1, 8)])
+def test_attention_producer_matches_conv3d_softmax(device, B, H1, W1, L, K):
+    from separableflowthesis_amd import MemorySaver
+    g = torch.Generator().manual_seed(11)
+    sep = torch.randn(B, H1, W1, 2, L, generator=g)
+    w = torch.randn(K, 2, 3, 3, 3, generator=g) * 0.3
+    bias = torch.randn(K, generator=g)
+    grad = torch.randn(B, H1, W1, K, L, generator=g)
+    r = [t.double().requires_grad_() for t in (sep, w, bias)]
+    ra = O.attention_weights(*r)
+    (ra * grad.double()).sum().backward()
+    d = lambda t: t.to(device)
+    a = MemorySaver.attention_forward(d(sep), d(w), d(bias))
+    assert_close(a, ra, "attention weights")
+    ds, dw, db = MemorySaver.attention_backward(d(sep), d(w), a, d(grad))
+    assert_close(ds, r[0].grad, "d_sep", scale_atol=True)
+    assert_close(dw, r[1].grad, "d_weight", scale_atol=True)
+    assert_close(db, r[2].grad, "d_bias", scale_atol=True)
+    again = MemorySaver.attention_backward(d(sep), d(w), a, d(grad))
+    assert all(torch.equal(x, y) for x, y in zip((ds, dw, db), again))
+    # without bias
+    a2 = MemorySaver.attention_forward(d(sep), d(w), None)
+    assert_close(a2, O.attention_weights(sep.double(), w.double(), None), "attention weights, no bias")
+
+
 def _native():
     from separableflowthesis_amd import MemorySaver
     return MemorySaver

@@ -280,6 +280,44 @@ def test_out_of_range_argmax_selects_nothing():
     assert np.all(l1 == 0) and np.all(l2 == 0)
 
 
+# ---- attention-weight producer ---------------------------------------------------------------------
+
+def test_attention_weights_closed_forms():
+    g = gen(21)
+    B, H1, W1, L, K = 1, 3, 4, 6, 2
+    sep = rnd(B, H1, W1, 2, L, g=g)
+    w = torch.zeros(K, 2, 3, 3, 3, dtype=D)
+    # zero weights: uniform softmax, whatever the bias
+    a = O.attention_weights(sep, w, torch.tensor([0.3, -2.0], dtype=D))
+    assert a.shape == (B, H1, W1, K, L) and torch.allclose(a, torch.full_like(a, 1 / L))
+    # centre tap on channel c: softmax of the pixel's own row
+    w[0, 1, 1, 1, 1] = 2.0
+    a = O.attention_weights(sep, w, None)
+    assert torch.allclose(a[:, :, :, 0], (2.0 * sep[:, :, :, 1]).softmax(-1))
+    # tap dl=2 reads l+1 (cross-correlation, zero padded); tap di=0 reads row i-1; tap dj=2 reads column j+1
+    w.zero_(); w[1, 0, 2, 1, 1] = 1.0
+    shifted = torch.cat((sep[:, :, :, 0, 1:], torch.zeros(B, H1, W1, 1, dtype=D)), dim=-1)
+    assert torch.allclose(O.attention_weights(sep, w, None)[:, :, :, 1], shifted.softmax(-1))
+    w.zero_(); w[0, 0, 1, 0, 1] = 1.0
+    up = torch.cat((torch.zeros(B, 1, W1, L, dtype=D), sep[:, :-1, :, 0]), dim=1)
+    assert torch.allclose(O.attention_weights(sep, w, None)[:, :, :, 0], up.softmax(-1))
+    w.zero_(); w[0, 1, 1, 1, 2] = 1.0
+    right = torch.cat((sep[:, :, 1:, 1], torch.zeros(B, H1, 1, L, dtype=D)), dim=2)
+    assert torch.allclose(O.attention_weights(sep, w, None)[:, :, :, 0], right.softmax(-1))
+    # rows sum to one
+    a = O.attention_weights(sep, rnd(K, 2, 3, 3, 3, g=g), rnd(K, g=g))
+    assert torch.allclose(a.sum(-1), torch.ones(B, H1, W1, K, dtype=D))
+
+
+def test_attention_weights_equal_the_module_path():
+    # the same numbers as the caller's torch.nn.Conv3d module applied to the permuted volume
+    torch.manual_seed(3)
+    conv = torch.nn.Conv3d(2, 3, 3, padding=1).double()
+    sep = rnd(2, 4, 5, 2, 7)
+    ref = conv(sep.permute(0, 3, 4, 1, 2)).softmax(dim=2).permute(0, 3, 4, 1, 2)
+    assert torch.allclose(O.attention_weights(sep, conv.weight, conv.bias), ref, atol=1e-14)
+
+
 # ---- module level ---------------------------------------------------------------------------------
 
 def test_corrblock4d_level0_equals_op_level_and_scaling():
