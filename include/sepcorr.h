@@ -143,6 +143,22 @@ int sepcorr_attention_backward(const float *sep, const float *weight, const floa
                                int B, int H1, int W1, int L, int K,
                                void *workspace, size_t workspace_bytes, void *stream);
 
+/*
+ * Assembly of a module-level volume from operator-level outputs.  Writes channels [c0, c0+ch) of
+ * dst (B,CT,L0,H1,W1) from src (B,H1,W1,ch,Li):
+ *   dst[b,c0+c,l0,i,j] = linear interpolation (align_corners=True) of src[b,i,j,c,:] at l0 * (Li-1)/(L0-1).
+ * Replaces, per level and per operator output, the caller's permute(0,3,4,1,2), torch.cat over channels,
+ * F.interpolate(..., [L0,h1,w1], mode='trilinear', align_corners=True) and the torch.cat over levels
+ * (core/corr.py:428-429, 451-475); H1 and W1 keep their size there, so only L is interpolated.
+ * Limits: Li and L0 up to about 500 (one LDS tile), B*ch < 65536.
+ */
+int sepcorr_assemble_forward(const float *src, float *dst, int B, int H1, int W1, int ch, int Li,
+                             int CT, int c0, int L0, void *stream);
+
+/* Adjoint of the above: grad_src (B,H1,W1,ch,Li), fully overwritten, from grad_dst (B,CT,L0,H1,W1). */
+int sepcorr_assemble_backward(const float *grad_dst, float *grad_src, int B, int H1, int W1, int ch, int Li,
+                              int CT, int c0, int L0, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -192,3 +192,40 @@ def attention_backward(sep, weight, a, grad_a, need_bias=True):
                                                   d_sep.data_ptr(), d_w.data_ptr(), d_b.data_ptr() if need_bias else None,
                                                   B, H1, W1, L, K, ws.data_ptr(), n, _stream()))
     return [d_sep, d_w, d_b]
+
+
+def assemble_forward(srcs, L0):
+    """srcs: operator outputs (B,H1,W1,ch_n,L_n) in channel order -> (B, sum ch_n, L0, H1, W1), each one
+    transposed and linearly interpolated along its last axis to length L0 (align_corners=True)."""
+    for n, t in enumerate(srcs):
+        _check(f"srcs[{n}]", t, ndim=5)
+    B, H1, W1 = srcs[0].shape[:3]
+    CT = sum(t.shape[3] for t in srcs)
+    lib = _lib.load()
+    with torch.cuda.device(srcs[0].device):
+        dst = torch.empty((B, CT, L0, H1, W1), dtype=srcs[0].dtype, device=srcs[0].device)
+        c0 = 0
+        for t in srcs:
+            if tuple(t.shape[:3]) != (B, H1, W1) or t.device != dst.device:
+                raise RuntimeError("assemble: all sources must share batch, H1, W1 and device")
+            _lib.check(lib.sepcorr_assemble_forward(t.data_ptr(), dst.data_ptr(), B, H1, W1, t.shape[3], t.shape[4],
+                                                    CT, c0, L0, _stream()))
+            c0 += t.shape[3]
+    return dst
+
+
+def assemble_backward(grad_dst, shapes):
+    """grad_dst (B,CT,L0,H1,W1) -> list of gradients with the given source shapes (B,H1,W1,ch_n,L_n)."""
+    _check("grad_dst", grad_dst, ndim=5)
+    B, CT, L0, H1, W1 = grad_dst.shape
+    lib = _lib.load()
+    out = []
+    with torch.cuda.device(grad_dst.device):
+        c0 = 0
+        for shp in shapes:
+            g = torch.empty(shp, dtype=grad_dst.dtype, device=grad_dst.device)
+            _lib.check(lib.sepcorr_assemble_backward(grad_dst.data_ptr(), g.data_ptr(), B, H1, W1, shp[3], shp[4],
+                                                     CT, c0, L0, _stream()))
+            c0 += shp[3]
+            out.append(g)
+    return out

@@ -27,6 +27,8 @@ SIGNATURES = {
     "sepcorr_attention_forward": (_I, [_P] * 4 + [_I] * 5 + [_P]),
     "sepcorr_attention_workspace_bytes": (_SZ, [_I] * 5),
     "sepcorr_attention_backward": (_I, [_P] * 7 + [_I] * 5 + [_P, _SZ, _P]),
+    "sepcorr_assemble_forward": (_I, [_P] * 2 + [_I] * 8 + [_P]),
+    "sepcorr_assemble_backward": (_I, [_P] * 2 + [_I] * 8 + [_P]),
 }
 
 _lib = None

@@ -10,8 +10,8 @@ trilinearly upsampled (align_corners=True) to the level-0 displacement length.
 import torch
 import torch.nn.functional as F
 
-from .functions import (AttentionWeightsFunction, ComputeMaxArgmaxAvgFunction, ComputeMaxAvgFunction,
-                        ComputeSelfCompressionFunction)
+from .functions import (AssembleVolumeFunction, AttentionWeightsFunction, ComputeMaxArgmaxAvgFunction,
+                        ComputeMaxAvgFunction, ComputeSelfCompressionFunction)
 
 
 def _is_reference_attention(m):
@@ -46,12 +46,27 @@ class AlternateCorrBlockSepflow:
     def separate(self, attention_weights):
         batch, fdim, h1, w1 = self.fmap1_l0.shape
         h2, w2 = h1, w1
-        sep_u_lvls, sep_v_lvls = [], []
         # the scaled NHWC copy of fmap1 is level independent; made once (the reference redoes it per level)
         fmap1 = self.fmap1_l0.permute(0, 2, 3, 1).contiguous() / torch.sqrt(torch.tensor(fdim).float())
+        fused = fmap1.is_cuda and max(h2, w2) <= 500 and (
+            attention_weights is None or all(_is_reference_attention(m) for m in attention_weights))
+        parts_u, parts_v = [], []      # operator outputs in final channel order (fused path)
+        sep_u_lvls, sep_v_lvls = [], []
         for i in range(self.num_levels):
             fmap2 = self.pyramid[i].permute(0, 2, 3, 1).contiguous()
             maxavg_u, maxavg_v = self.max_avg_function.apply(fmap1, fmap2)
+            if fused:
+                # everything stays in the operator's layout; one kernel per output assembles the result
+                parts_u.append(maxavg_v)
+                parts_v.append(maxavg_u)
+                if attention_weights is not None:
+                    attention1, attention2 = attention_weights
+                    a_u = AttentionWeightsFunction.apply(maxavg_v, attention1.weight.contiguous(), attention1.bias)
+                    a_v = AttentionWeightsFunction.apply(maxavg_u, attention2.weight.contiguous(), attention2.bias)
+                    adaptive_corr_u, adaptive_corr_v = ComputeSelfCompressionFunction.apply(fmap1, fmap2, a_u, a_v)
+                    parts_v.append(adaptive_corr_u)
+                    parts_u.append(adaptive_corr_v)
+                continue
             sep_v = maxavg_u.permute(0, 3, 4, 1, 2).contiguous()   # (B,2,H2_i,h1,w1)
             sep_u = maxavg_v.permute(0, 3, 4, 1, 2).contiguous()   # (B,2,W2_i,h1,w1)
             if attention_weights is not None:
@@ -64,6 +79,8 @@ class AlternateCorrBlockSepflow:
                 sep_u = torch.cat((sep_u, adaptive_corr_v.permute(0, 3, 4, 1, 2)), dim=1)
             sep_u_lvls.append(F.interpolate(sep_u, [w2, h1, w1], mode='trilinear', align_corners=True))
             sep_v_lvls.append(F.interpolate(sep_v, [h2, h1, w1], mode='trilinear', align_corners=True))
+        if fused:
+            return AssembleVolumeFunction.apply(w2, *parts_u), AssembleVolumeFunction.apply(h2, *parts_v)
         return torch.cat(sep_u_lvls, dim=1), torch.cat(sep_v_lvls, dim=1)
 
     def __call__(self, coords, sep=False, attention_weights=None):

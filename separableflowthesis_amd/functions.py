@@ -99,3 +99,21 @@ class AttentionWeightsFunction(Function):
         sep, weight, a = ctx.saved_tensors
         d_sep, d_w, d_b = MemorySaver.attention_backward(sep, weight, a, grad_a.contiguous(), need_bias=ctx.has_bias)
         return d_sep, d_w, d_b
+
+
+class AssembleVolumeFunction(Function):
+    """Operator outputs of all levels -> one module-level volume (B, channels, L0, H1, W1).
+
+    Not a class of the reference: it stands for the caller's permute / cat / trilinear interpolate / cat
+    chain (core/corr.py:428-429, 451-475) with the same result.
+    """
+
+    @staticmethod
+    def forward(ctx, L0, *srcs):
+        _contig(*srcs)
+        ctx.shapes = [tuple(t.shape) for t in srcs]
+        return MemorySaver.assemble_forward(srcs, L0)
+
+    @staticmethod
+    def backward(ctx, grad):
+        return (None,) + tuple(MemorySaver.assemble_backward(grad.contiguous(), ctx.shapes))

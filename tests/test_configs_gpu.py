@@ -80,6 +80,28 @@ def test_attention_producer_matches_conv3d_softmax(device, B, H1, W1, L, K):
     assert_close(a2, O.attention_weights(sep.double(), w.double(), None), "attention weights, no bias")
 
 
+@pytest.mark.parametrize("B,H1,W1,L0,specs", [
+    (1, 3, 5, 8, [(2, 8), (3, 8), (2, 4), (1, 2), (2, 1)]),
+    (2, 7, 40, 33, [(2, 33), (4, 33), (2, 16), (4, 16), (2, 8), (2, 4)]),
+    (1, 2, 3, 1, [(2, 1)]),
+])
+def test_assemble_matches_permute_cat_interpolate(device, B, H1, W1, L0, specs):
+    from separableflowthesis_amd import MemorySaver
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(4)
+    srcs = [torch.randn(B, H1, W1, ch, Li, generator=g) for ch, Li in specs]
+    ref_in = [t.double().requires_grad_() for t in srcs]
+    ref = torch.cat([F.interpolate(t.permute(0, 3, 4, 1, 2), [L0, H1, W1], mode='trilinear', align_corners=True)
+                     for t in ref_in], dim=1)
+    got = MemorySaver.assemble_forward([t.to(device) for t in srcs], L0)
+    assert_close(got, ref, "assembled volume")
+    grad = torch.randn(ref.shape, generator=g)
+    (ref * grad.double()).sum().backward()
+    back = MemorySaver.assemble_backward(grad.to(device), [tuple(t.shape) for t in srcs])
+    for x, r, n in zip(back, ref_in, range(len(srcs))):
+        assert_close(x, r.grad, f"grad of source {n}")
+
+
 def _native():
     from separableflowthesis_amd import MemorySaver
     return MemorySaver
