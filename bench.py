@@ -99,6 +99,36 @@ def cpu_baseline(B, H, W, C, Kp, ops, torch, budget_s=20.0):
     }
 
 
+def module_level(B, H, W, C, Kp, torch, dev, reps=5):
+    """The caller's whole separate() over 4 pyramid levels through the drop-in classes (untimed extra):
+    NHWC copies, both operators per level, the fused attention producer and volume assembly, autograd."""
+    from separableflowthesis_amd import AlternateCorrBlockSepflow
+    g = torch.Generator().manual_seed(1234)
+    fmap1 = torch.randn(B, C, H, W, generator=g).to(dev).requires_grad_()
+    fmap2 = torch.randn(B, C, H, W, generator=g).to(dev).requires_grad_()
+    torch.manual_seed(1234)
+    att = tuple(torch.nn.Conv3d(2, Kp, 3, padding=1).to(dev) for _ in range(2)) if Kp else None
+
+    def run(backward):
+        blk = AlternateCorrBlockSepflow(fmap1, fmap2, None, 4, 4, support_backward=backward)
+        c1, c2 = blk(None, sep=True, attention_weights=att)
+        if backward:
+            (c1.sum() + c2.sum()).backward()
+
+    out = {}
+    for name, bw in (("forward_ms", False), ("forward_backward_ms", True)):
+        for _ in range(2):
+            run(bw)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            run(bw)
+        torch.cuda.synchronize()
+        out[name] = round((time.perf_counter() - t0) / reps * 1e3, 3)
+    out["what"] = f"AlternateCorrBlockSepflow.separate, 4 levels, B={B}, C={C}, {H}x{W}, K'={Kp}, torch autograd around the native ops"
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -229,6 +259,7 @@ def main():
         "kernels": kernels,
     }
     if not args.no_cpu_baseline:
+        out["module_level"] = module_level(B, H, W, C, Kp, torch, dev)
         out["cpu_baseline"] = cpu_baseline(B, H, W, C, Kp, ops, torch)
     print(json.dumps(out))
 
