@@ -269,16 +269,21 @@ __global__ void __launch_bounds__(256) att_weight_backward_kernel(const AttArgs 
             dst[K * 54 + t] = red[0][6 * MAXK + t] + red[1][6 * MAXK + t] + red[2][6 * MAXK + t] + red[3][6 * MAXK + t];
 }
 
-// Stage 2: out[t] = sum over workgroups of partial[x][t], in order.  One workgroup per 256 outputs.
+// Stage 2: out[t] = sum over workgroups of partial[x][t].  One wave per output: lane l adds the partials
+// x = l, l+64, ... in order, then the 64 lane sums are added by a fixed butterfly: deterministic.
 __global__ void __launch_bounds__(256) att_weight_reduce_kernel(const float *partial, float *d_weight, float *d_bias, int nwg,
                                                                 int K) {
     const int n = K * 54 + K;
-    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (t >= n) return;
     float s = 0.f;
-    for (int x = 0; x < nwg; ++x) s += partial[(long)x * n + t];
-    if (t < K * 54) d_weight[t] = s;
-    else if (d_bias) d_bias[t - K * 54] = s;
+    for (int x = lane; x < nwg; x += 64) s += partial[(long)x * n + t];
+    s = wave_sum(s);
+    if (lane == 0) {
+        if (t < K * 54) d_weight[t] = s;
+        else if (d_bias) d_bias[t - K * 54] = s;
+    }
 }
 
 int check(const void *p, const char *name) {
@@ -367,7 +372,7 @@ int sepcorr_attention_backward(const float *sep, const float *weight, const floa
     hipLaunchKernelGGL(att_weight_backward_kernel, dim3(nwg, 9), dim3(256), 0, s, args);
     if (int rc = launched("attention weight gradient kernel")) return rc;
     const int n = K * 54 + K;
-    hipLaunchKernelGGL(att_weight_reduce_kernel, dim3((n + 255) / 256), dim3(256), 0, s, args.partial, d_weight, d_bias, nwg, K);
+    hipLaunchKernelGGL(att_weight_reduce_kernel, dim3((n + 3) / 4), dim3(256), 0, s, args.partial, d_weight, d_bias, nwg, K);
     return launched("attention weight gradient reduction");
 }
 
