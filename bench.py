@@ -139,7 +139,12 @@ def main():
     ap.add_argument("--profile-steps", type=int, default=5)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three 256 MiB device copies (known traffic) for scaling rocprofv3 FETCH_SIZE/WRITE_SIZE")
+    ap.add_argument("--single-stream", action="store_true",
+                    help="keep all kernels of a call on the caller's stream (per-kernel durations under a profiler are "
+                         "then those of kernels running alone)")
     args = ap.parse_args()
+    if args.single_stream:
+        os.environ["SEPCORR_SINGLE_STREAM"] = "1"
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
 
