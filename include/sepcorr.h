@@ -85,7 +85,7 @@ int sepcorr_compression_forward(const float *f1, const float *f2, const float *a
                                 float *comp_u, float *comp_v,
                                 int B, int H1, int W1, int H2, int W2, int C, int K, void *stream);
 
-/* Scratch bytes needed by either backward entry point for these sizes (0 is possible). */
+/* Scratch bytes needed by any of the three backward entry points for these sizes (0 is possible). */
 size_t sepcorr_backward_workspace_bytes(int B, int H1, int W1, int H2, int W2, int C);
 
 /*
@@ -110,12 +110,30 @@ int sepcorr_max_argmax_avg_backward(const float *f1, const float *f2,
  *   G = sum_k a_u[..,k,v]*g_cu[..,k,u] + a_v[..,k,u]*g_cv[..,k,v]
  *   d_f1 = sum_{u,v} G f2      d_f2 = sum_{i,j} G f1
  *   d_a_u[b,i,j,k,v] = sum_u S * g_cu[b,i,j,k,u]      d_a_v[b,i,j,k,u] = sum_v S * g_cv[b,i,j,k,v]
+ * d_f1 and d_f2 may both be NULL: then only d_a_u and d_a_v are computed (one sweep, no workspace needed).
  */
 int sepcorr_compression_backward(const float *f1, const float *f2, const float *a_u, const float *a_v,
                                  const float *g_cu, const float *g_cv,
                                  float *d_f1, float *d_f2, float *d_a_u, float *d_a_v,
                                  int B, int H1, int W1, int H2, int W2, int C, int K,
                                  void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Feature gradients of both operators of one pyramid level in one pass; no counterpart in the reference,
+ * whose two backward functions (MemorySaver_cuda.cpp:55-103) each contract their own dL/dS.  With G the sum
+ * of the two expressions given above for sepcorr_max_argmax_avg_backward and sepcorr_compression_backward,
+ *   d_f1 = sum_{u,v} G f2      d_f2 = sum_{i,j} G f1
+ * i.e. the sum of the d_f1 (d_f2) the two calls would return, from 2 sweeps over the volume instead of 4.
+ * For callers that have the complete gradient of the max/avg outputs before they need feature gradients
+ * (in core/corr.py:437-448 it arrives through d_a_u/d_a_v and the attention weights' producer).
+ */
+int sepcorr_fused_backward(const float *f1, const float *f2,
+                           const int32_t *argmax_u, const int32_t *argmax_v,
+                           const float *grad_u, const float *grad_v,
+                           const float *a_u, const float *a_v, const float *g_cu, const float *g_cv,
+                           float *d_f1, float *d_f2,
+                           int B, int H1, int W1, int H2, int W2, int C, int K,
+                           void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * Attention-weight producer in the operator's layout.  Replaces, for one of the two volumes, the caller's

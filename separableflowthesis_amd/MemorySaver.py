@@ -151,6 +151,63 @@ def compression_backward(img1_features_l0, img2_features_lk, attention_weights_u
     return [d1, d2, da_u, da_v]
 
 
+# --- not part of the reference's native module: both backward passes of one pyramid level in one
+
+def compression_weight_gradients(img1_features_l0, img2_features_lk, attention_weights_u, attention_weights_v,
+                                 grad_compressed_output_u, grad_compressed_output_v):
+    """-> [grad_attention_u (B,H1,W1,K,W2), grad_attention_v (B,H1,W1,K,H2)]: compression_backward without the
+    feature gradients (one sweep over the volume instead of three)."""
+    f1, f2 = img1_features_l0, img2_features_lk
+    B, H1, W1, H2, W2, C = _dims(f1, f2)
+    dev = f1.device
+    _check("attention_weights_u", attention_weights_u, ndim=5)
+    K = attention_weights_u.shape[3]
+    _expect("attention_weights_u", attention_weights_u, (B, H1, W1, K, W2), dev)
+    _expect("attention_weights_v", attention_weights_v, (B, H1, W1, K, H2), dev)
+    _expect("grad_compressed_output_u", grad_compressed_output_u, (B, H1, W1, K, H2), dev)
+    _expect("grad_compressed_output_v", grad_compressed_output_v, (B, H1, W1, K, W2), dev)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        da_u = torch.empty_like(attention_weights_u)
+        da_v = torch.empty_like(attention_weights_v)
+        _lib.check(lib.sepcorr_compression_backward(
+            f1.data_ptr(), f2.data_ptr(), attention_weights_u.data_ptr(), attention_weights_v.data_ptr(),
+            grad_compressed_output_u.data_ptr(), grad_compressed_output_v.data_ptr(),
+            None, None, da_u.data_ptr(), da_v.data_ptr(), B, H1, W1, H2, W2, C, K, None, 0, _stream()))
+    return [da_u, da_v]
+
+
+def fused_backward(img1_features_l0, img2_features_lk, argmax_output_u, argmax_output_v, grad_MaxAvg_u, grad_MaxAvg_v,
+                   attention_weights_u, attention_weights_v, grad_compressed_output_u, grad_compressed_output_v):
+    """-> [grad_fmap1_l0, grad_fmap2_lk]: the sum of what max_argmax_avg_backward and compression_backward return
+    for the features, from one contraction per output (dL/dS of both operators is added before it is used)."""
+    f1, f2 = img1_features_l0, img2_features_lk
+    B, H1, W1, H2, W2, C = _dims(f1, f2)
+    dev = f1.device
+    _check("attention_weights_u", attention_weights_u, ndim=5)
+    K = attention_weights_u.shape[3]
+    _expect("argmax_output_u", argmax_output_u, (B, H1, W1, 1, H2), dev, torch.int32)
+    _expect("argmax_output_v", argmax_output_v, (B, H1, W1, 1, W2), dev, torch.int32)
+    _expect("grad_MaxAvg_u", grad_MaxAvg_u, (B, H1, W1, 2, H2), dev)
+    _expect("grad_MaxAvg_v", grad_MaxAvg_v, (B, H1, W1, 2, W2), dev)
+    _expect("attention_weights_u", attention_weights_u, (B, H1, W1, K, W2), dev)
+    _expect("attention_weights_v", attention_weights_v, (B, H1, W1, K, H2), dev)
+    _expect("grad_compressed_output_u", grad_compressed_output_u, (B, H1, W1, K, H2), dev)
+    _expect("grad_compressed_output_v", grad_compressed_output_v, (B, H1, W1, K, W2), dev)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        d1 = torch.empty_like(f1)
+        d2 = torch.empty_like(f2)
+        ws, n = _workspace(lib, (B, H1, W1, H2, W2, C), dev)
+        _lib.check(lib.sepcorr_fused_backward(
+            f1.data_ptr(), f2.data_ptr(), argmax_output_u.data_ptr(), argmax_output_v.data_ptr(),
+            grad_MaxAvg_u.data_ptr(), grad_MaxAvg_v.data_ptr(),
+            attention_weights_u.data_ptr(), attention_weights_v.data_ptr(),
+            grad_compressed_output_u.data_ptr(), grad_compressed_output_v.data_ptr(),
+            d1.data_ptr(), d2.data_ptr(), B, H1, W1, H2, W2, C, K, ws.data_ptr(), n, _stream()))
+    return [d1, d2]
+
+
 # --- not part of the reference's native module: the attention-weight producer the caller runs between
 # --- the two operators (core/corr.py:437-446), fused and in the operator's layout
 

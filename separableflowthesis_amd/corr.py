@@ -11,7 +11,7 @@ import torch
 import torch.nn.functional as F
 
 from .functions import (AssembleVolumeFunction, AttentionWeightsFunction, ComputeMaxArgmaxAvgFunction,
-                        ComputeMaxAvgFunction, ComputeSelfCompressionFunction)
+                        ComputeMaxAvgFunction, ComputeSelfCompressionFunction, SeparateLevelFunction)
 
 
 def _is_reference_attention(m):
@@ -54,6 +54,15 @@ class AlternateCorrBlockSepflow:
         sep_u_lvls, sep_v_lvls = [], []
         for i in range(self.num_levels):
             fmap2 = self.pyramid[i].permute(0, 2, 3, 1).contiguous()
+            if fused and attention_weights is not None and self.max_avg_function is ComputeMaxArgmaxAvgFunction:
+                # the whole level as one autograd node: its backward contracts dL/dS of both operators once
+                attention1, attention2 = attention_weights
+                maxavg_u, maxavg_v, adaptive_corr_u, adaptive_corr_v = SeparateLevelFunction.apply(
+                    fmap1, fmap2, attention1.weight.contiguous(), attention1.bias,
+                    attention2.weight.contiguous(), attention2.bias)
+                parts_u += [maxavg_v, adaptive_corr_v]
+                parts_v += [maxavg_u, adaptive_corr_u]
+                continue
             maxavg_u, maxavg_v = self.max_avg_function.apply(fmap1, fmap2)
             if fused:
                 # everything stays in the operator's layout; one kernel per output assembles the result

@@ -652,7 +652,10 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
 // ------------------------------------------------------------------------------------------
 // backward: G synthesis shared by df1 / df2
 // ------------------------------------------------------------------------------------------
-enum { GMODE_MAXAVG = 0, GMODE_COMP = 1 };
+// GMODE_BOTH: G is the sum of the two, so that one contraction serves both gradients
+enum { GMODE_MAXAVG = 0, GMODE_COMP = 1, GMODE_BOTH = 2 };
+constexpr bool g_has_comp(int gmode) { return gmode != GMODE_MAXAVG; }
+constexpr bool g_has_maxavg(int gmode) { return gmode != GMODE_COMP; }
 
 struct BwdArgs {
     const float *f1, *f2;
@@ -671,34 +674,39 @@ struct BwdArgs {
     int accumulate;                  // add to the destination instead of overwriting
 };
 
-// Weights of one lane that depend on (p, v) and on (p, u).
+// Weights of one lane that depend on (p, v) and on (p, u).  Members a mode does not use stay unset and
+// cost no registers.
 template <int GMODE, int KC>
 struct VW {
-    float a[GMODE == GMODE_COMP ? KC : 1];   // maxavg: g_v[max];        comp: a_u[k]
-    float g[GMODE == GMODE_COMP ? KC : 1];   // maxavg: g_v[avg] / H2;   comp: g_cv[k]
-    int am;                                  // maxavg: argmax_v
+    float a[KC];   // comp: a_u[k]
+    float g[KC];   // comp: g_cv[k]
+    float ma;      // maxavg: g_v[max]
+    float mg;      // maxavg: g_v[avg] / H2
+    int am;        // maxavg: argmax_v
 };
 template <int GMODE, int KC>
 struct UW {
-    float a[GMODE == GMODE_COMP ? KC : 1];   // maxavg: g_u[max];        comp: a_v[k]
-    float g[GMODE == GMODE_COMP ? KC : 1];   // maxavg: g_u[avg] / W2;   comp: g_cu[k]
-    int am;                                  // maxavg: argmax_u
+    float a[KC];   // comp: a_v[k]
+    float g[KC];   // comp: g_cu[k]
+    float ma;      // maxavg: g_u[max]
+    float mg;      // maxavg: g_u[avg] / W2
+    int am;        // maxavg: argmax_u
 };
 
 template <int GMODE, int KC>
 __device__ __forceinline__ VW<GMODE, KC> load_vw(const BwdArgs &a, size_t bp, int v, bool ok) {
     VW<GMODE, KC> w;
-    if constexpr (GMODE == GMODE_COMP) {
+    if constexpr (g_has_comp(GMODE)) {
 #pragma unroll
         for (int k = 0; k < KC; ++k) {
             const size_t o = (bp * a.KT + a.k0 + k) * a.W2 + v;
             w.a[k] = ok ? a.a_u[o] : 0.f;
             w.g[k] = ok ? a.g_cv[o] : 0.f;
         }
-        w.am = 0;
-    } else {
-        w.a[0] = ok ? a.g_v[(bp * 2 + 0) * a.W2 + v] : 0.f;
-        w.g[0] = ok ? a.g_v[(bp * 2 + 1) * a.W2 + v] / (float)a.H2 : 0.f;
+    }
+    if constexpr (g_has_maxavg(GMODE)) {
+        w.ma = ok ? a.g_v[(bp * 2 + 0) * a.W2 + v] : 0.f;
+        w.mg = ok ? a.g_v[(bp * 2 + 1) * a.W2 + v] / (float)a.H2 : 0.f;
         w.am = ok ? a.am_v[bp * a.W2 + v] : -1;
     }
     return w;
@@ -706,17 +714,17 @@ __device__ __forceinline__ VW<GMODE, KC> load_vw(const BwdArgs &a, size_t bp, in
 template <int GMODE, int KC>
 __device__ __forceinline__ UW<GMODE, KC> load_uw(const BwdArgs &a, size_t bp, int u, bool ok) {
     UW<GMODE, KC> w;
-    if constexpr (GMODE == GMODE_COMP) {
+    if constexpr (g_has_comp(GMODE)) {
 #pragma unroll
         for (int k = 0; k < KC; ++k) {
             const size_t o = (bp * a.KT + a.k0 + k) * a.H2 + u;
             w.a[k] = ok ? a.a_v[o] : 0.f;
             w.g[k] = ok ? a.g_cu[o] : 0.f;
         }
-        w.am = 0;
-    } else {
-        w.a[0] = ok ? a.g_u[(bp * 2 + 0) * a.H2 + u] : 0.f;
-        w.g[0] = ok ? a.g_u[(bp * 2 + 1) * a.H2 + u] / (float)a.W2 : 0.f;
+    }
+    if constexpr (g_has_maxavg(GMODE)) {
+        w.ma = ok ? a.g_u[(bp * 2 + 0) * a.H2 + u] : 0.f;
+        w.mg = ok ? a.g_u[(bp * 2 + 1) * a.H2 + u] / (float)a.W2 : 0.f;
         w.am = ok ? a.am_u[bp * a.H2 + u] : -1;
     }
     return w;
@@ -725,13 +733,14 @@ __device__ __forceinline__ UW<GMODE, KC> load_uw(const BwdArgs &a, size_t bp, in
 template <int GMODE, int KC>
 __device__ __forceinline__ float gval(const VW<GMODE, KC> &wv, const UW<GMODE, KC> &wu, int u, int v, bool ok) {
     float g = 0.f;
-    if constexpr (GMODE == GMODE_COMP) {
+    if constexpr (g_has_comp(GMODE)) {
 #pragma unroll
         for (int k = 0; k < KC; ++k) g += wv.a[k] * wu.g[k] + wu.a[k] * wv.g[k];
-    } else {
-        g = wu.g[0] + wv.g[0];
-        if (wu.am == v) g += wu.a[0];
-        if (wv.am == u) g += wv.a[0];
+    }
+    if constexpr (g_has_maxavg(GMODE)) {
+        g += wu.mg + wv.mg;
+        if (wu.am == v) g += wu.ma;
+        if (wv.am == u) g += wv.ma;
     }
     return ok ? g : 0.f;
 }
@@ -999,16 +1008,21 @@ __device__ __forceinline__ void dma16(__amdgpu_buffer_rsrc_t r, float *lds_chunk
 }
 constexpr unsigned DMA_OOB = 0x80000000u;   // above every buffer size used here: reads as zero
 
-template <int GMODE, int KC, int NCB>
-__global__ void __launch_bounds__(256) df2_tiled_kernel(const BwdArgs a, int nvc, int nug) {
-    constexpr int NWV = 4;
-    constexpr int NV = GMODE == GMODE_COMP ? 2 * KC : 3;
+// buffers of the (p,u)-indexed weights per wave: the combined mode has LDS for one only
+constexpr int df2_tiled_ubuf(int gmode) { return gmode == GMODE_BOTH ? 1 : 2; }
+
+template <int GMODE, int KC, int NCB, int NWV>
+__global__ void __launch_bounds__(64 * NWV) df2_tiled_kernel(const BwdArgs a, int nvc, int nug) {
+    constexpr bool HC = g_has_comp(GMODE), HM = g_has_maxavg(GMODE);
+    constexpr int NVC = HC ? 2 * KC : 0;       // weight tensors of the compression part: a_u[k].., g_cv[k]..
+    constexpr int NV = NVC + (HM ? 3 : 0);     // then g_v[max], g_v[avg], argmax_v
     constexpr int NUP = (NV + 3) & ~3;
+    constexpr int UBUF = df2_tiled_ubuf(GMODE);
     constexpr int CB = 128 * NCB;
     extern __shared__ float smem[];
     float *F1s = smem;                         // [2][32][CB]
     float *VWs = F1s + 2 * 32 * CB;            // [2][NV][32 p][32 v]
-    float *UWs = VWs + 2 * NV * 1024;          // [NWV][2][32 p][NUP]
+    float *UWs = VWs + 2 * NV * 1024;          // [NWV][UBUF][32 p][NUP]
     const int tid = threadIdx.x, lane = tid & 63, pl = lane & 31, h = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int N1 = a.N1, H2 = a.H2, W2 = a.W2, C = a.C;
@@ -1039,27 +1053,26 @@ __global__ void __launch_bounds__(256) df2_tiled_kernel(const BwdArgs a, int nvc
         // buffer resources end at pixel `pend`: rows of later pixels read as zero
         const unsigned up = (unsigned)pend;
         const __amdgpu_buffer_rsrc_t rs_f1 = make_rsrc(a.f1 + (size_t)b * N1 * C, up * C * 4u);
-        __amdgpu_buffer_rsrc_t rs_va, rs_vb;   // the two (p,v)-indexed tensors
-        unsigned pstride_v;                    // floats per pixel in them
-        if constexpr (GMODE == GMODE_COMP) {
-            pstride_v = (unsigned)a.KT * W2;
-            rs_va = make_rsrc(a.a_u + (size_t)b * N1 * pstride_v, up * pstride_v * 4u);
-            rs_vb = make_rsrc(a.g_cv + (size_t)b * N1 * pstride_v, up * pstride_v * 4u);
-        } else {
-            pstride_v = 2u * W2;
-            rs_va = make_rsrc(a.g_v + (size_t)b * N1 * pstride_v, up * pstride_v * 4u);
-            rs_vb = make_rsrc(a.am_v + (size_t)b * N1 * W2, up * W2 * 4u);
+        // the (p,v)-indexed tensors: a_u, g_cv (KT*W2 floats per pixel); g_v (2*W2), argmax_v (W2)
+        __amdgpu_buffer_rsrc_t rs_va, rs_vb, rs_vc, rs_vd;
+        const unsigned pstride_c = (unsigned)a.KT * W2;
+        if constexpr (HC) {
+            rs_va = make_rsrc(a.a_u + (size_t)b * N1 * pstride_c, up * pstride_c * 4u);
+            rs_vb = make_rsrc(a.g_cv + (size_t)b * N1 * pstride_c, up * pstride_c * 4u);
+        }
+        if constexpr (HM) {
+            rs_vc = make_rsrc(a.g_v + (size_t)b * N1 * 2u * W2, up * 2u * W2 * 4u);
+            rs_vd = make_rsrc(a.am_v + (size_t)b * N1 * W2, up * W2 * 4u);
         }
         // lane-constant parts of the DMA offsets
         const int frow = (lane * 4) / CB, fcol = (lane * 4) % CB;        // within a 256-float chunk of the f1 tile
         const unsigned fcoff = (cb0 + fcol < C) ? (unsigned)(cb0 + fcol) * 4u : DMA_OOB;
-        const int vrow = 8 * wave + (lane >> 3);                          // pixel row of this lane in the weight tile
         const unsigned vcol = (unsigned)(v0 + 4 * (lane & 7)) * 4u;
 
         auto issue_tile = [&](int tile, int bi) {
             const int pt0 = pbeg + tile * TP;
             float *fdst = F1s + bi * 32 * CB;
-            constexpr int FCH = CB / 32;   // 256-float chunks per wave
+            constexpr int FCH = CB / 8 / NWV;   // 256-float chunks per wave
 #pragma unroll
             for (int i = 0; i < FCH; ++i) {
                 const int ch = wave * FCH + i;
@@ -1067,16 +1080,21 @@ __global__ void __launch_bounds__(256) df2_tiled_kernel(const BwdArgs a, int nvc
                 dma16(rs_f1, fdst + ch * 256, (unsigned)(pt0 + row) * C * 4u + fcoff);
             }
             float *vdst = VWs + bi * NV * 1024;
-            const unsigned p = (unsigned)(pt0 + vrow);
+            // the weight tile of one tensor is four 256-float chunks (8 pixels each); chunk c = 4*kk + quarter
 #pragma unroll
-            for (int kk = 0; kk < NV; ++kk) {
-                float *dst = vdst + kk * 1024 + wave * 256;
-                if constexpr (GMODE == GMODE_COMP) {
-                    const unsigned off = (p * pstride_v + (unsigned)(a.k0 + (kk % KC)) * W2) * 4u + vcol;
-                    dma16(kk < KC ? rs_va : rs_vb, dst, off);
-                } else {
-                    if (kk < 2) dma16(rs_va, dst, (p * pstride_v + (unsigned)kk * W2) * 4u + vcol);
-                    else dma16(rs_vb, dst, p * W2 * 4u + vcol);
+            for (int i = 0; i < (4 * NV + NWV - 1) / NWV; ++i) {
+                const int c = wave + NWV * i;
+                if (4 * NV % NWV != 0 && c >= 4 * NV) break;
+                const int kk = c >> 2, quarter = c & 3;
+                const unsigned p = (unsigned)(pt0 + 8 * quarter + (lane >> 3));
+                float *dst = vdst + c * 256;
+                if (HC && kk < NVC) {
+                    const unsigned off = (p * pstride_c + (unsigned)(a.k0 + (kk % KC)) * W2) * 4u + vcol;
+                    if constexpr (HC) dma16(kk < KC ? rs_va : rs_vb, dst, off);
+                } else if constexpr (HM) {
+                    const int m = kk - NVC;
+                    if (m < 2) dma16(rs_vc, dst, (p * 2u * W2 + (unsigned)m * W2) * 4u + vcol);
+                    else dma16(rs_vd, dst, p * W2 * 4u + vcol);
                 }
             }
         };
@@ -1086,21 +1104,24 @@ __global__ void __launch_bounds__(256) df2_tiled_kernel(const BwdArgs a, int nvc
             const size_t bp = (size_t)b * N1 + p;
 #pragma unroll
             for (int i = 0; i < NUP; ++i) r[i] = 0.f;
-            if constexpr (GMODE == GMODE_COMP) {
+            if constexpr (HC) {
 #pragma unroll
                 for (int k = 0; k < KC; ++k) {
                     const size_t o = (bp * a.KT + a.k0 + k) * H2 + u;
                     r[k] = a.a_v[o];
                     r[KC + k] = a.g_cu[o];
                 }
-            } else {
-                r[0] = a.g_u[(bp * 2 + 0) * H2 + u];
-                r[1] = a.g_u[(bp * 2 + 1) * H2 + u];
-                r[2] = __int_as_float(a.am_u[bp * H2 + u]);
+            }
+            if constexpr (HM) {
+                r[NVC + 0] = a.g_u[(bp * 2 + 0) * H2 + u];
+                r[NVC + 1] = a.g_u[(bp * 2 + 1) * H2 + u];
+                r[NVC + 2] = __int_as_float(a.am_u[bp * H2 + u]);
             }
         };
+        // With one buffer the rows of the next tile replace those of the current one after its last read:
+        // the region is private to the wave and a wave's LDS accesses complete in order.
         auto store_uw_tile = [&](int bi, const float(&r)[NUP]) {
-            float *dst = UWs + ((wave * 2 + bi) * 32 + pl) * NUP;
+            float *dst = UWs + ((wave * UBUF + (UBUF == 2 ? bi : 0)) * 32 + pl) * NUP;
 #pragma unroll
             for (int i = 0; i < NUP; i += 4) {
                 const v4f x = {r[i], r[i + 1], r[i + 2], r[i + 3]};
@@ -1124,7 +1145,7 @@ __global__ void __launch_bounds__(256) df2_tiled_kernel(const BwdArgs a, int nvc
             }
             const float *fs = F1s + bi * 32 * CB;
             const float *vs = VWs + bi * NV * 1024;
-            const float *us = UWs + (wave * 2 + bi) * 32 * NUP;
+            const float *us = UWs + (wave * UBUF + (UBUF == 2 ? bi : 0)) * 32 * NUP;
             const int pt0 = pbeg + tile * TP;
             // Software pipeline over the 16 MFMA steps of the tile: the LDS operands of step s+1 are
             // fetched before the MFMAs of step s and its G is computed between them, so the matrix
@@ -1147,13 +1168,14 @@ __global__ void __launch_bounds__(256) df2_tiled_kernel(const BwdArgs a, int nvc
             };
             auto g_of = [&](int s, const StepOps &o) {
                 float G = 0.f;
-                if constexpr (GMODE == GMODE_COMP) {
+                if constexpr (HC) {
 #pragma unroll
                     for (int k = 0; k < KC; ++k) G += o.vw[k] * o.uw[KC + k] + o.uw[k] * o.vw[KC + k];
-                } else {
-                    G = o.uw[1] * inv_w2 + o.vw[1] * inv_h2;
-                    if (__float_as_int(o.uw[2]) == v) G += o.uw[0];
-                    if (__float_as_int(o.vw[2]) == u) G += o.vw[0];
+                }
+                if constexpr (HM) {
+                    G += o.uw[NVC + 1] * inv_w2 + o.vw[NVC + 1] * inv_h2;
+                    if (__float_as_int(o.uw[NVC + 2]) == v) G += o.uw[NVC];
+                    if (__float_as_int(o.vw[NVC + 2]) == u) G += o.vw[NVC];
                 }
                 // No mask needed: pixels at or beyond `pend` have all-zero f1 rows and (p,v) weights (DMA
                 // bounds), so whatever finite G they get multiplies zeros; columns beyond W2 are not stored.
@@ -1369,15 +1391,25 @@ int weighted_forward(const Dims &d, const float *f1, const float *f2, const floa
     return SEPCORR_OK;
 }
 
+// fmap2 rows (= waves) per workgroup of the tiled d_f2 kernel: 8 (two waves per SIMD sharing one LDS tile)
+// unless that pads the row count more than 4 does.
+// The combined mode keeps more weight tiles in LDS and has room for 4 rows only.
+int df2_rows_per_wg(const Dims &d, bool both) {
+    if (both) return 4;
+    return (d.H2 + 7) / 8 * 8 <= (d.H2 + 3) / 4 * 4 ? 8 : 4;
+}
+
 struct Df2Plan {
     bool tiled;
     int nsplit;
+    int rows;
 };
 
 // How d_f2 is computed for these sizes.  The p range is split over workgroups so that the grid fills
 // the 256 CUs evenly; each split writes a partial d_f2 to scratch, summed in split order afterwards.
-Df2Plan df2_plan(const Dims &d) {
+Df2Plan df2_plan(const Dims &d, bool both) {
     Df2Plan pl;
+    pl.rows = df2_rows_per_wg(d, both);
     const size_t big = (size_t)1 << 30;
     const size_t n1 = (size_t)d.H1 * d.W1;
     pl.tiled = d.C % 4 == 0 && d.W2 % 4 == 0 && n1 * d.C * 4 <= big && n1 * MAX_K * d.W2 * 4 <= big;
@@ -1385,7 +1417,8 @@ Df2Plan df2_plan(const Dims &d) {
     const int nvc = (d.W2 + 31) / 32;
     const int cblocks = (d.C + 255) / 256;
     if (pl.tiled) {
-        const long base = (long)d.B * ((d.H2 + 3) / 4) * nvc * (d.C <= 128 ? 1 : cblocks);
+        const int rows = pl.rows;
+        const long base = (long)d.B * ((d.H2 + rows - 1) / rows) * nvc * (d.C <= 128 ? 1 : cblocks);
         double best = -1.0;
         pl.nsplit = 1;
         for (int ns = 1; ns <= 16 && ns <= tiles; ++ns) {
@@ -1424,7 +1457,7 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s
         const size_t lds = (size_t)TP * (128 * ncb + 4) * sizeof(float);
 #define SEPCORR_DF1(NCB, CV, MT)                                                                   \
     do {                                                                                           \
-        ProfScope ps(GMODE == GMODE_COMP ? "df1_comp" : "df1_maxavg", s1);                         \
+        ProfScope ps(GMODE == GMODE_COMP ? "df1_comp" : GMODE == GMODE_BOTH ? "df1_both" : "df1_maxavg", s1); \
         hipLaunchKernelGGL((df1_kernel<GMODE, KC, NCB, CV, MT>), grid, block, lds, s1, a);         \
     } while (0)
         if (nW > 4) { if (cvec) SEPCORR_DF1(1, true, 512); else SEPCORR_DF1(1, false, 512); }
@@ -1437,33 +1470,36 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s
         const int ncb = d.C <= 128 ? 1 : 2;
         const int cblocks = (d.C + 128 * ncb - 1) / (128 * ncb);
         const int tiles = a.tiles_per_batch;
-        const Df2Plan plan = df2_plan(d);
+        const Df2Plan plan = df2_plan(d, GMODE == GMODE_BOTH);
         a.nsplit = plan.nsplit;
         a.tiles_per_split = (tiles + a.nsplit - 1) / a.nsplit;
         const int nvc = nvc_all;
         float *d2 = a.d2;
         if (a.nsplit > 1) a.d2 = static_cast<float *>(ws);
         if (plan.tiled) {
-            constexpr int NV = GMODE == GMODE_COMP ? 2 * KC : 3;
+            constexpr int NV = (g_has_comp(GMODE) ? 2 * KC : 0) + (g_has_maxavg(GMODE) ? 3 : 0);
             constexpr int NUP = (NV + 3) & ~3;
-            const int nug = (d.H2 + 3) / 4;
-            const dim3 grid(d.B * a.nsplit * nug * nvc, cblocks), block(256);
-            const size_t lds = ((size_t)2 * 32 * 128 * ncb + 2 * NV * 1024 + 4 * 2 * 32 * NUP) * sizeof(float);
-#define SEPCORR_DF2T(NCB)                                                                          \
+            constexpr int UBUF = df2_tiled_ubuf(GMODE);
+            const int rows = plan.rows;
+            const int nug = (d.H2 + rows - 1) / rows;
+            const dim3 grid(d.B * a.nsplit * nug * nvc, cblocks), block(64 * rows);
+            const size_t lds = ((size_t)2 * 32 * 128 * ncb + 2 * NV * 1024 + rows * UBUF * 32 * NUP) * sizeof(float);
+#define SEPCORR_DF2T(NCB, NWV)                                                                     \
     do {                                                                                           \
-        auto k = df2_tiled_kernel<GMODE, KC, NCB>;                                                 \
+        auto k = df2_tiled_kernel<GMODE, KC, NCB, NWV>;                                            \
         if (int rc = set_lds(k, lds)) return rc;                                                   \
-        ProfScope ps(GMODE == GMODE_COMP ? "df2_comp" : "df2_maxavg", s);                          \
+        ProfScope ps(GMODE == GMODE_COMP ? "df2_comp" : GMODE == GMODE_BOTH ? "df2_both" : "df2_maxavg", s); \
         hipLaunchKernelGGL(k, grid, block, lds, s, a, nvc, nug);                                   \
     } while (0)
-            if (ncb == 1) SEPCORR_DF2T(1); else SEPCORR_DF2T(2);
+            if (rows == 8) { if (ncb == 1) SEPCORR_DF2T(1, 8); else SEPCORR_DF2T(2, 8); }
+            else           { if (ncb == 1) SEPCORR_DF2T(1, 4); else SEPCORR_DF2T(2, 4); }
 #undef SEPCORR_DF2T
         } else {
         const int ntasks = d.B * a.nsplit * d.H2 * nvc;
         const dim3 grid((ntasks + 3) / 4, cblocks), block(256);
 #define SEPCORR_DF2(NCB, CV)                                                                       \
     do {                                                                                           \
-        ProfScope ps(GMODE == GMODE_COMP ? "df2_comp" : "df2_maxavg", s);                          \
+        ProfScope ps(GMODE == GMODE_COMP ? "df2_comp" : GMODE == GMODE_BOTH ? "df2_both" : "df2_maxavg", s); \
         hipLaunchKernelGGL((df2_kernel<GMODE, KC, NCB, CV>), grid, block, 0, s, a, ntasks, nvc);   \
     } while (0)
         if (ncb == 1) { if (cvec) SEPCORR_DF2(1, true); else SEPCORR_DF2(1, false); }
@@ -1628,7 +1664,8 @@ int sepcorr_compression_forward(const float *f1, const float *f2, const float *a
 size_t sepcorr_backward_workspace_bytes(int B, int H1, int W1, int H2, int W2, int C) {
     if (B < 1 || H1 < 1 || W1 < 1 || H2 < 1 || W2 < 1 || C < 1) return 0;
     const Dims d = {B, H1, W1, H2, W2, C};
-    const int ns = df2_plan(d).nsplit;
+    const int n0 = df2_plan(d, false).nsplit, n1 = df2_plan(d, true).nsplit;
+    const int ns = n0 > n1 ? n0 : n1;   // one size serves every backward entry point
     return ns > 1 ? (size_t)ns * B * H2 * W2 * C * sizeof(float) : 0;
 }
 
@@ -1656,9 +1693,13 @@ int sepcorr_compression_backward(const float *f1, const float *f2, const float *
                                  int W1, int H2, int W2, int C, int K, void *workspace, size_t workspace_bytes,
                                  void *stream) {
     REQUIRE_PTR(f1); REQUIRE_PTR(f2); REQUIRE_PTR(a_u); REQUIRE_PTR(a_v); REQUIRE_PTR(g_cu); REQUIRE_PTR(g_cv);
-    REQUIRE_PTR(d_f1); REQUIRE_PTR(d_f2); REQUIRE_PTR(d_a_u); REQUIRE_PTR(d_a_v);
+    REQUIRE_PTR(d_a_u); REQUIRE_PTR(d_a_v);
     const Dims d = {B, H1, W1, H2, W2, C};
     if (int rc = check_dims(d, K)) return rc;
+    if ((d_f1 == nullptr) != (d_f2 == nullptr))
+        return fail(SEPCORR_EINVAL, "sepcorr: d_f1 and d_f2 must be given together or both be NULL");
+    if (d_f1 == nullptr)   // only the gradients of the weights: one sweep, no scratch
+        return weighted_forward(d, f1, f2, g_cv, g_cu, d_a_v, d_a_u, K, static_cast<hipStream_t>(stream));
     if (int rc = check_workspace(d, workspace, workspace_bytes)) return rc;
     ForkJoin fj(static_cast<hipStream_t>(stream));
     // d_a_v[k,u] = sum_v S g_cv[k,v];  d_a_u[k,v] = sum_u S g_cu[k,u]: the forward's weighted sums
@@ -1680,6 +1721,53 @@ int sepcorr_compression_backward(const float *f1, const float *f2, const float *
             case 3: rc = launch_bwd<GMODE_COMP, 3>(a, d, workspace, fj.sa, fj.sb); break;
             default: rc = launch_bwd<GMODE_COMP, 4>(a, d, workspace, fj.sa, fj.sb); break;
         }
+    }
+    const int rj = fj.join();
+    return rc ? rc : rj;
+}
+
+int sepcorr_fused_backward(const float *f1, const float *f2, const int32_t *argmax_u, const int32_t *argmax_v,
+                           const float *grad_u, const float *grad_v, const float *a_u, const float *a_v,
+                           const float *g_cu, const float *g_cv, float *d_f1, float *d_f2, int B, int H1, int W1, int H2,
+                           int W2, int C, int K, void *workspace, size_t workspace_bytes, void *stream) {
+    REQUIRE_PTR(f1); REQUIRE_PTR(f2); REQUIRE_PTR(argmax_u); REQUIRE_PTR(argmax_v); REQUIRE_PTR(grad_u); REQUIRE_PTR(grad_v);
+    REQUIRE_PTR(a_u); REQUIRE_PTR(a_v); REQUIRE_PTR(g_cu); REQUIRE_PTR(g_cv); REQUIRE_PTR(d_f1); REQUIRE_PTR(d_f2);
+    const Dims d = {B, H1, W1, H2, W2, C};
+    if (int rc = check_dims(d, K)) return rc;
+    if (int rc = check_workspace(d, workspace, workspace_bytes)) return rc;
+    BwdArgs a;
+    memset(&a, 0, sizeof(a));
+    a.f1 = f1; a.f2 = f2; a.am_u = argmax_u; a.am_v = argmax_v; a.g_u = grad_u; a.g_v = grad_v;
+    a.a_u = a_u; a.a_v = a_v; a.g_cu = g_cu; a.g_cv = g_cv;
+    a.d1 = d_f1; a.d2 = d_f2;
+    a.B = B; a.N1 = H1 * W1; a.H2 = H2; a.W2 = W2; a.C = C; a.KT = K;
+    ForkJoin fj(static_cast<hipStream_t>(stream));
+    const int kch = W2 > 128 ? 2 : KCH;
+    const int kc0 = K < kch ? K : kch;
+    // The first chunk of weight channels carries the max/avg terms of G along (built for 2 and 4 channels);
+    // otherwise they follow as one more accumulating launch.
+    const bool first_carries = kc0 == 2 || kc0 == 4;
+    int rc = SEPCORR_OK;
+    for (int k0 = 0; k0 < K && rc == SEPCORR_OK; k0 += kch) {
+        a.k0 = k0;
+        a.accumulate = k0 > 0;
+        const int kc = K - k0 < kch ? K - k0 : kch;
+        if (k0 == 0 && first_carries) {
+            rc = kc == 2 ? launch_bwd<GMODE_BOTH, 2>(a, d, workspace, fj.sa, fj.user)
+                         : launch_bwd<GMODE_BOTH, 4>(a, d, workspace, fj.sa, fj.user);
+            continue;
+        }
+        switch (kc) {
+            case 1: rc = launch_bwd<GMODE_COMP, 1>(a, d, workspace, fj.sa, fj.user); break;
+            case 2: rc = launch_bwd<GMODE_COMP, 2>(a, d, workspace, fj.sa, fj.user); break;
+            case 3: rc = launch_bwd<GMODE_COMP, 3>(a, d, workspace, fj.sa, fj.user); break;
+            default: rc = launch_bwd<GMODE_COMP, 4>(a, d, workspace, fj.sa, fj.user); break;
+        }
+    }
+    if (!first_carries && rc == SEPCORR_OK) {
+        a.k0 = 0; a.KT = 1;
+        a.accumulate = 1;
+        rc = launch_bwd<GMODE_MAXAVG, 1>(a, d, workspace, fj.sa, fj.user);
     }
     const int rj = fj.join();
     return rc ? rc : rj;

@@ -101,6 +101,45 @@ class AttentionWeightsFunction(Function):
         return d_sep, d_w, d_b
 
 
+class SeparateLevelFunction(Function):
+    """One pyramid level of the caller's loop (core/corr.py:416-457) as a single autograd node:
+    max/argmax/avg forward -> attention weights of both volumes -> compression forward.
+
+    Not a class of the reference.  Results equal the chain ComputeMaxArgmaxAvgFunction ->
+    AttentionWeightsFunction x2 -> ComputeSelfCompressionFunction; the point is the backward pass: the
+    gradient of the max/avg outputs is complete before any feature gradient is needed, so dL/dS of both
+    operators is added and contracted once (3 sweeps over the volume instead of 5).
+
+    forward(f1, f2, weight1, bias1, weight2, bias2) -> (max_avg_u, max_avg_v, comp_u, comp_v), operator layouts;
+    attention 1 reads max_avg_v and weights the sums over v, attention 2 reads max_avg_u (core/corr.py:437-448).
+    """
+
+    @staticmethod
+    def forward(ctx, f1, f2, weight1, bias1, weight2, bias2):
+        _contig(f1, f2, weight1, weight2)
+        with torch.cuda.device_of(f1):
+            out_u, out_v, am_u, am_v = MemorySaver.max_argmax_avg_forward(f1, f2)
+            a_u = MemorySaver.attention_forward(out_v, weight1, bias1)
+            a_v = MemorySaver.attention_forward(out_u, weight2, bias2)
+            cu, cv = MemorySaver.compression_forward(f1, f2, a_u, a_v)
+        ctx.save_for_backward(f1, f2, am_u, am_v, out_u, out_v, a_u, a_v, weight1, weight2)
+        ctx.has_bias = (bias1 is not None, bias2 is not None)
+        return out_u, out_v, cu, cv
+
+    @staticmethod
+    def backward(ctx, g_u, g_v, g_cu, g_cv):
+        f1, f2, am_u, am_v, out_u, out_v, a_u, a_v, weight1, weight2 = ctx.saved_tensors
+        g_u, g_v, g_cu, g_cv = (g.contiguous() for g in (g_u, g_v, g_cu, g_cv))
+        with torch.cuda.device_of(f1):
+            da_u, da_v = MemorySaver.compression_weight_gradients(f1, f2, a_u, a_v, g_cu, g_cv)
+            d_out_v, d_w1, d_b1 = MemorySaver.attention_backward(out_v, weight1, a_u, da_u, need_bias=ctx.has_bias[0])
+            d_out_u, d_w2, d_b2 = MemorySaver.attention_backward(out_u, weight2, a_v, da_v, need_bias=ctx.has_bias[1])
+            d_out_u += g_u
+            d_out_v += g_v
+            d1, d2 = MemorySaver.fused_backward(f1, f2, am_u, am_v, d_out_u, d_out_v, a_u, a_v, g_cu, g_cv)
+        return d1, d2, d_w1, d_b1, d_w2, d_b2
+
+
 class AssembleVolumeFunction(Function):
     """Operator outputs of all levels -> one module-level volume (B, channels, L0, H1, W1).
 

@@ -149,6 +149,34 @@ def test_compression_backward(device, shape, K):
     assert all(torch.equal(x, y) for x, y in zip(got, again))
 
 
+@pytest.mark.parametrize("shape", SHAPES[1:7] + SHAPES[9:])
+@pytest.mark.parametrize("K", [1, 2, 3, 4, 6])
+def test_fused_backward_is_the_sum_of_both_backwards(device, shape, K):
+    # G of the two operators added before the contraction: the oracle is the sum of its two backward functions
+    B, H1, W1, H2, W2, C = shape
+    f1, f2, g = op_inputs(B, H1, W1, H2, W2, C, seed=51 + K)
+    a_u = softmax_weights(B, H1, W1, K, W2, g)
+    a_v = softmax_weights(B, H1, W1, K, H2, g)
+    g_cu = torch.randn(B, H1, W1, K, H2, generator=g)
+    g_cv = torch.randn(B, H1, W1, K, W2, generator=g)
+    g_u = torch.randn(B, H1, W1, 2, H2, generator=g)
+    g_v = torch.randn(B, H1, W1, 2, W2, generator=g)
+    d = lambda t: t.to(device)
+    ms = _native()
+    _, _, au, av = ms.max_argmax_avg_forward(d(f1), d(f2))
+    d1, d2 = ms.fused_backward(d(f1), d(f2), au, av, d(g_u), d(g_v), d(a_u), d(a_v), d(g_cu), d(g_cv))
+    m1, m2 = O.max_argmax_avg_backward(f1.double(), f2.double(), au.cpu(), av.cpu(), g_u.double(), g_v.double())
+    c1, c2, ra_u, ra_v = O.compression_backward(*(t.double() for t in (f1, f2, a_u, a_v, g_cu, g_cv)))
+    assert_close(d1, m1 + c1, "grad_fmap1_l0", scale_atol=True)
+    assert_close(d2, m2 + c2, "grad_fmap2_lk", scale_atol=True)
+    e1, e2 = ms.fused_backward(d(f1), d(f2), au, av, d(g_u), d(g_v), d(a_u), d(a_v), d(g_cu), d(g_cv))
+    assert torch.equal(d1, e1) and torch.equal(d2, e2)
+    # the weight gradients alone (compression backward without feature gradients)
+    da_u, da_v = ms.compression_weight_gradients(d(f1), d(f2), d(a_u), d(a_v), d(g_cu), d(g_cv))
+    assert_close(da_u, ra_u, "grad_attention_u", scale_atol=True)
+    assert_close(da_v, ra_v, "grad_attention_v", scale_atol=True)
+
+
 def test_autograd_functions_match_autograd_through_4d(device):
     # mirrors overall_grad_test (scripts/test_maxavg_autograd.py:478-502, test_compression_autograd.py:442-484):
     # loss = sum of MSE(channel, 0) over all output channels, at a pooled level
