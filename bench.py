@@ -30,7 +30,7 @@ WORKLOADS = {
 }
 PASSES = {"f": 1, "c": 1, "C": 3, "F": 2}
 # contraction passes (units of W = 2*B*N1*N2*C flops) executed by one launch of each kernel
-KERNEL_PASSES = {"fwd_maxavg": 1, "fwd_weighted": 1, "df1_comp": 1, "df2_comp": 1, "df1_maxavg": 1, "df2_maxavg": 1}
+KERNEL_PASSES = {"df1_both": 1, "df2_both": 1, "fwd_maxavg": 1, "fwd_weighted": 1, "df1_comp": 1, "df2_comp": 1, "df1_maxavg": 1, "df2_maxavg": 1}
 # HBM bytes per launch at cfg4 from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by the factors a
 # 256 MiB device copy gives in the same run (profiles/cfg4_fwd_bwd_kernels.txt); None = not measured
 _MIB = 2 ** 20
@@ -263,6 +263,31 @@ def main():
                      "frac": round(ach / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": TRAFFIC_BYTES_CFG4.get(dom) if args.workload == "cfg4" else None},
         "kernels": kernels,
     }
+    if "C" in ops and "F" in ops:
+        # The same job through the entry points that have no counterpart in the reference's two-operator API:
+        # weight gradients alone, then one contraction per feature gradient with dL/dS of both operators added
+        # (5 sweeps over the volume instead of 7).  Reported beside the headline, never as `value`.
+        def fused_step():
+            op_f()
+            op_c()
+            _lib.check(lib.sepcorr_compression_backward(P(f1), P(f2), P(a_u), P(a_v), P(gr["g_cu"]), P(gr["g_cv"]),
+                                                        None, None, P(da_u), P(da_v), *dims, Kp, None, 0, stream))
+            _lib.check(lib.sepcorr_fused_backward(P(f1), P(f2), P(am_u), P(am_v), P(gr["g_u"]), P(gr["g_v"]),
+                                                  P(a_u), P(a_v), P(gr["g_cu"]), P(gr["g_cv"]), P(d1), P(d2),
+                                                  *dims, Kp, P(ws), nws, stream))
+        for _ in range(args.warmup):
+            fused_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fused_step()
+        torch.cuda.synchronize()
+        fms = (time.perf_counter() - t0) / args.steps * 1e3
+        out["fused_level"] = {
+            "ms_per_step": round(fms, 4), "contraction_passes_executed": 5,
+            "tflops_executed": round(5 * Wf / (fms * 1e-3) / 1e12, 2),
+            "what": "same inputs and outputs as the headline step (d_f1, d_f2 are the sums of the two operators' "
+                    "gradients), via sepcorr_compression_backward(d_f1=d_f2=NULL) + sepcorr_fused_backward"}
     if not args.no_cpu_baseline:
         out["module_level"] = module_level(B, H, W, C, Kp, torch, dev)
         out["cpu_baseline"] = cpu_baseline(B, H, W, C, Kp, ops, torch)

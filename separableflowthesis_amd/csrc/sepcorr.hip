@@ -126,6 +126,14 @@ __device__ __forceinline__ v16f mfma(float a, float b, v16f c) {
 // ------------------------------------------------------------------------------------------
 enum { MODE_MAXAVG = 0, MODE_ARGMAX = 1, MODE_WEIGHTED = 2 };
 
+// Workgroups are handed to the 8 XCDs round-robin by linear id, and each XCD has its own L2.  This maps the
+// hardware id to a logical one such that every XCD works on one contiguous range of logical ids: neighbours in
+// the range (same batch image, same pixel split) stream the same operand rows through the same L2.
+__device__ __forceinline__ int xcd_contiguous(int bid, int n) {
+    const int c = bid & 7, slot = bid >> 3, q = n >> 3, r = n & 7;
+    return c * q + (c < r ? c : r) + slot;
+}
+
 struct FwdArgs {
     const float *f1, *f2;
     const float *wv;   // MODE_WEIGHTED: weights indexed by v, (B,N1,KT,W2)
@@ -139,6 +147,7 @@ struct FwdArgs {
     int nvc;           // column chunks of 32 handled per pass = min(8, ceil(W2 / 32))
     int vpasses;       // passes of 256 columns = ceil(W2 / 256)
     int stage;         // collect the rows of out_u in LDS and store them coalesced at the end
+    int xcd_order;     // map workgroup ids so that each XCD gets a contiguous range
 };
 
 // CMODE: 0 = any C (scalar loads), 1 = C % 4 == 0 (16-byte loads), 2 = C % 32 == 0 (branch-free fast path),
@@ -160,8 +169,9 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     const int nvc = RG ? a.nvc : nW, NUG = RG ? nW / nvc : 1;
     const int vcw = RG ? wave % nvc : wave, ug = RG ? wave / nvc : 0;
     const int vpasses = (WM == 2) ? a.vpasses : 1;
-    const int b = blockIdx.x / a.tiles_per_batch;
-    const int p0 = (blockIdx.x % a.tiles_per_batch) * TP;
+    const int wg = a.xcd_order ? xcd_contiguous(blockIdx.x, gridDim.x) : (int)blockIdx.x;
+    const int b = wg / a.tiles_per_batch;
+    const int p0 = (wg % a.tiles_per_batch) * TP;
     const int N1 = a.N1, H2 = a.H2, W2 = a.W2, C = a.C;
     const int LS = a.CP + 4;
     float *f1s = smem;
@@ -672,6 +682,7 @@ struct BwdArgs {
     int tiles_per_batch;             // df1: p tiles per batch
     int nsplit, tiles_per_split;     // df2: split of the p range
     int accumulate;                  // add to the destination instead of overwriting
+    int xcd_order;                   // map workgroup ids so that each XCD gets a contiguous range
 };
 
 // Weights of one lane that depend on (p, v) and on (p, u).  Members a mode does not use stay unset and
@@ -758,8 +769,9 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
     // wave (vcw, ug): columns [32 vcw, 32 vcw + 32), rows ug, ug + NUG, ... (see fwd_kernel)
     const int nvc = a.nvc, NUG = nW / nvc;
     const int vcw = wave % nvc, ug = wave / nvc;
-    const int b = blockIdx.x / a.tiles_per_batch;
-    const int p0 = (blockIdx.x % a.tiles_per_batch) * TP;
+    const int wg = a.xcd_order ? xcd_contiguous(blockIdx.x, gridDim.x) : (int)blockIdx.x;
+    const int b = wg / a.tiles_per_batch;
+    const int p0 = (wg % a.tiles_per_batch) * TP;
     const int cb0 = blockIdx.y * CB;
     const int N1 = a.N1, H2 = a.H2, W2 = a.W2, C = a.C;
     const int pix = p0 + pl;
@@ -1026,7 +1038,7 @@ __global__ void __launch_bounds__(64 * NWV) df2_tiled_kernel(const BwdArgs a, in
     const int tid = threadIdx.x, lane = tid & 63, pl = lane & 31, h = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int N1 = a.N1, H2 = a.H2, W2 = a.W2, C = a.C;
-    int task = blockIdx.x;
+    int task = a.xcd_order ? xcd_contiguous(blockIdx.x, gridDim.x) : (int)blockIdx.x;
     const int vc = task % nvc; task /= nvc;
     const int ug = task % nug; task /= nug;
     const int split = task % a.nsplit;
@@ -1365,6 +1377,12 @@ int launch_fwd_weighted_k(const FwdArgs &a, int kc, int B, hipStream_t s) {
     }
 }
 
+// SEPCORR_NO_XCD_ORDER=1 keeps the hardware order of workgroups (for measurements).
+int xcd_order_enabled() {
+    static const int on = getenv("SEPCORR_NO_XCD_ORDER") == nullptr;
+    return on;
+}
+
 FwdArgs fwd_args(const Dims &d) {
     FwdArgs a;
     memset(&a, 0, sizeof(a));
@@ -1374,6 +1392,7 @@ FwdArgs fwd_args(const Dims &d) {
     a.C = d.C;
     a.CP = (d.C + 7) & ~7;
     a.tiles_per_batch = (a.N1 + TP - 1) / TP;
+    a.xcd_order = xcd_order_enabled();
     return a;
 }
 
@@ -1679,6 +1698,7 @@ int sepcorr_max_argmax_avg_backward(const float *f1, const float *f2, const int3
     if (int rc = check_workspace(d, workspace, workspace_bytes)) return rc;
     BwdArgs a;
     memset(&a, 0, sizeof(a));
+    a.xcd_order = xcd_order_enabled();
     a.f1 = f1; a.f2 = f2; a.am_u = argmax_u; a.am_v = argmax_v; a.g_u = grad_u; a.g_v = grad_v;
     a.d1 = d_f1; a.d2 = d_f2;
     a.B = B; a.N1 = H1 * W1; a.H2 = H2; a.W2 = W2; a.C = C; a.KT = 1;
@@ -1706,6 +1726,7 @@ int sepcorr_compression_backward(const float *f1, const float *f2, const float *
     int rc = weighted_forward(d, f1, f2, g_cv, g_cu, d_a_v, d_a_u, K, fj.user);
     BwdArgs a;
     memset(&a, 0, sizeof(a));
+    a.xcd_order = xcd_order_enabled();
     a.f1 = f1; a.f2 = f2; a.a_u = a_u; a.a_v = a_v; a.g_cu = g_cu; a.g_cv = g_cv;
     a.d1 = d_f1; a.d2 = d_f2;
     a.B = B; a.N1 = H1 * W1; a.H2 = H2; a.W2 = W2; a.C = C; a.KT = K;
@@ -1737,6 +1758,7 @@ int sepcorr_fused_backward(const float *f1, const float *f2, const int32_t *argm
     if (int rc = check_workspace(d, workspace, workspace_bytes)) return rc;
     BwdArgs a;
     memset(&a, 0, sizeof(a));
+    a.xcd_order = xcd_order_enabled();
     a.f1 = f1; a.f2 = f2; a.am_u = argmax_u; a.am_v = argmax_v; a.g_u = grad_u; a.g_v = grad_v;
     a.a_u = a_u; a.a_v = a_v; a.g_cu = g_cu; a.g_cv = g_cv;
     a.d1 = d_f1; a.d2 = d_f2;
