@@ -117,6 +117,18 @@ __device__ __forceinline__ v4f buf_load4(__amdgpu_buffer_rsrc_t r, unsigned byte
     return __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 0));
 }
 
+constexpr unsigned DMA_OOB = 0x80000000u;   // a byte offset above every buffer size used here: reads as zero
+
+// The same with a wave-uniform byte offset added by the hardware (it takes no part in the bounds check, so an
+// out-of-range marker in byte_off stays one).
+__device__ __forceinline__ v4f buf_load4s(__amdgpu_buffer_rsrc_t r, unsigned byte_off, unsigned uniform_off) {
+    return __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, uniform_off, 0));
+}
+
+__device__ __forceinline__ float buf_load1s(__amdgpu_buffer_rsrc_t r, unsigned byte_off, unsigned uniform_off) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, byte_off, uniform_off, 0));
+}
+
 __device__ __forceinline__ v16f mfma(float a, float b, v16f c) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
 }
@@ -310,8 +322,10 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                     }
                 }
             }
+            if constexpr (CMODE != 3) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) acc[ru][e] = 0.f;
+                for (int e = 0; e < 16; ++e) acc[ru][e] = 0.f;
+            }
         }
         __syncthreads();
         // combine the per-wave partials in wave order and store the finished rows
@@ -448,18 +462,23 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                     }
                 }
             }
+            // C == 256 instantiation: the first MFMA of a row takes a literal zero as its addend, which saves
+            // clearing the 16 accumulator registers after every row (vector moves are not free here: they run
+            // on the same lanes as the fp32 MFMA)
+            const v16f zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
             auto mfma_tq = [&](int tq, const v4f &bv) {
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
+                    const bool first = CMODE == 3 && J == 0 && tq == 0;
                     if constexpr (DUAL) {
                         // one row per step: split the contraction over two accumulators so that
                         // consecutive MFMAs are independent (skipped where registers are short: the
                         // matrix pipe accepts back-to-back dependent MFMAs without a bubble)
-                        if (t & 1) acc_alt = mfma(buf[0][tq][t], bv[t], acc_alt);
-                        else acc[0] = mfma(buf[0][tq][t], bv[t], acc[0]);
+                        if (t & 1) acc_alt = mfma(buf[0][tq][t], bv[t], first && t == 1 ? zero16 : acc_alt);
+                        else acc[0] = mfma(buf[0][tq][t], bv[t], first && t == 0 ? zero16 : acc[0]);
                     } else {
 #pragma unroll
-                        for (int r = 0; r < UR; ++r) acc[r] = mfma(buf[r][tq][t], bv[t], acc[r]);
+                        for (int r = 0; r < UR; ++r) acc[r] = mfma(buf[r][tq][t], bv[t], first && t == 0 ? zero16 : acc[r]);
                     }
                 }
             };
@@ -494,8 +513,10 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
 #endif
                 if constexpr (DUAL) {
                     acc[0] += acc_alt;
+                    if constexpr (CMODE != 3) {
 #pragma unroll
-                    for (int e = 0; e < 16; ++e) acc_alt[e] = 0.f;
+                        for (int e = 0; e < 16; ++e) acc_alt[e] = 0.f;
+                    }
                 }
                 epilogue(step);
             }
@@ -717,7 +738,7 @@ __device__ __forceinline__ VW<GMODE, KC> load_vw(const BwdArgs &a, size_t bp, in
     }
     if constexpr (g_has_maxavg(GMODE)) {
         w.ma = ok ? a.g_v[(bp * 2 + 0) * a.W2 + v] : 0.f;
-        w.mg = ok ? a.g_v[(bp * 2 + 1) * a.W2 + v] / (float)a.H2 : 0.f;
+        w.mg = ok ? a.g_v[(bp * 2 + 1) * a.W2 + v] * (1.f / (float)a.H2) : 0.f;
         w.am = ok ? a.am_v[bp * a.W2 + v] : -1;
     }
     return w;
@@ -735,7 +756,7 @@ __device__ __forceinline__ UW<GMODE, KC> load_uw(const BwdArgs &a, size_t bp, in
     }
     if constexpr (g_has_maxavg(GMODE)) {
         w.ma = ok ? a.g_u[(bp * 2 + 0) * a.H2 + u] : 0.f;
-        w.mg = ok ? a.g_u[(bp * 2 + 1) * a.H2 + u] / (float)a.W2 : 0.f;
+        w.mg = ok ? a.g_u[(bp * 2 + 1) * a.H2 + u] * (1.f / (float)a.W2) : 0.f;
         w.am = ok ? a.am_u[bp * a.H2 + u] : -1;
     }
     return w;
@@ -746,7 +767,10 @@ __device__ __forceinline__ float gval(const VW<GMODE, KC> &wv, const UW<GMODE, K
     float g = 0.f;
     if constexpr (g_has_comp(GMODE)) {
 #pragma unroll
-        for (int k = 0; k < KC; ++k) g += wv.a[k] * wu.g[k] + wu.a[k] * wv.g[k];
+        for (int k = 0; k < KC; ++k) {   // two fused multiply-adds per channel (a sum of two products would take three)
+            g = fmaf(wv.a[k], wu.g[k], g);
+            g = fmaf(wu.a[k], wv.g[k], g);
+        }
     }
     if constexpr (g_has_maxavg(GMODE)) {
         g += wu.mg + wv.mg;
@@ -757,14 +781,21 @@ __device__ __forceinline__ float gval(const VW<GMODE, KC> &wv, const UW<GMODE, K
 }
 
 // d_f1[p, c] = sum_q G[p,q] f2[q,c].  Grid: (B * tiles_per_batch, channel blocks of 128*NCB).
-template <int GMODE, int KC, int NCB, bool CVEC, int MAXT>
+// FAST (C == 256, W2 % 4 == 0, both channel blocks in one workgroup): the operand loads take no address
+// arithmetic at all -- a per-lane offset for each group of 4 columns is kept in a register, the row advances
+// through the scalar offset and the column within the group and the channel block through the immediate.
+// (fp32 MFMA and vector instructions share the SIMD's arithmetic lanes here: every vector instruction in the
+// loop costs its issue time, nothing hides behind the matrix work.)
+template <int GMODE, int KC, int NCB, bool CVEC, int MAXT, bool FAST = false>
 __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
+    static_assert(!FAST || (CVEC && NCB == 2), "fast loads: 16-byte loads, 256 channels per workgroup");
     constexpr int GS = 2;            // MFMA k-steps (pairs of v) per prefetch group
     constexpr int NG = 16 / GS;
     constexpr int CB = 128 * NCB;
     constexpr int RS = CB + 4;
     extern __shared__ float smem[];  // [TP][RS] cross-wave sum
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, pl = lane & 31, h = lane >> 5;
+    const int tid = threadIdx.x, lane = tid & 63, pl = lane & 31, h = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nW = blockDim.x >> 6;
     // wave (vcw, ug): columns [32 vcw, 32 vcw + 32), rows ug, ug + NUG, ... (see fwd_kernel)
     const int nvc = a.nvc, NUG = nW / nvc;
@@ -806,9 +837,23 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
         const int c = cb0 + 128 * cb + 4 * pl;
         coff[cb] = c < C ? (unsigned)c * 4u : nbytes;
     }
+    // FAST: byte offset of (column 8 q + 4 h of this wave's chunk, channel 4 pl) or the out-of-range marker
+    unsigned voffq[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int v = vbase + 32 * vcw + vmap(4 * q, h);
+        voffq[q] = v < W2 ? ((unsigned)v * 256u + 4u * pl) * 4u : DMA_OOB;
+    }
     auto issue = [&](int u, int g, v4f(&buf)[GS][NCB]) {
 #pragma unroll
         for (int ss = 0; ss < GS; ++ss) {
+            if constexpr (FAST) {
+                const int r = g * GS + ss;
+                const unsigned row = (unsigned)u * ((unsigned)W2 * 1024u);
+#pragma unroll
+                for (int cb = 0; cb < NCB; ++cb) buf[ss][cb] = buf_load4s(rsrc, voffq[r >> 2], row + (1024u * (r & 3) + 512u * cb));
+                continue;
+            }
             const int v = vbase + 32 * vcw + vmap(g * GS + ss, h);
             const bool ok = v < W2;
             if constexpr (CVEC) {
@@ -826,18 +871,56 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
     // G of the current row lives in G[]; G of this wave's next row (u + NUG) is computed two values per
     // MFMA group, between the group's MFMAs, so the arithmetic runs in the shadow of the matrix pipe.
     float G[16], Gn[16];
-    UW<GMODE, KC> wu_n = load_uw<GMODE, KC>(a, bp, min(ug, H2 - 1), true);   // bp is clamped: always a valid pixel
+    // FAST: the (p,u)-indexed weights come through buffer loads as well: a per-lane offset to the pixel's first
+    // entry, channel and row in the scalar offset
+    const unsigned pixb = pok ? (unsigned)pix : 0u;
+    const unsigned uwoff_c = (pixb * a.KT + a.k0) * H2 * 4u, uwoff_2 = pixb * 2u * H2 * 4u, uwoff_1 = pixb * H2 * 4u;
+    __amdgpu_buffer_rsrc_t rs_av, rs_gcu, rs_gu, rs_amu;
+    if constexpr (FAST) {
+        if constexpr (g_has_comp(GMODE)) {
+            rs_av = make_rsrc(a.a_v + (size_t)b * N1 * a.KT * H2, (unsigned)N1 * a.KT * H2 * 4u);
+            rs_gcu = make_rsrc(a.g_cu + (size_t)b * N1 * a.KT * H2, (unsigned)N1 * a.KT * H2 * 4u);
+        }
+        if constexpr (g_has_maxavg(GMODE)) {
+            rs_gu = make_rsrc(a.g_u + (size_t)b * N1 * 2 * H2, (unsigned)N1 * 2u * H2 * 4u);
+            rs_amu = make_rsrc(a.am_u + (size_t)b * N1 * H2, (unsigned)N1 * H2 * 4u);
+        }
+    }
+    const float inv_w2 = 1.f / (float)W2;
+    auto load_uw_row = [&](int u) {
+        if constexpr (!FAST) {
+            return load_uw<GMODE, KC>(a, bp, u, true);   // bp is clamped: always a valid pixel
+        } else {
+            UW<GMODE, KC> w;
+            if constexpr (g_has_comp(GMODE)) {
+#pragma unroll
+                for (int k = 0; k < KC; ++k) {
+                    w.a[k] = buf_load1s(rs_av, uwoff_c, (unsigned)(k * H2 + u) * 4u);
+                    w.g[k] = buf_load1s(rs_gcu, uwoff_c, (unsigned)(k * H2 + u) * 4u);
+                }
+            }
+            if constexpr (g_has_maxavg(GMODE)) {
+                w.ma = buf_load1s(rs_gu, uwoff_2, (unsigned)u * 4u);
+                w.mg = buf_load1s(rs_gu, uwoff_2, (unsigned)(H2 + u) * 4u) * inv_w2;
+                w.am = __float_as_int(buf_load1s(rs_amu, uwoff_1, (unsigned)u * 4u));
+            }
+            return w;
+        }
+    };
+    UW<GMODE, KC> wu_n = load_uw_row(min(ug, H2 - 1));
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
         const int v = vbase + 32 * vcw + vmap(r, h);
-        G[r] = gval<GMODE, KC>(wv[r], wu_n, ug, v, pok && v < W2);
+        // no mask: a column outside the image has an all-zero A operand and the column of a pixel outside the
+        // image is never stored; the weights behind both are those of real entries, so G stays finite
+        G[r] = gval<GMODE, KC>(wv[r], wu_n, ug, v, true);
     }
-    UW<GMODE, KC> wu_next = load_uw<GMODE, KC>(a, bp, min(ug + NUG, H2 - 1), true);
+    UW<GMODE, KC> wu_next = load_uw_row(min(ug + NUG, H2 - 1));
     auto compute = [&](int u, int g, v4f(&buf)[GS][NCB]) {
         static_assert(GS == 2, "two G values are produced per group");
         if (g == 0) {
             wu_n = wu_next;                                                       // weights of row u + NUG
-            wu_next = load_uw<GMODE, KC>(a, bp, min(u + 2 * NUG, H2 - 1), true);  // and of the row after it
+            wu_next = load_uw_row(min(u + 2 * NUG, H2 - 1));                      // and of the row after it
         }
 #pragma unroll
         for (int cb = 0; cb < NCB; ++cb)
@@ -848,7 +931,7 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
         for (int ss = 0; ss < GS; ++ss) {
             const int r = g * GS + ss;
             const int v = vbase + 32 * vcw + vmap(r, h);
-            Gn[r] = gval<GMODE, KC>(wv[r], wu_n, u + NUG, v, pok && v < W2);
+            Gn[r] = gval<GMODE, KC>(wv[r], wu_n, u + NUG, v, true);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -1018,7 +1101,6 @@ __global__ void __launch_bounds__(256) df2_kernel(const BwdArgs a, int ntasks, i
 __device__ __forceinline__ void dma16(__amdgpu_buffer_rsrc_t r, float *lds_chunk, unsigned voff) {
     __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void *)lds_chunk, 16, voff, 0, 0, 0);
 }
-constexpr unsigned DMA_OOB = 0x80000000u;   // above every buffer size used here: reads as zero
 
 // buffers of the (p,u)-indexed weights per wave: the combined mode has LDS for one only
 constexpr int df2_tiled_ubuf(int gmode) { return gmode == GMODE_BOTH ? 1 : 2; }
@@ -1076,21 +1158,25 @@ __global__ void __launch_bounds__(64 * NWV) df2_tiled_kernel(const BwdArgs a, in
             rs_vc = make_rsrc(a.g_v + (size_t)b * N1 * 2u * W2, up * 2u * W2 * 4u);
             rs_vd = make_rsrc(a.am_v + (size_t)b * N1 * W2, up * W2 * 4u);
         }
-        // lane-constant parts of the DMA offsets
+        // DMA offsets = a lane-constant part (kept in registers) + a wave-uniform part that moves with the tile:
+        // one vector add per transfer.  The pixel index stays inside the checked offset, so rows at or beyond
+        // `pend` still read as zero.
+        constexpr int FCH = CB / 8 / NWV;   // 256-float chunks of the f1 tile per wave
         const int frow = (lane * 4) / CB, fcol = (lane * 4) % CB;        // within a 256-float chunk of the f1 tile
         const unsigned fcoff = (cb0 + fcol < C) ? (unsigned)(cb0 + fcol) * 4u : DMA_OOB;
+        unsigned f_lane[FCH];
+#pragma unroll
+        for (int i = 0; i < FCH; ++i) f_lane[i] = (unsigned)((wave * FCH + i) * (256 / CB) + frow) * C * 4u + fcoff;
         const unsigned vcol = (unsigned)(v0 + 4 * (lane & 7)) * 4u;
+        const unsigned prow = (unsigned)(lane >> 3);                      // pixel of this lane within a weight chunk
+        const unsigned wl_c = prow * pstride_c * 4u + vcol, wl_2 = prow * 2u * W2 * 4u + vcol, wl_1 = prow * W2 * 4u + vcol;
 
         auto issue_tile = [&](int tile, int bi) {
-            const int pt0 = pbeg + tile * TP;
+            const unsigned pt0 = (unsigned)(pbeg + tile * TP);
             float *fdst = F1s + bi * 32 * CB;
-            constexpr int FCH = CB / 8 / NWV;   // 256-float chunks per wave
+            const unsigned tf = pt0 * C * 4u;
 #pragma unroll
-            for (int i = 0; i < FCH; ++i) {
-                const int ch = wave * FCH + i;
-                const int row = ch * (256 / CB) + frow;
-                dma16(rs_f1, fdst + ch * 256, (unsigned)(pt0 + row) * C * 4u + fcoff);
-            }
+            for (int i = 0; i < FCH; ++i) dma16(rs_f1, fdst + (wave * FCH + i) * 256, f_lane[i] + tf);
             float *vdst = VWs + bi * NV * 1024;
             // the weight tile of one tensor is four 256-float chunks (8 pixels each); chunk c = 4*kk + quarter
 #pragma unroll
@@ -1098,36 +1184,50 @@ __global__ void __launch_bounds__(64 * NWV) df2_tiled_kernel(const BwdArgs a, in
                 const int c = wave + NWV * i;
                 if (4 * NV % NWV != 0 && c >= 4 * NV) break;
                 const int kk = c >> 2, quarter = c & 3;
-                const unsigned p = (unsigned)(pt0 + 8 * quarter + (lane >> 3));
+                const unsigned p8 = pt0 + 8u * quarter;   // first pixel of the chunk (uniform)
                 float *dst = vdst + c * 256;
                 if (HC && kk < NVC) {
-                    const unsigned off = (p * pstride_c + (unsigned)(a.k0 + (kk % KC)) * W2) * 4u + vcol;
-                    if constexpr (HC) dma16(kk < KC ? rs_va : rs_vb, dst, off);
+                    const unsigned uni = (p8 * pstride_c + (unsigned)(a.k0 + (kk % KC)) * W2) * 4u;
+                    if constexpr (HC) dma16(kk < KC ? rs_va : rs_vb, dst, wl_c + uni);
                 } else if constexpr (HM) {
                     const int m = kk - NVC;
-                    if (m < 2) dma16(rs_vc, dst, (p * 2u * W2 + (unsigned)m * W2) * 4u + vcol);
-                    else dma16(rs_vd, dst, p * W2 * 4u + vcol);
+                    if (m < 2) dma16(rs_vc, dst, wl_2 + (p8 * 2u * W2 + (unsigned)m * W2) * 4u);
+                    else dma16(rs_vd, dst, wl_1 + p8 * W2 * 4u);
                 }
             }
         };
-        // (p,u)-indexed weights of this wave's row: lane pl fetches pixel pt0+pl (both halves the same)
+        // (p,u)-indexed weights of this wave's row: lane pl fetches pixel pt0+pl (both halves the same), through
+        // buffer loads whose channel/row part is a scalar offset
+        __amdgpu_buffer_rsrc_t rs_av, rs_gcu, rs_gu, rs_amu;
+        if constexpr (HC) {
+            rs_av = make_rsrc(a.a_v + (size_t)b * N1 * a.KT * H2, (unsigned)N1 * a.KT * H2 * 4u);
+            rs_gcu = make_rsrc(a.g_cu + (size_t)b * N1 * a.KT * H2, (unsigned)N1 * a.KT * H2 * 4u);
+        }
+        if constexpr (HM) {
+            rs_gu = make_rsrc(a.g_u + (size_t)b * N1 * 2 * H2, (unsigned)N1 * 2u * H2 * 4u);
+            rs_amu = make_rsrc(a.am_u + (size_t)b * N1 * H2, (unsigned)N1 * H2 * 4u);
+        }
         auto load_uw_tile = [&](int tile, float(&r)[NUP]) {
-            const int p = min(pbeg + tile * TP + pl, pend - 1);
-            const size_t bp = (size_t)b * N1 + p;
+            const unsigned p = (unsigned)min(pbeg + tile * TP + pl, pend - 1);
+            const unsigned o1 = p * H2 * 4u;   // byte offset of the pixel's first entry in a 1-channel tensor
 #pragma unroll
             for (int i = 0; i < NUP; ++i) r[i] = 0.f;
             if constexpr (HC) {
+                const unsigned oc = o1 * a.KT;
 #pragma unroll
                 for (int k = 0; k < KC; ++k) {
-                    const size_t o = (bp * a.KT + a.k0 + k) * H2 + u;
-                    r[k] = a.a_v[o];
-                    r[KC + k] = a.g_cu[o];
+                    const unsigned so = (unsigned)((a.k0 + k) * H2 + u) * 4u;
+                    r[k] = buf_load1s(rs_av, oc, so);
+                    r[KC + k] = buf_load1s(rs_gcu, oc, so);
                 }
             }
             if constexpr (HM) {
-                r[NVC + 0] = a.g_u[(bp * 2 + 0) * H2 + u];
-                r[NVC + 1] = a.g_u[(bp * 2 + 1) * H2 + u];
-                r[NVC + 2] = __int_as_float(a.am_u[bp * H2 + u]);
+                // stored as: value if the row's argmax is this column, value otherwise, argmax
+                const float ma = buf_load1s(rs_gu, o1 * 2u, (unsigned)u * 4u);
+                const float mg = buf_load1s(rs_gu, o1 * 2u, (unsigned)(H2 + u) * 4u) * inv_w2;
+                r[NVC + 0] = mg + ma;
+                r[NVC + 1] = mg;
+                r[NVC + 2] = buf_load1s(rs_amu, o1, (unsigned)u * 4u);
             }
         };
         // With one buffer the rows of the next tile replace those of the current one after its last read:
@@ -1166,27 +1266,32 @@ __global__ void __launch_bounds__(64 * NWV) df2_tiled_kernel(const BwdArgs a, in
                 float uw[NUP], vw[NV];
                 v4f fa[NCB];
             };
+            // one lane-dependent base address per LDS region and tile; every step is a constant offset from it
+            // (an immediate of the LDS instruction, no address arithmetic in the loop)
+            const float *us_l = us + h * NUP, *vs_l = vs + h * 32 + pl, *fs_l = fs + h * CB + 4 * pl;
             auto lds_fetch = [&](int s, StepOps &o) {
-                const int row = 2 * s + h;
 #pragma unroll
                 for (int i = 0; i < NUP; i += 4) {
-                    const v4f x = *reinterpret_cast<const v4f *>(us + row * NUP + i);
+                    const v4f x = *reinterpret_cast<const v4f *>(us_l + 2 * s * NUP + i);
                     o.uw[i] = x[0]; o.uw[i + 1] = x[1]; o.uw[i + 2] = x[2]; o.uw[i + 3] = x[3];
                 }
 #pragma unroll
-                for (int kk = 0; kk < NV; ++kk) o.vw[kk] = vs[kk * 1024 + row * 32 + pl];
+                for (int kk = 0; kk < NV; ++kk) o.vw[kk] = vs_l[kk * 1024 + 2 * s * 32];
 #pragma unroll
-                for (int cb = 0; cb < NCB; ++cb) o.fa[cb] = *reinterpret_cast<const v4f *>(fs + row * CB + 128 * cb + 4 * pl);
+                for (int cb = 0; cb < NCB; ++cb) o.fa[cb] = *reinterpret_cast<const v4f *>(fs_l + 2 * s * CB + 128 * cb);
             };
             auto g_of = [&](int s, const StepOps &o) {
                 float G = 0.f;
                 if constexpr (HC) {
 #pragma unroll
-                    for (int k = 0; k < KC; ++k) G += o.vw[k] * o.uw[KC + k] + o.uw[k] * o.vw[KC + k];
+                    for (int k = 0; k < KC; ++k) {
+                        G = fmaf(o.vw[k], o.uw[KC + k], G);
+                        G = fmaf(o.uw[k], o.vw[KC + k], G);
+                    }
                 }
                 if constexpr (HM) {
-                    G += o.uw[NVC + 1] * inv_w2 + o.vw[NVC + 1] * inv_h2;
-                    if (__float_as_int(o.uw[NVC + 2]) == v) G += o.uw[NVC];
+                    G += __float_as_int(o.uw[NVC + 2]) == v ? o.uw[NVC] : o.uw[NVC + 1];
+                    G = fmaf(o.vw[NVC + 1], inv_h2, G);
                     if (__float_as_int(o.vw[NVC + 2]) == u) G += o.vw[NVC];
                 }
                 // No mask needed: pixels at or beyond `pend` have all-zero f1 rows and (p,v) weights (DMA
@@ -1431,7 +1536,8 @@ Df2Plan df2_plan(const Dims &d, bool both) {
     pl.rows = df2_rows_per_wg(d, both);
     const size_t big = (size_t)1 << 30;
     const size_t n1 = (size_t)d.H1 * d.W1;
-    pl.tiled = d.C % 4 == 0 && d.W2 % 4 == 0 && n1 * d.C * 4 <= big && n1 * MAX_K * d.W2 * 4 <= big;
+    pl.tiled = d.C % 4 == 0 && d.W2 % 4 == 0 && n1 * d.C * 4 <= big && n1 * MAX_K * d.W2 * 4 <= big &&
+               n1 * MAX_K * d.H2 * 4 <= big;
     const int tiles = (int)((n1 + TP - 1) / TP);
     const int nvc = (d.W2 + 31) / 32;
     const int cblocks = (d.C + 255) / 256;
@@ -1481,6 +1587,10 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s
     } while (0)
         if (nW > 4) { if (cvec) SEPCORR_DF1(1, true, 512); else SEPCORR_DF1(1, false, 512); }
         else if (ncb == 1) { if (cvec) SEPCORR_DF1(1, true, 256); else SEPCORR_DF1(1, false, 256); }
+        else if (cvec && d.C == 256 && d.W2 % 4 == 0) {
+            ProfScope ps(GMODE == GMODE_COMP ? "df1_comp" : GMODE == GMODE_BOTH ? "df1_both" : "df1_maxavg", s1);
+            hipLaunchKernelGGL((df1_kernel<GMODE, KC, 2, true, 256, true>), grid, block, lds, s1, a);
+        }
         else { if (cvec) SEPCORR_DF1(2, true, 256); else SEPCORR_DF1(2, false, 256); }
 #undef SEPCORR_DF1
         if (int rc = check_launch("d_f1 kernel")) return rc;
