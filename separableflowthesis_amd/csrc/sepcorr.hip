@@ -1426,6 +1426,8 @@ WaveGrid wave_grid(int B, int tiles_per_batch, int W2, int H2) {
         g.nug = 4 / g.nvc;                                        // 4 waves
         if ((long)B * tiles_per_batch * 4 < 1536) g.nug *= 2;     // small problem: 8 waves fill more SIMDs
         while (g.nug > 1 && g.nug > H2) g.nug /= 2;
+    } else if (g.nvc <= 4 && (long)B * tiles_per_batch <= 256 && H2 >= 8) {
+        g.nug = 2;   // at most one workgroup per CU: two row groups give every SIMD a second wave
     }
     return g;
 }
