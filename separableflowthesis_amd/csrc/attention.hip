@@ -43,13 +43,16 @@ struct AttArgs {
     int B, H1, W1, L, K;
 };
 
-// Forward.  NCH = ceil(L / 64) chunks per row held in registers.
+// Forward.  NCH = ceil(L / 64) chunks per row.  A lane first gathers the 54 inputs of each of its positions (9
+// neighbouring pixels x 2 channels x 3 shifts along L, zero outside the volume) into registers, then runs the K
+// filters over them with the weights read from LDS four at a time: 54 FMAs per position and filter, no load in
+// the filter loop.
 template <int NCH>
 __global__ void __launch_bounds__(64 * WPB) att_forward_kernel(const AttArgs a) {
-    __shared__ float ws[MAXK * 54 + MAXK];
+    __shared__ __attribute__((aligned(16))) float ws[MAXK * 56 + MAXK];   // [k][56]: 54 weights (c, dl, di, dj) + 2 pad
     const int K = a.K, L = a.L, H1 = a.H1, W1 = a.W1;
-    for (int t = threadIdx.x; t < K * 54; t += blockDim.x) ws[t] = a.weight[t];
-    for (int t = threadIdx.x; t < K; t += blockDim.x) ws[MAXK * 54 + t] = a.bias ? a.bias[t] : 0.f;
+    for (int t = threadIdx.x; t < K * 54; t += blockDim.x) ws[(t / 54) * 56 + t % 54] = a.weight[t];
+    for (int t = threadIdx.x; t < K; t += blockDim.x) ws[MAXK * 56 + t] = a.bias ? a.bias[t] : 0.f;
     __syncthreads();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const long pix = (long)blockIdx.x * WPB + wave;       // flattened (b,i,j)
@@ -57,30 +60,38 @@ __global__ void __launch_bounds__(64 * WPB) att_forward_kernel(const AttArgs a) 
     if (pix >= npix) return;
     const int j = (int)(pix % W1), i = (int)((pix / W1) % H1);
 
+    float x[NCH][2][3][9];   // [chunk][c][dl][neighbour di*3+dj]: the order of the weights
+#pragma unroll
+    for (int n = 0; n < 9; ++n) {
+        const int ii = i + n / 3 - 1, jj = j + n % 3 - 1;
+        const bool inb = ii >= 0 && ii < H1 && jj >= 0 && jj < W1;   // wave-uniform
+        const float *row = a.sep + (pix + (long)(n / 3 - 1) * W1 + (n % 3 - 1)) * 2 * L;
+#pragma unroll
+        for (int ch = 0; ch < NCH; ++ch)
+#pragma unroll
+            for (int c = 0; c < 2; ++c)
+#pragma unroll
+                for (int dl = 0; dl < 3; ++dl) {
+                    const int ll = ch * 64 + lane + dl - 1;
+                    x[ch][c][dl][n] = (inb && ll >= 0 && ll < L) ? row[c * L + ll] : 0.f;
+                }
+    }
+
     for (int k = 0; k < K; ++k) {
         float logit[NCH];
 #pragma unroll
-        for (int c = 0; c < NCH; ++c) logit[c] = ws[MAXK * 54 + k];
-        for (int di = 0; di < 3; ++di) {
-            const int ii = i + di - 1;
-            if (ii < 0 || ii >= H1) continue;
-            for (int dj = 0; dj < 3; ++dj) {
-                const int jj = j + dj - 1;
-                if (jj < 0 || jj >= W1) continue;
-                const float *row = a.sep + (pix + (long)(di - 1) * W1 + (dj - 1)) * 2 * L;
+        for (int ch = 0; ch < NCH; ++ch) logit[ch] = ws[MAXK * 56 + k];
 #pragma unroll
-                for (int c = 0; c < 2; ++c) {
-                    const float w0 = ws[((k * 2 + c) * 3 + 0) * 9 + di * 3 + dj];
-                    const float w1 = ws[((k * 2 + c) * 3 + 1) * 9 + di * 3 + dj];
-                    const float w2 = ws[((k * 2 + c) * 3 + 2) * 9 + di * 3 + dj];
+        for (int q = 0; q < 14; ++q) {   // 56 floats = 14 reads of 16 bytes, the same address in every lane
+            const float4 w4 = *reinterpret_cast<const float4 *>(&ws[k * 56 + 4 * q]);
+            const float wq[4] = {w4.x, w4.y, w4.z, w4.w};
 #pragma unroll
-                    for (int ch = 0; ch < NCH; ++ch) {
-                        const int l = ch * 64 + lane;
-                        const float x0 = (l - 1 >= 0 && l - 1 < L) ? row[c * L + l - 1] : 0.f;
-                        const float x1 = (l < L) ? row[c * L + l] : 0.f;
-                        const float x2 = (l + 1 < L) ? row[c * L + l + 1] : 0.f;
-                        logit[ch] += w0 * x0 + w1 * x1 + w2 * x2;
-                    }
+            for (int e = 0; e < 4; ++e) {
+                const int t = 4 * q + e;
+                if (t < 54) {
+                    const int c = t / 27, dl = (t / 9) % 3, n = t % 9;
+#pragma unroll
+                    for (int ch = 0; ch < NCH; ++ch) logit[ch] = fmaf(wq[e], x[ch][c][dl][n], logit[ch]);
                 }
             }
         }
@@ -168,10 +179,12 @@ __global__ void __launch_bounds__(64 * WPB) att_softmax_backward_kernel(const At
 }
 
 // d_sep[(i,j),c,l] = sum_{k,dl,di,dj} w[k][c][dl][di][dj] * dlogits[(i-di+1, j-dj+1), k, l-dl+1]
+// Per filter k a lane gathers the 27 logit gradients it needs (9 neighbouring pixels x 3 shifts, zero outside the
+// volume), then applies the two 27-tap rows of the filter, read from LDS four weights at a time.
 __global__ void __launch_bounds__(64 * WPB) att_input_backward_kernel(const AttArgs a) {
-    __shared__ float ws[MAXK * 54];
+    __shared__ __attribute__((aligned(16))) float ws[MAXK * 2 * 28];   // [k][c][28]: 27 weights (dl, di, dj) + 1 pad
     const int K = a.K, L = a.L, H1 = a.H1, W1 = a.W1;
-    for (int t = threadIdx.x; t < K * 54; t += blockDim.x) ws[t] = a.weight[t];
+    for (int t = threadIdx.x; t < K * 54; t += blockDim.x) ws[(t / 27) * 28 + t % 27] = a.weight[t];
     __syncthreads();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const long pix = (long)blockIdx.x * WPB + wave;
@@ -179,21 +192,29 @@ __global__ void __launch_bounds__(64 * WPB) att_input_backward_kernel(const AttA
     const int j = (int)(pix % W1), i = (int)((pix / W1) % H1);
     for (int l = lane; l < L; l += 64) {
         float d0 = 0.f, d1 = 0.f;
-        for (int di = 0; di < 3; ++di) {
-            const int ii = i - di + 1;
-            if (ii < 0 || ii >= H1) continue;
-            for (int dj = 0; dj < 3; ++dj) {
-                const int jj = j - dj + 1;
-                if (jj < 0 || jj >= W1) continue;
-                const float *g = a.dlogits + (pix + (long)(1 - di) * W1 + (1 - dj)) * K * L;
-                for (int k = 0; k < K; ++k)
-                    for (int dl = 0; dl < 3; ++dl) {
-                        const int ll = l - dl + 1;
-                        if (ll >= 0 && ll < L) {
-                            const float gv = g[k * L + ll];
-                            d0 += ws[((k * 2 + 0) * 3 + dl) * 9 + di * 3 + dj] * gv;
-                            d1 += ws[((k * 2 + 1) * 3 + dl) * 9 + di * 3 + dj] * gv;
-                        }
+        for (int k = 0; k < K; ++k) {
+            float x[27];   // [dl][di*3+dj]: the order of the weights
+#pragma unroll
+            for (int n = 0; n < 9; ++n) {
+                const int ii = i - n / 3 + 1, jj = j - n % 3 + 1;
+                const bool inb = ii >= 0 && ii < H1 && jj >= 0 && jj < W1;   // wave-uniform
+                const float *g = a.dlogits + ((pix + (long)(1 - n / 3) * W1 + (1 - n % 3)) * K + k) * L;
+#pragma unroll
+                for (int dl = 0; dl < 3; ++dl) {
+                    const int ll = l - dl + 1;
+                    x[dl * 9 + n] = (inb && ll >= 0 && ll < L) ? g[ll] : 0.f;
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < 7; ++q) {   // 28 floats = 7 reads of 16 bytes per channel, the same address in every lane
+                const float4 u4 = *reinterpret_cast<const float4 *>(&ws[(k * 2 + 0) * 28 + 4 * q]);
+                const float4 v4 = *reinterpret_cast<const float4 *>(&ws[(k * 2 + 1) * 28 + 4 * q]);
+                const float u[4] = {u4.x, u4.y, u4.z, u4.w}, v[4] = {v4.x, v4.y, v4.z, v4.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (4 * q + e < 27) {
+                        d0 = fmaf(u[e], x[4 * q + e], d0);
+                        d1 = fmaf(v[e], x[4 * q + e], d1);
                     }
             }
         }
@@ -202,71 +223,104 @@ __global__ void __launch_bounds__(64 * WPB) att_input_backward_kernel(const AttA
     }
 }
 
-// Weight and bias gradient, stage 1.  Workgroup (x, y): pixels [x*DW_PIX, ...), neighbour y = di*3+dj.
-// Wave w of the 4 handles every 4th pixel; per lane 6*K accumulators (c, dl, k); reduced over lanes and
-// waves, written as partial[x][...].
+// Sum over the 64 lanes with data-parallel-primitive adds (one vector instruction per step, no LDS traffic);
+// the total is returned by lane 63.
+__device__ __forceinline__ float wave_sum_dpp(float x) {
+    // row_shr:1, 2, 3 gather a row's four-lane groups; row_shr:4 and 8 (bank masked) complete the row of 16;
+    // row_bcast:15 / 31 carry the row totals across rows
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x111, 0xf, 0xf, true));
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x112, 0xf, 0xf, true));
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x114, 0xf, 0xe, true));
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x118, 0xf, 0xc, true));
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x142, 0xa, 0xf, true));
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x143, 0xc, 0xf, true));
+    return x;
+}
+
+// Weight and bias gradient, stage 1.  Workgroup (x, y): pixels [x*DW_PIX, ...), input channel c = y % 2, weight
+// channels [4 (y/2), +4).  Wave w of the 4 handles every 4th pixel, lanes run along L.  Per position a lane gathers
+// the 27 inputs of its channel (9 neighbouring pixels x 3 shifts along L, zero outside the volume) and the 4 logit
+// gradients, then updates 27 x 4 accumulators (108 registers: two waves fit a SIMD); these are reduced over lanes
+// and waves in a fixed order and written as partial[x][...].
+constexpr int DW_KC = 4;
 __global__ void __launch_bounds__(256) att_weight_backward_kernel(const AttArgs a) {
-    __shared__ float red[4][6 * MAXK + MAXK];
+    __shared__ float red[4][27 * DW_KC + DW_KC];
     const int K = a.K, L = a.L, H1 = a.H1, W1 = a.W1;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int di = blockIdx.y / 3, dj = blockIdx.y % 3;
+    const int c = blockIdx.y & 1, k0 = (blockIdx.y >> 1) * DW_KC;
     const long npix = (long)a.B * H1 * W1;
     const long p0 = (long)blockIdx.x * DW_PIX;
-    float acc[6 * MAXK], accb[MAXK];
+    float acc[27][DW_KC], accb[DW_KC];
 #pragma unroll
-    for (int t = 0; t < 6 * MAXK; ++t) acc[t] = 0.f;
+    for (int t = 0; t < 27; ++t)
 #pragma unroll
-    for (int t = 0; t < MAXK; ++t) accb[t] = 0.f;
-    for (int q = wave; q < DW_PIX; q += 4) {
-        const long pix = p0 + q;
-        if (pix >= npix) break;
+        for (int k = 0; k < DW_KC; ++k) acc[t][k] = 0.f;
+#pragma unroll
+    for (int k = 0; k < DW_KC; ++k) accb[k] = 0.f;
+    // iterations = (pixel of this wave, chunk of 64 positions); the inputs of the next iteration are fetched while
+    // the accumulators are updated with the current ones
+    const int nch = (L + 63) >> 6;
+    const long left = npix - p0;
+    const int npx = (int)(left < DW_PIX ? left : DW_PIX);
+    const int nit = ((npx - wave + 3) / 4) * nch;   // pixels wave, wave + 4, ... below npx
+    auto fetch = [&](int it, float(&x)[27], float(&gv)[DW_KC]) {
+        const long pix = p0 + wave + 4 * (it / nch);
+        const int l = (it % nch) * 64 + lane;
         const int j = (int)(pix % W1), i = (int)((pix / W1) % H1);
-        const int ii = i + di - 1, jj = j + dj - 1;
-        const bool inb = ii >= 0 && ii < H1 && jj >= 0 && jj < W1;
-        const float *g = a.dlogits + pix * K * L;
-        const float *row = a.sep + (pix + (long)(di - 1) * W1 + (dj - 1)) * 2 * L;
-        for (int l = lane; l < L; l += 64) {
-            float x[2][3];
 #pragma unroll
-            for (int c = 0; c < 2; ++c)
+        for (int n = 0; n < 9; ++n) {
+            const int ii = i + n / 3 - 1, jj = j + n % 3 - 1;
+            const bool inb = ii >= 0 && ii < H1 && jj >= 0 && jj < W1;   // wave-uniform
+            const float *row = a.sep + ((pix + (long)(n / 3 - 1) * W1 + (n % 3 - 1)) * 2 + c) * L;
 #pragma unroll
-                for (int dl = 0; dl < 3; ++dl) {
-                    const int ll = l + dl - 1;
-                    x[c][dl] = (inb && ll >= 0 && ll < L) ? row[c * L + ll] : 0.f;
-                }
-#pragma unroll
-            for (int k = 0; k < MAXK; ++k) {
-                if (k < K) {
-                    const float gv = g[k * L + l];
-                    if (blockIdx.y == 4) accb[k] += gv;   // bias: counted once, by the centre tap
-#pragma unroll
-                    for (int c = 0; c < 2; ++c)
-#pragma unroll
-                        for (int dl = 0; dl < 3; ++dl) acc[(k * 2 + c) * 3 + dl] += gv * x[c][dl];
-                }
+            for (int dl = 0; dl < 3; ++dl) {
+                const int ll = l + dl - 1;
+                x[dl * 9 + n] = (inb && ll >= 0 && ll < L) ? row[ll] : 0.f;   // [dl][neighbour]: the order of the weights
             }
         }
+        const float *g = a.dlogits + pix * K * L;
+#pragma unroll
+        for (int k = 0; k < DW_KC; ++k) gv[k] = (k0 + k < K && l < L) ? g[(k0 + k) * L + l] : 0.f;
+    };
+    auto update = [&](const float(&x)[27], const float(&gv)[DW_KC]) {
+#pragma unroll
+        for (int k = 0; k < DW_KC; ++k) {
+            accb[k] += gv[k];
+#pragma unroll
+            for (int t = 0; t < 27; ++t) acc[t][k] = fmaf(gv[k], x[t], acc[t][k]);
+        }
+    };
+    float xa[27], xb[27], ga[DW_KC], gb[DW_KC];
+    if (nit > 0) fetch(0, xa, ga);
+    for (int it = 0; it < nit; it += 2) {
+        if (it + 1 < nit) fetch(it + 1, xb, gb);
+        update(xa, ga);
+        if (it + 2 < nit) fetch(it + 2, xa, ga);
+        if (it + 1 < nit) update(xb, gb);
     }
 #pragma unroll
-    for (int t = 0; t < 6 * MAXK; ++t) {
-        const float r = wave_sum(acc[t]);
-        if (lane == 0) red[wave][t] = r;
-    }
+    for (int t = 0; t < 27; ++t)
 #pragma unroll
-    for (int t = 0; t < MAXK; ++t) {
-        const float r = wave_sum(accb[t]);
-        if (lane == 0) red[wave][6 * MAXK + t] = r;
+        for (int k = 0; k < DW_KC; ++k) {
+            const float r = wave_sum_dpp(acc[t][k]);
+            if (lane == 63) red[wave][t * DW_KC + k] = r;
+        }
+#pragma unroll
+    for (int k = 0; k < DW_KC; ++k) {
+        const float r = wave_sum_dpp(accb[k]);
+        if (lane == 63) red[wave][27 * DW_KC + k] = r;
     }
     __syncthreads();
-    // partial layout per workgroup x: [K*54 weights in weight order][K biases]
+    // partial layout per workgroup x: [K*54 weights in weight order (k, c, dl, di, dj)][K biases]
     float *dst = a.partial + (long)blockIdx.x * (K * 54 + K);
-    for (int t = threadIdx.x; t < 6 * K; t += blockDim.x) {
-        const int k = t / 6, c = (t / 3) % 2, dl = t % 3;
-        dst[((k * 2 + c) * 3 + dl) * 9 + di * 3 + dj] = red[0][t] + red[1][t] + red[2][t] + red[3][t];
+    for (int t = threadIdx.x; t < 27 * DW_KC; t += blockDim.x) {
+        const int k = t % DW_KC, tap = t / DW_KC;
+        if (k0 + k < K) dst[(k0 + k) * 54 + c * 27 + tap] = red[0][t] + red[1][t] + red[2][t] + red[3][t];
     }
-    if (blockIdx.y == 4)
-        for (int t = threadIdx.x; t < K; t += blockDim.x)
-            dst[K * 54 + t] = red[0][6 * MAXK + t] + red[1][6 * MAXK + t] + red[2][6 * MAXK + t] + red[3][6 * MAXK + t];
+    if (c == 0)   // the bias gradient is counted once
+        for (int t = threadIdx.x; t < DW_KC; t += blockDim.x)
+            if (k0 + t < K)
+                dst[K * 54 + k0 + t] = red[0][27 * DW_KC + t] + red[1][27 * DW_KC + t] + red[2][27 * DW_KC + t] + red[3][27 * DW_KC + t];
 }
 
 // Stage 2: out[t] = sum over workgroups of partial[x][t].  One wave per output: lane l adds the partials
@@ -369,7 +423,7 @@ int sepcorr_attention_backward(const float *sep, const float *weight, const floa
     args.out = d_sep;
     hipLaunchKernelGGL(att_input_backward_kernel, grid, block, 0, s, args);
     if (int rc = launched("attention input gradient kernel")) return rc;
-    hipLaunchKernelGGL(att_weight_backward_kernel, dim3(nwg, 9), dim3(256), 0, s, args);
+    hipLaunchKernelGGL(att_weight_backward_kernel, dim3(nwg, 2 * ((K + DW_KC - 1) / DW_KC)), dim3(256), 0, s, args);
     if (int rc = launched("attention weight gradient kernel")) return rc;
     const int n = K * 54 + K;
     hipLaunchKernelGGL(att_weight_reduce_kernel, dim3((n + 3) / 4), dim3(256), 0, s, args.partial, d_weight, d_bias, nwg, K);
