@@ -34,6 +34,17 @@ __device__ __forceinline__ float wave_sum(float x) {
     for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o);
     return x;
 }
+// The same over aligned groups of `lw` lanes (16, 32 or 64): short rows put several pixels into one wave.
+__device__ __forceinline__ float group_max(float x, int lw) {
+    for (int o = lw >> 1; o > 0; o >>= 1) x = fmaxf(x, __shfl_xor(x, o));
+    return x;
+}
+__device__ __forceinline__ float group_sum(float x, int lw) {
+    for (int o = lw >> 1; o > 0; o >>= 1) x += __shfl_xor(x, o);
+    return x;
+}
+// lanes per pixel for rows of L entries
+__host__ __device__ inline int lanes_per_pixel(int L) { return L <= 16 ? 16 : L <= 32 ? 32 : 64; }
 
 struct AttArgs {
     const float *sep, *weight, *bias, *a, *grad_a;
@@ -54,17 +65,19 @@ __global__ void __launch_bounds__(64 * WPB) att_forward_kernel(const AttArgs a) 
     for (int t = threadIdx.x; t < K * 54; t += blockDim.x) ws[(t / 54) * 56 + t % 54] = a.weight[t];
     for (int t = threadIdx.x; t < K; t += blockDim.x) ws[MAXK * 56 + t] = a.bias ? a.bias[t] : 0.f;
     __syncthreads();
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const long pix = (long)blockIdx.x * WPB + wave;       // flattened (b,i,j)
+    // rows of up to 32 (16) entries: 2 (4) pixels per wave, a group of lw lanes each
+    const int lw = NCH == 1 ? lanes_per_pixel(L) : 64;
+    const int lane = threadIdx.x & (lw - 1), wave = threadIdx.x >> 6, sub = (threadIdx.x & 63) / lw;
+    const long pix = ((long)blockIdx.x * WPB + wave) * (64 / lw) + sub;       // flattened (b,i,j)
     const long npix = (long)a.B * H1 * W1;
-    if (pix >= npix) return;
+    if (pix >= npix) return;   // whole groups leave: the reductions below stay inside a group
     const int j = (int)(pix % W1), i = (int)((pix / W1) % H1);
 
     float x[NCH][2][3][9];   // [chunk][c][dl][neighbour di*3+dj]: the order of the weights
 #pragma unroll
     for (int n = 0; n < 9; ++n) {
         const int ii = i + n / 3 - 1, jj = j + n % 3 - 1;
-        const bool inb = ii >= 0 && ii < H1 && jj >= 0 && jj < W1;   // wave-uniform
+        const bool inb = ii >= 0 && ii < H1 && jj >= 0 && jj < W1;
         const float *row = a.sep + (pix + (long)(n / 3 - 1) * W1 + (n % 3 - 1)) * 2 * L;
 #pragma unroll
         for (int ch = 0; ch < NCH; ++ch)
@@ -99,14 +112,14 @@ __global__ void __launch_bounds__(64 * WPB) att_forward_kernel(const AttArgs a) 
 #pragma unroll
         for (int ch = 0; ch < NCH; ++ch)
             if (ch * 64 + lane < L) m = fmaxf(m, logit[ch]);
-        m = wave_max(m);
+        m = group_max(m, lw);
         float s = 0.f;
 #pragma unroll
         for (int ch = 0; ch < NCH; ++ch) {
             logit[ch] = (ch * 64 + lane < L) ? __expf(logit[ch] - m) : 0.f;
             s += logit[ch];
         }
-        s = wave_sum(s);
+        s = group_sum(s, lw);
         const float inv = 1.f / s;
         float *dst = a.out + (pix * K + k) * L;
 #pragma unroll
@@ -165,16 +178,17 @@ __global__ void __launch_bounds__(64 * WPB) att_forward_long_kernel(const AttArg
 // dlogits = a * (grad_a - sum_l a * grad_a), one wave per pixel.
 __global__ void __launch_bounds__(64 * WPB) att_softmax_backward_kernel(const AttArgs a) {
     const int K = a.K, L = a.L;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const long pix = (long)blockIdx.x * WPB + wave;
+    const int lw = lanes_per_pixel(L);
+    const int lane = threadIdx.x & (lw - 1), wave = threadIdx.x >> 6, sub = (threadIdx.x & 63) / lw;
+    const long pix = ((long)blockIdx.x * WPB + wave) * (64 / lw) + sub;
     if (pix >= (long)a.B * a.H1 * a.W1) return;
     for (int k = 0; k < K; ++k) {
         const float *pa = a.a + (pix * K + k) * L, *pg = a.grad_a + (pix * K + k) * L;
         float dot = 0.f;
-        for (int l = lane; l < L; l += 64) dot += pa[l] * pg[l];
-        dot = wave_sum(dot);
+        for (int l = lane; l < L; l += lw) dot += pa[l] * pg[l];
+        dot = group_sum(dot, lw);
         float *dst = a.dlogits + (pix * K + k) * L;
-        for (int l = lane; l < L; l += 64) dst[l] = pa[l] * (pg[l] - dot);
+        for (int l = lane; l < L; l += lw) dst[l] = pa[l] * (pg[l] - dot);
     }
 }
 
@@ -186,18 +200,19 @@ __global__ void __launch_bounds__(64 * WPB) att_input_backward_kernel(const AttA
     const int K = a.K, L = a.L, H1 = a.H1, W1 = a.W1;
     for (int t = threadIdx.x; t < K * 54; t += blockDim.x) ws[(t / 27) * 28 + t % 27] = a.weight[t];
     __syncthreads();
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const long pix = (long)blockIdx.x * WPB + wave;
+    const int lw = lanes_per_pixel(L);
+    const int lane = threadIdx.x & (lw - 1), wave = threadIdx.x >> 6, sub = (threadIdx.x & 63) / lw;
+    const long pix = ((long)blockIdx.x * WPB + wave) * (64 / lw) + sub;
     if (pix >= (long)a.B * H1 * W1) return;
     const int j = (int)(pix % W1), i = (int)((pix / W1) % H1);
-    for (int l = lane; l < L; l += 64) {
+    for (int l = lane; l < L; l += lw) {
         float d0 = 0.f, d1 = 0.f;
         for (int k = 0; k < K; ++k) {
             float x[27];   // [dl][di*3+dj]: the order of the weights
 #pragma unroll
             for (int n = 0; n < 9; ++n) {
                 const int ii = i - n / 3 + 1, jj = j - n % 3 + 1;
-                const bool inb = ii >= 0 && ii < H1 && jj >= 0 && jj < W1;   // wave-uniform
+                const bool inb = ii >= 0 && ii < H1 && jj >= 0 && jj < W1;
                 const float *g = a.dlogits + ((pix + (long)(1 - n / 3) * W1 + (1 - n % 3)) * K + k) * L;
 #pragma unroll
                 for (int dl = 0; dl < 3; ++dl) {
@@ -246,7 +261,8 @@ constexpr int DW_KC = 4;
 __global__ void __launch_bounds__(256) att_weight_backward_kernel(const AttArgs a) {
     __shared__ float red[4][27 * DW_KC + DW_KC];
     const int K = a.K, L = a.L, H1 = a.H1, W1 = a.W1;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lw = lanes_per_pixel(L), ppw = 64 / lw;   // short rows: ppw pixels per wave and iteration
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, sub = lane / lw, ll0 = lane & (lw - 1);
     const int c = blockIdx.y & 1, k0 = (blockIdx.y >> 1) * DW_KC;
     const long npix = (long)a.B * H1 * W1;
     const long p0 = (long)blockIdx.x * DW_PIX;
@@ -262,15 +278,18 @@ __global__ void __launch_bounds__(256) att_weight_backward_kernel(const AttArgs 
     const int nch = (L + 63) >> 6;
     const long left = npix - p0;
     const int npx = (int)(left < DW_PIX ? left : DW_PIX);
-    const int nit = ((npx - wave + 3) / 4) * nch;   // pixels wave, wave + 4, ... below npx
+    const int ngr = (npx + ppw - 1) / ppw;           // pixel groups of this workgroup
+    const int nit = ((ngr - wave + 3) / 4) * nch;    // groups wave, wave + 4, ... below ngr
     auto fetch = [&](int it, float(&x)[27], float(&gv)[DW_KC]) {
-        const long pix = p0 + wave + 4 * (it / nch);
-        const int l = (it % nch) * 64 + lane;
+        const int q = (wave + 4 * (it / nch)) * ppw + sub;
+        const bool pok = q < npx;
+        const long pix = p0 + (pok ? q : 0);
+        const int l = (it % nch) * 64 + ll0;
         const int j = (int)(pix % W1), i = (int)((pix / W1) % H1);
 #pragma unroll
         for (int n = 0; n < 9; ++n) {
             const int ii = i + n / 3 - 1, jj = j + n % 3 - 1;
-            const bool inb = ii >= 0 && ii < H1 && jj >= 0 && jj < W1;   // wave-uniform
+            const bool inb = pok && ii >= 0 && ii < H1 && jj >= 0 && jj < W1;
             const float *row = a.sep + ((pix + (long)(n / 3 - 1) * W1 + (n % 3 - 1)) * 2 + c) * L;
 #pragma unroll
             for (int dl = 0; dl < 3; ++dl) {
@@ -280,7 +299,7 @@ __global__ void __launch_bounds__(256) att_weight_backward_kernel(const AttArgs 
         }
         const float *g = a.dlogits + pix * K * L;
 #pragma unroll
-        for (int k = 0; k < DW_KC; ++k) gv[k] = (k0 + k < K && l < L) ? g[(k0 + k) * L + l] : 0.f;
+        for (int k = 0; k < DW_KC; ++k) gv[k] = (pok && k0 + k < K && l < L) ? g[(k0 + k) * L + l] : 0.f;
     };
     auto update = [&](const float(&x)[27], const float(&gv)[DW_KC]) {
 #pragma unroll
@@ -381,7 +400,8 @@ int sepcorr_attention_forward(const float *sep, const float *weight, const float
     args.sep = sep; args.weight = weight; args.bias = bias; args.out = a;
     args.B = B; args.H1 = H1; args.W1 = W1; args.L = L; args.K = K;
     const long npix = (long)B * H1 * W1;
-    const dim3 grid((unsigned)((npix + WPB - 1) / WPB)), block(64 * WPB);
+    const long ppg = (long)WPB * (64 / lanes_per_pixel(L));   // pixels per workgroup
+    const dim3 grid((unsigned)((npix + ppg - 1) / ppg)), block(64 * WPB);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (L <= 64) hipLaunchKernelGGL(att_forward_kernel<1>, grid, block, 0, s, args);
     else if (L <= 128) hipLaunchKernelGGL(att_forward_kernel<2>, grid, block, 0, s, args);
@@ -417,7 +437,8 @@ int sepcorr_attention_backward(const float *sep, const float *weight, const floa
     args.partial = reinterpret_cast<float *>(static_cast<char *>(workspace) + align256((size_t)npix * K * L * sizeof(float)));
     args.B = B; args.H1 = H1; args.W1 = W1; args.L = L; args.K = K;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const dim3 grid((unsigned)((npix + WPB - 1) / WPB)), block(64 * WPB);
+    const long ppg = (long)WPB * (64 / lanes_per_pixel(L));   // pixels per workgroup
+    const dim3 grid((unsigned)((npix + ppg - 1) / ppg)), block(64 * WPB);
     hipLaunchKernelGGL(att_softmax_backward_kernel, grid, block, 0, s, args);
     if (int rc = launched("attention softmax backward kernel")) return rc;
     args.out = d_sep;
