@@ -140,6 +140,10 @@ def main():
     ap.add_argument("--profile-steps", type=int, default=5)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three 256 MiB device copies (known traffic) for scaling rocprofv3 FETCH_SIZE/WRITE_SIZE")
+    ap.add_argument("--module-level", action="store_true",
+                    help="measure the caller's whole separate() too even with --no-cpu-baseline")
+    ap.add_argument("--only-module-level", action="store_true",
+                    help="measure nothing but the caller's whole separate() (for kernel traces of that path)")
     ap.add_argument("--single-stream", action="store_true",
                     help="keep all kernels of a call on the caller's stream (per-kernel durations under a profiler are "
                          "then those of kernels running alone)")
@@ -160,6 +164,9 @@ def main():
     B, H, W, Kp, ops = WORKLOADS[args.workload]
     C = 256
     N = H * W
+    if args.only_module_level:
+        print(json.dumps({"workload": args.workload, "module_level": module_level(B, H, W, C, Kp, torch, dev)}))
+        return
     f1c, f2c, gr, att = make_inputs(B, H, W, C, Kp, torch)
     f1, f2 = f1c.to(dev), f2c.to(dev)
     gr = {k: v.to(dev) for k, v in gr.items()}
@@ -180,9 +187,10 @@ def main():
     if Kp:
         # attention weights as the caller produces them: Conv3d on the (max,avg) volumes, softmax over the
         # kept axis, back to (B,H1,W1,K',L) (core/corr.py:437-446)
+        from separableflowthesis_amd import MemorySaver
         with torch.no_grad():
-            a_u = att[0].to(dev)(out_v.permute(0, 3, 4, 1, 2)).softmax(dim=2).permute(0, 3, 4, 1, 2).contiguous()
-            a_v = att[1].to(dev)(out_u.permute(0, 3, 4, 1, 2)).softmax(dim=2).permute(0, 3, 4, 1, 2).contiguous()
+            a_u = MemorySaver.attention_forward(out_v, att[0].weight.to(dev).contiguous(), att[0].bias.to(dev))
+            a_v = MemorySaver.attention_forward(out_u, att[1].weight.to(dev).contiguous(), att[1].bias.to(dev))
         cu, cv = E(B, H, W, Kp, H), E(B, H, W, Kp, W)
         da_u, da_v = torch.empty_like(a_u), torch.empty_like(a_v)
 
@@ -289,8 +297,9 @@ def main():
             "tflops_executed": round(5 * Wf / (fms * 1e-3) / 1e12, 2),
             "what": "same inputs and outputs as the headline step (d_f1, d_f2 are the sums of the two operators' "
                     "gradients), via sepcorr_compression_backward(d_f1=d_f2=NULL) + sepcorr_fused_backward"}
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline or args.module_level:
         out["module_level"] = module_level(B, H, W, C, Kp, torch, dev)
+    if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(B, H, W, C, Kp, ops, torch)
     print(json.dumps(out))
 
