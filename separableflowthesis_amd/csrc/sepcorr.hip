@@ -443,9 +443,6 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                 const unsigned off = lane_off + (unsigned)((step * NUG + ug) * UR + r) * rowbytes + (unsigned)J * 128u;
 #pragma unroll
                 for (int tq = 0; tq < 4; ++tq) {
-#if defined(SEPCORR_EXP) && SEPCORR_EXP == 2
-                    if (step == 0 && J == 0)   // experiment: load only once
-#endif
                     buf[r][tq] = buf_load4(rsrc, off + 16u * tq);
                 }
             }
@@ -506,11 +503,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                 for (int tq = 0; tq < 4; ++tq) mfma_tq(tq, bv[tq]);
             }
             __builtin_amdgcn_sched_barrier(0);
-#if defined(SEPCORR_EXP) && SEPCORR_EXP == 1
-            if (J == NJB - 1 && step == nsteps - 1) {   // experiment: epilogue only once
-#else
             if (J == NJB - 1) {
-#endif
                 if constexpr (DUAL) {
                     acc[0] += acc_alt;
                     if constexpr (CMODE != 3) {
@@ -712,17 +705,17 @@ template <int GMODE, int KC>
 struct VW {
     float a[KC];   // comp: a_u[k]
     float g[KC];   // comp: g_cv[k]
-    float ma;      // maxavg: g_v[max]
-    float mg;      // maxavg: g_v[avg] / H2
+    float ma;      // maxavg: g_v[avg] / H2 + g_v[max]  (the value where the row index equals argmax_v)
+    float mg;      // maxavg: g_v[avg] / H2             (the value elsewhere)
     int am;        // maxavg: argmax_v
 };
 template <int GMODE, int KC>
 struct UW {
     float a[KC];   // comp: a_v[k]
     float g[KC];   // comp: g_cu[k]
-    float ma;      // maxavg: g_u[max]
-    float mg;      // maxavg: g_u[avg] / W2
-    int am;        // maxavg: argmax_u
+    float ma;      // maxavg: g_u[avg] / W2 + g_u[max]  (the value where the column index equals argmax_u)
+    float mg;      // maxavg: g_u[avg] / W2             (the value elsewhere)
+    int am;        // maxavg: argmax_u (callers may store it relative to a lane's first column)
 };
 
 template <int GMODE, int KC>
@@ -737,8 +730,8 @@ __device__ __forceinline__ VW<GMODE, KC> load_vw(const BwdArgs &a, size_t bp, in
         }
     }
     if constexpr (g_has_maxavg(GMODE)) {
-        w.ma = ok ? a.g_v[(bp * 2 + 0) * a.W2 + v] : 0.f;
         w.mg = ok ? a.g_v[(bp * 2 + 1) * a.W2 + v] * (1.f / (float)a.H2) : 0.f;
+        w.ma = ok ? w.mg + a.g_v[(bp * 2 + 0) * a.W2 + v] : 0.f;
         w.am = ok ? a.am_v[bp * a.W2 + v] : -1;
     }
     return w;
@@ -755,8 +748,8 @@ __device__ __forceinline__ UW<GMODE, KC> load_uw(const BwdArgs &a, size_t bp, in
         }
     }
     if constexpr (g_has_maxavg(GMODE)) {
-        w.ma = ok ? a.g_u[(bp * 2 + 0) * a.H2 + u] : 0.f;
         w.mg = ok ? a.g_u[(bp * 2 + 1) * a.H2 + u] * (1.f / (float)a.W2) : 0.f;
+        w.ma = ok ? w.mg + a.g_u[(bp * 2 + 0) * a.H2 + u] : 0.f;
         w.am = ok ? a.am_u[bp * a.H2 + u] : -1;
     }
     return w;
@@ -765,17 +758,14 @@ __device__ __forceinline__ UW<GMODE, KC> load_uw(const BwdArgs &a, size_t bp, in
 template <int GMODE, int KC>
 __device__ __forceinline__ float gval(const VW<GMODE, KC> &wv, const UW<GMODE, KC> &wu, int u, int v, bool ok) {
     float g = 0.f;
+    // max/avg terms: two selects and one add (the sums with and without the max gradient are kept ready)
+    if constexpr (g_has_maxavg(GMODE)) g = (wu.am == v ? wu.ma : wu.mg) + (wv.am == u ? wv.ma : wv.mg);
     if constexpr (g_has_comp(GMODE)) {
 #pragma unroll
         for (int k = 0; k < KC; ++k) {   // two fused multiply-adds per channel (a sum of two products would take three)
             g = fmaf(wv.a[k], wu.g[k], g);
             g = fmaf(wu.a[k], wv.g[k], g);
         }
-    }
-    if constexpr (g_has_maxavg(GMODE)) {
-        g += wu.mg + wv.mg;
-        if (wu.am == v) g += wu.ma;
-        if (wv.am == u) g += wv.ma;
     }
     return ok ? g : 0.f;
 }
@@ -887,9 +877,14 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
         }
     }
     const float inv_w2 = 1.f / (float)W2;
+    // argmax_u is kept relative to this lane's first column: register r then compares against the constant
+    // 8 (r / 4) + r % 4 instead of a column index that would have to be formed for every element
+    const int lanebase = vbase + 32 * vcw + 4 * h;
     auto load_uw_row = [&](int u) {
         if constexpr (!FAST) {
-            return load_uw<GMODE, KC>(a, bp, u, true);   // bp is clamped: always a valid pixel
+            UW<GMODE, KC> w = load_uw<GMODE, KC>(a, bp, u, true);   // bp is clamped: always a valid pixel
+            if constexpr (g_has_maxavg(GMODE)) w.am -= lanebase;
+            return w;
         } else {
             UW<GMODE, KC> w;
             if constexpr (g_has_comp(GMODE)) {
@@ -900,9 +895,9 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
                 }
             }
             if constexpr (g_has_maxavg(GMODE)) {
-                w.ma = buf_load1s(rs_gu, uwoff_2, (unsigned)u * 4u);
                 w.mg = buf_load1s(rs_gu, uwoff_2, (unsigned)(H2 + u) * 4u) * inv_w2;
-                w.am = __float_as_int(buf_load1s(rs_amu, uwoff_1, (unsigned)u * 4u));
+                w.ma = w.mg + buf_load1s(rs_gu, uwoff_2, (unsigned)u * 4u);
+                w.am = __float_as_int(buf_load1s(rs_amu, uwoff_1, (unsigned)u * 4u)) - lanebase;
             }
             return w;
         }
@@ -910,10 +905,9 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
     UW<GMODE, KC> wu_n = load_uw_row(min(ug, H2 - 1));
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-        const int v = vbase + 32 * vcw + vmap(r, h);
         // no mask: a column outside the image has an all-zero A operand and the column of a pixel outside the
         // image is never stored; the weights behind both are those of real entries, so G stays finite
-        G[r] = gval<GMODE, KC>(wv[r], wu_n, ug, v, true);
+        G[r] = gval<GMODE, KC>(wv[r], wu_n, ug, vmap(r, 0), true);
     }
     UW<GMODE, KC> wu_next = load_uw_row(min(ug + NUG, H2 - 1));
     auto compute = [&](int u, int g, v4f(&buf)[GS][NCB]) {
@@ -930,8 +924,11 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
 #pragma unroll
         for (int ss = 0; ss < GS; ++ss) {
             const int r = g * GS + ss;
-            const int v = vbase + 32 * vcw + vmap(r, h);
-            Gn[r] = gval<GMODE, KC>(wv[r], wu_n, u + NUG, v, true);
+            // the row index as an opaque scalar: otherwise the comparison with argmax_v is rewritten into
+            // (argmax_v - row) == 0 with one more vector add per element
+            int un = u + NUG;
+            asm volatile("" : "+s"(un));
+            Gn[r] = gval<GMODE, KC>(wv[r], wu_n, un, vmap(r, 0), true);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -1258,7 +1255,6 @@ __global__ void __launch_bounds__(64 * NWV) df2_tiled_kernel(const BwdArgs a, in
             const float *fs = F1s + bi * 32 * CB;
             const float *vs = VWs + bi * NV * 1024;
             const float *us = UWs + (wave * UBUF + (UBUF == 2 ? bi : 0)) * 32 * NUP;
-            const int pt0 = pbeg + tile * TP;
             // Software pipeline over the 16 MFMA steps of the tile: the LDS operands of step s+1 are
             // fetched before the MFMAs of step s and its G is computed between them, so the matrix
             // pipe does not wait for LDS latency or for the G arithmetic.
