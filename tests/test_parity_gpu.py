@@ -27,6 +27,8 @@ SHAPES = [
     (1, 4, 40, 3, 300, 32),     # rows wider than 256 columns: two column passes
     (1, 5, 24, 2, 520, 20),     # three column passes, last one ragged
     (1, 3, 11, 2, 301, 7),      # wide rows on the generic load paths
+    (1, 2, 3, 1, 2048, 8),      # the widest supported row: 8 column passes
+    (1, 2, 5, 2, 8, 1024),      # the most channels supported: 4 channel blocks in the backward kernels
 ]
 
 
