@@ -230,3 +230,56 @@ def test_error_conventions_on_device(device):
         ms.max_avg_forward(torch.randn(1, 1, 2, 4, device=device), torch.randn(1, 1, 2100, 4, device=device))
     with pytest.raises(RuntimeError, match="shape"):
         ms.compression_forward(f, f, torch.randn(1, 4, 4, 2, 4, device=device), torch.randn(1, 4, 4, 2, 5, device=device))
+
+
+def _all_ops(ms, t):
+    ou, ov, au, av = ms.max_argmax_avg_forward(t["f1"], t["f2"])
+    cu, cv = ms.compression_forward(t["f1"], t["f2"], t["a_u"], t["a_v"])
+    c1, c2, da_u, da_v = ms.compression_backward(t["f1"], t["f2"], t["a_u"], t["a_v"], t["g_cu"], t["g_cv"])
+    m1, m2 = ms.max_argmax_avg_backward(t["f1"], t["f2"], au, av, t["g_u"], t["g_v"])
+    f1, f2 = ms.fused_backward(t["f1"], t["f2"], au, av, t["g_u"], t["g_v"], t["a_u"], t["a_v"], t["g_cu"], t["g_cv"])
+    return [ou, ov, au, av, cu, cv, c1, c2, da_u, da_v, m1, m2, f1, f2]
+
+
+def _op_tensors(device, seed, B=2, H1=9, W1=20, H2=9, W2=20, C=64, K=4):
+    f1, f2, g = op_inputs(B, H1, W1, H2, W2, C, seed=seed)
+    t = dict(f1=f1, f2=f2, a_u=softmax_weights(B, H1, W1, K, W2, g), a_v=softmax_weights(B, H1, W1, K, H2, g),
+             g_u=torch.randn(B, H1, W1, 2, H2, generator=g), g_v=torch.randn(B, H1, W1, 2, W2, generator=g),
+             g_cu=torch.randn(B, H1, W1, K, H2, generator=g), g_cv=torch.randn(B, H1, W1, K, W2, generator=g))
+    return {k: v.to(device) for k, v in t.items()}
+
+
+def test_ops_follow_the_callers_stream(device):
+    # work queued on a side stream right after the inputs were produced there; the library's own side streams
+    # fork from and join back into that stream
+    ms = _native()
+    ref = _all_ops(ms, _op_tensors(device, seed=71))
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        t = _op_tensors(device, seed=71)
+        t = {k: v * 1.0 for k, v in t.items()}   # produced on s: the ops must wait for it
+        got = _all_ops(ms, t)
+    s.synchronize()
+    assert all(torch.equal(x, y) for x, y in zip(got, ref))
+
+
+def test_ops_replay_correctly_from_a_captured_graph(device):
+    # all five reference functions and the fused backward in one captured graph (outputs and scratch come from
+    # the graph's pool); every replay is checked against the eager result for the inputs of that replay
+    ms = _native()
+    static = _op_tensors(device, seed=81)
+    _all_ops(ms, static)                      # warm-up outside the capture (lazy initialisations)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = _all_ops(ms, static)
+    for seed in (82, 83, 84):
+        fresh = _op_tensors(device, seed=seed)
+        ref = _all_ops(ms, fresh)             # eager work between the replays
+        torch.cuda.synchronize()
+        for k in static:
+            static[k].copy_(fresh[k])
+        graph.replay()
+        torch.cuda.synchronize()
+        assert all(torch.equal(x, y) for x, y in zip(outs, ref)), f"replay with seed {seed} differs from eager"
