@@ -1585,7 +1585,8 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s
     } while (0)
         if (nW > 4) { if (cvec) SEPCORR_DF1(1, true, 512); else SEPCORR_DF1(1, false, 512); }
         else if (ncb == 1) { if (cvec) SEPCORR_DF1(1, true, 256); else SEPCORR_DF1(1, false, 256); }
-        else if (cvec && d.C == 256 && d.W2 % 4 == 0) {
+        // (the fast variant addresses the (p,u)-indexed tensors of one batch image with 32-bit byte offsets)
+        else if (cvec && d.C == 256 && d.W2 % 4 == 0 && (size_t)d.H1 * d.W1 * MAX_K * d.H2 * 4 <= big) {
             ProfScope ps(GMODE == GMODE_COMP ? "df1_comp" : GMODE == GMODE_BOTH ? "df1_both" : "df1_maxavg", s1);
             hipLaunchKernelGGL((df1_kernel<GMODE, KC, 2, true, 256, true>), grid, block, lds, s1, a);
         }
