@@ -54,6 +54,41 @@ def test_corr_block_matches_full_4d_corr_block(device, B, C, H, W, K, backward):
             assert_close(m.bias.grad, rm.bias.grad, n + ".bias.grad", scale_atol=True)
 
 
+@pytest.mark.parametrize("kind,backward", [("reference", False), ("pointwise", True), ("pointwise", False)])
+def test_corr_block_other_paths(device, kind, backward):
+    """The paths the test above does not take: the reference's attention without a backward pass (separate
+    Functions per operator), and an attention module that is not the reference's Conv3d(2, K, 3, padding=1), for
+    which the caller's torch glue (permute / module / softmax / cat / interpolate) runs around the operators."""
+    from separableflowthesis_amd import AlternateCorrBlockSepflow
+    B, C, H, W, K = 1, 64, 12, 20, 3
+    fmap1, fmap2, _, _ = O.make_inputs(B, H, W, C, seed=91)
+    torch.manual_seed(9)
+    if kind == "reference":
+        att = (torch.nn.Conv3d(2, K, 3, padding=1), torch.nn.Conv3d(2, K, 3, padding=1))
+    else:
+        att = (torch.nn.Conv3d(2, K, 1), torch.nn.Conv3d(2, K, 1))
+    r1 = fmap1.double().requires_grad_(backward)
+    r2 = fmap2.double().requires_grad_(backward)
+    ratt = tuple(copy.deepcopy(m).double() for m in att)
+    rc1, rc2 = O.CorrBlock4D(r1, r2, num_levels=4).separate(ratt)
+    g1 = fmap1.to(device).requires_grad_(backward)
+    g2 = fmap2.to(device).requires_grad_(backward)
+    gatt = tuple(copy.deepcopy(m).to(device) for m in att)
+    c1, c2 = AlternateCorrBlockSepflow(g1, g2, None, num_levels=4, support_backward=backward)(None, sep=True, attention_weights=gatt)
+    assert_close(c1, rc1, "corr1")
+    assert_close(c2, rc2, "corr2")
+    if backward:
+        gen = torch.Generator().manual_seed(4)
+        w1 = torch.randn(rc1.shape, generator=gen) / 64
+        w2 = torch.randn(rc2.shape, generator=gen) / 64
+        ((rc1 * w1.double()).sum() + (rc2 * w2.double()).sum()).backward()
+        ((c1 * w1.to(device)).sum() + (c2 * w2.to(device)).sum()).backward()
+        assert_close(g1.grad, r1.grad, "grad fmap1", scale_atol=True)
+        assert_close(g2.grad, r2.grad, "grad fmap2", scale_atol=True)
+        for m, rm, n in zip(gatt, ratt, ("attention1", "attention2")):
+            assert_close(m.weight.grad, rm.weight.grad, n + ".weight.grad", scale_atol=True)
+
+
 @pytest.mark.parametrize("B,H1,W1,L,K", [(1, 3, 4, 5, 1), (2, 9, 13, 70, 4), (1, 6, 10, 128, 4), (1, 4, 5, 200, 3),
                                           (1, 3, 6, 300, 2), (1, 2, 3, 1, 8)])
 def test_attention_producer_matches_conv3d_softmax(device, B, H1, W1, L, K):
