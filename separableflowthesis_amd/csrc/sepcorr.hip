@@ -133,6 +133,57 @@ __device__ __forceinline__ v16f mfma(float a, float b, v16f c) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
 }
 
+// Experimental contraction in three bf16 planes.  x = h + m + l with h = bf16(x), m = bf16(x - h), l = bf16(x - h - m)
+// is exact for fp32 x (8 + 8 + 8 significant bits); the product of two such numbers is taken as
+// hh + hm + mh + hl + lh + mm (what is dropped is below 2^-25 of the product) with six bf16 MFMAs that accumulate
+// in fp32.  A bf16 MFMA has 16x the rate of the fp32 one here and, unlike it, leaves the vector lanes free.
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ void split8(const float (&x)[8], v8bf &h, v8bf &m, v8bf &l) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const __bf16 hh = (__bf16)x[e];
+        const float r1 = x[e] - (float)hh;
+        const __bf16 mm = (__bf16)r1;
+        const float r2 = r1 - (float)mm;
+        h[e] = hh; m[e] = mm; l[e] = (__bf16)r2;
+    }
+}
+__device__ __forceinline__ v16f mfma_bf(v8bf a, v8bf b, v16f c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+constexpr int BF_LSB = 264;   // bf16 per pixel row of an f1 plane in LDS (256 + 8: 16-byte reads hit distinct banks)
+constexpr int BF_LS = 3 * BF_LSB / 2;   // the same in floats per pixel, all three planes
+// fmap2 as bf16 planes in device memory (C == 256), ordered the way the sweep reads them: one 48 KB block per
+// (image, row u, chunk of 32 columns), and inside it one KB per (32-channel block J, plane, k-step s2) holding the
+// 16 bytes of each of the 64 lanes in lane order (lane = 32 h + column, channels 32J + 16h + 8 s2 + 0..7).  Every
+// operand load of a wave is then one contiguous KB.  Rows are padded to whole chunks and to an even row count,
+// the padding reads as zero.
+constexpr unsigned BF_CHUNK = 8 * 6 * 1024;
+__global__ void __launch_bounds__(256) split_planes_kernel(const float *__restrict__ f2, char *__restrict__ planes, int H2,
+                                                           int W2, int H2p, int nvc, long nunits) {
+    const long t = (long)blockIdx.x * 256 + threadIdx.x;   // one thread per lane and (J, s2) of a chunk
+    if (t >= nunits) return;
+    const int lane = (int)(t & 63), pl = lane & 31, h = lane >> 5;
+    long r = t >> 6;
+    const int s2 = (int)(r & 1), J = (int)((r >> 1) & 7);
+    r >>= 4;                                                // chunk index = (b * H2p + u) * nvc + vc
+    const int vc = (int)(r % nvc);
+    const long bu = r / nvc;
+    const int u = (int)(bu % H2p), v = 32 * vc + pl;
+    const long b = bu / H2p;
+    float xs[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (u < H2 && v < W2) {
+        const float *src = f2 + ((b * H2 + u) * W2 + v) * 256 + 32 * J + 16 * h + 8 * s2;
+        const v4f x0 = *reinterpret_cast<const v4f *>(src), x1 = *reinterpret_cast<const v4f *>(src + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { xs[e] = x0[e]; xs[4 + e] = x1[e]; }
+    }
+    v8bf ph, pm, pl3;
+    split8(xs, ph, pm, pl3);
+    char *dst = planes + r * BF_CHUNK + (J * 6 + s2) * 1024 + lane * 16;   // KB index in a chunk: 6 J + 2 plane + s2
+    *reinterpret_cast<v8bf *>(dst) = ph;
+    *reinterpret_cast<v8bf *>(dst + 2048) = pm;
+    *reinterpret_cast<v8bf *>(dst + 4096) = pl3;
+}
+
 // ------------------------------------------------------------------------------------------
 // forward
 // ------------------------------------------------------------------------------------------
@@ -148,6 +199,7 @@ __device__ __forceinline__ int xcd_contiguous(int bid, int n) {
 
 struct FwdArgs {
     const float *f1, *f2;
+    const char *f2_planes;   // bf16-plane variant: fmap2 split by split_planes_kernel
     const float *wv;   // MODE_WEIGHTED: weights indexed by v, (B,N1,KT,W2)
     const float *wu;   // MODE_WEIGHTED: weights indexed by u, (B,N1,KT,H2)
     float *out_u;      // (B,N1,CH,H2)
@@ -166,8 +218,10 @@ struct FwdArgs {
 //        3 = C == 256 (fast path with the channel loop unrolled: every load offset is an immediate)
 // WM: 0 = one pass, one row group (both compile-time constants: the lean common case),
 //     1 = row groups enabled (narrow rows), 2 = column passes enabled (rows wider than 256).
-template <int MODE, int KC, int UR, int CMODE, int WM>
+// BF: the experimental bf16-plane contraction (C == 256, one pass, one row group, max/avg modes)
+template <int MODE, int KC, int UR, int CMODE, int WM, bool BF = false>
 __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
+    static_assert(!BF || (CMODE == 3 && WM == 0 && UR == 2), "bf16 planes: C == 256, one pass, one row group, two rows per step");
     constexpr bool CVEC = CMODE >= 1;
     constexpr int GJ = 2;  // 8-channel slices per prefetch group
     constexpr int NPART = (MODE == MODE_WEIGHTED) ? KC : 3;
@@ -185,8 +239,9 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     const int b = wg / a.tiles_per_batch;
     const int p0 = (wg % a.tiles_per_batch) * TP;
     const int N1 = a.N1, H2 = a.H2, W2 = a.W2, C = a.C;
-    const int LS = a.CP + 4;
+    const int LS = BF ? BF_LS : a.CP + 4;
     float *f1s = smem;
+    __bf16 *f1b = reinterpret_cast<__bf16 *>(smem);   // BF: [plane][TP][BF_LSB]
     float *part = smem + TP * LS;
     constexpr int NCHO = (MODE == MODE_WEIGHTED) ? KC : 2;            // out_u channels of this launch
     float *ostage = part + 2 * UR * NPART * (blockDim.x >> 6) * 32;   // [32 p][NCHO][H2] when a.stage
@@ -198,7 +253,20 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
             const int row = idx / c4n, c = (idx - row * c4n) * 4;
             const bool ok = p0 + row < N1;
             const float *src = a.f1 + ((size_t)b * N1 + (ok ? p0 + row : 0)) * C;
-            *reinterpret_cast<v4f *>(f1s + row * LS + c) = load4<CVEC>(src, c, C, ok);
+            const v4f x = load4<CVEC>(src, c, C, ok);
+            if constexpr (BF) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const __bf16 hh = (__bf16)x[e];
+                    const float r1 = x[e] - (float)hh;
+                    const __bf16 mm = (__bf16)r1;
+                    f1b[(0 * TP + row) * BF_LSB + c + e] = hh;
+                    f1b[(1 * TP + row) * BF_LSB + c + e] = mm;
+                    f1b[(2 * TP + row) * BF_LSB + c + e] = (__bf16)(r1 - (float)mm);
+                }
+            } else {
+                *reinterpret_cast<v4f *>(f1s + row * LS + c) = x;
+            }
         }
     }
     __syncthreads();
@@ -418,7 +486,65 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         if (g == NG - 1) epilogue(step);
     };
 
-    if constexpr (CMODE >= 2) {
+    if constexpr (BF) {
+        // bf16 planes: per 32-channel block and row, six 16-byte loads (plane x k-step) feed twelve MFMAs of two rows
+        const int nvcp = (W2 + 31) >> 5, H2p = (H2 + 1) & ~1;
+        const unsigned rowbytes = (unsigned)nvcp * BF_CHUNK;
+        const unsigned nbytes = (unsigned)H2p * rowbytes;
+        const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(a.f2_planes + (size_t)b * nbytes, nbytes);
+        const unsigned lane_off = (unsigned)vcw * BF_CHUNK + 16u * lane;
+        const v16f zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        v4f ring[2][UR][6];
+        auto issueB = [&](int step, int J, v4f(&buf)[UR][6]) {
+#pragma unroll
+            for (int r = 0; r < UR; ++r) {
+                const unsigned row = (unsigned)(step * UR + r) * rowbytes;   // wave-uniform: travels in a scalar register
+#pragma unroll
+                for (int i = 0; i < 6; ++i) buf[r][i] = buf_load4s(rsrc, lane_off, row + (unsigned)(J * 6 + i) * 1024u);   // i = 2 plane + k-step
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        auto computeB = [&](int step, int J, v4f(&buf)[UR][6]) {
+            if constexpr (MODE == MODE_WEIGHTED) {
+                if (J == 0) {
+#pragma unroll
+                    for (int r = 0; r < UR; ++r) {
+                        const int u = min(step * UR + r, H2 - 1);
+#pragma unroll
+                        for (int k = 0; k < KC; ++k) wur[r][k] = a.wu[(bp * a.KT + a.k0 + k) * H2 + u];
+                    }
+                }
+            }
+            const __bf16 *bb = f1b + pl * BF_LSB + 32 * J + 16 * h;
+            v8bf bq[3][2];
+#pragma unroll
+            for (int q = 0; q < 3; ++q)
+#pragma unroll
+                for (int s2 = 0; s2 < 2; ++s2) bq[q][s2] = *reinterpret_cast<const v8bf *>(bb + q * TP * BF_LSB + 8 * s2);
+            // plane pairs (f2, f1) in the order of growing magnitude: l.h, h.l, m.m, m.h, h.m, h.h
+            constexpr int PA[6] = {2, 0, 1, 1, 0, 0}, PB[6] = {0, 2, 1, 0, 1, 0};
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+                for (int t = 0; t < 6; ++t)
+#pragma unroll
+                    for (int r = 0; r < UR; ++r) {
+                        const bool first = J == 0 && s2 == 0 && t == 0;
+                        acc[r] = mfma_bf(__builtin_bit_cast(v8bf, buf[r][2 * PA[t] + s2]), bq[PB[t]][s2], first ? zero16 : acc[r]);
+                    }
+            __builtin_amdgcn_sched_barrier(0);
+            if (J == 7) epilogue(step);
+        };
+        issueB(0, 0, ring[0]);
+        for (int step = 0; step < nsteps; ++step) {
+#pragma unroll
+            for (int J = 0; J < 8; ++J) {
+                if (J + 1 < 8) issueB(step, J + 1, ring[(J + 1) & 1]);
+                else if (step + 1 < nsteps) issueB(step + 1, 0, ring[0]);
+                computeB(step, J, ring[J & 1]);
+            }
+        }
+    } else if constexpr (CMODE >= 2) {
         // Fast path.  Contraction index permuted so that a lane reads 64 contiguous bytes of its fmap2
         // pixel per 32-channel block J: MFMA step (tq,t) of block J contracts channels 32J+4tq+t (lanes
         // 0..31) and 32J+16+4tq+t (lanes 32..63); the f1 tile in LDS is read with the same mapping.
@@ -1463,6 +1589,21 @@ int launch_fwd(FwdArgs a, int B, hipStream_t s) {
         if (cmode == 3) SEPCORR_FWD(3, 1); else if (cmode == 2) SEPCORR_FWD(2, 1);
         else if (cmode == 1) SEPCORR_FWD(1, 1); else SEPCORR_FWD(0, 1);
     } else {
+        if constexpr (UR == 2) {
+            if (cmode == 3 && a.f2_planes) {   // bf16-plane variant: the caller has split fmap2
+                // LDS with the larger f1 tile (three bf16 planes); out_u staging only if two workgroups still fit a CU
+                constexpr int NCHO = (MODE == MODE_WEIGHTED) ? KC : 2;
+                lds = ((size_t)TP * BF_LS + 2 * UR * NPART * nW * 32) * sizeof(float);
+                const size_t extra = (size_t)TP * (NCHO + (MODE == MODE_ARGMAX ? 1 : 0)) * a.H2 * sizeof(float);
+                a.stage = lds + extra <= 80 * 1024;
+                if (a.stage) lds += extra;
+                auto k = fwd_kernel<MODE, KC, UR, 3, 0, true>;
+                if (int rc = set_lds(k, lds)) return rc;
+                ProfScope ps(MODE == MODE_WEIGHTED ? "fwd_weighted_bf16x3" : "fwd_maxavg_bf16x3", s);
+                hipLaunchKernelGGL(k, grid, block, lds, s, a);
+                return check_launch("forward kernel (bf16 planes)");
+            }
+        }
         if (cmode == 3) SEPCORR_FWD(3, 0); else if (cmode == 2) SEPCORR_FWD(2, 0);
         else if (cmode == 1) SEPCORR_FWD(1, 0); else SEPCORR_FWD(0, 0);
     }
@@ -1486,6 +1627,31 @@ int xcd_order_enabled() {
     return on;
 }
 
+// SEPCORR_BF16X3=1 selects the experimental forward sweeps that contract in three bf16 planes (C == 256, rows of
+// 97..256 columns or enough workgroups that a wave owns one column chunk).  fmap2 is split once per call into
+// stream-ordered memory that is released, in stream order, when the call returns.
+struct Bf16Planes {
+    void *ptr = nullptr;
+    hipStream_t s = nullptr;
+    ~Bf16Planes() { if (ptr) (void)hipFreeAsync(ptr, s); }
+    int make(const Dims &d, const float *f2, hipStream_t stream) {
+        static const bool on = [] { const char *e = getenv("SEPCORR_BF16X3"); return e && e[0] == '1'; }();
+        const WaveGrid wg = wave_grid(d.B, (d.H1 * d.W1 + TP - 1) / TP, d.W2, d.H2);
+        const int nvcp = (d.W2 + 31) / 32, H2p = (d.H2 + 1) & ~1;
+        const size_t batch_bytes = (size_t)H2p * nvcp * BF_CHUNK;
+        if (!on || d.C != 256 || wg.vpasses > 1 || wg.nug > 1 || batch_bytes > (1u << 30)) return SEPCORR_OK;
+        const size_t nchunks = (size_t)d.B * H2p * nvcp;
+        s = stream;
+        const hipError_t e = hipMallocAsync(&ptr, nchunks * BF_CHUNK, s);
+        if (e != hipSuccess) { ptr = nullptr; return fail(SEPCORR_ELAUNCH, "sepcorr: bf16 planes: %s", hipGetErrorString(e)); }
+        ProfScope ps("split_planes", s);
+        const long nunits = (long)nchunks * 16 * 64;
+        hipLaunchKernelGGL(split_planes_kernel, dim3((unsigned)((nunits + 255) / 256)), dim3(256), 0, s, f2,
+                           static_cast<char *>(ptr), d.H2, d.W2, H2p, nvcp, nunits);
+        return check_launch("split_planes");
+    }
+};
+
 FwdArgs fwd_args(const Dims &d) {
     FwdArgs a;
     memset(&a, 0, sizeof(a));
@@ -1505,6 +1671,9 @@ int weighted_forward(const Dims &d, const float *f1, const float *f2, const floa
     FwdArgs a = fwd_args(d);
     a.f1 = f1; a.f2 = f2; a.wv = wv; a.wu = wu; a.out_u = out_u; a.out_v = out_v;
     a.KT = K;
+    Bf16Planes planes;
+    if (int rc = planes.make(d, f2, s)) return rc;
+    a.f2_planes = static_cast<const char *>(planes.ptr);
     for (int k0 = 0; k0 < K; k0 += KCH) {
         a.k0 = k0;
         const int kc = K - k0 < KCH ? K - k0 : KCH;
@@ -1768,6 +1937,9 @@ int sepcorr_max_avg_forward(const float *f1, const float *f2, float *out_u, floa
     if (int rc = check_dims(d, 2)) return rc;
     FwdArgs a = fwd_args(d);
     a.f1 = f1; a.f2 = f2; a.out_u = out_u; a.out_v = out_v;
+    Bf16Planes planes;
+    if (int rc = planes.make(d, f2, static_cast<hipStream_t>(stream))) return rc;
+    a.f2_planes = static_cast<const char *>(planes.ptr);
     return launch_fwd<MODE_MAXAVG, 1, 2>(a, B, static_cast<hipStream_t>(stream));
 }
 
@@ -1778,6 +1950,9 @@ int sepcorr_max_argmax_avg_forward(const float *f1, const float *f2, float *out_
     if (int rc = check_dims(d, 2)) return rc;
     FwdArgs a = fwd_args(d);
     a.f1 = f1; a.f2 = f2; a.out_u = out_u; a.out_v = out_v; a.am_u = argmax_u; a.am_v = argmax_v;
+    Bf16Planes planes;
+    if (int rc = planes.make(d, f2, static_cast<hipStream_t>(stream))) return rc;
+    a.f2_planes = static_cast<const char *>(planes.ptr);
     return launch_fwd<MODE_ARGMAX, 1, 2>(a, B, static_cast<hipStream_t>(stream));
 }
 
