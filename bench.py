@@ -297,6 +297,38 @@ def main():
             "tflops_executed": round(5 * Wf / (fms * 1e-3) / 1e12, 2),
             "what": "same inputs and outputs as the headline step (d_f1, d_f2 are the sums of the two operators' "
                     "gradients), via sepcorr_compression_backward(d_f1=d_f2=NULL) + sepcorr_fused_backward"}
+    # The same headline step with the forward sweeps contracting in three bf16 planes per operand (an option of
+    # this library with the same accuracy bar, see sepcorr_set_contraction).  Reported beside the headline, never
+    # as `value`: the headline arithmetic is fp32 MFMA throughout.
+    prev_mode = lib.sepcorr_set_contraction(1)
+    try:
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        pms = (time.perf_counter() - t0) / args.steps * 1e3
+        lib.sepcorr_profile_enable(1)
+        step()
+        torch.cuda.synchronize()
+        names = ctypes.create_string_buffer(1 << 16)
+        tms = (ctypes.c_float * 4096)()
+        n = lib.sepcorr_profile_collect(names, len(names), tms, 4096)
+        lib.sepcorr_profile_enable(0)
+        pk = {}
+        for nm, t in zip(names.value.decode().split("\n")[:n], list(tms)[:n]):
+            if nm.endswith("bf16x3") or nm == "split_planes":
+                pk.setdefault(nm, []).append(t)
+        out["bf16_planes"] = {
+            "ms_per_step": round(pms, 4), "tflops_fp32_equivalent": round(passes * Wf / (pms * 1e-3) / 1e12, 2),
+            "kernels_ms": {k: round(sum(v) / len(v), 4) for k, v in pk.items()},
+            "what": "headline step with sepcorr_set_contraction(SEPCORR_CONTRACT_BF16X3): forward-type sweeps "
+                    "(max/argmax/avg, compression forward, attention gradients) in bf16 planes, feature gradients "
+                    "in fp32 MFMA"}
+    finally:
+        lib.sepcorr_set_contraction(prev_mode)
     if not args.no_cpu_baseline or args.module_level:
         out["module_level"] = module_level(B, H, W, C, Kp, torch, dev)
     if not args.no_cpu_baseline:

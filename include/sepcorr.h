@@ -56,6 +56,25 @@ int sepcorr_profile_enable(int on);
 int sepcorr_profile_collect(char *names, size_t names_cap, float *ms, int cap);
 
 /*
+ * Arithmetic of the contraction over channels in the forward sweeps (max/avg, max/argmax/avg, compression
+ * forward and the attention-gradient pass of the compression backward); no counterpart in the reference.
+ *   SEPCORR_CONTRACT_FP32    fp32 MFMA (the initial choice).
+ *   SEPCORR_CONTRACT_BF16X3  every fp32 operand is written exactly as the sum of three bf16 numbers and the
+ *                            product taken as the six largest of the nine plane products, with bf16 MFMA
+ *                            accumulating in fp32.  What is dropped is below 2^-24 of each product, so results
+ *                            agree with the fp32 contraction to its own rounding error; argmax may differ
+ *                            where two maxima are that close.  Used where C == 256 and a row of fmap2 has at
+ *                            most 256 columns, silently fp32 elsewhere.  Takes B*H2*W2*1536 bytes (rows and
+ *                            columns padded to 2 and 32) from the stream's memory pool (hipMallocAsync)
+ *                            for the duration of each call.
+ * The setting is process-wide and read when a call is enqueued.  Returns the previous mode; an unknown mode
+ * changes nothing.  SEPCORR_BF16X3=1 in the environment makes BF16X3 the initial choice.
+ */
+#define SEPCORR_CONTRACT_FP32 0
+#define SEPCORR_CONTRACT_BF16X3 1
+int sepcorr_set_contraction(int mode);
+
+/*
  * Replaces MemorySaver.max_avg_forward (MemorySaver_cuda.cpp:10-21 -> max_avg_cuda_forward,
  * MemorySaver_kernel_forward.cu:901-949).
  *   out_u[b,i,j,0,u] = max_v S   out_u[b,i,j,1,u] = (sum_v S) / W2      (B,H1,W1,2,H2)

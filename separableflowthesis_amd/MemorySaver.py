@@ -286,3 +286,14 @@ def assemble_backward(grad_dst, shapes):
             c0 += shp[3]
             out.append(g)
     return out
+
+
+CONTRACT_FP32, CONTRACT_BF16X3 = 0, 1
+
+
+def set_contraction(mode):
+    """Arithmetic of the forward sweeps' contraction: CONTRACT_FP32 (fp32 MFMA) or CONTRACT_BF16X3 (three bf16
+    planes per operand, fp32 accumulation; C == 256 only, fp32 elsewhere).  Process-wide; returns the previous mode.
+    Not a function of the reference."""
+    return _lib.load().sepcorr_set_contraction(int(mode))
+

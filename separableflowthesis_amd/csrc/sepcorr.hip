@@ -29,6 +29,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
 #include <mutex>
 #include <string>
 #include <vector>
@@ -221,7 +222,7 @@ struct FwdArgs {
 // BF: the experimental bf16-plane contraction (C == 256, one pass, one row group, max/avg modes)
 template <int MODE, int KC, int UR, int CMODE, int WM, bool BF = false>
 __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
-    static_assert(!BF || (CMODE == 3 && WM == 0 && UR == 2), "bf16 planes: C == 256, one pass, one row group, two rows per step");
+    static_assert(!BF || (CMODE == 3 && WM == 0), "bf16 planes: C == 256, one pass, one row group");
     constexpr bool CVEC = CMODE >= 1;
     constexpr int GJ = 2;  // 8-channel slices per prefetch group
     constexpr int NPART = (MODE == MODE_WEIGHTED) ? KC : 3;
@@ -1589,7 +1590,7 @@ int launch_fwd(FwdArgs a, int B, hipStream_t s) {
         if (cmode == 3) SEPCORR_FWD(3, 1); else if (cmode == 2) SEPCORR_FWD(2, 1);
         else if (cmode == 1) SEPCORR_FWD(1, 1); else SEPCORR_FWD(0, 1);
     } else {
-        if constexpr (UR == 2) {
+        {
             if (cmode == 3 && a.f2_planes) {   // bf16-plane variant: the caller has split fmap2
                 // LDS with the larger f1 tile (three bf16 planes); out_u staging only if two workgroups still fit a CU
                 constexpr int NCHO = (MODE == MODE_WEIGHTED) ? KC : 2;
@@ -1627,15 +1628,20 @@ int xcd_order_enabled() {
     return on;
 }
 
-// SEPCORR_BF16X3=1 selects the experimental forward sweeps that contract in three bf16 planes (C == 256, rows of
-// 97..256 columns or enough workgroups that a wave owns one column chunk).  fmap2 is split once per call into
+// Contraction of the forward sweeps: fp32 MFMA, or three bf16 planes where the shape allows (C == 256, rows of
+// 97..256 columns or enough workgroups that a wave owns one column chunk).  sepcorr_set_contraction() selects;
+// SEPCORR_BF16X3=1 in the environment makes the planes the initial choice.  fmap2 is split once per call into
 // stream-ordered memory that is released, in stream order, when the call returns.
+std::atomic<int> g_contraction{[] {
+    const char *e = getenv("SEPCORR_BF16X3");
+    return e && e[0] == '1' ? SEPCORR_CONTRACT_BF16X3 : SEPCORR_CONTRACT_FP32;
+}()};
 struct Bf16Planes {
     void *ptr = nullptr;
     hipStream_t s = nullptr;
     ~Bf16Planes() { if (ptr) (void)hipFreeAsync(ptr, s); }
     int make(const Dims &d, const float *f2, hipStream_t stream) {
-        static const bool on = [] { const char *e = getenv("SEPCORR_BF16X3"); return e && e[0] == '1'; }();
+        const bool on = g_contraction.load(std::memory_order_relaxed) == SEPCORR_CONTRACT_BF16X3;
         const WaveGrid wg = wave_grid(d.B, (d.H1 * d.W1 + TP - 1) / TP, d.W2, d.H2);
         const int nvcp = (d.W2 + 31) / 32, H2p = (d.H2 + 1) & ~1;
         const size_t batch_bytes = (size_t)H2p * nvcp * BF_CHUNK;
@@ -1902,6 +1908,11 @@ extern "C" {
 
 const char *sepcorr_last_error(void) { return g_err; }
 int sepcorr_abi_version(void) { return 1; }
+
+int sepcorr_set_contraction(int mode) {
+    if (mode != SEPCORR_CONTRACT_FP32 && mode != SEPCORR_CONTRACT_BF16X3) return g_contraction.load();
+    return g_contraction.exchange(mode);
+}
 
 int sepcorr_profile_enable(int on) {
     std::lock_guard<std::mutex> lk(g_prof_mu);
