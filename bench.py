@@ -319,7 +319,7 @@ def main():
         lib.sepcorr_profile_enable(0)
         pk = {}
         for nm, t in zip(names.value.decode().split("\n")[:n], list(tms)[:n]):
-            if nm.endswith("bf16x3") or nm == "split_planes":
+            if nm.endswith("bf16x3") or nm.startswith("split_planes") or nm == "df1_reduce_chunks":
                 pk.setdefault(nm, []).append(t)
         out["bf16_planes"] = {
             "ms_per_step": round(pms, 4), "tflops_fp32_equivalent": round(passes * Wf / (pms * 1e-3) / 1e12, 2),

@@ -185,6 +185,31 @@ __global__ void __launch_bounds__(256) split_planes_kernel(const float *__restri
     *reinterpret_cast<v8bf *>(dst + 4096) = pl3;
 }
 
+// The same planes with the roles of pixel and channel exchanged, for contractions over fmap2 pixels (d_f1): one
+// 48 KB block per (image, row u, chunk of 32 columns); inside it one KB per (16-column half s, 32-channel block cb,
+// plane): lane 32 h + i holds channel 32 cb + i at the 8 columns 32 vc + 16 s + 8 h + 0..7.
+__global__ void __launch_bounds__(256) split_planes_t_kernel(const float *__restrict__ f2, char *__restrict__ planes, int W2,
+                                                             int nvc, long nunits) {
+    const long t = (long)blockIdx.x * 256 + threadIdx.x;   // one thread per lane and (s, cb) of a chunk
+    if (t >= nunits) return;
+    const int lane = (int)(t & 63), i = lane & 31, h = lane >> 5;
+    long r = t >> 6;
+    const int cb = (int)(r & 7), s = (int)((r >> 3) & 1);
+    r >>= 4;                                                // chunk index = (b * H2 + u) * nvc + vc
+    const int vc = (int)(r % nvc);
+    const long bu = r / nvc;
+    const int v0 = 32 * vc + 16 * s + 8 * h;
+    float xs[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) xs[e] = v0 + e < W2 ? f2[(bu * W2 + v0 + e) * 256 + 32 * cb + i] : 0.f;
+    v8bf ph, pm, pl3;
+    split8(xs, ph, pm, pl3);
+    char *dst = planes + r * BF_CHUNK + ((s * 8 + cb) * 3) * 1024 + lane * 16;
+    *reinterpret_cast<v8bf *>(dst) = ph;
+    *reinterpret_cast<v8bf *>(dst + 1024) = pm;
+    *reinterpret_cast<v8bf *>(dst + 2048) = pl3;
+}
+
 // ------------------------------------------------------------------------------------------
 // forward
 // ------------------------------------------------------------------------------------------
@@ -1459,6 +1484,169 @@ __global__ void __launch_bounds__(64 * NWV) df2_tiled_kernel(const BwdArgs a, in
     }
 }
 
+// d_f1 in bf16 planes (C == 256, rows of at most 256 columns).  Workgroup = 4 waves = 128 pixels p x one chunk of 32
+// columns; it sweeps the rows u.  Per row the 48 KB block of transposed fmap2 planes is DMA'd into LDS (double
+// buffered, one barrier per row) and shared by the four waves, each of which owns 32 pixels and all 256 channels
+// (128 accumulator registers).  dL/dS of the next row is synthesised and split into planes between the MFMAs of
+// the current one.  The workgroups of the column chunks of a row leave partial sums [chunk][B, N1, 256] that
+// reduce_splits_kernel adds in chunk order (no atomics).
+__device__ __forceinline__ void dma16s(__amdgpu_buffer_rsrc_t r, float *lds_chunk, unsigned voff, unsigned soff) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void *)lds_chunk, 16, voff, soff, 0, 0);
+}
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+constexpr int DF1BF_RS = 260;   // floats per pixel row of the output transpose in LDS
+
+template <int GMODE, int KC>
+__global__ void __launch_bounds__(256) df1_bf_kernel(const BwdArgs a, const char *__restrict__ planes, float *__restrict__ dst,
+                                                     int nvc, int ptiles) {
+    extern __shared__ float smem[];   // two 48 KB row blocks; reused for the output transpose
+    const int tid = threadIdx.x, lane = tid & 63, pl = lane & 31, h = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wg = a.xcd_order ? xcd_contiguous(blockIdx.x, gridDim.x) : (int)blockIdx.x;
+    const int ptile = wg % ptiles, vc = (wg / ptiles) % nvc, b = wg / (ptiles * nvc);
+    const int N1 = a.N1, H2 = a.H2, W2 = a.W2;
+    const int pix = ptile * 128 + 32 * wave + pl;
+    const bool pok = pix < N1;
+    const size_t bp = (size_t)b * N1 + (pok ? pix : 0);
+
+    v16f acc[8];
+#pragma unroll
+    for (int cb = 0; cb < 8; ++cb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[cb][e] = 0.f;
+
+    // register r = 8 s + e of a lane belongs to column 32 vc + 16 s + 8 h + e
+    const int lanebase = 32 * vc + 8 * h;
+    VW<GMODE, KC> wv[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int v = lanebase + 16 * (r >> 3) + (r & 7);
+        wv[r] = load_vw<GMODE, KC>(a, bp, v < W2 ? v : 0, pok && v < W2);
+    }
+
+    const unsigned pixb = pok ? (unsigned)pix : 0u;
+    const unsigned uwoff_c = (pixb * a.KT + a.k0) * H2 * 4u, uwoff_2 = pixb * 2u * H2 * 4u, uwoff_1 = pixb * H2 * 4u;
+    __amdgpu_buffer_rsrc_t rs_av, rs_gcu, rs_gu, rs_amu;
+    if constexpr (g_has_comp(GMODE)) {
+        rs_av = make_rsrc(a.a_v + (size_t)b * N1 * a.KT * H2, (unsigned)N1 * a.KT * H2 * 4u);
+        rs_gcu = make_rsrc(a.g_cu + (size_t)b * N1 * a.KT * H2, (unsigned)N1 * a.KT * H2 * 4u);
+    }
+    if constexpr (g_has_maxavg(GMODE)) {
+        rs_gu = make_rsrc(a.g_u + (size_t)b * N1 * 2 * H2, (unsigned)N1 * 2u * H2 * 4u);
+        rs_amu = make_rsrc(a.am_u + (size_t)b * N1 * H2, (unsigned)N1 * H2 * 4u);
+    }
+    const float inv_w2 = 1.f / (float)W2;
+    auto load_uw_row = [&](int u) {
+        UW<GMODE, KC> w;
+        if constexpr (g_has_comp(GMODE)) {
+#pragma unroll
+            for (int k = 0; k < KC; ++k) {
+                w.a[k] = buf_load1s(rs_av, uwoff_c, (unsigned)(k * H2 + u) * 4u);
+                w.g[k] = buf_load1s(rs_gcu, uwoff_c, (unsigned)(k * H2 + u) * 4u);
+            }
+        }
+        if constexpr (g_has_maxavg(GMODE)) {
+            w.mg = buf_load1s(rs_gu, uwoff_2, (unsigned)(H2 + u) * 4u) * inv_w2;
+            w.ma = w.mg + buf_load1s(rs_gu, uwoff_2, (unsigned)u * 4u);
+            w.am = __float_as_int(buf_load1s(rs_amu, uwoff_1, (unsigned)u * 4u)) - lanebase;
+        }
+        return w;
+    };
+
+    const unsigned nbytes = (unsigned)H2 * nvc * BF_CHUNK;
+    const __amdgpu_buffer_rsrc_t rs_pl = make_rsrc(planes + (size_t)b * nbytes, nbytes);
+    auto issue_row = [&](int u, int bi) {   // each wave moves 12 of the 48 KB
+        const unsigned blk = (unsigned)(u * nvc + vc) * BF_CHUNK;
+#pragma unroll
+        for (int i = 0; i < 12; ++i) {
+            const int kb = wave * 12 + i;
+            dma16s(rs_pl, smem + bi * (BF_CHUNK / 4) + kb * 256, 16u * lane, blk + (unsigned)kb * 1024u);
+        }
+    };
+
+    // G of a row as bf16 planes: dword j of plane q holds registers 2j, 2j+1
+    unsigned gp[3][8], gn[3][8];
+    auto g_pair = [&](const UW<GMODE, KC> &wu, int u, int j, unsigned(&out)[3][8]) {
+        int un = u;
+        asm volatile("" : "+s"(un));   // (keeps the comparison with argmax_v a compare against a scalar)
+        const float x0 = gval<GMODE, KC>(wv[2 * j], wu, un, 16 * ((2 * j) >> 3) + ((2 * j) & 7), true);
+        const float x1 = gval<GMODE, KC>(wv[2 * j + 1], wu, un, 16 * ((2 * j + 1) >> 3) + ((2 * j + 1) & 7), true);
+        const v2bf hh = {(__bf16)x0, (__bf16)x1};
+        const float r0 = x0 - (float)hh[0], r1 = x1 - (float)hh[1];
+        const v2bf mm = {(__bf16)r0, (__bf16)r1};
+        const v2bf ll = {(__bf16)(r0 - (float)mm[0]), (__bf16)(r1 - (float)mm[1])};
+        out[0][j] = __builtin_bit_cast(unsigned, hh);
+        out[1][j] = __builtin_bit_cast(unsigned, mm);
+        out[2][j] = __builtin_bit_cast(unsigned, ll);
+    };
+
+    UW<GMODE, KC> wu_n = load_uw_row(0);
+    issue_row(0, 0);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) g_pair(wu_n, 0, j, gp);
+    wu_n = load_uw_row(min(1, H2 - 1));
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's DMA has landed
+    __syncthreads();
+
+    constexpr int PA[6] = {2, 0, 1, 1, 0, 0}, PB[6] = {0, 2, 1, 0, 1, 0};   // (fmap2 plane, G plane), small products first
+    for (int u = 0; u < H2; ++u) {
+        const int bi = u & 1;
+        if (u + 1 < H2) issue_row(u + 1, bi ^ 1);
+        const UW<GMODE, KC> wu_c = wu_n;                       // weights of row u + 1
+        wu_n = load_uw_row(min(u + 2, H2 - 1));
+        const char *abase = reinterpret_cast<const char *>(smem) + bi * BF_CHUNK + 16 * lane;
+        v8bf an[3], ac[3];
+#pragma unroll
+        for (int q = 0; q < 3; ++q) an[q] = *reinterpret_cast<const v8bf *>(abase + q * 1024);
+#pragma unroll
+        for (int g = 0; g < 16; ++g) {   // g = 8 s + cb
+            const int s = g >> 3, cb = g & 7;
+#pragma unroll
+            for (int q = 0; q < 3; ++q) ac[q] = an[q];
+            if (g + 1 < 16) {
+#pragma unroll
+                for (int q = 0; q < 3; ++q) an[q] = *reinterpret_cast<const v8bf *>(abase + ((g + 1) * 3 + q) * 1024);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = 0; t < 6; ++t) {
+                const v4u gb = {gp[PB[t]][4 * s], gp[PB[t]][4 * s + 1], gp[PB[t]][4 * s + 2], gp[PB[t]][4 * s + 3]};
+                acc[cb] = mfma_bf(ac[PA[t]], __builtin_bit_cast(v8bf, gb), acc[cb]);
+                if (t == 2 && (g & 1) == 0) g_pair(wu_c, u + 1, g >> 1, gn);   // runs beside the MFMAs
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int q = 0; q < 3; ++q)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) gp[q][j] = gn[q][j];
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+    }
+
+    // transpose through LDS (one region per wave): a pixel's 256 channels leave as one contiguous KB
+    float *reg = smem + wave * 32 * DF1BF_RS;
+#pragma unroll
+    for (int cb = 0; cb < 8; ++cb)
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+            const v4f x = {acc[cb][4 * rq], acc[cb][4 * rq + 1], acc[cb][4 * rq + 2], acc[cb][4 * rq + 3]};
+            *reinterpret_cast<v4f *>(reg + pl * DF1BF_RS + 32 * cb + 8 * rq + 4 * h) = x;
+        }
+    __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): the wave's own LDS writes are done (no other wave reads them)
+    float *out = dst + ((size_t)(nvc > 1 ? vc : 0) * a.B + b) * N1 * 256;
+    const bool accum = nvc == 1 && a.accumulate != 0;
+    for (int j = 0; j < 32; ++j) {
+        const int p = ptile * 128 + 32 * wave + j;
+        if (p < N1) {
+            v4f x = *reinterpret_cast<const v4f *>(reg + j * DF1BF_RS + 4 * lane);
+            v4f *o = reinterpret_cast<v4f *>(out + (size_t)p * 256 + 4 * lane);
+            if (accum) x += *o;
+            *o = x;
+        }
+    }
+}
+
 // out[i] (+)= sum_s part[s*n + i], in split order.
 __global__ void __launch_bounds__(256) reduce_splits_kernel(const float *part, float *out, size_t n, int nsplit,
                                                             int accumulate) {
@@ -1758,7 +1946,46 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s
         ProfScope ps(GMODE == GMODE_COMP ? "df1_comp" : GMODE == GMODE_BOTH ? "df1_both" : "df1_maxavg", s1); \
         hipLaunchKernelGGL((df1_kernel<GMODE, KC, NCB, CV, MT>), grid, block, lds, s1, a);         \
     } while (0)
-        if (nW > 4) { if (cvec) SEPCORR_DF1(1, true, 512); else SEPCORR_DF1(1, false, 512); }
+        const bool planes = g_contraction.load(std::memory_order_relaxed) == SEPCORR_CONTRACT_BF16X3 && d.C == 256 &&
+                            wg.vpasses == 1 && cvec && (size_t)d.H1 * d.W1 * MAX_K * d.H2 * 4 <= big &&
+                            (size_t)d.H2 * nvc_all * BF_CHUNK <= big;
+        if (planes) {
+            // bf16 planes: transposed fmap2 planes and the per-chunk partial sums live in stream-ordered memory
+            const int nvc = nvc_all, ptiles = (a.N1 + 127) / 128;
+            const size_t planes_bytes = (size_t)d.B * d.H2 * nvc * BF_CHUNK;
+            const size_t n = (size_t)d.B * a.N1 * 256;
+            const size_t part_bytes = nvc > 1 ? (size_t)nvc * n * sizeof(float) : 0;
+            void *buf = nullptr;
+            hipError_t e = hipMallocAsync(&buf, planes_bytes + part_bytes, s1);
+            if (e != hipSuccess) return fail(SEPCORR_ELAUNCH, "sepcorr: bf16 planes: %s", hipGetErrorString(e));
+            char *pl = static_cast<char *>(buf);
+            float *part = nvc > 1 ? reinterpret_cast<float *>(pl + planes_bytes) : a.d1;
+            {
+                ProfScope ps("split_planes_t", s1);
+                const long nunits = (long)d.B * d.H2 * nvc * 16 * 64;
+                hipLaunchKernelGGL(split_planes_t_kernel, dim3((unsigned)((nunits + 255) / 256)), dim3(256), 0, s1, a.f2, pl,
+                                   d.W2, nvc, nunits);
+            }
+            auto k = df1_bf_kernel<GMODE, KC>;
+            const size_t ldsb = 4 * 32 * DF1BF_RS * sizeof(float);   // output transpose; covers the two 48 KB row blocks
+            int rc = set_lds(k, ldsb);
+            if (rc == SEPCORR_OK) {
+                {
+                    ProfScope ps(GMODE == GMODE_COMP ? "df1_comp_bf16x3" : GMODE == GMODE_BOTH ? "df1_both_bf16x3" : "df1_maxavg_bf16x3", s1);
+                    hipLaunchKernelGGL(k, dim3(d.B * ptiles * nvc), dim3(256), ldsb, s1, a, pl, part, nvc, ptiles);
+                }
+                if (nvc > 1) {
+                    const int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+                    ProfScope ps("df1_reduce_chunks", s1);
+                    hipLaunchKernelGGL(reduce_splits_kernel, dim3(blocks), dim3(256), 0, s1, part, a.d1, n, nvc, a.accumulate);
+                }
+                rc = check_launch("d_f1 kernel (bf16 planes)");
+            }
+            e = hipFreeAsync(buf, s1);
+            if (rc) return rc;
+            if (e != hipSuccess) return fail(SEPCORR_ELAUNCH, "sepcorr: bf16 planes: %s", hipGetErrorString(e));
+        }
+        else if (nW > 4) { if (cvec) SEPCORR_DF1(1, true, 512); else SEPCORR_DF1(1, false, 512); }
         else if (ncb == 1) { if (cvec) SEPCORR_DF1(1, true, 256); else SEPCORR_DF1(1, false, 256); }
         // (the fast variant addresses the (p,u)-indexed tensors of one batch image with 32-bit byte offsets)
         else if (cvec && d.C == 256 && d.W2 % 4 == 0 && (size_t)d.H1 * d.W1 * MAX_K * d.H2 * 4 <= big) {

@@ -101,6 +101,64 @@ def test_compression_backward_attention_gradients(device, planes):
         assert_close(x, y, n, scale_atol=True)
 
 
+BWD_SHAPES = SHAPES[:3] + [(2, 9, 20, 9, 20, 256)]   # the last: one ragged chunk, the partial sums go straight to d_f1
+
+
+@pytest.mark.parametrize("shape", BWD_SHAPES)
+def test_max_argmax_avg_backward(device, planes, shape):
+    B, H1, W1, H2, W2, C = shape
+    f1, f2, g = op_inputs(B, H1, W1, H2, W2, C, seed=21)
+    s64 = O.corr_volume(f1.double(), f2.double())
+    _, _, am_u, am_v = O.max_argmax_avg_from_volume(s64)
+    g_u = torch.randn(B, H1, W1, 2, H2, generator=g)
+    g_v = torch.randn(B, H1, W1, 2, W2, generator=g)
+    d = lambda t: t.to(device)
+    got, labels = _labels_of(lambda: planes.max_argmax_avg_backward(d(f1), d(f2), d(am_u), d(am_v), d(g_u), d(g_v)))
+    assert "df1_maxavg_bf16x3" in labels, labels
+    ref = O.max_argmax_avg_backward(f1.double(), f2.double(), am_u, am_v, g_u.double(), g_v.double())
+    for x, y, n in zip(got, ref, ("grad_fmap1_l0", "grad_fmap2_lk")):
+        assert_close(x, y, n, scale_atol=True)
+
+
+@pytest.mark.parametrize("shape", BWD_SHAPES)
+@pytest.mark.parametrize("K", [1, 2, 3, 4, 6])
+def test_compression_backward(device, planes, shape, K):
+    B, H1, W1, H2, W2, C = shape
+    f1, f2, g = op_inputs(B, H1, W1, H2, W2, C, seed=31 + K)
+    a_u = softmax_weights(B, H1, W1, K, W2, g)
+    a_v = softmax_weights(B, H1, W1, K, H2, g)
+    g_cu = torch.randn(B, H1, W1, K, H2, generator=g)
+    g_cv = torch.randn(B, H1, W1, K, W2, generator=g)
+    d = lambda t: t.to(device)
+    got, labels = _labels_of(lambda: planes.compression_backward(d(f1), d(f2), d(a_u), d(a_v), d(g_cu), d(g_cv)))
+    assert "df1_comp_bf16x3" in labels, labels
+    ref = O.compression_backward(*(t.double() for t in (f1, f2, a_u, a_v, g_cu, g_cv)))
+    for x, y, n in zip(got, ref, ("grad_fmap1_l0", "grad_fmap2_lk", "grad_attention_u", "grad_attention_v")):
+        assert_close(x, y, n, scale_atol=True)
+
+
+@pytest.mark.parametrize("K", [2, 4, 3])
+def test_fused_backward(device, planes, K):
+    B, H1, W1, H2, W2, C = SHAPES[0]
+    f1, f2, g = op_inputs(B, H1, W1, H2, W2, C, seed=51 + K)
+    a_u = softmax_weights(B, H1, W1, K, W2, g)
+    a_v = softmax_weights(B, H1, W1, K, H2, g)
+    g_cu = torch.randn(B, H1, W1, K, H2, generator=g)
+    g_cv = torch.randn(B, H1, W1, K, W2, generator=g)
+    g_u = torch.randn(B, H1, W1, 2, H2, generator=g)
+    g_v = torch.randn(B, H1, W1, 2, W2, generator=g)
+    s64 = O.corr_volume(f1.double(), f2.double())
+    _, _, am_u, am_v = O.max_argmax_avg_from_volume(s64)
+    d = lambda t: t.to(device)
+    got, labels = _labels_of(lambda: planes.fused_backward(d(f1), d(f2), d(am_u), d(am_v), d(g_u), d(g_v),
+                                                           d(a_u), d(a_v), d(g_cu), d(g_cv)))
+    assert any(l.startswith("df1_") and l.endswith("bf16x3") for l in labels), labels
+    r1 = O.max_argmax_avg_backward(f1.double(), f2.double(), am_u, am_v, g_u.double(), g_v.double())
+    r2 = O.compression_backward(*(t.double() for t in (f1, f2, a_u, a_v, g_cu, g_cv)))
+    assert_close(got[0], r1[0] + r2[0], "grad_fmap1_l0", scale_atol=True)
+    assert_close(got[1], r1[1] + r2[1], "grad_fmap2_lk", scale_atol=True)
+
+
 def test_ineligible_shapes_stay_fp32(device, planes):
     # C != 256, and a narrow row that is swept by row groups: both silently use the fp32 MFMA kernels
     for shape in [(1, 8, 150, 8, 150, 64), (1, 12, 40, 12, 40, 256)]:
