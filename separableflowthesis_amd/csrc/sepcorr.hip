@@ -1496,8 +1496,9 @@ __device__ __forceinline__ void dma16s(__amdgpu_buffer_rsrc_t r, float *lds_chun
 typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
 constexpr int DF1BF_RS = 260;   // floats per pixel row of the output transpose in LDS
 
-template <int GMODE, int KC>
-__global__ void __launch_bounds__(256) df1_bf_kernel(const BwdArgs a, const char *__restrict__ planes, float *__restrict__ dst,
+// NW: waves per workgroup: 4 (one per SIMD, up to 512 registers) or 8 (two per SIMD, where 256 registers suffice)
+template <int GMODE, int KC, int NW>
+__global__ void __launch_bounds__(64 * NW) df1_bf_kernel(const BwdArgs a, const char *__restrict__ planes, float *__restrict__ dst,
                                                      int nvc, int ptiles) {
     extern __shared__ float smem[];   // two 48 KB row blocks; reused for the output transpose
     const int tid = threadIdx.x, lane = tid & 63, pl = lane & 31, h = lane >> 5;
@@ -1505,7 +1506,7 @@ __global__ void __launch_bounds__(256) df1_bf_kernel(const BwdArgs a, const char
     const int wg = a.xcd_order ? xcd_contiguous(blockIdx.x, gridDim.x) : (int)blockIdx.x;
     const int ptile = wg % ptiles, vc = (wg / ptiles) % nvc, b = wg / (ptiles * nvc);
     const int N1 = a.N1, H2 = a.H2, W2 = a.W2;
-    const int pix = ptile * 128 + 32 * wave + pl;
+    const int pix = ptile * (32 * NW) + 32 * wave + pl;
     const bool pok = pix < N1;
     const size_t bp = (size_t)b * N1 + (pok ? pix : 0);
 
@@ -1536,8 +1537,11 @@ __global__ void __launch_bounds__(256) df1_bf_kernel(const BwdArgs a, const char
         rs_amu = make_rsrc(a.am_u + (size_t)b * N1 * H2, (unsigned)N1 * H2 * 4u);
     }
     const float inv_w2 = 1.f / (float)W2;
-    auto load_uw_row = [&](int u) {
-        UW<GMODE, KC> w;
+    // The loads of a row's (p,u)-indexed weights are issued ahead of the row block's DMA and finished (scaled,
+    // made relative) only after the row's MFMAs: waiting for one of them then never waits for the DMA behind it.
+    struct UWRaw { float a[KC], g[KC], avg, mx, am; };
+    auto issue_uw_row = [&](int u) {
+        UWRaw w;
         if constexpr (g_has_comp(GMODE)) {
 #pragma unroll
             for (int k = 0; k < KC; ++k) {
@@ -1546,27 +1550,42 @@ __global__ void __launch_bounds__(256) df1_bf_kernel(const BwdArgs a, const char
             }
         }
         if constexpr (g_has_maxavg(GMODE)) {
-            w.mg = buf_load1s(rs_gu, uwoff_2, (unsigned)(H2 + u) * 4u) * inv_w2;
-            w.ma = w.mg + buf_load1s(rs_gu, uwoff_2, (unsigned)u * 4u);
-            w.am = __float_as_int(buf_load1s(rs_amu, uwoff_1, (unsigned)u * 4u)) - lanebase;
+            w.avg = buf_load1s(rs_gu, uwoff_2, (unsigned)(H2 + u) * 4u);
+            w.mx = buf_load1s(rs_gu, uwoff_2, (unsigned)u * 4u);
+            w.am = buf_load1s(rs_amu, uwoff_1, (unsigned)u * 4u);
         }
         return w;
     };
+    auto finish_uw_row = [&](const UWRaw &r) {
+        UW<GMODE, KC> w;
+        if constexpr (g_has_comp(GMODE)) {
+#pragma unroll
+            for (int k = 0; k < KC; ++k) { w.a[k] = r.a[k]; w.g[k] = r.g[k]; }
+        }
+        if constexpr (g_has_maxavg(GMODE)) {
+            w.mg = r.avg * inv_w2;
+            w.ma = w.mg + r.mx;
+            w.am = __float_as_int(r.am) - lanebase;
+        }
+        return w;
+    };
+    auto load_uw_row = [&](int u) { return finish_uw_row(issue_uw_row(u)); };
 
     const unsigned nbytes = (unsigned)H2 * nvc * BF_CHUNK;
     const __amdgpu_buffer_rsrc_t rs_pl = make_rsrc(planes + (size_t)b * nbytes, nbytes);
-    auto issue_row = [&](int u, int bi) {   // each wave moves 12 of the 48 KB
+    constexpr int KBW = 48 / NW;   // KB of a row block moved by each wave
+    auto issue_row = [&](int u, int bi) {
         const unsigned blk = (unsigned)(u * nvc + vc) * BF_CHUNK;
 #pragma unroll
-        for (int i = 0; i < 12; ++i) {
-            const int kb = wave * 12 + i;
+        for (int i = 0; i < KBW; ++i) {
+            const int kb = wave * KBW + i;
             dma16s(rs_pl, smem + bi * (BF_CHUNK / 4) + kb * 256, 16u * lane, blk + (unsigned)kb * 1024u);
         }
     };
 
-    // G of a row as bf16 planes: dword j of plane q holds registers 2j, 2j+1
-    unsigned gp[3][8], gn[3][8];
-    auto g_pair = [&](const UW<GMODE, KC> &wu, int u, int j, unsigned(&out)[3][8]) {
+    // G of a row as bf16 planes: dword j of plane q holds registers 2j, 2j+1 (half s = j / 4)
+    v4u gp[3][2], gn[3][2];
+    auto g_pair = [&](const UW<GMODE, KC> &wu, int u, int j, v4u(&out)[3][2]) {
         int un = u;
         asm volatile("" : "+s"(un));   // (keeps the comparison with argmax_v a compare against a scalar)
         const float x0 = gval<GMODE, KC>(wv[2 * j], wu, un, 16 * ((2 * j) >> 3) + ((2 * j) & 7), true);
@@ -1575,9 +1594,9 @@ __global__ void __launch_bounds__(256) df1_bf_kernel(const BwdArgs a, const char
         const float r0 = x0 - (float)hh[0], r1 = x1 - (float)hh[1];
         const v2bf mm = {(__bf16)r0, (__bf16)r1};
         const v2bf ll = {(__bf16)(r0 - (float)mm[0]), (__bf16)(r1 - (float)mm[1])};
-        out[0][j] = __builtin_bit_cast(unsigned, hh);
-        out[1][j] = __builtin_bit_cast(unsigned, mm);
-        out[2][j] = __builtin_bit_cast(unsigned, ll);
+        out[0][j >> 2][j & 3] = __builtin_bit_cast(unsigned, hh);
+        out[1][j >> 2][j & 3] = __builtin_bit_cast(unsigned, mm);
+        out[2][j >> 2][j & 3] = __builtin_bit_cast(unsigned, ll);
     };
 
     UW<GMODE, KC> wu_n = load_uw_row(0);
@@ -1589,60 +1608,94 @@ __global__ void __launch_bounds__(256) df1_bf_kernel(const BwdArgs a, const char
     __syncthreads();
 
     constexpr int PA[6] = {2, 0, 1, 1, 0, 0}, PB[6] = {0, 2, 1, 0, 1, 0};   // (fmap2 plane, G plane), small products first
+    // One row = 8 regions of two channel blocks (same column half): 12 MFMAs that alternate between the two
+    // accumulators, the 6 LDS reads of the next region and one pair of next-row G values.  A wave is alone on its
+    // SIMD and issues in order, so the vector work only overlaps the matrix pipe if it sits between the MFMAs:
+    // the group barriers below ask for that interleaving.
     for (int u = 0; u < H2; ++u) {
+        const v4u(&gc)[3][2] = gp;
+        v4u(&gx)[3][2] = gn;
         const int bi = u & 1;
-        if (u + 1 < H2) issue_row(u + 1, bi ^ 1);
         const UW<GMODE, KC> wu_c = wu_n;                       // weights of row u + 1
-        wu_n = load_uw_row(min(u + 2, H2 - 1));
+        const UWRaw wu_raw = issue_uw_row(min(u + 2, H2 - 1));
+        __builtin_amdgcn_sched_barrier(0);
         const char *abase = reinterpret_cast<const char *>(smem) + bi * BF_CHUNK + 16 * lane;
-        v8bf an[3], ac[3];
+        v8bf A[2][2][3];
 #pragma unroll
-        for (int q = 0; q < 3; ++q) an[q] = *reinterpret_cast<const v8bf *>(abase + q * 1024);
+        for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int g = 0; g < 16; ++g) {   // g = 8 s + cb
-            const int s = g >> 3, cb = g & 7;
+            for (int q = 0; q < 3; ++q) A[0][i][q] = *reinterpret_cast<const v8bf *>(abase + (i * 3 + q) * 1024);
 #pragma unroll
-            for (int q = 0; q < 3; ++q) ac[q] = an[q];
-            if (g + 1 < 16) {
-#pragma unroll
-                for (int q = 0; q < 3; ++q) an[q] = *reinterpret_cast<const v8bf *>(abase + ((g + 1) * 3 + q) * 1024);
-            }
+        for (int R = 0; R < 8; ++R) {   // groups g = 8 s + cb: 2R and 2R + 1
+            const int s = R >> 2, cb0 = 2 * (R & 3), cur = R & 1;
             __builtin_amdgcn_sched_barrier(0);
+            if (R + 1 < 8) {
 #pragma unroll
-            for (int t = 0; t < 6; ++t) {
-                const v4u gb = {gp[PB[t]][4 * s], gp[PB[t]][4 * s + 1], gp[PB[t]][4 * s + 2], gp[PB[t]][4 * s + 3]};
-                acc[cb] = mfma_bf(ac[PA[t]], __builtin_bit_cast(v8bf, gb), acc[cb]);
-                if (t == 2 && (g & 1) == 0) g_pair(wu_c, u + 1, g >> 1, gn);   // runs beside the MFMAs
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int q = 0; q < 3; ++q)
+                        A[cur ^ 1][i][q] = *reinterpret_cast<const v8bf *>(abase + ((2 * R + 2 + i) * 3 + q) * 1024);
             }
-            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = 0; t < 6; ++t)
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+                    acc[cb0 + i] = mfma_bf(A[cur][i][PA[t]], __builtin_bit_cast(v8bf, gc[PB[t]][s]), acc[cb0 + i]);
+            g_pair(wu_c, u + 1, R, gx);
+            // the next row's block: this wave's KBs spread over the first six regions (issuing a DMA holds the
+            // wave for a while; spread out, that time falls into the shadow of the MFMAs)
+            if (R < 6 && u + 1 < H2) {
+                const unsigned blk = (unsigned)((u + 1) * nvc + vc) * BF_CHUNK;
+#pragma unroll
+                for (int i = 0; i < KBW / 6; ++i) {
+                    const int kb = wave * KBW + (KBW / 6) * R + i;
+                    dma16s(rs_pl, smem + (bi ^ 1) * (BF_CHUNK / 4) + kb * 256, 16u * lane, blk + (unsigned)kb * 1024u);
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < 12; ++k) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);               // one MFMA
+                if (k < 6) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);    // one LDS read
+                __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);               // up to four vector instructions
+                if (k == 1 || (k == 3 && KBW == 12)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // one DMA
+            }
         }
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int q = 0; q < 3; ++q)
 #pragma unroll
-            for (int j = 0; j < 8; ++j) gp[q][j] = gn[q][j];
+            for (int i = 0; i < 2; ++i) gp[q][i] = gn[q][i];
         __builtin_amdgcn_s_waitcnt(0x0F70);
+        wu_n = finish_uw_row(wu_raw);
         __syncthreads();
     }
 
-    // transpose through LDS (one region per wave): a pixel's 256 channels leave as one contiguous KB
-    float *reg = smem + wave * 32 * DF1BF_RS;
-#pragma unroll
-    for (int cb = 0; cb < 8; ++cb)
-#pragma unroll
-        for (int rq = 0; rq < 4; ++rq) {
-            const v4f x = {acc[cb][4 * rq], acc[cb][4 * rq + 1], acc[cb][4 * rq + 2], acc[cb][4 * rq + 3]};
-            *reinterpret_cast<v4f *>(reg + pl * DF1BF_RS + 32 * cb + 8 * rq + 4 * h) = x;
-        }
-    __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): the wave's own LDS writes are done (no other wave reads them)
+    // transpose through LDS (one region per wave, four waves at a time): a pixel's 256 channels leave as one
+    // contiguous KB
+    float *reg = smem + (wave & 3) * 32 * DF1BF_RS;
     float *out = dst + ((size_t)(nvc > 1 ? vc : 0) * a.B + b) * N1 * 256;
     const bool accum = nvc == 1 && a.accumulate != 0;
-    for (int j = 0; j < 32; ++j) {
-        const int p = ptile * 128 + 32 * wave + j;
-        if (p < N1) {
-            v4f x = *reinterpret_cast<const v4f *>(reg + j * DF1BF_RS + 4 * lane);
-            v4f *o = reinterpret_cast<v4f *>(out + (size_t)p * 256 + 4 * lane);
-            if (accum) x += *o;
-            *o = x;
+#pragma unroll
+    for (int half = 0; half < NW / 4; ++half) {
+        if (half > 0) __syncthreads();
+        if ((wave >> 2) == half) {
+#pragma unroll
+            for (int cb = 0; cb < 8; ++cb)
+#pragma unroll
+                for (int rq = 0; rq < 4; ++rq) {
+                    const v4f x = {acc[cb][4 * rq], acc[cb][4 * rq + 1], acc[cb][4 * rq + 2], acc[cb][4 * rq + 3]};
+                    *reinterpret_cast<v4f *>(reg + pl * DF1BF_RS + 32 * cb + 8 * rq + 4 * h) = x;
+                }
+            __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): the wave's own LDS writes are done (no other wave reads them)
+            for (int j = 0; j < 32; ++j) {
+                const int p = ptile * (32 * NW) + 32 * wave + j;
+                if (p < N1) {
+                    v4f x = *reinterpret_cast<const v4f *>(reg + j * DF1BF_RS + 4 * lane);
+                    v4f *o = reinterpret_cast<v4f *>(out + (size_t)p * 256 + 4 * lane);
+                    if (accum) x += *o;
+                    *o = x;
+                }
+            }
         }
     }
 }
@@ -1951,7 +2004,12 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s
                             (size_t)d.H2 * nvc_all * BF_CHUNK <= big;
         if (planes) {
             // bf16 planes: transposed fmap2 planes and the per-chunk partial sums live in stream-ordered memory
-            const int nvc = nvc_all, ptiles = (a.N1 + 127) / 128;
+            // eight waves (two per SIMD, 256 registers) where the weights are few enough and the larger pixel
+            // tile does not cost a further round of workgroups
+            const int nvc = nvc_all;
+            const long w4 = (long)d.B * ((a.N1 + 127) / 128) * nvc, w8 = (long)d.B * ((a.N1 + 255) / 256) * nvc;
+            const bool eight = GMODE == GMODE_MAXAVG && ((w8 + 255) / 256) * 8 <= ((w4 + 255) / 256) * 4;
+            const int ptiles = eight ? (a.N1 + 255) / 256 : (a.N1 + 127) / 128;
             const size_t planes_bytes = (size_t)d.B * d.H2 * nvc * BF_CHUNK;
             const size_t n = (size_t)d.B * a.N1 * 256;
             const size_t part_bytes = nvc > 1 ? (size_t)nvc * n * sizeof(float) : 0;
@@ -1966,13 +2024,15 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s
                 hipLaunchKernelGGL(split_planes_t_kernel, dim3((unsigned)((nunits + 255) / 256)), dim3(256), 0, s1, a.f2, pl,
                                    d.W2, nvc, nunits);
             }
-            auto k = df1_bf_kernel<GMODE, KC>;
             const size_t ldsb = 4 * 32 * DF1BF_RS * sizeof(float);   // output transpose; covers the two 48 KB row blocks
-            int rc = set_lds(k, ldsb);
+            auto k4 = df1_bf_kernel<GMODE, KC, 4>;
+            auto k8 = df1_bf_kernel<GMODE, GMODE == GMODE_MAXAVG ? KC : 1, GMODE == GMODE_MAXAVG ? 8 : 4>;
+            int rc = eight ? set_lds(k8, ldsb) : set_lds(k4, ldsb);
             if (rc == SEPCORR_OK) {
                 {
                     ProfScope ps(GMODE == GMODE_COMP ? "df1_comp_bf16x3" : GMODE == GMODE_BOTH ? "df1_both_bf16x3" : "df1_maxavg_bf16x3", s1);
-                    hipLaunchKernelGGL(k, dim3(d.B * ptiles * nvc), dim3(256), ldsb, s1, a, pl, part, nvc, ptiles);
+                    if (eight) hipLaunchKernelGGL(k8, dim3(d.B * ptiles * nvc), dim3(512), ldsb, s1, a, pl, part, nvc, ptiles);
+                    else hipLaunchKernelGGL(k4, dim3(d.B * ptiles * nvc), dim3(256), ldsb, s1, a, pl, part, nvc, ptiles);
                 }
                 if (nvc > 1) {
                     const int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
