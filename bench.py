@@ -272,6 +272,7 @@ def main():
                      "frac": round(ach / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": TRAFFIC_BYTES_CFG4.get(dom) if args.workload == "cfg4" else None},
         "kernels": kernels,
     }
+    fused_step = None
     if "C" in ops and "F" in ops:
         # The same job through the entry points that have no counterpart in the reference's two-operator API:
         # weight gradients alone, then one contraction per feature gradient with dL/dS of both operators added
@@ -325,8 +326,17 @@ def main():
             "ms_per_step": round(pms, 4), "tflops_fp32_equivalent": round(passes * Wf / (pms * 1e-3) / 1e12, 2),
             "kernels_ms": {k: round(sum(v) / len(v), 4) for k, v in pk.items()},
             "what": "headline step with sepcorr_set_contraction(SEPCORR_CONTRACT_BF16X3): forward-type sweeps "
-                    "(max/argmax/avg, compression forward, attention gradients) in bf16 planes, feature gradients "
+                    "(max/argmax/avg, compression forward, attention gradients) and d_f1 in bf16 planes, d_f2 "
                     "in fp32 MFMA"}
+        if fused_step is not None:
+            for _ in range(args.warmup):
+                fused_step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                fused_step()
+            torch.cuda.synchronize()
+            out["bf16_planes"]["fused_level_ms_per_step"] = round((time.perf_counter() - t0) / args.steps * 1e3, 4)
     finally:
         lib.sepcorr_set_contraction(prev_mode)
     if not args.no_cpu_baseline or args.module_level:

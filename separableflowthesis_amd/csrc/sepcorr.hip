@@ -839,6 +839,7 @@ struct BwdArgs {
     const float *g_u, *g_v;          // GMODE_MAXAVG: (B,N1,2,H2), (B,N1,2,W2)
     const float *a_u, *a_v;          // GMODE_COMP:   (B,N1,KT,W2), (B,N1,KT,H2)
     const float *g_cu, *g_cv;        // GMODE_COMP:   (B,N1,KT,H2), (B,N1,KT,W2)
+    const float *uwt;                // fast d_f1: the (p,u)-indexed weights transposed to [b][u][field][p]
     float *d1;                       // (B,N1,C)
     float *d2;                       // (B,N2,C) or scratch [nsplit][B,N2,C]
     int B, N1, H2, W2, C;
@@ -1013,21 +1014,15 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
     // G of the current row lives in G[]; G of this wave's next row (u + NUG) is computed two values per
     // MFMA group, between the group's MFMAs, so the arithmetic runs in the shadow of the matrix pipe.
     float G[16], Gn[16];
-    // FAST: the (p,u)-indexed weights come through buffer loads as well: a per-lane offset to the pixel's first
-    // entry, channel and row in the scalar offset
-    const unsigned pixb = pok ? (unsigned)pix : 0u;
-    const unsigned uwoff_c = (pixb * a.KT + a.k0) * H2 * 4u, uwoff_2 = pixb * 2u * H2 * 4u, uwoff_1 = pixb * H2 * 4u;
-    __amdgpu_buffer_rsrc_t rs_av, rs_gcu, rs_gu, rs_amu;
-    if constexpr (FAST) {
-        if constexpr (g_has_comp(GMODE)) {
-            rs_av = make_rsrc(a.a_v + (size_t)b * N1 * a.KT * H2, (unsigned)N1 * a.KT * H2 * 4u);
-            rs_gcu = make_rsrc(a.g_cu + (size_t)b * N1 * a.KT * H2, (unsigned)N1 * a.KT * H2 * 4u);
-        }
-        if constexpr (g_has_maxavg(GMODE)) {
-            rs_gu = make_rsrc(a.g_u + (size_t)b * N1 * 2 * H2, (unsigned)N1 * 2u * H2 * 4u);
-            rs_amu = make_rsrc(a.am_u + (size_t)b * N1 * H2, (unsigned)N1 * H2 * 4u);
-        }
-    }
+    // FAST: the (p,u)-indexed weights come through buffer loads as well, from their transposed copy [u][field][p]:
+    // the pixel in the per-lane offset, row and field in the scalar offset; a load then reads 128 contiguous bytes
+    // (in the operator's layout every lane would touch a line of its own, and with eight or more fields those
+    // lines do not survive in cache from one row to the next)
+    constexpr int NVC = g_has_comp(GMODE) ? 2 * KC : 0;
+    constexpr int NF = NVC + (g_has_maxavg(GMODE) ? 3 : 0);
+    const unsigned pix4 = (pok ? (unsigned)pix : 0u) * 4u;
+    __amdgpu_buffer_rsrc_t rs_uw;
+    if constexpr (FAST) rs_uw = make_rsrc(a.uwt + (size_t)b * H2 * NF * N1, (unsigned)H2 * NF * N1 * 4u);
     const float inv_w2 = 1.f / (float)W2;
     // argmax_u is kept relative to this lane's first column: register r then compares against the constant
     // 8 (r / 4) + r % 4 instead of a column index that would have to be formed for every element
@@ -1039,17 +1034,18 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
             return w;
         } else {
             UW<GMODE, KC> w;
+            const unsigned row = (unsigned)u * NF * N1 * 4u;
             if constexpr (g_has_comp(GMODE)) {
 #pragma unroll
                 for (int k = 0; k < KC; ++k) {
-                    w.a[k] = buf_load1s(rs_av, uwoff_c, (unsigned)(k * H2 + u) * 4u);
-                    w.g[k] = buf_load1s(rs_gcu, uwoff_c, (unsigned)(k * H2 + u) * 4u);
+                    w.a[k] = buf_load1s(rs_uw, pix4, row + (unsigned)k * N1 * 4u);
+                    w.g[k] = buf_load1s(rs_uw, pix4, row + (unsigned)(KC + k) * N1 * 4u);
                 }
             }
             if constexpr (g_has_maxavg(GMODE)) {
-                w.mg = buf_load1s(rs_gu, uwoff_2, (unsigned)(H2 + u) * 4u) * inv_w2;
-                w.ma = w.mg + buf_load1s(rs_gu, uwoff_2, (unsigned)u * 4u);
-                w.am = __float_as_int(buf_load1s(rs_amu, uwoff_1, (unsigned)u * 4u)) - lanebase;
+                w.mg = buf_load1s(rs_uw, pix4, row + (unsigned)(NVC + 1) * N1 * 4u) * inv_w2;
+                w.ma = w.mg + buf_load1s(rs_uw, pix4, row + (unsigned)NVC * N1 * 4u);
+                w.am = __float_as_int(buf_load1s(rs_uw, pix4, row + (unsigned)(NVC + 2) * N1 * 4u)) - lanebase;
             }
             return w;
         }
@@ -1496,10 +1492,56 @@ __device__ __forceinline__ void dma16s(__amdgpu_buffer_rsrc_t r, float *lds_chun
 typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
 constexpr int DF1BF_RS = 260;   // floats per pixel row of the output transpose in LDS
 
+// The (p,u)-indexed weights of d_f1 in row-major order of u: out[b][u][f][p], fields f = a_v[k], g_cu[k] (k < KC),
+// then g_u max, g_u avg, argmax_u as the mode has them.  In the operator's layout a lane's weight of row u is 4 bytes
+// of its own pixel's line, so the 64 lanes of a load touch 64 lines and the lines of all pixels have to stay cached
+// from one row to the next; with more than a few fields they do not, and every row fetches them from HBM again.
+// Transposed, a wave's load is 128 contiguous bytes that are used once.
+// Grid: (B * ceil(N1 / 64), fields); 256 threads.
+template <int GMODE>
+__global__ void __launch_bounds__(256) transpose_uw_kernel(const BwdArgs a, int KC, float *__restrict__ out) {
+    __shared__ float tile[64 * 65];
+    const int NF = (g_has_comp(GMODE) ? 2 * KC : 0) + (g_has_maxavg(GMODE) ? 3 : 0);
+    const int tiles = (a.N1 + 63) / 64;
+    const int b = blockIdx.x / tiles, p0 = (blockIdx.x % tiles) * 64, f = blockIdx.y;
+    const int H2 = a.H2, N1 = a.N1;
+    const int np = min(64, N1 - p0);
+    // source row of pixel p for this field: H2 contiguous floats
+    const float *src;
+    size_t pstride;
+    const int fm = f - (g_has_comp(GMODE) ? 2 * KC : 0);
+    if (g_has_comp(GMODE) && f < 2 * KC) {
+        const float *base = f < KC ? a.a_v : a.g_cu;
+        const int kk = f < KC ? f : f - KC;
+        src = base + (((size_t)b * N1 + p0) * a.KT + a.k0 + kk) * H2;
+        pstride = (size_t)a.KT * H2;
+    } else if (fm < 2) {
+        src = a.g_u + (((size_t)b * N1 + p0) * 2 + fm) * H2;
+        pstride = (size_t)2 * H2;
+    } else {
+        src = reinterpret_cast<const float *>(a.am_u) + ((size_t)b * N1 + p0) * H2;
+        pstride = (size_t)H2;
+    }
+    for (int u0 = 0; u0 < H2; u0 += 64) {
+        const int nu = min(64, H2 - u0);
+        for (int idx = threadIdx.x; idx < np * nu; idx += 256) {
+            const int p = idx / nu, u = idx - p * nu;
+            tile[p * 65 + u] = src[p * pstride + u0 + u];
+        }
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < nu * np; idx += 256) {
+            const int u = idx / np, p = idx - u * np;
+            out[(((size_t)b * H2 + u0 + u) * NF + f) * N1 + p0 + p] = tile[p * 65 + u];
+        }
+        __syncthreads();
+    }
+}
+
 // NW: waves per workgroup: 4 (one per SIMD, up to 512 registers) or 8 (two per SIMD, where 256 registers suffice)
 template <int GMODE, int KC, int NW>
-__global__ void __launch_bounds__(64 * NW) df1_bf_kernel(const BwdArgs a, const char *__restrict__ planes, float *__restrict__ dst,
-                                                     int nvc, int ptiles) {
+__global__ void __launch_bounds__(64 * NW) df1_bf_kernel(const BwdArgs a, const char *__restrict__ planes,
+                                                         const float *__restrict__ uwt, float *__restrict__ dst, int nvc,
+                                                         int ptiles) {
     extern __shared__ float smem[];   // two 48 KB row blocks; reused for the output transpose
     const int tid = threadIdx.x, lane = tid & 63, pl = lane & 31, h = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1525,34 +1567,29 @@ __global__ void __launch_bounds__(64 * NW) df1_bf_kernel(const BwdArgs a, const 
         wv[r] = load_vw<GMODE, KC>(a, bp, v < W2 ? v : 0, pok && v < W2);
     }
 
-    const unsigned pixb = pok ? (unsigned)pix : 0u;
-    const unsigned uwoff_c = (pixb * a.KT + a.k0) * H2 * 4u, uwoff_2 = pixb * 2u * H2 * 4u, uwoff_1 = pixb * H2 * 4u;
-    __amdgpu_buffer_rsrc_t rs_av, rs_gcu, rs_gu, rs_amu;
-    if constexpr (g_has_comp(GMODE)) {
-        rs_av = make_rsrc(a.a_v + (size_t)b * N1 * a.KT * H2, (unsigned)N1 * a.KT * H2 * 4u);
-        rs_gcu = make_rsrc(a.g_cu + (size_t)b * N1 * a.KT * H2, (unsigned)N1 * a.KT * H2 * 4u);
-    }
-    if constexpr (g_has_maxavg(GMODE)) {
-        rs_gu = make_rsrc(a.g_u + (size_t)b * N1 * 2 * H2, (unsigned)N1 * 2u * H2 * 4u);
-        rs_amu = make_rsrc(a.am_u + (size_t)b * N1 * H2, (unsigned)N1 * H2 * 4u);
-    }
+    // transposed (p,u) weights of this image: [u][field][p]
+    constexpr int NVC = g_has_comp(GMODE) ? 2 * KC : 0;
+    constexpr int NF = NVC + (g_has_maxavg(GMODE) ? 3 : 0);
+    const unsigned pix4 = (pok ? (unsigned)pix : 0u) * 4u;
+    const __amdgpu_buffer_rsrc_t rs_uw = make_rsrc(uwt + (size_t)b * H2 * NF * N1, (unsigned)H2 * NF * N1 * 4u);
     const float inv_w2 = 1.f / (float)W2;
     // The loads of a row's (p,u)-indexed weights are issued ahead of the row block's DMA and finished (scaled,
     // made relative) only after the row's MFMAs: waiting for one of them then never waits for the DMA behind it.
     struct UWRaw { float a[KC], g[KC], avg, mx, am; };
     auto issue_uw_row = [&](int u) {
         UWRaw w;
+        const unsigned row = (unsigned)u * NF * N1 * 4u;
         if constexpr (g_has_comp(GMODE)) {
 #pragma unroll
             for (int k = 0; k < KC; ++k) {
-                w.a[k] = buf_load1s(rs_av, uwoff_c, (unsigned)(k * H2 + u) * 4u);
-                w.g[k] = buf_load1s(rs_gcu, uwoff_c, (unsigned)(k * H2 + u) * 4u);
+                w.a[k] = buf_load1s(rs_uw, pix4, row + (unsigned)k * N1 * 4u);
+                w.g[k] = buf_load1s(rs_uw, pix4, row + (unsigned)(KC + k) * N1 * 4u);
             }
         }
         if constexpr (g_has_maxavg(GMODE)) {
-            w.avg = buf_load1s(rs_gu, uwoff_2, (unsigned)(H2 + u) * 4u);
-            w.mx = buf_load1s(rs_gu, uwoff_2, (unsigned)u * 4u);
-            w.am = buf_load1s(rs_amu, uwoff_1, (unsigned)u * 4u);
+            w.mx = buf_load1s(rs_uw, pix4, row + (unsigned)NVC * N1 * 4u);
+            w.avg = buf_load1s(rs_uw, pix4, row + (unsigned)(NVC + 1) * N1 * 4u);
+            w.am = buf_load1s(rs_uw, pix4, row + (unsigned)(NVC + 2) * N1 * 4u);
         }
         return w;
     };
@@ -1976,6 +2013,18 @@ Df2Plan df2_plan(const Dims &d, bool both) {
     return pl;
 }
 
+// Workspace of a backward call: the split partial sums of d_f2, then the transposed (p,u) weights of the fast d_f1
+// kernel (C == 256; sized for the most fields one launch can have).
+size_t df2_part_bytes(const Dims &d) {
+    const int n0 = df2_plan(d, false).nsplit, n1 = df2_plan(d, true).nsplit;
+    const int ns = n0 > n1 ? n0 : n1;   // one size serves every backward entry point
+    const size_t bytes = ns > 1 ? (size_t)ns * d.B * d.H2 * d.W2 * d.C * sizeof(float) : 0;
+    return (bytes + 255) & ~(size_t)255;
+}
+size_t df1_uwt_bytes(const Dims &d) {
+    return d.C == 256 ? (size_t)d.B * d.H2 * (2 * KCH + 3) * d.H1 * d.W1 * sizeof(float) : 0;
+}
+
 template <int GMODE, int KC>
 int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s) {
     // s1: stream of the d_f1 kernel; s: stream of the d_f2 kernel and its split reduction
@@ -2001,7 +2050,7 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s
     } while (0)
         const bool planes = g_contraction.load(std::memory_order_relaxed) == SEPCORR_CONTRACT_BF16X3 && d.C == 256 &&
                             wg.vpasses == 1 && cvec && (size_t)d.H1 * d.W1 * MAX_K * d.H2 * 4 <= big &&
-                            (size_t)d.H2 * nvc_all * BF_CHUNK <= big;
+                            (size_t)d.H2 * nvc_all * BF_CHUNK <= big && (size_t)d.H2 * (2 * MAX_K + 3) * d.H1 * d.W1 * 4 <= big;
         if (planes) {
             // bf16 planes: transposed fmap2 planes and the per-chunk partial sums live in stream-ordered memory
             // eight waves (two per SIMD, 256 registers) where the weights are few enough and the larger pixel
@@ -2013,11 +2062,18 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s
             const size_t planes_bytes = (size_t)d.B * d.H2 * nvc * BF_CHUNK;
             const size_t n = (size_t)d.B * a.N1 * 256;
             const size_t part_bytes = nvc > 1 ? (size_t)nvc * n * sizeof(float) : 0;
+            constexpr int NF = (g_has_comp(GMODE) ? 2 * KC : 0) + (g_has_maxavg(GMODE) ? 3 : 0);
+            const size_t uwt_bytes = (size_t)d.B * d.H2 * NF * a.N1 * sizeof(float);
             void *buf = nullptr;
-            hipError_t e = hipMallocAsync(&buf, planes_bytes + part_bytes, s1);
+            hipError_t e = hipMallocAsync(&buf, planes_bytes + part_bytes + uwt_bytes, s1);
             if (e != hipSuccess) return fail(SEPCORR_ELAUNCH, "sepcorr: bf16 planes: %s", hipGetErrorString(e));
             char *pl = static_cast<char *>(buf);
             float *part = nvc > 1 ? reinterpret_cast<float *>(pl + planes_bytes) : a.d1;
+            float *uwt = reinterpret_cast<float *>(pl + planes_bytes + part_bytes);
+            {
+                ProfScope ps("transpose_uw", s1);
+                hipLaunchKernelGGL(transpose_uw_kernel<GMODE>, dim3(d.B * ((a.N1 + 63) / 64), NF), dim3(256), 0, s1, a, KC, uwt);
+            }
             {
                 ProfScope ps("split_planes_t", s1);
                 const long nunits = (long)d.B * d.H2 * nvc * 16 * 64;
@@ -2031,8 +2087,8 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s
             if (rc == SEPCORR_OK) {
                 {
                     ProfScope ps(GMODE == GMODE_COMP ? "df1_comp_bf16x3" : GMODE == GMODE_BOTH ? "df1_both_bf16x3" : "df1_maxavg_bf16x3", s1);
-                    if (eight) hipLaunchKernelGGL(k8, dim3(d.B * ptiles * nvc), dim3(512), ldsb, s1, a, pl, part, nvc, ptiles);
-                    else hipLaunchKernelGGL(k4, dim3(d.B * ptiles * nvc), dim3(256), ldsb, s1, a, pl, part, nvc, ptiles);
+                    if (eight) hipLaunchKernelGGL(k8, dim3(d.B * ptiles * nvc), dim3(512), ldsb, s1, a, pl, uwt, part, nvc, ptiles);
+                    else hipLaunchKernelGGL(k4, dim3(d.B * ptiles * nvc), dim3(256), ldsb, s1, a, pl, uwt, part, nvc, ptiles);
                 }
                 if (nvc > 1) {
                     const int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
@@ -2048,7 +2104,14 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s
         else if (nW > 4) { if (cvec) SEPCORR_DF1(1, true, 512); else SEPCORR_DF1(1, false, 512); }
         else if (ncb == 1) { if (cvec) SEPCORR_DF1(1, true, 256); else SEPCORR_DF1(1, false, 256); }
         // (the fast variant addresses the (p,u)-indexed tensors of one batch image with 32-bit byte offsets)
-        else if (cvec && d.C == 256 && d.W2 % 4 == 0 && (size_t)d.H1 * d.W1 * MAX_K * d.H2 * 4 <= big) {
+        else if (cvec && d.C == 256 && d.W2 % 4 == 0 && (size_t)d.H2 * (2 * KCH + 3) * d.H1 * d.W1 * 4 <= big) {
+            constexpr int NF = (g_has_comp(GMODE) ? 2 * KC : 0) + (g_has_maxavg(GMODE) ? 3 : 0);
+            float *uwt = reinterpret_cast<float *>(static_cast<char *>(ws) + df2_part_bytes(d));
+            {
+                ProfScope ps("transpose_uw", s1);
+                hipLaunchKernelGGL(transpose_uw_kernel<GMODE>, dim3(d.B * ((a.N1 + 63) / 64), NF), dim3(256), 0, s1, a, KC, uwt);
+            }
+            a.uwt = uwt;
             ProfScope ps(GMODE == GMODE_COMP ? "df1_comp" : GMODE == GMODE_BOTH ? "df1_both" : "df1_maxavg", s1);
             hipLaunchKernelGGL((df1_kernel<GMODE, KC, 2, true, 256, true>), grid, block, lds, s1, a);
         }
@@ -2265,9 +2328,7 @@ int sepcorr_compression_forward(const float *f1, const float *f2, const float *a
 size_t sepcorr_backward_workspace_bytes(int B, int H1, int W1, int H2, int W2, int C) {
     if (B < 1 || H1 < 1 || W1 < 1 || H2 < 1 || W2 < 1 || C < 1) return 0;
     const Dims d = {B, H1, W1, H2, W2, C};
-    const int n0 = df2_plan(d, false).nsplit, n1 = df2_plan(d, true).nsplit;
-    const int ns = n0 > n1 ? n0 : n1;   // one size serves every backward entry point
-    return ns > 1 ? (size_t)ns * B * H2 * W2 * C * sizeof(float) : 0;
+    return df2_part_bytes(d) + df1_uwt_bytes(d);
 }
 
 int sepcorr_max_argmax_avg_backward(const float *f1, const float *f2, const int32_t *argmax_u, const int32_t *argmax_v,
