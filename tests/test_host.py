@@ -34,7 +34,10 @@ def test_abi_version_and_workspace_query():
     assert lib.sepcorr_abi_version() == 1
     assert lib.sepcorr_backward_workspace_bytes(0, 1, 1, 1, 1, 1) == 0
     n = lib.sepcorr_backward_workspace_bytes(2, 55, 128, 55, 128, 256)
-    assert n % (2 * 55 * 128 * 256 * 4) == 0          # a whole number of d_f2-sized partial buffers
+    # d_f2-sized partial buffers, then (C == 256) the transposed copy of up to 11 weight fields of size B*H2*N1
+    part, fields = 2 * 55 * 128 * 256 * 4, 11 * 2 * 55 * (55 * 128) * 4
+    assert n > fields and (n - fields) % part == 0
+    assert lib.sepcorr_backward_workspace_bytes(2, 55, 128, 55, 128, 64) % (2 * 55 * 128 * 64 * 4) == 0
 
 
 def test_argument_checks_precede_any_launch():
