@@ -56,17 +56,18 @@ int sepcorr_profile_enable(int on);
 int sepcorr_profile_collect(char *names, size_t names_cap, float *ms, int cap);
 
 /*
- * Arithmetic of the contraction over channels in the forward sweeps (max/avg, max/argmax/avg, compression
- * forward and the attention-gradient pass of the compression backward); no counterpart in the reference.
+ * Arithmetic of the contractions of the forward sweeps (max/avg, max/argmax/avg, compression forward and the
+ * attention-gradient pass of the compression backward) and of d_f1; no counterpart in the reference.
  *   SEPCORR_CONTRACT_FP32    fp32 MFMA (the initial choice).
  *   SEPCORR_CONTRACT_BF16X3  every fp32 operand is written exactly as the sum of three bf16 numbers and the
  *                            product taken as the six largest of the nine plane products, with bf16 MFMA
  *                            accumulating in fp32.  What is dropped is below 2^-24 of each product, so results
  *                            agree with the fp32 contraction to its own rounding error; argmax may differ
  *                            where two maxima are that close.  Used where C == 256 and a row of fmap2 has at
- *                            most 256 columns, silently fp32 elsewhere.  Takes B*H2*W2*1536 bytes (rows and
- *                            columns padded to 2 and 32) from the stream's memory pool (hipMallocAsync)
- *                            for the duration of each call.
+ *                            most 256 columns, silently fp32 elsewhere.  Takes its scratch memory (about
+ *                            B*H2*W2*1536 bytes of planes; for d_f1 also ceil(W2/32) partial copies of d_f1 and
+ *                            the transposed weights) from the stream's memory pool (hipMallocAsync) for the
+ *                            duration of each call.
  * The setting is process-wide and read when a call is enqueued.  Returns the previous mode; an unknown mode
  * changes nothing.  SEPCORR_BF16X3=1 in the environment makes BF16X3 the initial choice.
  */
