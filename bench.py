@@ -337,6 +337,9 @@ def main():
                 fused_step()
             torch.cuda.synchronize()
             out["bf16_planes"]["fused_level_ms_per_step"] = round((time.perf_counter() - t0) / args.steps * 1e3, 4)
+        if not args.no_cpu_baseline or args.module_level:
+            ml = module_level(B, H, W, C, Kp, torch, dev)
+            out["bf16_planes"]["module_level"] = {k: v for k, v in ml.items() if k != "what"}
     finally:
         lib.sepcorr_set_contraction(prev_mode)
     if not args.no_cpu_baseline or args.module_level:
