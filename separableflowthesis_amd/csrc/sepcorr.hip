@@ -1537,7 +1537,8 @@ __global__ void __launch_bounds__(256) transpose_uw_kernel(const BwdArgs a, int 
     }
 }
 
-// NW: waves per workgroup: 4 (one per SIMD, up to 512 registers) or 8 (two per SIMD, where 256 registers suffice)
+// NW: waves per workgroup.  4 (one per SIMD, up to 512 registers) is what is launched; 8 (two per SIMD) fits the
+// max/avg mode only with spills and measured the same.
 template <int GMODE, int KC, int NW>
 __global__ void __launch_bounds__(64 * NW) df1_bf_kernel(const BwdArgs a, const char *__restrict__ planes,
                                                          const float *__restrict__ uwt, float *__restrict__ dst, int nvc,
@@ -1681,8 +1682,10 @@ __global__ void __launch_bounds__(64 * NW) df1_bf_kernel(const BwdArgs a, const 
             g_pair(wu_c, u + 1, R, gx);
             // the next row's block: this wave's KBs spread over the first six regions (issuing a DMA holds the
             // wave for a while; spread out, that time falls into the shadow of the MFMAs)
-            if (R < 6 && u + 1 < H2) {
-                const unsigned blk = (unsigned)((u + 1) * nvc + vc) * BF_CHUNK;
+            // (no branch on the last row: it fetches its own block once more, into the buffer nobody reads again;
+            // a branch here would split the loop body and undo the interleaving)
+            if (R < 6) {
+                const unsigned blk = (unsigned)(min(u + 1, H2 - 1) * nvc + vc) * BF_CHUNK;
 #pragma unroll
                 for (int i = 0; i < KBW / 6; ++i) {
                     const int kb = wave * KBW + (KBW / 6) * R + i;
@@ -2053,12 +2056,7 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s
                             (size_t)d.H2 * nvc_all * BF_CHUNK <= big && (size_t)d.H2 * (2 * MAX_K + 3) * d.H1 * d.W1 * 4 <= big;
         if (planes) {
             // bf16 planes: transposed fmap2 planes and the per-chunk partial sums live in stream-ordered memory
-            // eight waves (two per SIMD, 256 registers) where the weights are few enough and the larger pixel
-            // tile does not cost a further round of workgroups
-            const int nvc = nvc_all;
-            const long w4 = (long)d.B * ((a.N1 + 127) / 128) * nvc, w8 = (long)d.B * ((a.N1 + 255) / 256) * nvc;
-            const bool eight = GMODE == GMODE_MAXAVG && ((w8 + 255) / 256) * 8 <= ((w4 + 255) / 256) * 4;
-            const int ptiles = eight ? (a.N1 + 255) / 256 : (a.N1 + 127) / 128;
+            const int nvc = nvc_all, ptiles = (a.N1 + 127) / 128;
             const size_t planes_bytes = (size_t)d.B * d.H2 * nvc * BF_CHUNK;
             const size_t n = (size_t)d.B * a.N1 * 256;
             const size_t part_bytes = nvc > 1 ? (size_t)nvc * n * sizeof(float) : 0;
@@ -2082,13 +2080,11 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s
             }
             const size_t ldsb = 4 * 32 * DF1BF_RS * sizeof(float);   // output transpose; covers the two 48 KB row blocks
             auto k4 = df1_bf_kernel<GMODE, KC, 4>;
-            auto k8 = df1_bf_kernel<GMODE, GMODE == GMODE_MAXAVG ? KC : 1, GMODE == GMODE_MAXAVG ? 8 : 4>;
-            int rc = eight ? set_lds(k8, ldsb) : set_lds(k4, ldsb);
+            int rc = set_lds(k4, ldsb);
             if (rc == SEPCORR_OK) {
                 {
                     ProfScope ps(GMODE == GMODE_COMP ? "df1_comp_bf16x3" : GMODE == GMODE_BOTH ? "df1_both_bf16x3" : "df1_maxavg_bf16x3", s1);
-                    if (eight) hipLaunchKernelGGL(k8, dim3(d.B * ptiles * nvc), dim3(512), ldsb, s1, a, pl, uwt, part, nvc, ptiles);
-                    else hipLaunchKernelGGL(k4, dim3(d.B * ptiles * nvc), dim3(256), ldsb, s1, a, pl, uwt, part, nvc, ptiles);
+                    hipLaunchKernelGGL(k4, dim3(d.B * ptiles * nvc), dim3(256), ldsb, s1, a, pl, uwt, part, nvc, ptiles);
                 }
                 if (nvc > 1) {
                     const int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
