@@ -159,6 +159,39 @@ def test_fused_backward(device, planes, K):
     assert_close(got[1], r1[1] + r2[1], "grad_fmap2_lk", scale_atol=True)
 
 
+def test_corr_block_with_planes(device, planes):
+    # the caller's separate() over a two-level pyramid, forward and gradients, against the full-4D oracle
+    import copy
+    from separableflowthesis_amd import AlternateCorrBlockSepflow
+    B, C, H, W, K = 1, 256, 6, 100, 2
+    fmap1, fmap2, _, _ = O.make_inputs(B, H, W, C, seed=9)
+    torch.manual_seed(4)
+    att = (torch.nn.Conv3d(2, K, 3, padding=1), torch.nn.Conv3d(2, K, 3, padding=1))
+    r1, r2 = fmap1.double().requires_grad_(), fmap2.double().requires_grad_()
+    ratt = tuple(copy.deepcopy(m).double() for m in att)
+    rc1, rc2 = O.CorrBlock4D(r1, r2, num_levels=2).separate(ratt)
+    g1, g2 = fmap1.to(device).requires_grad_(), fmap2.to(device).requires_grad_()
+    gatt = tuple(copy.deepcopy(m).to(device) for m in att)
+
+    def run():
+        blk = AlternateCorrBlockSepflow(g1, g2, None, num_levels=2, support_backward=True)
+        c1, c2 = blk(None, sep=True, attention_weights=gatt)
+        gen = torch.Generator().manual_seed(3)
+        w1, w2 = torch.randn(rc1.shape, generator=gen) / 64, torch.randn(rc2.shape, generator=gen) / 64
+        ((c1 * w1.to(device)).sum() + (c2 * w2.to(device)).sum()).backward()
+        return c1, c2, w1, w2
+
+    (c1, c2, w1, w2), labels = _labels_of(run)
+    assert {"fwd_maxavg_bf16x3", "fwd_weighted_bf16x3", "df1_both_bf16x3"} <= labels, labels
+    assert_close(c1, rc1, "corr1")
+    assert_close(c2, rc2, "corr2")
+    ((rc1 * w1.double()).sum() + (rc2 * w2.double()).sum()).backward()
+    assert_close(g1.grad, r1.grad, "grad fmap1", scale_atol=True)
+    assert_close(g2.grad, r2.grad, "grad fmap2", scale_atol=True)
+    for m, rm, n in zip(gatt, ratt, ("attention1", "attention2")):
+        assert_close(m.weight.grad, rm.weight.grad, n + ".weight.grad", scale_atol=True)
+
+
 def test_ineligible_shapes_stay_fp32(device, planes):
     # C != 256, and a narrow row that is swept by row groups: both silently use the fp32 MFMA kernels
     for shape in [(1, 8, 150, 8, 150, 64), (1, 12, 40, 12, 40, 256)]:
