@@ -889,6 +889,40 @@ __device__ __forceinline__ VW<GMODE, KC> load_vw(const BwdArgs &a, size_t bp, in
     }
     return w;
 }
+// The (p,v)-indexed weights of a lane's 16 columns, field by field.  The 16 values of one field lie in one or two
+// cache lines of the lane's pixel, so 16 consecutive loads of the same field hit the lines the first one brought
+// in; column by column (all fields of a column, then the next column) a wave cycles through 32 lines per field and
+// with 8 or more fields nothing survives until the next column: the workgroups of an XCD then overflow its L2 and
+// every column refetches its lines from memory (0.9 GB per launch at B=2, 55x128, 11 fields).
+template <int GMODE, int KC>
+__device__ __forceinline__ void load_vw16(const BwdArgs &a, size_t bp, const int (&v)[16], const bool (&ok)[16],
+                                          VW<GMODE, KC> (&w)[16]) {
+    if constexpr (g_has_comp(GMODE)) {
+#pragma unroll
+        for (int k = 0; k < KC; ++k) {
+            const float *row = a.a_u + (bp * a.KT + a.k0 + k) * a.W2;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) w[r].a[k] = ok[r] ? row[v[r]] : 0.f;
+        }
+#pragma unroll
+        for (int k = 0; k < KC; ++k) {
+            const float *row = a.g_cv + (bp * a.KT + a.k0 + k) * a.W2;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) w[r].g[k] = ok[r] ? row[v[r]] : 0.f;
+        }
+    }
+    if constexpr (g_has_maxavg(GMODE)) {
+        const float inv_h2 = 1.f / (float)a.H2;
+        const float *ravg = a.g_v + (bp * 2 + 1) * a.W2, *rmax = a.g_v + (bp * 2 + 0) * a.W2;
+        const int *ram = a.am_v + bp * a.W2;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) w[r].mg = ok[r] ? ravg[v[r]] * inv_h2 : 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) w[r].ma = ok[r] ? w[r].mg + rmax[v[r]] : 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) w[r].am = ok[r] ? ram[v[r]] : -1;
+    }
+}
 template <int GMODE, int KC>
 __device__ __forceinline__ UW<GMODE, KC> load_uw(const BwdArgs &a, size_t bp, int u, bool ok) {
     UW<GMODE, KC> w;
@@ -964,10 +998,16 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
     for (int vp = 0; vp < a.vpasses; ++vp) {
     const int vbase = vp * 256;
     VW<GMODE, KC> wv[16];
+    {
+        int vs[16];
+        bool oks[16];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const int v = vbase + 32 * vcw + vmap(r, h);
-        wv[r] = load_vw<GMODE, KC>(a, bp, v < W2 ? v : 0, pok && v < W2);
+        for (int r = 0; r < 16; ++r) {
+            const int v = vbase + 32 * vcw + vmap(r, h);
+            vs[r] = v < W2 ? v : 0;
+            oks[r] = pok && v < W2;
+        }
+        load_vw16<GMODE, KC>(a, bp, vs, oks, wv);
     }
 
     const float *f2b = a.f2 + (size_t)b * H2 * W2 * C;
@@ -1562,10 +1602,16 @@ __global__ void __launch_bounds__(64 * NW) df1_bf_kernel(const BwdArgs a, const 
     // register r = 8 s + e of a lane belongs to column 32 vc + 16 s + 8 h + e
     const int lanebase = 32 * vc + 8 * h;
     VW<GMODE, KC> wv[16];
+    {
+        int vs[16];
+        bool oks[16];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const int v = lanebase + 16 * (r >> 3) + (r & 7);
-        wv[r] = load_vw<GMODE, KC>(a, bp, v < W2 ? v : 0, pok && v < W2);
+        for (int r = 0; r < 16; ++r) {
+            const int v = lanebase + 16 * (r >> 3) + (r & 7);
+            vs[r] = v < W2 ? v : 0;
+            oks[r] = pok && v < W2;
+        }
+        load_vw16<GMODE, KC>(a, bp, vs, oks, wv);
     }
 
     // transposed (p,u) weights of this image: [u][field][p]
