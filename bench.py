@@ -34,9 +34,9 @@ KERNEL_PASSES = {"df1_both": 1, "df2_both": 1, "fwd_maxavg": 1, "fwd_weighted": 
 # HBM bytes per launch at cfg4 from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by the factors a
 # 256 MiB device copy gives in the same run (profiles/cfg4_fwd_bwd_kernels.txt); None = not measured
 _MIB = 2 ** 20
-TRAFFIC_BYTES_CFG4 = {"fwd_maxavg": 116.3 * _MIB, "fwd_weighted": 187.6 * _MIB, "df1_comp": 206.7 * _MIB,
-                      "df2_comp": 289.0 * _MIB, "df1_maxavg": 153.4 * _MIB, "df2_maxavg": 203.7 * _MIB,
-                      "df1_both": 927.0 * _MIB, "df2_both": 438.4 * _MIB}
+TRAFFIC_BYTES_CFG4 = {"fwd_maxavg": 115.9 * _MIB, "fwd_weighted": 187.6 * _MIB, "df1_comp": 202.6 * _MIB,
+                      "df2_comp": 289.1 * _MIB, "df1_maxavg": 153.4 * _MIB, "df2_maxavg": 203.7 * _MIB,
+                      "df1_both": 232.1 * _MIB, "df2_both": 438.6 * _MIB}
 
 
 def make_inputs(B, H, W, C, Kp, torch):
