@@ -224,3 +224,33 @@ def test_full_size_agrees_with_fp32_mfma(device, planes):
         if bool(mism.any()):
             pass_gap = (ou[:, :, :, 0] - ou0[:, :, :, 0]).abs() if n == "argmax_u" else (ov[:, :, :, 0] - ov0[:, :, :, 0]).abs()
             assert float(pass_gap[mism].max()) <= 1e-5, n
+
+
+def test_full_size_backward_agrees_with_fp32_mfma(device, planes):
+    # B=2, 55x128, C=256, K'=4: d_f1 of both backward operators and of the fused one, planes against fp32 MFMA
+    B, H, W, C, K = 2, 55, 128, 256, 4
+    f1, f2, g = op_inputs(B, H, W, H, W, C, seed=2)
+    a_u = softmax_weights(B, H, W, K, W, g)
+    a_v = softmax_weights(B, H, W, K, H, g)
+    g_cu, g_cv = torch.randn(B, H, W, K, H, generator=g), torch.randn(B, H, W, K, W, generator=g)
+    g_u, g_v = torch.randn(B, H, W, 2, H, generator=g), torch.randn(B, H, W, 2, W, generator=g)
+    am_u = torch.randint(0, W, (B, H, W, 1, H), generator=g, dtype=torch.int32)
+    am_v = torch.randint(0, H, (B, H, W, 1, W), generator=g, dtype=torch.int32)
+    d = lambda t: t.to(device)
+    f1, f2, a_u, a_v, g_cu, g_cv, g_u, g_v, am_u, am_v = map(d, (f1, f2, a_u, a_v, g_cu, g_cv, g_u, g_v, am_u, am_v))
+
+    def all_three():
+        return (planes.compression_backward(f1, f2, a_u, a_v, g_cu, g_cv)[0],
+                planes.max_argmax_avg_backward(f1, f2, am_u, am_v, g_u, g_v)[0],
+                planes.fused_backward(f1, f2, am_u, am_v, g_u, g_v, a_u, a_v, g_cu, g_cv)[0])
+
+    got, labels = _labels_of(all_three)
+    assert {"df1_comp_bf16x3", "df1_maxavg_bf16x3", "df1_both_bf16x3"} <= labels, labels
+    prev = planes.set_contraction(planes.CONTRACT_FP32)
+    ref = all_three()
+    planes.set_contraction(prev)
+    for x, y, n in zip(got, ref, ("compression d_f1", "max/avg d_f1", "fused d_f1")):
+        assert_close(x, y, n, scale_atol=True)
+    # the fused gradient is the sum of the two
+    assert_close(got[2], got[0].double() + got[1].double(), "fused = sum", scale_atol=True)
+
