@@ -226,6 +226,7 @@ __device__ __forceinline__ int xcd_contiguous(int bid, int n) {
 struct FwdArgs {
     const float *f1, *f2;
     const char *f2_planes;   // bf16-plane variant: fmap2 split by split_planes_kernel
+    int H2p;                 //   its row count, padded to whole steps of all row groups
     const float *wv;   // MODE_WEIGHTED: weights indexed by v, (B,N1,KT,W2)
     const float *wu;   // MODE_WEIGHTED: weights indexed by u, (B,N1,KT,H2)
     float *out_u;      // (B,N1,CH,H2)
@@ -247,7 +248,7 @@ struct FwdArgs {
 // BF: the experimental bf16-plane contraction (C == 256, one pass, one row group, max/avg modes)
 template <int MODE, int KC, int UR, int CMODE, int WM, bool BF = false>
 __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
-    static_assert(!BF || (CMODE == 3 && WM == 0), "bf16 planes: C == 256, one pass, one row group");
+    static_assert(!BF || (CMODE == 3 && WM <= 1), "bf16 planes: C == 256, one column pass");
     constexpr bool CVEC = CMODE >= 1;
     constexpr int GJ = 2;  // 8-channel slices per prefetch group
     constexpr int NPART = (MODE == MODE_WEIGHTED) ? KC : 3;
@@ -514,7 +515,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
 
     if constexpr (BF) {
         // bf16 planes: per 32-channel block and row, six 16-byte loads (plane x k-step) feed twelve MFMAs of two rows
-        const int nvcp = (W2 + 31) >> 5, H2p = (H2 + 1) & ~1;
+        const int nvcp = (W2 + 31) >> 5, H2p = a.H2p;
         const unsigned rowbytes = (unsigned)nvcp * BF_CHUNK;
         const unsigned nbytes = (unsigned)H2p * rowbytes;
         const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(a.f2_planes + (size_t)b * nbytes, nbytes);
@@ -524,7 +525,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         auto issueB = [&](int step, int J, v4f(&buf)[UR][6]) {
 #pragma unroll
             for (int r = 0; r < UR; ++r) {
-                const unsigned row = (unsigned)(step * UR + r) * rowbytes;   // wave-uniform: travels in a scalar register
+                const unsigned row = (unsigned)((step * NUG + ug) * UR + r) * rowbytes;   // wave-uniform: travels in a scalar register
 #pragma unroll
                 for (int i = 0; i < 6; ++i) buf[r][i] = buf_load4s(rsrc, lane_off, row + (unsigned)(J * 6 + i) * 1024u);   // i = 2 plane + k-step
             }
@@ -535,7 +536,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                 if (J == 0) {
 #pragma unroll
                     for (int r = 0; r < UR; ++r) {
-                        const int u = min(step * UR + r, H2 - 1);
+                        const int u = min((step * NUG + ug) * UR + r, H2 - 1);
 #pragma unroll
                         for (int k = 0; k < KC; ++k) wur[r][k] = a.wu[(bp * a.KT + a.k0 + k) * H2 + u];
                     }
@@ -1911,27 +1912,33 @@ int launch_fwd(FwdArgs a, int B, hipStream_t s) {
     } while (0)
     // Always built for two waves per SIMD (256 registers): the accumulators then stay in ordinary
     // VGPRs, where the epilogue reads them without accumulator-register copies.
+    if (wg.vpasses == 1 && cmode == 3 && a.f2_planes) {   // bf16-plane variant: the caller has split fmap2
+        // LDS with the larger f1 tile (three bf16 planes); out_u staging only if two workgroups still fit a CU
+        constexpr int NCHO = (MODE == MODE_WEIGHTED) ? KC : 2;
+        lds = ((size_t)TP * BF_LS + 2 * UR * NPART * nW * 32) * sizeof(float);
+        const size_t extra = (size_t)TP * (NCHO + (MODE == MODE_ARGMAX ? 1 : 0)) * a.H2 * sizeof(float);
+        a.stage = lds + extra <= 80 * 1024;
+        if (a.stage) lds += extra;
+        const size_t merge = wg.nug > 1 ? (size_t)wg.nvc * NPART * 16 * 64 * sizeof(float) : 0;
+        if (lds < merge) lds = merge;
+        ProfScope ps(MODE == MODE_WEIGHTED ? "fwd_weighted_bf16x3" : "fwd_maxavg_bf16x3", s);
+        if (wg.nug > 1) {
+            auto k = fwd_kernel<MODE, KC, UR, 3, 1, true>;
+            if (int rc = set_lds(k, lds)) return rc;
+            hipLaunchKernelGGL(k, grid, block, lds, s, a);
+        } else {
+            auto k = fwd_kernel<MODE, KC, UR, 3, 0, true>;
+            if (int rc = set_lds(k, lds)) return rc;
+            hipLaunchKernelGGL(k, grid, block, lds, s, a);
+        }
+        return check_launch("forward kernel (bf16 planes)");
+    }
     if (wg.vpasses > 1) {
         if (cmode >= 2) SEPCORR_FWD(2, 2); else if (cmode == 1) SEPCORR_FWD(1, 2); else SEPCORR_FWD(0, 2);
     } else if (wg.nug > 1) {
         if (cmode == 3) SEPCORR_FWD(3, 1); else if (cmode == 2) SEPCORR_FWD(2, 1);
         else if (cmode == 1) SEPCORR_FWD(1, 1); else SEPCORR_FWD(0, 1);
     } else {
-        {
-            if (cmode == 3 && a.f2_planes) {   // bf16-plane variant: the caller has split fmap2
-                // LDS with the larger f1 tile (three bf16 planes); out_u staging only if two workgroups still fit a CU
-                constexpr int NCHO = (MODE == MODE_WEIGHTED) ? KC : 2;
-                lds = ((size_t)TP * BF_LS + 2 * UR * NPART * nW * 32) * sizeof(float);
-                const size_t extra = (size_t)TP * (NCHO + (MODE == MODE_ARGMAX ? 1 : 0)) * a.H2 * sizeof(float);
-                a.stage = lds + extra <= 80 * 1024;
-                if (a.stage) lds += extra;
-                auto k = fwd_kernel<MODE, KC, UR, 3, 0, true>;
-                if (int rc = set_lds(k, lds)) return rc;
-                ProfScope ps(MODE == MODE_WEIGHTED ? "fwd_weighted_bf16x3" : "fwd_maxavg_bf16x3", s);
-                hipLaunchKernelGGL(k, grid, block, lds, s, a);
-                return check_launch("forward kernel (bf16 planes)");
-            }
-        }
         if (cmode == 3) SEPCORR_FWD(3, 0); else if (cmode == 2) SEPCORR_FWD(2, 0);
         else if (cmode == 1) SEPCORR_FWD(1, 0); else SEPCORR_FWD(0, 0);
     }
@@ -1955,8 +1962,8 @@ int xcd_order_enabled() {
     return on;
 }
 
-// Contraction of the forward sweeps: fp32 MFMA, or three bf16 planes where the shape allows (C == 256, rows of
-// 97..256 columns or enough workgroups that a wave owns one column chunk).  sepcorr_set_contraction() selects;
+// Contraction of the forward sweeps: fp32 MFMA, or three bf16 planes where the shape allows (C == 256, rows of at
+// most 256 columns).  sepcorr_set_contraction() selects;
 // SEPCORR_BF16X3=1 in the environment makes the planes the initial choice.  fmap2 is split once per call into
 // stream-ordered memory that is released, in stream order, when the call returns.
 std::atomic<int> g_contraction{[] {
@@ -1965,14 +1972,16 @@ std::atomic<int> g_contraction{[] {
 }()};
 struct Bf16Planes {
     void *ptr = nullptr;
+    int H2p = 0;
     hipStream_t s = nullptr;
     ~Bf16Planes() { if (ptr) (void)hipFreeAsync(ptr, s); }
     int make(const Dims &d, const float *f2, hipStream_t stream) {
         const bool on = g_contraction.load(std::memory_order_relaxed) == SEPCORR_CONTRACT_BF16X3;
         const WaveGrid wg = wave_grid(d.B, (d.H1 * d.W1 + TP - 1) / TP, d.W2, d.H2);
-        const int nvcp = (d.W2 + 31) / 32, H2p = (d.H2 + 1) & ~1;
+        const int nvcp = (d.W2 + 31) / 32;
+        H2p = (d.H2 + 2 * wg.nug - 1) / (2 * wg.nug) * (2 * wg.nug);   // whole steps of two rows for every row group
         const size_t batch_bytes = (size_t)H2p * nvcp * BF_CHUNK;
-        if (!on || d.C != 256 || wg.vpasses > 1 || wg.nug > 1 || batch_bytes > (1u << 30)) return SEPCORR_OK;
+        if (!on || d.C != 256 || wg.vpasses > 1 || batch_bytes > (1u << 30)) return SEPCORR_OK;
         const size_t nchunks = (size_t)d.B * H2p * nvcp;
         s = stream;
         const hipError_t e = hipMallocAsync(&ptr, nchunks * BF_CHUNK, s);
@@ -2007,6 +2016,7 @@ int weighted_forward(const Dims &d, const float *f1, const float *f2, const floa
     Bf16Planes planes;
     if (int rc = planes.make(d, f2, s)) return rc;
     a.f2_planes = static_cast<const char *>(planes.ptr);
+    a.H2p = planes.H2p;
     for (int k0 = 0; k0 < K; k0 += KCH) {
         a.k0 = k0;
         const int kc = K - k0 < KCH ? K - k0 : KCH;
@@ -2343,6 +2353,7 @@ int sepcorr_max_avg_forward(const float *f1, const float *f2, float *out_u, floa
     Bf16Planes planes;
     if (int rc = planes.make(d, f2, static_cast<hipStream_t>(stream))) return rc;
     a.f2_planes = static_cast<const char *>(planes.ptr);
+    a.H2p = planes.H2p;
     return launch_fwd<MODE_MAXAVG, 1, 2>(a, B, static_cast<hipStream_t>(stream));
 }
 
@@ -2356,6 +2367,7 @@ int sepcorr_max_argmax_avg_forward(const float *f1, const float *f2, float *out_
     Bf16Planes planes;
     if (int rc = planes.make(d, f2, static_cast<hipStream_t>(stream))) return rc;
     a.f2_planes = static_cast<const char *>(planes.ptr);
+    a.H2p = planes.H2p;
     return launch_fwd<MODE_ARGMAX, 1, 2>(a, B, static_cast<hipStream_t>(stream));
 }
 

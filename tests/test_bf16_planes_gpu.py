@@ -13,12 +13,15 @@ from tests._util import assert_close, check_argmax, op_inputs, softmax_weights
 
 pytestmark = pytest.mark.gpu
 
-# (B, H1, W1, H2, W2, C), all with C == 256 and one column chunk per wave, one row group
+# (B, H1, W1, H2, W2, C), all with C == 256 and rows of at most 256 columns
 SHAPES = [
     (1, 7, 100, 7, 100, 256),    # ragged last chunk, odd row count (one padded row)
     (1, 9, 160, 9, 160, 256),    # five chunks
     (3, 48, 64, 24, 96, 256),    # pooled fmap2, three chunks, more than 256 workgroups
     (1, 4, 256, 4, 256, 256),    # widest row of a single pass
+    (1, 12, 40, 12, 40, 256),    # narrow rows: two column chunks x row groups
+    (2, 24, 32, 11, 17, 256),    # one ragged column chunk, row groups, rows padded to whole steps
+    (1, 16, 128, 16, 128, 256),  # four chunks x two row groups (few workgroups)
 ]
 
 
@@ -70,7 +73,7 @@ def test_max_argmax_avg_forward(device, planes, shape):
     assert torch.equal(ou, ou2) and torch.equal(ov, ov2)
 
 
-@pytest.mark.parametrize("shape", SHAPES[:3])
+@pytest.mark.parametrize("shape", SHAPES[:3] + SHAPES[4:])
 @pytest.mark.parametrize("K", [1, 2, 3, 5])
 def test_compression_forward(device, planes, shape, K):
     B, H1, W1, H2, W2, C = shape
@@ -193,8 +196,8 @@ def test_corr_block_with_planes(device, planes):
 
 
 def test_ineligible_shapes_stay_fp32(device, planes):
-    # C != 256, and a narrow row that is swept by row groups: both silently use the fp32 MFMA kernels
-    for shape in [(1, 8, 150, 8, 150, 64), (1, 12, 40, 12, 40, 256)]:
+    # C != 256, and rows wider than one column pass: both silently use the fp32 MFMA kernels
+    for shape in [(1, 8, 150, 8, 150, 64), (1, 2, 300, 2, 300, 256)]:
         B, H1, W1, H2, W2, C = shape
         f1, f2, _ = op_inputs(B, H1, W1, H2, W2, C, seed=3)
         (ou, ov), labels = _labels_of(lambda: planes.max_avg_forward(f1.to(device), f2.to(device)))
