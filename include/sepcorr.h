@@ -197,6 +197,28 @@ int sepcorr_assemble_forward(const float *src, float *dst, int B, int H1, int W1
 int sepcorr_assemble_backward(const float *grad_dst, float *grad_src, int B, int H1, int W1, int ch, int Li,
                               int CT, int c0, int L0, void *stream);
 
+/*
+ * Windowed bilinear lookup of the correlation pyramid without the 4D volume: what the caller's
+ * corr_fn(coords) returns on the stored-volume path (CorrBlock.__call__, core/corr.py:193-248), for the block
+ * that never stores the volume (AlternateCorrBlockSepflow.__call__, core/corr.py:479-510, which raises
+ * NotImplementedError in the reference: its native part, RAFT's alt_cuda_corr.forward, is not in the tree).
+ *   f1         (B,H1,W1,C)       unscaled NHWC fmap1 (core/corr.py:500)
+ *   f2_levels  host array of L device pointers; level l is the pooled NHWC fmap2 (B,h2[l],w2[l],C)
+ *              (core/corr.py:377-382, 501); h2, w2 are host arrays of L ints
+ *   coords     (B,2,H1,W1)       channel 0 = x (fmap2 column), channel 1 = y (fmap2 row), level-0 pixels;
+ *                                level l samples at coords / 2^l (core/corr.py:219, 503)
+ *   out        (B, L*n*n, H1, W1), n = 2*radius+1, fully overwritten:
+ *              out[b, l*n*n + a*n + c, i, j] = scale * bilinear(S_l[b,i,j,:,:])(x/2^l + a - radius, y/2^l + c - radius)
+ *              with S_l = <f1[b,i,j,:], f2_l[b,u,v,:]>, corners outside the level counting as zero
+ *              (grid_sample with align_corners=True, core/utils/utils.py:110-118); the x offset runs with the
+ *              first window index as in the reference (core/corr.py:213-226).  scale = 1/sqrt(C) reproduces
+ *              core/corr.py:282, 509.
+ * Limits: C <= 1024, L <= 8, radius 1..8.
+ */
+int sepcorr_lookup_forward(const float *f1, const float *const *f2_levels, const int *h2, const int *w2,
+                           const float *coords, float *out, int B, int H1, int W1, int C, int L, int radius,
+                           float scale, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

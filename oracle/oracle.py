@@ -252,8 +252,9 @@ def loops_forward(f1, f2, a_u=None, a_v=None):
 class CorrBlock4D:
     """Restatement of CorrBlock.__init__/corr_compute/separate (core/corr.py:19-165, 251-302).
 
-    NCHW fmaps in, (corr1 (B,K*L,W,H1,W1), corr2 (B,K*L,H,H1,W1)) out.  The 4D
-    lookup (__call__ with coords) and NLF aggregation are not part of the path.
+    NCHW fmaps in, (corr1 (B,K*L,W,H1,W1), corr2 (B,K*L,H,H1,W1)) out.  `lookup`
+    restates __call__ with coords (core/corr.py:193-248); NLF aggregation is not
+    part of the path.
     """
 
     def __init__(self, fmap1, fmap2, num_levels=4):
@@ -290,6 +291,80 @@ class CorrBlock4D:
             us.append(F.interpolate(sep_u, [w2, h1, w1], mode='trilinear', align_corners=True))
             vs.append(F.interpolate(sep_v, [h2, h1, w1], mode='trilinear', align_corners=True))
         return torch.cat(us, dim=1), torch.cat(vs, dim=1)
+
+
+    def lookup(self, coords, radius=4):
+        """Windowed bilinear lookup in every pyramid level (core/corr.py:193-248).
+
+        coords (B,2,h1,w1): channel 0 = x (fmap2 column), channel 1 = y (fmap2 row),
+        in level-0 pixels.  Returns (B, levels*(2r+1)^2, h1, w1); within a level the
+        channel index is a*(2r+1)+b and samples (x/2^l + a - r, y/2^l + b - r): the
+        x offset runs with the *first* window index, because the reference stacks
+        meshgrid(dy, dx) onto (x, y) coordinates (core/corr.py:213, 226).  Sampling is
+        grid_sample(bilinear, align_corners=True, zero padding) on pixel coordinates
+        normalised as core/utils/utils.py:110-118.
+        """
+        r = radius
+        B, h1, w1, _, _ = self.shape
+        coords = coords.permute(0, 2, 3, 1)
+        d = torch.linspace(-r, r, 2 * r + 1, dtype=coords.dtype)
+        delta = torch.stack(torch.meshgrid(d, d, indexing='ij'), dim=-1).view(1, 2 * r + 1, 2 * r + 1, 2)
+        out = []
+        for i, corr in enumerate(self.pyramid):
+            H, W = corr.shape[-2:]
+            c = coords.reshape(B * h1 * w1, 1, 1, 2) / 2 ** i + delta
+            xg = 2 * c[..., 0:1] / (W - 1) - 1
+            yg = 2 * c[..., 1:2] / (H - 1) - 1
+            smp = F.grid_sample(corr, torch.cat([xg, yg], dim=-1), mode='bilinear', padding_mode='zeros',
+                                align_corners=True)
+            out.append(smp.view(B, h1, w1, -1))
+        return torch.cat(out, dim=-1).permute(0, 3, 1, 2).contiguous()
+
+
+def lookup_direct(fmap1, fmap2, coords, num_levels=4, radius=4):
+    """The same lookup from its definition, without a 4D volume and without grid_sample.
+
+    Bilinear sampling is linear in the sampled image and the level-l volume is
+    S(f1, avgpool^l f2) (pooling commutes with the contraction), so every sample is
+    <fmap1[:,i,j], bilinear(avgpool^l fmap2)(x, y)> / sqrt(C) with corners outside the
+    image counted as zero.  Independent of `CorrBlock4D.lookup` in everything but the
+    definition; the two are compared in tests/test_oracle.py.
+    """
+    B, C, h1, w1 = fmap1.shape
+    r = radius
+    n = 2 * r + 1
+    f1 = fmap1.permute(0, 2, 3, 1)                                 # (B,h1,w1,C)
+    x = coords[:, 0]
+    y = coords[:, 1]
+    off = torch.arange(-r, r + 1, dtype=coords.dtype)
+    outs = []
+    f2 = fmap2
+    for lvl in range(num_levels):
+        if lvl:
+            f2 = F.avg_pool2d(f2, 2, stride=2)
+        H, W = f2.shape[-2:]
+        f2n = f2.permute(0, 2, 3, 1)                               # (B,H,W,C)
+        xs = (x / 2 ** lvl)[..., None, None] + off.view(1, 1, 1, n, 1)   # (B,h1,w1,a,1): x moves with a
+        ys = (y / 2 ** lvl)[..., None, None] + off.view(1, 1, 1, 1, n)   # (B,h1,w1,1,b): y moves with b
+        xs, ys = torch.broadcast_tensors(xs, ys)
+        x0 = torch.floor(xs)
+        y0 = torch.floor(ys)
+        fx = xs - x0
+        fy = ys - y0
+        acc = torch.zeros(B, h1, w1, n, n, dtype=fmap1.dtype)
+        bidx = torch.arange(B).view(B, 1, 1, 1, 1).expand_as(x0)
+        for dy, wy in ((0, 1 - fy), (1, fy)):
+            for dx, wx in ((0, 1 - fx), (1, fx)):
+                xi = (x0 + dx).long()
+                yi = (y0 + dy).long()
+                ok = (xi >= 0) & (xi < W) & (yi >= 0) & (yi < H)
+                g = f2n[bidx, yi.clamp(0, H - 1), xi.clamp(0, W - 1)]          # (B,h1,w1,n,n,C)
+                dot = (g * f1[:, :, :, None, None, :]).sum(-1)
+                acc = acc + torch.where(ok, wx * wy * dot, torch.zeros_like(dot))
+        outs.append(acc.reshape(B, h1, w1, n * n))
+    # the reference divides by the fp32 square root (core/corr.py:282, 509)
+    out = torch.cat(outs, dim=-1) / torch.sqrt(torch.tensor(C).float()).to(fmap1.dtype)
+    return out.permute(0, 3, 1, 2).contiguous()
 
 
 def make_inputs(B, H, W, C, seed=1234, dtype=torch.float32):

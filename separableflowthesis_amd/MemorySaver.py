@@ -288,6 +288,39 @@ def assemble_backward(grad_dst, shapes):
     return out
 
 
+def lookup_forward(img1_features_l0, img2_features_lvls, coords, radius, scale):
+    """Windowed bilinear lookup of the correlation pyramid, never holding the 4D volume.
+
+    img1_features_l0 (B,H1,W1,C) unscaled, img2_features_lvls: list of pooled NHWC fmap2 levels (B,H2_l,W2_l,C),
+    coords (B,2,H1,W1) with x in channel 0 -> (B, levels*(2*radius+1)^2, H1, W1), multiplied by `scale`.
+    Stands where the reference calls alt_cuda_corr.forward once per level (core/corr.py:497-509); not a function
+    of the reference's MemorySaver module.
+    """
+    import ctypes
+    f1 = img1_features_l0
+    _check("img1_features_l0", f1, ndim=4)
+    B, H1, W1, C = f1.shape
+    _expect("coords", coords, (B, 2, H1, W1), f1.device)
+    lvls = list(img2_features_lvls)
+    if not lvls:
+        raise RuntimeError("at least one fmap2 level is needed")
+    for n, t in enumerate(lvls):
+        _check(f"img2_features_lvls[{n}]", t, ndim=4)
+        if t.shape[0] != B or t.shape[3] != C or t.device != f1.device:
+            raise RuntimeError(f"img2_features_lvls[{n}]: batch/feature size or device differs from img1_features_l0")
+    L = len(lvls)
+    n = 2 * int(radius) + 1
+    lib = _lib.load()
+    with torch.cuda.device(f1.device):
+        out = torch.empty((B, L * n * n, H1, W1), dtype=f1.dtype, device=f1.device)
+        ptrs = (ctypes.c_void_p * L)(*[t.data_ptr() for t in lvls])
+        h2 = (ctypes.c_int * L)(*[t.shape[1] for t in lvls])
+        w2 = (ctypes.c_int * L)(*[t.shape[2] for t in lvls])
+        _lib.check(lib.sepcorr_lookup_forward(f1.data_ptr(), ptrs, h2, w2, coords.data_ptr(), out.data_ptr(),
+                                              B, H1, W1, C, L, int(radius), float(scale), _stream()))
+    return out
+
+
 CONTRACT_FP32, CONTRACT_BF16X3 = 0, 1
 
 

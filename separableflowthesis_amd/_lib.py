@@ -31,6 +31,7 @@ SIGNATURES = {
     "sepcorr_attention_backward": (_I, [_P] * 7 + [_I] * 5 + [_P, _SZ, _P]),
     "sepcorr_assemble_forward": (_I, [_P] * 2 + [_I] * 8 + [_P]),
     "sepcorr_assemble_backward": (_I, [_P] * 2 + [_I] * 8 + [_P]),
+    "sepcorr_lookup_forward": (_I, [_P] * 6 + [_I] * 6 + [ctypes.c_float, _P]),
 }
 
 _lib = None

@@ -10,6 +10,7 @@ trilinearly upsampled (align_corners=True) to the level-0 displacement length.
 import torch
 import torch.nn.functional as F
 
+from . import MemorySaver
 from .functions import (AssembleVolumeFunction, AttentionWeightsFunction, ComputeMaxArgmaxAvgFunction,
                         ComputeMaxAvgFunction, ComputeSelfCompressionFunction, SeparateLevelFunction)
 
@@ -95,6 +96,24 @@ class AlternateCorrBlockSepflow:
     def __call__(self, coords, sep=False, attention_weights=None):
         if sep:
             return self.separate(attention_weights)
-        # core/corr.py:491-492
-        raise NotImplementedError("Missing the cpp/cuda part for lookup"
-                                  "of the 4d correlation volume without storing it")
+        return self.lookup(coords)
+
+    def lookup(self, coords):
+        """corr_fn(coords) without the 4D volume: (B, levels*(2r+1)^2, H1, W1).
+
+        The reference stops here with NotImplementedError (core/corr.py:491-492) because the native part its
+        draft calls (alt_cuda_corr.forward per level, core/corr.py:494-509) is not in its tree; the values are
+        those of the stored-volume block (CorrBlock.__call__, core/corr.py:193-248).  Forward only: the result
+        carries no autograd graph (the flow iterations that consume it detach coords anyway; gradients reach the
+        feature maps through separate()).
+        """
+        if not hasattr(self, "_lookup_inputs"):
+            with torch.no_grad():
+                f1 = self.fmap1_l0.permute(0, 2, 3, 1).contiguous().float()
+                f2s = [p.permute(0, 2, 3, 1).contiguous().float() for p in self.pyramid]
+            self._lookup_inputs = (f1, f2s)
+        f1, f2s = self._lookup_inputs
+        fdim = f1.shape[3]
+        with torch.no_grad():
+            return MemorySaver.lookup_forward(f1, f2s, coords.detach().contiguous().float(), self.radius,
+                                              1.0 / float(torch.sqrt(torch.tensor(fdim).float())))
