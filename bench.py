@@ -130,6 +130,47 @@ def module_level(B, H, W, C, Kp, torch, dev, reps=5):
     return out
 
 
+def lookup_level(B, H, W, C, torch, dev, reps=20):
+    """corr_fn(coords) of the block without the 4D volume (untimed extra): 4 levels, radius 4, a smooth flow field.
+    Forward = one gather kernel; backward = grid gradients, d_f1 gather, d_f2 by owner tiles, slice reduction."""
+    from separableflowthesis_amd import MemorySaver
+    g = torch.Generator().manual_seed(1234)
+    f1 = torch.randn(B, H, W, C, generator=g).to(dev)
+    f2s = [torch.randn(B, H >> l, W >> l, C, generator=g).to(dev) for l in range(4)]
+    yy, xx = torch.meshgrid(torch.arange(H), torch.arange(W), indexing="ij")
+    flow = torch.randn(B, 2, 1, 1, generator=g) * 4 + torch.randn(B, 2, H, W, generator=g) * 0.5
+    coords = (torch.stack([xx, yy]).float()[None] + flow).contiguous().to(dev)
+    up = torch.randn(B, 4 * 81, H, W, generator=g).to(dev)
+    scale = 1.0 / 16.0
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    fwd = timed(lambda: MemorySaver.lookup_forward(f1, f2s, coords, 4, scale))
+    bwd = timed(lambda: MemorySaver.lookup_backward(f1, f2s, coords, up, 4, scale))
+    pts = B * H * W * 4 * 100                       # (pixel, level, grid point) pairs: one C-long dot product each
+    alg = (f1.numel() + sum(t.numel() for t in f2s) + coords.numel() + up.numel()) * 4
+    return {
+        "forward_ms": round(fwd, 4), "backward_ms": round(bwd, 4),
+        "forward_gathered_gb_s": round(pts * C * 4 / fwd / 1e6, 1),
+        "forward_gflop_s": round(pts * C * 2 / fwd / 1e6, 1),
+        "forward_algorithmic_mib": round(alg / 2 ** 20, 1),
+        "forward_hbm_gb_s": round(alg / fwd / 1e6, 1),
+        "what": f"sepcorr_lookup_forward / sepcorr_lookup_backward, B={B}, C={C}, {H}x{W}, 4 levels, radius 4; "
+                "gathered = bytes of fmap2 rows fetched through the vector cache (2 flop per 4 bytes: bound by that "
+                "cache, peak 256 CU x 64 B/clk x 2.4 GHz = 39.3 TB/s); algorithmic = f1 + pyramid + coords + out once",
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -144,6 +185,7 @@ def main():
                     help="measure the caller's whole separate() too even with --no-cpu-baseline")
     ap.add_argument("--only-module-level", action="store_true",
                     help="measure nothing but the caller's whole separate() (for kernel traces of that path)")
+    ap.add_argument("--only-lookup", action="store_true", help="run only the pyramid-lookup extra (for profiling)")
     ap.add_argument("--single-stream", action="store_true",
                     help="keep all kernels of a call on the caller's stream (per-kernel durations under a profiler are "
                          "then those of kernels running alone)")
@@ -164,6 +206,9 @@ def main():
     B, H, W, Kp, ops = WORKLOADS[args.workload]
     C = 256
     N = H * W
+    if args.only_lookup:
+        print(json.dumps({"workload": args.workload, "lookup": lookup_level(B, H, W, C, torch, dev)}))
+        return
     if args.only_module_level:
         print(json.dumps({"workload": args.workload, "module_level": module_level(B, H, W, C, Kp, torch, dev)}))
         return
@@ -344,6 +389,8 @@ def main():
         lib.sepcorr_set_contraction(prev_mode)
     if not args.no_cpu_baseline or args.module_level:
         out["module_level"] = module_level(B, H, W, C, Kp, torch, dev)
+    if not args.no_cpu_baseline or args.module_level:
+        out["lookup"] = lookup_level(B, H, W, C, torch, dev)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(B, H, W, C, Kp, ops, torch)
     print(json.dumps(out))

@@ -219,6 +219,27 @@ int sepcorr_lookup_forward(const float *f1, const float *const *f2_levels, const
                            const float *coords, float *out, int B, int H1, int W1, int C, int L, int radius,
                            float scale, void *stream);
 
+/* Scratch bytes needed by sepcorr_lookup_backward (h2, w2: host arrays of L level sizes). 0 for invalid sizes. */
+size_t sepcorr_lookup_backward_workspace_bytes(const int *h2, const int *w2, int B, int H1, int W1, int C, int L,
+                                               int radius);
+
+/*
+ * Gradients of sepcorr_lookup_forward with respect to the feature maps: what torch autograd computes through
+ * bilinear_sampler and the stored pyramid on the reference's 4D path (core/corr.py:193-248, 19-38) and what
+ * alt_cuda_corr.backward would supply to the draft at core/corr.py:494-509.  coords receive no gradient (the flow
+ * iterations detach them, core/sepflow.py:194).
+ *   grad_out     (B, L*n*n, H1, W1)
+ *   d_f1         (B,H1,W1,C)                      fully overwritten
+ *   d_f2_levels  host array of L device pointers; level l (B,h2[l],w2[l],C), fully overwritten: the gradient of that
+ *                level's pooled fmap2 (the caller's avg_pool2d chain carries it on to fmap2)
+ * No atomics; sums run in a fixed order: results are run-to-run identical.  workspace: 256-byte aligned device memory
+ * of at least sepcorr_lookup_backward_workspace_bytes(...) bytes.
+ */
+int sepcorr_lookup_backward(const float *f1, const float *const *f2_levels, const int *h2, const int *w2,
+                            const float *coords, const float *grad_out, float *d_f1, float *const *d_f2_levels,
+                            int B, int H1, int W1, int C, int L, int radius, float scale,
+                            void *workspace, size_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -288,6 +288,24 @@ def assemble_backward(grad_dst, shapes):
     return out
 
 
+def _lookup_args(f1, lvls, coords):
+    import ctypes
+    _check("img1_features_l0", f1, ndim=4)
+    B, H1, W1, C = f1.shape
+    _expect("coords", coords, (B, 2, H1, W1), f1.device)
+    if not lvls:
+        raise RuntimeError("at least one fmap2 level is needed")
+    for n, t in enumerate(lvls):
+        _check(f"img2_features_lvls[{n}]", t, ndim=4)
+        if t.shape[0] != B or t.shape[3] != C or t.device != f1.device:
+            raise RuntimeError(f"img2_features_lvls[{n}]: batch/feature size or device differs from img1_features_l0")
+    L = len(lvls)
+    ptrs = (ctypes.c_void_p * L)(*[t.data_ptr() for t in lvls])
+    h2 = (ctypes.c_int * L)(*[t.shape[1] for t in lvls])
+    w2 = (ctypes.c_int * L)(*[t.shape[2] for t in lvls])
+    return B, H1, W1, C, L, ptrs, h2, w2
+
+
 def lookup_forward(img1_features_l0, img2_features_lvls, coords, radius, scale):
     """Windowed bilinear lookup of the correlation pyramid, never holding the 4D volume.
 
@@ -296,29 +314,35 @@ def lookup_forward(img1_features_l0, img2_features_lvls, coords, radius, scale):
     Stands where the reference calls alt_cuda_corr.forward once per level (core/corr.py:497-509); not a function
     of the reference's MemorySaver module.
     """
-    import ctypes
-    f1 = img1_features_l0
-    _check("img1_features_l0", f1, ndim=4)
-    B, H1, W1, C = f1.shape
-    _expect("coords", coords, (B, 2, H1, W1), f1.device)
-    lvls = list(img2_features_lvls)
-    if not lvls:
-        raise RuntimeError("at least one fmap2 level is needed")
-    for n, t in enumerate(lvls):
-        _check(f"img2_features_lvls[{n}]", t, ndim=4)
-        if t.shape[0] != B or t.shape[3] != C or t.device != f1.device:
-            raise RuntimeError(f"img2_features_lvls[{n}]: batch/feature size or device differs from img1_features_l0")
-    L = len(lvls)
+    f1, lvls = img1_features_l0, list(img2_features_lvls)
+    B, H1, W1, C, L, ptrs, h2, w2 = _lookup_args(f1, lvls, coords)
     n = 2 * int(radius) + 1
     lib = _lib.load()
     with torch.cuda.device(f1.device):
         out = torch.empty((B, L * n * n, H1, W1), dtype=f1.dtype, device=f1.device)
-        ptrs = (ctypes.c_void_p * L)(*[t.data_ptr() for t in lvls])
-        h2 = (ctypes.c_int * L)(*[t.shape[1] for t in lvls])
-        w2 = (ctypes.c_int * L)(*[t.shape[2] for t in lvls])
         _lib.check(lib.sepcorr_lookup_forward(f1.data_ptr(), ptrs, h2, w2, coords.data_ptr(), out.data_ptr(),
                                               B, H1, W1, C, L, int(radius), float(scale), _stream()))
     return out
+
+
+def lookup_backward(img1_features_l0, img2_features_lvls, coords, grad_out, radius, scale):
+    """Gradients of lookup_forward: -> [d_f1 (B,H1,W1,C), [d_f2 level (B,H2_l,W2_l,C) ...]].  coords get none."""
+    import ctypes
+    f1, lvls = img1_features_l0, list(img2_features_lvls)
+    B, H1, W1, C, L, ptrs, h2, w2 = _lookup_args(f1, lvls, coords)
+    n = 2 * int(radius) + 1
+    _expect("grad_out", grad_out, (B, L * n * n, H1, W1), f1.device)
+    lib = _lib.load()
+    with torch.cuda.device(f1.device):
+        d_f1 = torch.empty_like(f1)
+        d_f2 = [torch.empty_like(t) for t in lvls]
+        dptrs = (ctypes.c_void_p * L)(*[t.data_ptr() for t in d_f2])
+        nws = lib.sepcorr_lookup_backward_workspace_bytes(h2, w2, B, H1, W1, C, L, int(radius))
+        ws = torch.empty(max(nws, 1), dtype=torch.uint8, device=f1.device)
+        _lib.check(lib.sepcorr_lookup_backward(f1.data_ptr(), ptrs, h2, w2, coords.data_ptr(), grad_out.data_ptr(),
+                                               d_f1.data_ptr(), dptrs, B, H1, W1, C, L, int(radius), float(scale),
+                                               ws.data_ptr(), nws, _stream()))
+    return [d_f1, d_f2]
 
 
 CONTRACT_FP32, CONTRACT_BF16X3 = 0, 1

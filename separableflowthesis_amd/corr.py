@@ -10,9 +10,9 @@ trilinearly upsampled (align_corners=True) to the level-0 displacement length.
 import torch
 import torch.nn.functional as F
 
-from . import MemorySaver
 from .functions import (AssembleVolumeFunction, AttentionWeightsFunction, ComputeMaxArgmaxAvgFunction,
-                        ComputeMaxAvgFunction, ComputeSelfCompressionFunction, SeparateLevelFunction)
+                        ComputeMaxAvgFunction, ComputeSelfCompressionFunction, LookupFunction,
+                        SeparateLevelFunction)
 
 
 def _is_reference_attention(m):
@@ -39,6 +39,7 @@ class AlternateCorrBlockSepflow:
         self.num_levels = num_levels
         self.radius = radius
         self.fmap1_l0 = fmap1
+        self._lookup_inputs = None
         self.pyramid = [fmap2]
         for _ in range(self.num_levels - 1):
             fmap2 = F.avg_pool2d(fmap2, 2, stride=2)
@@ -103,17 +104,13 @@ class AlternateCorrBlockSepflow:
 
         The reference stops here with NotImplementedError (core/corr.py:491-492) because the native part its
         draft calls (alt_cuda_corr.forward per level, core/corr.py:494-509) is not in its tree; the values are
-        those of the stored-volume block (CorrBlock.__call__, core/corr.py:193-248).  Forward only: the result
-        carries no autograd graph (the flow iterations that consume it detach coords anyway; gradients reach the
-        feature maps through separate()).
+        those of the stored-volume block (CorrBlock.__call__, core/corr.py:193-248).  Gradients reach fmap1 and
+        fmap2 (through the pooled pyramid); coords get none, as the flow iterations detach them.
         """
-        if not hasattr(self, "_lookup_inputs"):
-            with torch.no_grad():
-                f1 = self.fmap1_l0.permute(0, 2, 3, 1).contiguous().float()
-                f2s = [p.permute(0, 2, 3, 1).contiguous().float() for p in self.pyramid]
-            self._lookup_inputs = (f1, f2s)
+        if self._lookup_inputs is None:
+            # NHWC copies are made once per block and shared by all flow iterations (the draft redoes them per call)
+            f1 = self.fmap1_l0.permute(0, 2, 3, 1).contiguous().float()
+            self._lookup_inputs = (f1, [p.permute(0, 2, 3, 1).contiguous().float() for p in self.pyramid])
         f1, f2s = self._lookup_inputs
-        fdim = f1.shape[3]
-        with torch.no_grad():
-            return MemorySaver.lookup_forward(f1, f2s, coords.detach().contiguous().float(), self.radius,
-                                              1.0 / float(torch.sqrt(torch.tensor(fdim).float())))
+        scale = 1.0 / float(torch.sqrt(torch.tensor(f1.shape[3]).float()))
+        return LookupFunction.apply(coords.detach().contiguous().float(), self.radius, scale, f1, *f2s)

@@ -153,6 +153,215 @@ __global__ void __launch_bounds__(256) lookup_forward_kernel(const LookupArgs a)
     }
 }
 
+
+// ------------------------------------------------------------------------------------------------------------
+// Backward: gradients of the lookup w.r.t. both feature maps (coords get none: the flow iterations detach them,
+// core/sepflow.py:194).  With W[p,l][gy][gx] = scale * sum over the samples (a,c) and corners (dy,dx) that read grid
+// point (gy,gx) = (c+dy, a+dx) of weight(dy,dx) * grad_out[b,l,a,c,p]:
+//   d_f1[p]        = sum_l sum_g W[p,l][g] * f2_l[origin_p + g]           (gather, same reads as the forward)
+//   d_f2_l[q]      = sum_p W[p,l][q - origin_p] * f1[p]                   (scatter, done by the owner of q)
+// Three kernels: W and the window origins go to scratch once; d_f1 is one thread per (pixel, channel); d_f2 is
+// owned by tiles of fmap2 positions that scan the pixels for windows touching the tile, in ascending pixel order,
+// so no atomics are used and sums are run-to-run identical.  Coarse levels have few positions but as many
+// (pixel, grid point) pairs as level 0: their pixel range is cut into S_l slices, each slice writes a partial
+// result, and a last kernel adds the slices in order.
+// ------------------------------------------------------------------------------------------------------------
+
+constexpr int TQX = 16, TQY = 4, TQ = TQX * TQY;   // fmap2 positions per d_f2 workgroup
+constexpr int CB = 32;                              // candidates staged per round in the d_f2 kernel
+
+struct LookupBwdArgs {
+    const float *f1, *coords, *gout;
+    float *d_f1;
+    const float *f2[MAXL];
+    float *d_f2[MAXL];
+    float *part[MAXL];          // S[l] partial results of d_f2[l] (unused when S[l] == 1)
+    float *wg;                  // (B,L,H1*W1,G*G)
+    int *org;                   // (B,L,H1*W1,2): x then y of the window's first grid point
+    int H2[MAXL], W2[MAXL], S[MAXL], tile0[MAXL + 1];
+    int B, H1, W1, C, L, r;
+    float scale;
+};
+
+__global__ void __launch_bounds__(256) lookup_grid_grad_kernel(const LookupBwdArgs a) {
+    extern __shared__ float lds[];
+    const int r = a.r, n = 2 * r + 1, G = n + 1, GG = G * G, NN = n * n;
+    float *gtile = lds;                                   // [NN][TP+1]
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int lvl = blockIdx.z % a.L, b = blockIdx.z / a.L;
+    const int i = blockIdx.y, j0 = blockIdx.x * TP;
+    const size_t plane = (size_t)a.H1 * a.W1;
+    const int nj = min(TP, a.W1 - j0);
+    const float *g0 = a.gout + (((size_t)b * a.L + lvl) * NN) * plane + (size_t)i * a.W1 + j0;
+    for (int t = threadIdx.x; t < NN * TP; t += 256) {
+        const int c = t / TP, jj = t % TP;
+        gtile[c * (TP + 1) + jj] = jj < nj ? g0[(size_t)c * plane + jj] : 0.f;
+    }
+    __syncthreads();
+    const float lscale = 1.f / (float)(1 << lvl);
+    for (int jj = wave; jj < nj; jj += 4) {
+        const int j = j0 + jj;
+        const float *cp = a.coords + (size_t)b * 2 * plane + (size_t)i * a.W1 + j;
+        int x0, y0;
+        float fx, fy;
+        split_coord(cp[0] * lscale, x0, fx);
+        split_coord(cp[plane] * lscale, y0, fy);
+        const float w[2][2] = {{(1.f - fx) * (1.f - fy), fx * (1.f - fy)}, {(1.f - fx) * fy, fx * fy}};   // [dy][dx]
+        const size_t pl = ((size_t)b * a.L + lvl) * plane + (size_t)i * a.W1 + j;
+        for (int g = lane; g < GG; g += 64) {
+            const int gy = g / G, gx = g - gy * G;
+            float sum = 0.f;
+#pragma unroll
+            for (int dy = 0; dy < 2; ++dy)
+#pragma unroll
+                for (int dx = 0; dx < 2; ++dx) {
+                    const int c = gy - dy, ax = gx - dx;
+                    if (c >= 0 && c < n && ax >= 0 && ax < n) sum = fmaf(w[dy][dx], gtile[(ax * n + c) * (TP + 1) + jj], sum);
+                }
+            a.wg[pl * GG + g] = a.scale * sum;
+        }
+        if (lane == 0) {
+            a.org[pl * 2] = x0 - r;
+            a.org[pl * 2 + 1] = y0 - r;
+        }
+    }
+}
+
+// one workgroup per image-1 pixel, thread = channel (channels beyond 256 in further passes)
+__global__ void __launch_bounds__(256) lookup_df1_kernel(const LookupBwdArgs a) {
+    const int G = 2 * a.r + 2, GG = G * G, C = a.C;
+    const size_t plane = (size_t)a.H1 * a.W1;
+    const size_t p = blockIdx.x % plane;
+    const int b = blockIdx.x / plane;
+    for (int c = threadIdx.x; c < C; c += 256) {
+        float acc0 = 0.f, acc1 = 0.f;
+        for (int l = 0; l < a.L; ++l) {
+            const int H2 = a.H2[l], W2 = a.W2[l];
+            const size_t pl = ((size_t)b * a.L + l) * plane + p;
+            const int ox = a.org[pl * 2], oy = a.org[pl * 2 + 1];
+            const float *w = a.wg + pl * GG;
+            const float *f2 = a.f2[l] + (size_t)b * H2 * W2 * C + c;
+            const int gy0 = max(0, -oy), gy1 = min(G, H2 - oy);       // rows and columns of the window inside the level
+            const int gx0 = max(0, -ox), gx1 = min(G, W2 - ox);
+            for (int gy = gy0; gy < gy1; ++gy) {
+                const float *rowp = f2 + ((size_t)(oy + gy) * W2 + ox) * C;
+                const float *wr = w + gy * G;
+                int gx = gx0;
+                for (; gx + 1 < gx1; gx += 2) {
+                    acc0 = fmaf(wr[gx], rowp[(size_t)gx * C], acc0);
+                    acc1 = fmaf(wr[gx + 1], rowp[(size_t)(gx + 1) * C], acc1);
+                }
+                if (gx < gx1) acc0 = fmaf(wr[gx], rowp[(size_t)gx * C], acc0);
+            }
+        }
+        a.d_f1[((size_t)b * plane + p) * C + c] = acc0 + acc1;
+    }
+}
+
+// workgroup = (tile of TQY x TQX positions of one level, pixel slice), blockIdx.y = block of 256 channels, z = batch
+__global__ void __launch_bounds__(256) lookup_df2_kernel(const LookupBwdArgs a) {
+    __shared__ int list[256];
+    __shared__ int lorg[256][2];
+    __shared__ int wcount[4];
+    __shared__ __attribute__((aligned(16))) float wt[CB][TQ];
+    const int G = 2 * a.r + 2, GG = G * G, C = a.C;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    int l = 0;
+    while (l + 1 < a.L && (int)blockIdx.x >= a.tile0[l + 1]) ++l;
+    const int H2 = a.H2[l], W2 = a.W2[l], S = a.S[l];
+    const int tx_n = (W2 + TQX - 1) / TQX, ty_n = (H2 + TQY - 1) / TQY;
+    int t = blockIdx.x - a.tile0[l];
+    const int slice = t / (tx_n * ty_n);
+    t -= slice * tx_n * ty_n;
+    const int ty0 = (t / tx_n) * TQY, tx0 = (t % tx_n) * TQX;
+    const int b = blockIdx.z, c = blockIdx.y * 256 + tid;
+    const int P = a.H1 * a.W1;
+    const int per = (P + S - 1) / S, p_begin = slice * per, p_end = min(P, p_begin + per);
+    const size_t pl0 = ((size_t)b * a.L + l) * P;
+    const int *org = a.org + pl0 * 2;
+    const float *wg = a.wg + pl0 * GG;
+    const float *f1 = a.f1 + (size_t)b * P * C;
+
+    float acc[TQ];
+#pragma unroll
+    for (int q = 0; q < TQ; ++q) acc[q] = 0.f;
+
+    for (int pc = p_begin; pc < p_end; pc += 256) {
+        // pixels of this chunk whose window touches the tile, kept in ascending order
+        const int p = pc + tid;
+        int ox = 0, oy = 0;
+        bool hit = false;
+        if (p < p_end) {
+            ox = org[(size_t)p * 2];
+            oy = org[(size_t)p * 2 + 1];
+            hit = ox < tx0 + TQX && ox + G > tx0 && oy < ty0 + TQY && oy + G > ty0;
+        }
+        const unsigned long long m = __ballot(hit);
+        if (lane == 0) wcount[wave] = __popcll(m);
+        __syncthreads();
+        int base = 0, ncand = 0;
+        for (int w = 0; w < 4; ++w) {
+            if (w < wave) base += wcount[w];
+            ncand += wcount[w];
+        }
+        if (hit) {
+            const int pos = base + __popcll(m & ((1ull << lane) - 1ull));
+            list[pos] = p;
+            lorg[pos][0] = ox;
+            lorg[pos][1] = oy;
+        }
+        __syncthreads();
+        for (int cb = 0; cb < ncand; cb += CB) {
+            const int nc = min(CB, ncand - cb);
+            for (int e = tid; e < CB * TQ; e += 256) {
+                const int cn = e / TQ, q = e - cn * TQ;
+                float v = 0.f;
+                if (cn < nc) {
+                    const int gy = ty0 + q / TQX - lorg[cb + cn][1], gx = tx0 + q % TQX - lorg[cb + cn][0];
+                    if (gy >= 0 && gy < G && gx >= 0 && gx < G) v = wg[(size_t)list[cb + cn] * GG + gy * G + gx];
+                }
+                wt[cn][q] = v;
+            }
+            __syncthreads();
+            if (c < C) {
+                for (int cn = 0; cn < nc; ++cn) {
+                    const float f = f1[(size_t)list[cb + cn] * C + c];
+                    const float4 *w4 = reinterpret_cast<const float4 *>(wt[cn]);
+#pragma unroll
+                    for (int q4 = 0; q4 < TQ / 4; ++q4) {
+                        const float4 w = w4[q4];
+                        acc[q4 * 4 + 0] = fmaf(w.x, f, acc[q4 * 4 + 0]);
+                        acc[q4 * 4 + 1] = fmaf(w.y, f, acc[q4 * 4 + 1]);
+                        acc[q4 * 4 + 2] = fmaf(w.z, f, acc[q4 * 4 + 2]);
+                        acc[q4 * 4 + 3] = fmaf(w.w, f, acc[q4 * 4 + 3]);
+                    }
+                }
+            }
+            __syncthreads();
+        }
+    }
+    if (c < C) {
+        const size_t lvl_elems = (size_t)a.B * H2 * W2 * C;
+        float *dst = (S == 1 ? a.d_f2[l] : a.part[l] + (size_t)slice * lvl_elems) + (size_t)b * H2 * W2 * C + c;
+#pragma unroll
+        for (int q = 0; q < TQ; ++q) {
+            const int y = ty0 + q / TQX, x = tx0 + q % TQX;
+            if (y < H2 && x < W2) dst[((size_t)y * W2 + x) * C] = acc[q];
+        }
+    }
+}
+
+// d_f2[l] = sum over the S[l] slices, in slice order
+__global__ void __launch_bounds__(256) lookup_df2_reduce_kernel(const LookupBwdArgs a, int l) {
+    const size_t n = (size_t)a.B * a.H2[l] * a.W2[l] * a.C;
+    const int S = a.S[l];
+    for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < n; e += (size_t)gridDim.x * 256) {
+        float s = 0.f;
+        for (int k = 0; k < S; ++k) s += a.part[l][(size_t)k * n + e];
+        a.d_f2[l][e] = s;
+    }
+}
+
 int bad(const char *msg) { return sepcorr_set_error(SEPCORR_EINVAL, msg); }
 
 template <int M, int RT, bool VEC>
@@ -171,6 +380,43 @@ void launch_c(const LookupArgs &a, dim3 grid, size_t lds, hipStream_t s) {
     else if (C <= 256) launch<4, RT, true>(a, grid, lds, s);
     else if (C <= 512) launch<8, RT, true>(a, grid, lds, s);
     else launch<16, RT, true>(a, grid, lds, s);
+}
+
+
+// slices of the pixel range for level l: as many as level 0 has more positions than level l, at most 64
+int level_slices(const int *h2, const int *w2, int l) {
+    const long n0 = (long)h2[0] * w2[0], nl = (long)h2[l] * w2[l];
+    long s = nl > 0 ? n0 / nl : 1;
+    return (int)(s < 1 ? 1 : s > 64 ? 64 : s);
+}
+
+int check_common(const void *f1, const float *const *f2_levels, const int *h2, const int *w2, const void *coords,
+                 int B, int H1, int W1, int C, int L, int radius) {
+    if (!f1 || !f2_levels || !h2 || !w2 || !coords) return bad("sepcorr: lookup: NULL pointer");
+    if (B < 1 || H1 < 1 || W1 < 1 || C < 1) return bad("sepcorr: lookup: sizes must be positive");
+    if (C > 1024) return bad("sepcorr: lookup: C above 1024 is not supported");
+    if (L < 1 || L > MAXL) return bad("sepcorr: lookup: 1 to 8 pyramid levels are supported");
+    if (radius < 1 || radius > MAXR) return bad("sepcorr: lookup: radius must be 1..8");
+    const int n = 2 * radius + 1;
+    if ((double)B * L * n * n * H1 * W1 > 2147483647.0 || (double)B * H1 * W1 * C > 2147483647.0)
+        return bad("sepcorr: a tensor would have 2^31 or more elements");
+    if ((long)B * L > 65535 || H1 > 65535) return bad("sepcorr: lookup: B*L and H1 must be below 65536");
+    for (int l = 0; l < L; ++l) {
+        if (!f2_levels[l]) return bad("sepcorr: lookup: NULL level pointer");
+        if (h2[l] < 1 || w2[l] < 1) return bad("sepcorr: lookup: level sizes must be positive");
+        if ((double)B * h2[l] * w2[l] * C > 2147483647.0) return bad("sepcorr: a tensor would have 2^31 or more elements");
+    }
+    return SEPCORR_OK;
+}
+
+size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+int launch_error(const char *what) {
+    const hipError_t e = hipGetLastError();
+    if (e == hipSuccess) return SEPCORR_OK;
+    char msg[160];
+    snprintf(msg, sizeof(msg), "sepcorr: %s: %s", what, hipGetErrorString(e));
+    return sepcorr_set_error(SEPCORR_ELAUNCH, msg);
 }
 
 }  // namespace
@@ -209,6 +455,71 @@ int sepcorr_lookup_forward(const float *f1, const float *const *f2_levels, const
         snprintf(msg, sizeof(msg), "sepcorr: lookup kernel: %s", hipGetErrorString(e));
         return sepcorr_set_error(SEPCORR_ELAUNCH, msg);
     }
+    return SEPCORR_OK;
+}
+
+size_t sepcorr_lookup_backward_workspace_bytes(const int *h2, const int *w2, int B, int H1, int W1, int C, int L,
+                                               int radius) {
+    if (!h2 || !w2 || B < 1 || H1 < 1 || W1 < 1 || C < 1 || L < 1 || L > MAXL || radius < 1 || radius > MAXR) return 0;
+    const size_t G = 2 * (size_t)radius + 2, pix = (size_t)B * L * H1 * W1;
+    size_t n = align256(pix * G * G * sizeof(float)) + align256(pix * 2 * sizeof(int));
+    for (int l = 0; l < L; ++l) {
+        if (h2[l] < 1 || w2[l] < 1) return 0;
+        const int S = level_slices(h2, w2, l);
+        if (S > 1) n += align256((size_t)S * B * h2[l] * w2[l] * C * sizeof(float));
+    }
+    return n;
+}
+
+int sepcorr_lookup_backward(const float *f1, const float *const *f2_levels, const int *h2, const int *w2,
+                            const float *coords, const float *grad_out, float *d_f1, float *const *d_f2_levels,
+                            int B, int H1, int W1, int C, int L, int radius, float scale,
+                            void *workspace, size_t workspace_bytes, void *stream) {
+    const int rc = check_common(f1, f2_levels, h2, w2, coords, B, H1, W1, C, L, radius);
+    if (rc != SEPCORR_OK) return rc;
+    if (!grad_out || !d_f1 || !d_f2_levels) return bad("sepcorr: lookup: NULL pointer");
+    const size_t need = sepcorr_lookup_backward_workspace_bytes(h2, w2, B, H1, W1, C, L, radius);
+    if (!workspace || workspace_bytes < need)
+        return sepcorr_set_error(SEPCORR_EWORKSPACE, "sepcorr: lookup backward: workspace missing or too small");
+    if ((uintptr_t)workspace % 256) return bad("sepcorr: lookup backward: workspace must be 256-byte aligned");
+    const int n = 2 * radius + 1, G = n + 1;
+    const size_t pix = (size_t)B * L * H1 * W1;
+    LookupBwdArgs a = {};
+    a.f1 = f1; a.coords = coords; a.gout = grad_out; a.d_f1 = d_f1;
+    char *ws = static_cast<char *>(workspace);
+    a.wg = reinterpret_cast<float *>(ws); ws += align256(pix * G * G * sizeof(float));
+    a.org = reinterpret_cast<int *>(ws); ws += align256(pix * 2 * sizeof(int));
+    long tiles = 0;
+    for (int l = 0; l < L; ++l) {
+        if (!d_f2_levels[l]) return bad("sepcorr: lookup: NULL level pointer");
+        a.f2[l] = f2_levels[l]; a.d_f2[l] = d_f2_levels[l]; a.H2[l] = h2[l]; a.W2[l] = w2[l];
+        a.S[l] = level_slices(h2, w2, l);
+        if (a.S[l] > 1) {
+            a.part[l] = reinterpret_cast<float *>(ws);
+            ws += align256((size_t)a.S[l] * B * h2[l] * w2[l] * C * sizeof(float));
+        }
+        a.tile0[l] = (int)tiles;
+        tiles += (long)((w2[l] + TQX - 1) / TQX) * ((h2[l] + TQY - 1) / TQY) * a.S[l];
+        if (tiles > 2147483647L) return bad("sepcorr: lookup backward: too many tiles");
+    }
+    a.tile0[L] = (int)tiles;
+    a.B = B; a.H1 = H1; a.W1 = W1; a.C = C; a.L = L; a.r = radius; a.scale = scale;
+    if (B > 65535) return bad("sepcorr: lookup backward: B must be below 65536");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t lds = (size_t)n * n * (TP + 1) * sizeof(float);
+    hipLaunchKernelGGL(lookup_grid_grad_kernel, dim3((W1 + TP - 1) / TP, H1, B * L), dim3(256), lds, s, a);
+    if (int e = launch_error("lookup grid-gradient kernel")) return e;
+    hipLaunchKernelGGL(lookup_df1_kernel, dim3((unsigned)((size_t)B * H1 * W1)), dim3(256), 0, s, a);
+    if (int e = launch_error("lookup d_f1 kernel")) return e;
+    hipLaunchKernelGGL(lookup_df2_kernel, dim3((unsigned)tiles, (C + 255) / 256, B), dim3(256), 0, s, a);
+    if (int e = launch_error("lookup d_f2 kernel")) return e;
+    for (int l = 0; l < L; ++l)
+        if (a.S[l] > 1) {
+            const size_t ne = (size_t)B * h2[l] * w2[l] * C;
+            const unsigned blocks = (unsigned)((ne + 255) / 256 < 4096 ? (ne + 255) / 256 : 4096);
+            hipLaunchKernelGGL(lookup_df2_reduce_kernel, dim3(blocks), dim3(256), 0, s, a, l);
+            if (int e = launch_error("lookup d_f2 reduction")) return e;
+        }
     return SEPCORR_OK;
 }
 

@@ -156,3 +156,30 @@ class AssembleVolumeFunction(Function):
     @staticmethod
     def backward(ctx, grad):
         return (None,) + tuple(MemorySaver.assemble_backward(grad.contiguous(), ctx.shapes))
+
+
+class LookupFunction(Function):
+    """corr_fn(coords) of the block that never stores the 4D volume: windowed bilinear lookup in every pyramid level.
+
+    apply(coords, radius, scale, f1, *f2_levels): f1 (B,H1,W1,C) and the pooled fmap2 levels (B,H2_l,W2_l,C) in NHWC,
+    coords (B,2,H1,W1) -> (B, levels*(2*radius+1)^2, H1, W1).  Values as CorrBlock.__call__ (core/corr.py:193-248);
+    the reference's own draft of this call raises NotImplementedError (core/corr.py:491-509).  Gradients go to f1 and
+    to every level; coords get none (the flow iterations detach them, core/sepflow.py:194).
+    """
+
+    @staticmethod
+    def forward(ctx, coords, radius, scale, f1, *f2_levels):
+        _contig(coords, f1, *f2_levels)
+        with torch.cuda.device_of(f1):
+            out = MemorySaver.lookup_forward(f1, f2_levels, coords, radius, scale)
+        ctx.save_for_backward(coords, f1, *f2_levels)
+        ctx.radius, ctx.scale = radius, scale
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        coords, f1, *f2_levels = ctx.saved_tensors
+        grad_out = grad_out.contiguous()
+        with torch.cuda.device_of(grad_out):
+            d_f1, d_f2 = MemorySaver.lookup_backward(f1, f2_levels, coords, grad_out, ctx.radius, ctx.scale)
+        return (None, None, None, d_f1, *d_f2)

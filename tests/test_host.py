@@ -22,7 +22,7 @@ def header_symbols():
 
 def test_library_exports_every_declared_symbol():
     names = header_symbols()
-    assert len(names) == 17
+    assert len(names) == 20
     lib = ctypes.CDLL(_lib.LIB_PATH)
     for n in names:
         assert hasattr(lib, n), f"libsepcorr.so does not export {n}"
@@ -110,7 +110,9 @@ def test_corr_block_guards_and_pyramid():
     assert [tuple(p.shape[2:]) for p in blk.pyramid] == [(11, 13), (5, 6), (2, 3), (1, 1)]
     assert blk.max_avg_function.__name__ == "ComputeMaxArgmaxAvgFunction"
     assert AlternateCorrBlockSepflow(fmap, fmap, None).max_avg_function.__name__ == "ComputeMaxAvgFunction"
-    with pytest.raises(NotImplementedError):
+    # the lookup is native as well (the reference raises NotImplementedError here, core/corr.py:491-492):
+    # CPU tensors are refused, there is no fallback
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
         blk(torch.zeros(1, 2, 11, 13))
 
 

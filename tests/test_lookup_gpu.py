@@ -85,3 +85,57 @@ def test_lookup_special_coordinates_and_errors(device):
         MemorySaver.lookup_forward(f1, [f2[..., :32].contiguous()], coords.to(device), 4, 1.0)
     with pytest.raises(RuntimeError):
         MemorySaver.lookup_forward(f1.cpu(), [f2], coords.to(device), 4, 1.0)
+
+
+@pytest.mark.parametrize("B,C,H,W,levels,r,spread", [
+    (2, 256, 16, 24, 3, 4, 3.0),
+    (1, 256, 28, 64, 4, 4, 6.0),      # half the benchmark shape: sliced pixel ranges on the coarse levels
+    (1, 64, 11, 37, 2, 4, 3.0),       # ragged tiles of fmap2 positions
+    (1, 100, 9, 20, 2, 3, 25.0),      # most windows outside, C not a multiple of 64
+    (1, 37, 8, 20, 2, 1, 2.0),
+    (1, 300, 8, 16, 2, 2, 2.0),       # two channel blocks in the d_f2 kernel
+])
+def test_lookup_gradients_match_autograd_through_the_oracle(device, B, C, H, W, levels, r, spread):
+    from separableflowthesis_amd import AlternateCorrBlockSepflow
+    g = torch.Generator().manual_seed(4321 + C + W)
+    fmap1 = torch.randn(B, C, H, W, generator=g)
+    fmap2 = torch.randn(B, C, H, W, generator=g)
+    coords = _coords(B, H, W, g, spread)
+    up = torch.randn(B, levels * (2 * r + 1) ** 2, H, W, generator=g)
+    r1 = fmap1.double().requires_grad_()
+    r2 = fmap2.double().requires_grad_()
+    (O.lookup_direct(r1, r2, coords.double(), levels, r) * up.double()).sum().backward()
+    g1 = fmap1.to(device).requires_grad_()
+    g2 = fmap2.to(device).requires_grad_()
+    blk = AlternateCorrBlockSepflow(g1, g2, None, num_levels=levels, radius=r)
+    out = blk(coords.to(device))
+    out.backward(up.to(device), retain_graph=True)       # the block's NHWC copies are shared by later calls
+    assert_close(g1.grad, r1.grad, "d_fmap1", scale_atol=True)
+    assert_close(g2.grad, r2.grad, "d_fmap2", scale_atol=True)
+    # a second call on the same block (next flow iteration) accumulates into the same leaves
+    blk(coords.to(device)).backward(up.to(device))
+    assert_close(g1.grad, 2 * r1.grad, "d_fmap1 accumulated", scale_atol=True)
+
+
+def test_lookup_backward_is_deterministic_and_checks_its_workspace(device):
+    import ctypes
+    from separableflowthesis_amd import MemorySaver, _lib
+    B, C, H, W, r = 1, 64, 12, 20, 4
+    g = torch.Generator().manual_seed(8)
+    f1 = torch.randn(B, H, W, C, generator=g).to(device)
+    f2s = [torch.randn(B, H >> l, W >> l, C, generator=g).to(device) for l in range(3)]
+    coords = _coords(B, H, W, g, 3.0).to(device)
+    up = torch.randn(B, 3 * 81, H, W, generator=g).to(device)
+    a = MemorySaver.lookup_backward(f1, f2s, coords, up, r, 0.125)
+    b = MemorySaver.lookup_backward(f1, f2s, coords, up, r, 0.125)
+    assert torch.equal(a[0], b[0]) and all(torch.equal(x, y) for x, y in zip(a[1], b[1]))
+    lib = _lib.load()
+    ptrs = (ctypes.c_void_p * 3)(*[t.data_ptr() for t in f2s])
+    h2 = (ctypes.c_int * 3)(*[t.shape[1] for t in f2s])
+    w2 = (ctypes.c_int * 3)(*[t.shape[2] for t in f2s])
+    need = lib.sepcorr_lookup_backward_workspace_bytes(h2, w2, B, H, W, C, 3, r)
+    assert need > 0
+    ws = torch.empty(need, dtype=torch.uint8, device=device)
+    rc = lib.sepcorr_lookup_backward(f1.data_ptr(), ptrs, h2, w2, coords.data_ptr(), up.data_ptr(), a[0].data_ptr(),
+                                     ptrs, B, H, W, C, 3, r, 0.125, ws.data_ptr(), need - 1, None)
+    assert rc == -3 and b"workspace" in lib.sepcorr_last_error()

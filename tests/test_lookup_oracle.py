@@ -113,3 +113,26 @@ def test_a_level_of_size_one_is_undefined_in_the_stored_volume_path_only():
     b = O.lookup_direct(fmap1, fmap2, coords, 2, 1)
     assert bool(torch.isnan(a[:, 9:]).any()) and bool(torch.isfinite(b).all())
     assert float((a[:, :9] - b[:, :9]).abs().max()) < 1e-12
+
+
+def test_gradients_of_both_formulations_agree():
+    # autograd through grid_sample on the stored pyramid against autograd through the gather formulation
+    B, C, H, W, levels, r = 1, 6, 8, 12, 2, 2
+    g = torch.Generator().manual_seed(21)
+    fmap1 = torch.randn(B, C, H, W, generator=g, dtype=torch.float64)
+    fmap2 = torch.randn(B, C, H, W, generator=g, dtype=torch.float64)
+    coords = _grid(B, H, W) + torch.randn(B, 2, H, W, generator=g, dtype=torch.float64) * 2
+    up = torch.randn(B, levels * (2 * r + 1) ** 2, H, W, generator=g, dtype=torch.float64)
+    grads = []
+    for fn in (lambda a, b: O.CorrBlock4D(a, b, num_levels=levels).lookup(coords, radius=r),
+               lambda a, b: O.lookup_direct(a, b, coords, levels, r)):
+        a = fmap1.clone().requires_grad_()
+        b = fmap2.clone().requires_grad_()
+        (fn(a, b) * up).sum().backward()
+        grads.append((a.grad, b.grad))
+    assert float((grads[0][0] - grads[1][0]).abs().max()) < 1e-11
+    assert float((grads[0][1] - grads[1][1]).abs().max()) < 1e-11
+    # the lookup is bilinear in (fmap1, fmap2): <up, out> = <d_fmap1, fmap1> = <d_fmap2, fmap2>
+    val = float((O.lookup_direct(fmap1, fmap2, coords, levels, r) * up).sum())
+    assert abs(float((grads[1][0] * fmap1).sum()) - val) < 1e-9 * max(1.0, abs(val))
+    assert abs(float((grads[1][1] * fmap2).sum()) - val) < 1e-9 * max(1.0, abs(val))
