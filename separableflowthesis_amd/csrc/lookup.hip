@@ -403,6 +403,95 @@ __global__ void __launch_bounds__(256) lookup_df1_kernel(const LookupBwdArgs a) 
     }
 }
 
+// d_f1 for C a multiple of 4: a wave takes NPX consecutive pixels and, level by level, walks the bounding box of their
+// windows once.  Lane = 4 channels (float4 fetch of a whole fmap2 row per wave and box point); the NPX weights of a box
+// point (zero outside a pixel's own window or outside the level) sit in a per-wave LDS table and arrive as one
+// broadcast read.  Scattered windows (box above BOXMAX points) are walked pixel by pixel with the same code.
+__global__ void __launch_bounds__(256) lookup_df1_group_kernel(const LookupBwdArgs a) {
+    __shared__ __attribute__((aligned(16))) float wtab[4][BOXMAX][NPX];
+    const int G = 2 * a.r + 2, GG = G * G, C = a.C;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int b = blockIdx.z, i = blockIdx.y, j0 = blockIdx.x * TPG + wave * NPX;
+    if (j0 >= a.W1) return;                                 // whole wave; the kernel has no workgroup barrier
+    const size_t plane = (size_t)a.H1 * a.W1;
+    float (*wt)[NPX] = wtab[wave];
+    for (int c0 = 0; c0 < C; c0 += 256) {
+        const int ch = c0 + lane * 4;
+        const int chl = ch < C ? ch : 0;                    // idle lanes re-read channel 0 and store nothing
+        float4 acc[NPX];
+#pragma unroll
+        for (int e = 0; e < NPX; ++e) acc[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int l = 0; l < a.L; ++l) {
+            const int H2 = a.H2[l], W2 = a.W2[l];
+            const float *f2 = a.f2[l] + (size_t)b * H2 * W2 * C + chl;
+            int ox[NPX], oy[NPX];
+            size_t pl[NPX];
+            int bx0 = 0, bx1 = 0, by0 = 0, by1 = 0;
+#pragma unroll
+            for (int e = 0; e < NPX; ++e) {
+                const int j = min(j0 + e, a.W1 - 1);
+                pl[e] = ((size_t)b * a.L + l) * plane + (size_t)i * a.W1 + j;
+                ox[e] = a.org[pl[e] * 2];
+                oy[e] = a.org[pl[e] * 2 + 1];
+                bx0 = e ? min(bx0, ox[e]) : ox[e];
+                bx1 = e ? max(bx1, ox[e]) : ox[e];
+                by0 = e ? min(by0, oy[e]) : oy[e];
+                by1 = e ? max(by1, oy[e]) : oy[e];
+            }
+            const long BWl = (long)bx1 - bx0 + G, BHl = (long)by1 - by0 + G;
+            const bool joint = BWl * BHl <= BOXMAX;
+            for (int sub = 0; sub < (joint ? 1 : NPX); ++sub) {
+                int qx0 = bx0, qy0 = by0, BW = (int)(joint ? BWl : G), BH = (int)(joint ? BHl : G);
+                if (!joint) {
+#pragma unroll
+                    for (int e = 0; e < NPX; ++e)
+                        if (e == sub) { qx0 = ox[e]; qy0 = oy[e]; }
+                }
+                const int npts = BW * BH;
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                for (int bp = lane; bp < npts; bp += 64) {
+                    const int by = bp / BW, bx = bp - by * BW;
+                    const int yy = qy0 + by, xx = qx0 + bx;
+                    const bool inside = yy >= 0 && yy < H2 && xx >= 0 && xx < W2;
+                    float w[NPX];
+#pragma unroll
+                    for (int e = 0; e < NPX; ++e) {
+                        const int gy = yy - oy[e], gx = xx - ox[e];
+                        const bool use = inside && (joint || e == sub) && j0 + e < a.W1 && gy >= 0 && gy < G && gx >= 0 && gx < G;
+                        w[e] = use ? a.wg[pl[e] * GG + gy * G + gx] : 0.f;
+                    }
+                    *reinterpret_cast<float4 *>(wt[bp]) = make_float4(w[0], w[1], w[2], w[3]);
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                int bx = 0, by = 0;
+#pragma unroll 2
+                for (int bp = 0; bp < npts; ++bp) {
+                    const int yc = min(max(qy0 + by, 0), H2 - 1), xc = min(max(qx0 + bx, 0), W2 - 1);
+                    const float4 v = *reinterpret_cast<const float4 *>(f2 + ((size_t)yc * W2 + xc) * C);
+                    const float4 w = *reinterpret_cast<const float4 *>(wt[bp]);
+                    const float ws[NPX] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+                    for (int e = 0; e < NPX; ++e) {
+                        acc[e].x = fmaf(ws[e], v.x, acc[e].x);
+                        acc[e].y = fmaf(ws[e], v.y, acc[e].y);
+                        acc[e].z = fmaf(ws[e], v.z, acc[e].z);
+                        acc[e].w = fmaf(ws[e], v.w, acc[e].w);
+                    }
+                    if (++bx == BW) { bx = 0; ++by; }
+                }
+            }
+        }
+        if (ch < C) {
+#pragma unroll
+            for (int e = 0; e < NPX; ++e)
+                if (j0 + e < a.W1)
+                    *reinterpret_cast<float4 *>(a.d_f1 + (((size_t)b * a.H1 + i) * a.W1 + j0 + e) * C + ch) = acc[e];
+        }
+    }
+}
+
 // workgroup = (tile of TQY x TQX positions of one level, pixel slice), blockIdx.y = block of 256 channels, z = batch
 __global__ void __launch_bounds__(256) lookup_df2_kernel(const LookupBwdArgs a) {
     __shared__ int list[256];
@@ -662,7 +751,10 @@ int sepcorr_lookup_backward(const float *f1, const float *const *f2_levels, cons
     const size_t lds = (size_t)n * n * (TP + 1) * sizeof(float);
     hipLaunchKernelGGL(lookup_grid_grad_kernel, dim3((W1 + TP - 1) / TP, H1, B * L), dim3(256), lds, s, a);
     if (int e = launch_error("lookup grid-gradient kernel")) return e;
-    hipLaunchKernelGGL(lookup_df1_kernel, dim3((unsigned)((size_t)B * H1 * W1)), dim3(256), 0, s, a);
+    bool vec = C % 4 == 0 && (uintptr_t)d_f1 % 16 == 0;
+    for (int l = 0; l < L; ++l) vec = vec && (uintptr_t)a.f2[l] % 16 == 0;
+    if (vec) hipLaunchKernelGGL(lookup_df1_group_kernel, dim3((W1 + TPG - 1) / TPG, H1, B), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL(lookup_df1_kernel, dim3((unsigned)((size_t)B * H1 * W1)), dim3(256), 0, s, a);
     if (int e = launch_error("lookup d_f1 kernel")) return e;
     hipLaunchKernelGGL(lookup_df2_kernel, dim3((unsigned)tiles, (C + 255) / 256, B), dim3(256), 0, s, a);
     if (int e = launch_error("lookup d_f2 kernel")) return e;
