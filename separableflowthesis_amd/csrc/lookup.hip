@@ -312,8 +312,9 @@ __global__ void __launch_bounds__(256) lookup_forward_group_kernel(const LookupA
 // result, and a last kernel adds the slices in order.
 // ------------------------------------------------------------------------------------------------------------
 
-constexpr int TQX = 16, TQY = 4, TQ = TQX * TQY;   // fmap2 positions per d_f2 workgroup
-constexpr int CB = 32;                              // candidates staged per round in the d_f2 kernel
+constexpr int TQX = 8, TQY = 8;                     // fmap2 positions per d_f2 wave (one per lane)
+constexpr int NCH = 64;                             // channels per d_f2 wave
+static_assert(TQX * TQY == 64, "one tile position per lane");
 
 struct LookupBwdArgs {
     const float *f1, *coords, *gout;
@@ -492,14 +493,17 @@ __global__ void __launch_bounds__(256) lookup_df1_group_kernel(const LookupBwdAr
     }
 }
 
-// workgroup = (tile of TQY x TQX positions of one level, pixel slice), blockIdx.y = block of 256 channels, z = batch
-__global__ void __launch_bounds__(256) lookup_df2_kernel(const LookupBwdArgs a) {
-    __shared__ int list[256];
-    __shared__ int lorg[256][2];
-    __shared__ int wcount[4];
-    __shared__ __attribute__((aligned(16))) float wt[CB][TQ];
+// One wave = (tile of TQY x TQX positions of one level, slice of the pixel range, block of NCH channels).  For the
+// tile, d_f2[pos, ch] = sum over pixels of W[pos, pixel] * f1[pixel, ch] is a small matrix product whose inner index
+// runs over the pixels whose window touches the tile.  The wave scans its pixels 64 at a time (origins stay in the
+// lanes' registers), takes the touching ones in ascending order, two per v_mfma_f32_32x32x2_f32: operand A = the two
+// pixels' window entries at the tile's positions (zero outside the window), operand B = their f1 channels, fetched as
+// contiguous runs.  Eight pixels are fetched before their MFMAs are issued.  No LDS, no barrier, no atomics.
+typedef float lk_v16f __attribute__((ext_vector_type(16)));
+
+__global__ void __launch_bounds__(64) lookup_df2_kernel(const LookupBwdArgs a) {
     const int G = 2 * a.r + 2, GG = G * G, C = a.C;
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int lane = threadIdx.x, half = lane >> 5, l32 = lane & 31;
     int l = 0;
     while (l + 1 < a.L && (int)blockIdx.x >= a.tile0[l + 1]) ++l;
     const int H2 = a.H2[l], W2 = a.W2[l], S = a.S[l];
@@ -508,21 +512,28 @@ __global__ void __launch_bounds__(256) lookup_df2_kernel(const LookupBwdArgs a) 
     const int slice = t / (tx_n * ty_n);
     t -= slice * tx_n * ty_n;
     const int ty0 = (t / tx_n) * TQY, tx0 = (t % tx_n) * TQX;
-    const int b = blockIdx.z, c = blockIdx.y * 256 + tid;
+    const int b = blockIdx.z, c0 = blockIdx.y * NCH;
     const int P = a.H1 * a.W1;
     const int per = (P + S - 1) / S, p_begin = slice * per, p_end = min(P, p_begin + per);
     const size_t pl0 = ((size_t)b * a.L + l) * P;
-    const int *org = a.org + pl0 * 2;
-    const float *wg = a.wg + pl0 * GG;
-    const float *f1 = a.f1 + (size_t)b * P * C;
+    const int *__restrict__ org = a.org + pl0 * 2;
+    const float *__restrict__ wg = a.wg + pl0 * GG;
+    const float *__restrict__ f1 = a.f1 + (size_t)b * P * C;
+    // operand A rows of this lane: tile positions l32 and 32 + l32
+    const int qy0 = ty0 + l32 / TQX, qy1 = qy0 + 32 / TQX, qx = tx0 + l32 % TQX;
+    // operand B columns of this lane: channels c0 + l32 and c0 + 32 + l32
+    const int cA = c0 + l32, cB = c0 + 32 + l32;
 
-    float acc[TQ];
+    lk_v16f acc[2][2];
 #pragma unroll
-    for (int q = 0; q < TQ; ++q) acc[q] = 0.f;
+    for (int ph = 0; ph < 2; ++ph)
+#pragma unroll
+        for (int ch = 0; ch < 2; ++ch)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[ph][ch][v] = 0.f;
 
-    for (int pc = p_begin; pc < p_end; pc += 256) {
-        // pixels of this chunk whose window touches the tile, kept in ascending order
-        const int p = pc + tid;
+    for (int pc = p_begin; pc < p_end; pc += 64) {
+        const int p = pc + lane;
         int ox = 0, oy = 0;
         bool hit = false;
         if (p < p_end) {
@@ -530,59 +541,55 @@ __global__ void __launch_bounds__(256) lookup_df2_kernel(const LookupBwdArgs a) 
             oy = org[(size_t)p * 2 + 1];
             hit = ox < tx0 + TQX && ox + G > tx0 && oy < ty0 + TQY && oy + G > ty0;
         }
-        const unsigned long long m = __ballot(hit);
-        if (lane == 0) wcount[wave] = __popcll(m);
-        __syncthreads();
-        int base = 0, ncand = 0;
-        for (int w = 0; w < 4; ++w) {
-            if (w < wave) base += wcount[w];
-            ncand += wcount[w];
-        }
-        if (hit) {
-            const int pos = base + __popcll(m & ((1ull << lane) - 1ull));
-            list[pos] = p;
-            lorg[pos][0] = ox;
-            lorg[pos][1] = oy;
-        }
-        __syncthreads();
-        for (int cb = 0; cb < ncand; cb += CB) {
-            const int nc = min(CB, ncand - cb);
-            for (int e = tid; e < CB * TQ; e += 256) {
-                const int cn = e / TQ, q = e - cn * TQ;
-                float v = 0.f;
-                if (cn < nc) {
-                    const int gy = ty0 + q / TQX - lorg[cb + cn][1], gx = tx0 + q % TQX - lorg[cb + cn][0];
-                    if (gy >= 0 && gy < G && gx >= 0 && gx < G) v = wg[(size_t)list[cb + cn] * GG + gy * G + gx];
-                }
-                wt[cn][q] = v;
-            }
-            __syncthreads();
-            if (c < C) {
-                for (int cn = 0; cn < nc; ++cn) {
-                    const float f = f1[(size_t)list[cb + cn] * C + c];
-                    const float4 *w4 = reinterpret_cast<const float4 *>(wt[cn]);
+        unsigned long long m = __ballot(hit);
+        while (m) {
+            float wa[4][2], fb[4][2];
+            bool any[4];
 #pragma unroll
-                    for (int q4 = 0; q4 < TQ / 4; ++q4) {
-                        const float4 w = w4[q4];
-                        acc[q4 * 4 + 0] = fmaf(w.x, f, acc[q4 * 4 + 0]);
-                        acc[q4 * 4 + 1] = fmaf(w.y, f, acc[q4 * 4 + 1]);
-                        acc[q4 * 4 + 2] = fmaf(w.z, f, acc[q4 * 4 + 2]);
-                        acc[q4 * 4 + 3] = fmaf(w.w, f, acc[q4 * 4 + 3]);
-                    }
-                }
+            for (int pr = 0; pr < 4; ++pr) {
+                any[pr] = m != 0;                              // wave-uniform
+                const int cn0 = m ? __builtin_ctzll(m) : 0;
+                m &= m - 1;
+                const bool two = m != 0;
+                const int cn1 = two ? __builtin_ctzll(m) : cn0;
+                m &= m - 1;
+                const bool mine = any[pr] && (half == 0 || two);
+                const int cn = half ? cn1 : cn0;
+                const int oxc = __shfl(ox, cn), oyc = __shfl(oy, cn);
+                const size_t pp = (size_t)(pc + cn);
+                const int gx = qx - oxc, gya = qy0 - oyc, gyb = qy1 - oyc;
+                const bool inx = mine && gx >= 0 && gx < G;
+                wa[pr][0] = inx && gya >= 0 && gya < G ? wg[pp * GG + gya * G + gx] : 0.f;
+                wa[pr][1] = inx && gyb >= 0 && gyb < G ? wg[pp * GG + gyb * G + gx] : 0.f;
+                fb[pr][0] = mine && cA < C ? f1[pp * C + cA] : 0.f;
+                fb[pr][1] = mine && cB < C ? f1[pp * C + cB] : 0.f;
             }
-            __syncthreads();
+#pragma unroll
+            for (int pr = 0; pr < 4; ++pr)
+                if (any[pr]) {
+#pragma unroll
+                    for (int ph = 0; ph < 2; ++ph)
+#pragma unroll
+                        for (int ch = 0; ch < 2; ++ch)
+                            acc[ph][ch] = __builtin_amdgcn_mfma_f32_32x32x2f32(wa[pr][ph], fb[pr][ch], acc[ph][ch], 0, 0, 0);
+                }
         }
     }
-    if (c < C) {
-        const size_t lvl_elems = (size_t)a.B * H2 * W2 * C;
-        float *dst = (S == 1 ? a.d_f2[l] : a.part[l] + (size_t)slice * lvl_elems) + (size_t)b * H2 * W2 * C + c;
+    // register v of lane (half, l32) holds tile position ph*32 + 8*(v/4) + 4*half + v%4, channel c0 + ch*32 + l32
+    const size_t lvl_elems = (size_t)a.B * H2 * W2 * C;
+    float *dst = (S == 1 ? a.d_f2[l] : a.part[l] + (size_t)slice * lvl_elems) + (size_t)b * H2 * W2 * C;
 #pragma unroll
-        for (int q = 0; q < TQ; ++q) {
-            const int y = ty0 + q / TQX, x = tx0 + q % TQX;
-            if (y < H2 && x < W2) dst[((size_t)y * W2 + x) * C] = acc[q];
+    for (int ph = 0; ph < 2; ++ph)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int pos = ph * 32 + 8 * (v / 4) + 4 * half + v % 4;
+            const int y = ty0 + pos / TQX, x = tx0 + pos % TQX;
+            if (y < H2 && x < W2) {
+                float *d = dst + ((size_t)y * W2 + x) * C;
+                if (cA < C) d[cA] = acc[ph][0][v];
+                if (cB < C) d[cB] = acc[ph][1][v];
+            }
         }
-    }
 }
 
 // d_f2[l] = sum over the S[l] slices, in slice order
@@ -756,7 +763,7 @@ int sepcorr_lookup_backward(const float *f1, const float *const *f2_levels, cons
     if (vec) hipLaunchKernelGGL(lookup_df1_group_kernel, dim3((W1 + TPG - 1) / TPG, H1, B), dim3(256), 0, s, a);
     else hipLaunchKernelGGL(lookup_df1_kernel, dim3((unsigned)((size_t)B * H1 * W1)), dim3(256), 0, s, a);
     if (int e = launch_error("lookup d_f1 kernel")) return e;
-    hipLaunchKernelGGL(lookup_df2_kernel, dim3((unsigned)tiles, (C + 255) / 256, B), dim3(256), 0, s, a);
+    hipLaunchKernelGGL(lookup_df2_kernel, dim3((unsigned)tiles, (C + NCH - 1) / NCH, B), dim3(64), 0, s, a);
     if (int e = launch_error("lookup d_f2 kernel")) return e;
     for (int l = 0; l < L; ++l)
         if (a.S[l] > 1) {
