@@ -158,16 +158,17 @@ def lookup_level(B, H, W, C, torch, dev, reps=20):
     fwd = timed(lambda: MemorySaver.lookup_forward(f1, f2s, coords, 4, scale))
     bwd = timed(lambda: MemorySaver.lookup_backward(f1, f2s, coords, up, 4, scale))
     pts = B * H * W * 4 * 100                       # (pixel, level, grid point) pairs: one C-long dot product each
-    alg = (f1.numel() + sum(t.numel() for t in f2s) + coords.numel() + up.numel()) * 4
+    alg = (f1.numel() + sum(t.numel() for t in f2s) + coords.numel() + up.numel()) * 4   # up has the output's size
     return {
         "forward_ms": round(fwd, 4), "backward_ms": round(bwd, 4),
-        "forward_gathered_gb_s": round(pts * C * 4 / fwd / 1e6, 1),
+        "forward_window_gb_s": round(pts * C * 4 / fwd / 1e6, 1),
         "forward_gflop_s": round(pts * C * 2 / fwd / 1e6, 1),
         "forward_algorithmic_mib": round(alg / 2 ** 20, 1),
         "forward_hbm_gb_s": round(alg / fwd / 1e6, 1),
         "what": f"sepcorr_lookup_forward / sepcorr_lookup_backward, B={B}, C={C}, {H}x{W}, 4 levels, radius 4; "
-                "gathered = bytes of fmap2 rows fetched through the vector cache (2 flop per 4 bytes: bound by that "
-                "cache, peak 256 CU x 64 B/clk x 2.4 GHz = 39.3 TB/s); algorithmic = f1 + pyramid + coords + out once",
+                "window = bytes of the fmap2 rows under all windows (one C-long dot product each, 2 flop per 4 bytes; "
+                "the kernel fetches a row once for four neighbouring pixels, so this may exceed the vector cache's "
+                "256 CU x 64 B/clk x 2.4 GHz = 39.3 TB/s); algorithmic = f1 + pyramid + coords + out once",
     }
 
 

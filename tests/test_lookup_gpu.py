@@ -139,3 +139,20 @@ def test_lookup_backward_is_deterministic_and_checks_its_workspace(device):
     rc = lib.sepcorr_lookup_backward(f1.data_ptr(), ptrs, h2, w2, coords.data_ptr(), up.data_ptr(), a[0].data_ptr(),
                                      ptrs, B, H, W, C, 3, r, 0.125, ws.data_ptr(), need - 1, None)
     assert rc == -3 and b"workspace" in lib.sepcorr_last_error()
+
+
+def test_lookup_matches_the_golden_vectors(device):
+    from separableflowthesis_amd import AlternateCorrBlockSepflow
+    from tests.test_lookup_oracle import _golden
+    n = 0
+    for name, z in _golden():
+        n += 1
+        g1 = z["in_fmap1"].to(device).requires_grad_()
+        g2 = z["in_fmap2"].to(device).requires_grad_()
+        blk = AlternateCorrBlockSepflow(g1, g2, None, num_levels=int(z["in_levels"]), radius=int(z["in_radius"]))
+        out = blk(z["in_coords"].to(device))
+        out.backward(z["in_up"].to(device))
+        assert_close(out, z["out_lookup"], name + " lookup")
+        assert_close(g1.grad, z["out_d_fmap1"], name + " d_fmap1", scale_atol=True)
+        assert_close(g2.grad, z["out_d_fmap2"], name + " d_fmap2", scale_atol=True)
+    assert n == 2

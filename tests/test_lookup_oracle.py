@@ -136,3 +136,28 @@ def test_gradients_of_both_formulations_agree():
     val = float((O.lookup_direct(fmap1, fmap2, coords, levels, r) * up).sum())
     assert abs(float((grads[1][0] * fmap1).sum()) - val) < 1e-9 * max(1.0, abs(val))
     assert abs(float((grads[1][1] * fmap2).sum()) - val) < 1e-9 * max(1.0, abs(val))
+
+
+def _golden():
+    import glob
+    import os
+    import numpy as np
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "lookup")
+    for f in sorted(glob.glob(os.path.join(here, "*.npz"))):
+        z = np.load(f, allow_pickle=False)
+        yield os.path.basename(f), {k: torch.from_numpy(z[k]) for k in z.files}
+
+
+def test_oracle_reproduces_the_lookup_golden_vectors():
+    names = []
+    for name, z in _golden():
+        names.append(name)
+        levels, r = int(z["in_levels"]), int(z["in_radius"])
+        a = z["in_fmap1"].double().requires_grad_()
+        b = z["in_fmap2"].double().requires_grad_()
+        out = O.lookup_direct(a, b, z["in_coords"].double(), levels, r)      # the formulation the files were not made with
+        (out * z["in_up"].double()).sum().backward()
+        assert torch.allclose(out.detach().float(), z["out_lookup"], rtol=1e-6, atol=1e-6), name
+        assert torch.allclose(a.grad.float(), z["out_d_fmap1"], rtol=1e-6, atol=1e-5), name
+        assert torch.allclose(b.grad.float(), z["out_d_fmap2"], rtol=1e-6, atol=1e-5), name
+    assert len(names) == 2
