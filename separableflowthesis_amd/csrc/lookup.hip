@@ -667,21 +667,13 @@ extern "C" {
 int sepcorr_lookup_forward(const float *f1, const float *const *f2_levels, const int *h2, const int *w2,
                            const float *coords, float *out, int B, int H1, int W1, int C, int L, int radius,
                            float scale, void *stream) {
-    if (!f1 || !f2_levels || !h2 || !w2 || !coords || !out) return bad("sepcorr: lookup: NULL pointer");
-    if (B < 1 || H1 < 1 || W1 < 1 || C < 1) return bad("sepcorr: lookup: sizes must be positive");
-    if (C > 1024) return bad("sepcorr: lookup: C above 1024 is not supported");
-    if (L < 1 || L > MAXL) return bad("sepcorr: lookup: 1 to 8 pyramid levels are supported");
-    if (radius < 1 || radius > MAXR) return bad("sepcorr: lookup: radius must be 1..8");
+    const int rc = check_common(f1, f2_levels, h2, w2, coords, B, H1, W1, C, L, radius);
+    if (rc != SEPCORR_OK) return rc;
+    if (!out) return bad("sepcorr: lookup: NULL pointer");
     const int n = 2 * radius + 1;
-    if ((double)B * L * n * n * H1 * W1 > 2147483647.0 || (double)B * H1 * W1 * C > 2147483647.0)
-        return bad("sepcorr: a tensor would have 2^31 or more elements");
-    if ((long)B * L > 65535 || H1 > 65535) return bad("sepcorr: lookup: B*L and H1 must be below 65536");
     LookupArgs a = {};
     a.f1 = f1; a.coords = coords; a.out = out;
     for (int l = 0; l < L; ++l) {
-        if (!f2_levels[l]) return bad("sepcorr: lookup: NULL level pointer");
-        if (h2[l] < 1 || w2[l] < 1) return bad("sepcorr: lookup: level sizes must be positive");
-        if ((double)B * h2[l] * w2[l] * C > 2147483647.0) return bad("sepcorr: a tensor would have 2^31 or more elements");
         a.f2[l] = f2_levels[l]; a.H2[l] = h2[l]; a.W2[l] = w2[l];
     }
     a.B = B; a.H1 = H1; a.W1 = W1; a.C = C; a.L = L; a.r = radius; a.scale = scale;
@@ -698,13 +690,7 @@ int sepcorr_lookup_forward(const float *f1, const float *const *f2_levels, const
         else hipLaunchKernelGGL(lookup_forward_group_kernel<4>, ggrid, dim3(256), glds, s, a);
     } else if (radius == 4) launch_c<4>(a, grid, lds, s);
     else launch_c<0>(a, grid, lds, s);
-    const hipError_t e = hipGetLastError();
-    if (e != hipSuccess) {
-        char msg[160];
-        snprintf(msg, sizeof(msg), "sepcorr: lookup kernel: %s", hipGetErrorString(e));
-        return sepcorr_set_error(SEPCORR_ELAUNCH, msg);
-    }
-    return SEPCORR_OK;
+    return launch_error("lookup kernel");
 }
 
 size_t sepcorr_lookup_backward_workspace_bytes(const int *h2, const int *w2, int B, int H1, int W1, int C, int L,

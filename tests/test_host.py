@@ -61,6 +61,27 @@ def test_argument_checks_precede_any_launch():
     assert b"workspace" in lib.sepcorr_last_error()
 
 
+def test_lookup_argument_checks_precede_any_launch():
+    lib = _lib.load()
+    one = ctypes.c_void_p(256)
+    lv = (ctypes.c_void_p * 2)(256, 256)
+    hw = (ctypes.c_int * 2)(4, 2)
+    f = lib.sepcorr_lookup_forward
+    assert f(None, lv, hw, hw, one, one, 1, 4, 4, 8, 2, 4, 1.0, None) == -1 and b"NULL" in lib.sepcorr_last_error()
+    assert f(one, lv, hw, hw, one, one, 1, 4, 4, 8, 2, 9, 1.0, None) == -1 and b"radius" in lib.sepcorr_last_error()
+    assert f(one, lv, hw, hw, one, one, 1, 4, 4, 8, 9, 4, 1.0, None) == -1 and b"levels" in lib.sepcorr_last_error()
+    assert f(one, lv, hw, hw, one, one, 1, 4, 4, 1025, 2, 4, 1.0, None) == -1
+    assert f(one, (ctypes.c_void_p * 2)(256, None), hw, hw, one, one, 1, 4, 4, 8, 2, 4, 1.0, None) == -1
+    assert f(one, lv, (ctypes.c_int * 2)(4, 0), hw, one, one, 1, 4, 4, 8, 2, 4, 1.0, None) == -1
+    n = lib.sepcorr_lookup_backward_workspace_bytes(hw, hw, 1, 4, 4, 8, 2, 4)
+    assert n > 0 and n % 256 == 0
+    assert lib.sepcorr_lookup_backward_workspace_bytes(hw, hw, 1, 4, 4, 8, 2, 0) == 0
+    b = lib.sepcorr_lookup_backward
+    assert b(one, lv, hw, hw, one, one, one, lv, 1, 4, 4, 8, 2, 4, 1.0, None, 0, None) == -3
+    assert b(one, lv, hw, hw, one, one, one, lv, 1, 4, 4, 8, 2, 4, 1.0, ctypes.c_void_p(257), n, None) == -1
+    assert b"aligned" in lib.sepcorr_last_error()
+
+
 def test_cpu_tensors_are_refused_like_check_cuda():
     from separableflowthesis_amd import MemorySaver
     f = torch.randn(1, 2, 2, 4)
