@@ -312,9 +312,9 @@ __global__ void __launch_bounds__(256) lookup_forward_group_kernel(const LookupA
 // result, and a last kernel adds the slices in order.
 // ------------------------------------------------------------------------------------------------------------
 
-constexpr int TQX = 8, TQY = 8;                     // fmap2 positions per d_f2 wave (one per lane)
-constexpr int NCH = 64;                             // channels per d_f2 wave
-static_assert(TQX * TQY == 64, "one tile position per lane");
+constexpr int TQX = 8, TQY = 4;                     // fmap2 positions per d_f2 wave: the 32 rows of one MFMA tile
+constexpr int NCH = 128;                            // channels per d_f2 wave
+static_assert(TQX * TQY == 32, "one tile position per MFMA row");
 
 struct LookupBwdArgs {
     const float *f1, *coords, *gout;
@@ -502,6 +502,7 @@ __global__ void __launch_bounds__(256) lookup_df1_group_kernel(const LookupBwdAr
 typedef float lk_v16f __attribute__((ext_vector_type(16)));
 
 __global__ void __launch_bounds__(64) lookup_df2_kernel(const LookupBwdArgs a) {
+    constexpr int NB = NCH / 32;                               // operand-B registers (32 channels each) per pixel pair
     const int G = 2 * a.r + 2, GG = G * G, C = a.C;
     const int lane = threadIdx.x, half = lane >> 5, l32 = lane & 31;
     int l = 0;
@@ -519,31 +520,26 @@ __global__ void __launch_bounds__(64) lookup_df2_kernel(const LookupBwdArgs a) {
     const int *__restrict__ org = a.org + pl0 * 2;
     const float *__restrict__ wg = a.wg + pl0 * GG;
     const float *__restrict__ f1 = a.f1 + (size_t)b * P * C;
-    // operand A rows of this lane: tile positions l32 and 32 + l32
-    const int qy0 = ty0 + l32 / TQX, qy1 = qy0 + 32 / TQX, qx = tx0 + l32 % TQX;
-    // operand B columns of this lane: channels c0 + l32 and c0 + 32 + l32
-    const int cA = c0 + l32, cB = c0 + 32 + l32;
+    // operand A row of this lane: tile position l32; operand B columns: channels c0 + 32*cb + l32
+    const int qy = ty0 + l32 / TQX, qx = tx0 + l32 % TQX;
 
-    lk_v16f acc[2][2];
+    lk_v16f acc[NB];
 #pragma unroll
-    for (int ph = 0; ph < 2; ++ph)
+    for (int cb = 0; cb < NB; ++cb)
 #pragma unroll
-        for (int ch = 0; ch < 2; ++ch)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[ph][ch][v] = 0.f;
+        for (int v = 0; v < 16; ++v) acc[cb][v] = 0.f;
 
+    // origins of the next 64 pixels are fetched while the current ones are worked on
+    int2 nxt = make_int2(0, 0);
+    if (p_begin + lane < p_end) nxt = *reinterpret_cast<const int2 *>(org + (size_t)(p_begin + lane) * 2);
     for (int pc = p_begin; pc < p_end; pc += 64) {
         const int p = pc + lane;
-        int ox = 0, oy = 0;
-        bool hit = false;
-        if (p < p_end) {
-            ox = org[(size_t)p * 2];
-            oy = org[(size_t)p * 2 + 1];
-            hit = ox < tx0 + TQX && ox + G > tx0 && oy < ty0 + TQY && oy + G > ty0;
-        }
+        const int ox = nxt.x, oy = nxt.y;
+        if (p + 64 < p_end) nxt = *reinterpret_cast<const int2 *>(org + (size_t)(p + 64) * 2);
+        const bool hit = p < p_end && ox < tx0 + TQX && ox + G > tx0 && oy < ty0 + TQY && oy + G > ty0;
         unsigned long long m = __ballot(hit);
         while (m) {
-            float wa[4][2], fb[4][2];
+            float wa[4], fb[4][NB];
             bool any[4];
 #pragma unroll
             for (int pr = 0; pr < 4; ++pr) {
@@ -557,39 +553,39 @@ __global__ void __launch_bounds__(64) lookup_df2_kernel(const LookupBwdArgs a) {
                 const int cn = half ? cn1 : cn0;
                 const int oxc = __shfl(ox, cn), oyc = __shfl(oy, cn);
                 const size_t pp = (size_t)(pc + cn);
-                const int gx = qx - oxc, gya = qy0 - oyc, gyb = qy1 - oyc;
-                const bool inx = mine && gx >= 0 && gx < G;
-                wa[pr][0] = inx && gya >= 0 && gya < G ? wg[pp * GG + gya * G + gx] : 0.f;
-                wa[pr][1] = inx && gyb >= 0 && gyb < G ? wg[pp * GG + gyb * G + gx] : 0.f;
-                fb[pr][0] = mine && cA < C ? f1[pp * C + cA] : 0.f;
-                fb[pr][1] = mine && cB < C ? f1[pp * C + cB] : 0.f;
+                const int gx = qx - oxc, gy = qy - oyc;
+                wa[pr] = mine && gx >= 0 && gx < G && gy >= 0 && gy < G ? wg[pp * GG + gy * G + gx] : 0.f;
+#pragma unroll
+                for (int cb = 0; cb < NB; ++cb) {
+                    const int c = c0 + 32 * cb + l32;
+                    fb[pr][cb] = mine && c < C ? f1[pp * C + c] : 0.f;
+                }
             }
 #pragma unroll
             for (int pr = 0; pr < 4; ++pr)
                 if (any[pr]) {
 #pragma unroll
-                    for (int ph = 0; ph < 2; ++ph)
-#pragma unroll
-                        for (int ch = 0; ch < 2; ++ch)
-                            acc[ph][ch] = __builtin_amdgcn_mfma_f32_32x32x2f32(wa[pr][ph], fb[pr][ch], acc[ph][ch], 0, 0, 0);
+                    for (int cb = 0; cb < NB; ++cb)
+                        acc[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(wa[pr], fb[pr][cb], acc[cb], 0, 0, 0);
                 }
         }
     }
-    // register v of lane (half, l32) holds tile position ph*32 + 8*(v/4) + 4*half + v%4, channel c0 + ch*32 + l32
+    // register v of lane (half, l32) holds tile position 8*(v/4) + 4*half + v%4, channel c0 + 32*cb + l32
     const size_t lvl_elems = (size_t)a.B * H2 * W2 * C;
     float *dst = (S == 1 ? a.d_f2[l] : a.part[l] + (size_t)slice * lvl_elems) + (size_t)b * H2 * W2 * C;
 #pragma unroll
-    for (int ph = 0; ph < 2; ++ph)
+    for (int v = 0; v < 16; ++v) {
+        const int pos = 8 * (v / 4) + 4 * half + v % 4;
+        const int y = ty0 + pos / TQX, x = tx0 + pos % TQX;
+        if (y < H2 && x < W2) {
+            float *d = dst + ((size_t)y * W2 + x) * C;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int pos = ph * 32 + 8 * (v / 4) + 4 * half + v % 4;
-            const int y = ty0 + pos / TQX, x = tx0 + pos % TQX;
-            if (y < H2 && x < W2) {
-                float *d = dst + ((size_t)y * W2 + x) * C;
-                if (cA < C) d[cA] = acc[ph][0][v];
-                if (cB < C) d[cB] = acc[ph][1][v];
+            for (int cb = 0; cb < NB; ++cb) {
+                const int c = c0 + 32 * cb + l32;
+                if (c < C) d[c] = acc[cb][v];
             }
         }
+    }
 }
 
 // d_f2[l] = sum over the S[l] slices, in slice order
