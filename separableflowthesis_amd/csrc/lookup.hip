@@ -588,14 +588,30 @@ __global__ void __launch_bounds__(64) lookup_df2_kernel(const LookupBwdArgs a) {
     }
 }
 
-// d_f2[l] = sum over the S[l] slices, in slice order
-__global__ void __launch_bounds__(256) lookup_df2_reduce_kernel(const LookupBwdArgs a, int l) {
-    const size_t n = (size_t)a.B * a.H2[l] * a.W2[l] * a.C;
+// d_f2[l] = sum over the S[l] slices, in slice order; blockIdx.y = level
+__global__ void __launch_bounds__(256) lookup_df2_reduce_kernel(const LookupBwdArgs a) {
+    const int l = blockIdx.y;
     const int S = a.S[l];
-    for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < n; e += (size_t)gridDim.x * 256) {
-        float s = 0.f;
-        for (int k = 0; k < S; ++k) s += a.part[l][(size_t)k * n + e];
-        a.d_f2[l][e] = s;
+    if (S == 1) return;
+    const size_t n = (size_t)a.B * a.H2[l] * a.W2[l] * a.C;
+    const float *__restrict__ part = a.part[l];
+    float *__restrict__ dst = a.d_f2[l];
+    const size_t stride = (size_t)gridDim.x * 256;
+    if (n % 4 == 0 && (uintptr_t)dst % 16 == 0) {
+        for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < n / 4; e += stride) {
+            float4 s = reinterpret_cast<const float4 *>(part)[e];
+            for (int k = 1; k < S; ++k) {
+                const float4 v = reinterpret_cast<const float4 *>(part + (size_t)k * n)[e];
+                s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+            }
+            reinterpret_cast<float4 *>(dst)[e] = s;
+        }
+    } else {
+        for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < n; e += stride) {
+            float s = part[e];
+            for (int k = 1; k < S; ++k) s += part[(size_t)k * n + e];
+            dst[e] = s;
+        }
     }
 }
 
@@ -620,11 +636,13 @@ void launch_c(const LookupArgs &a, dim3 grid, size_t lds, hipStream_t s) {
 }
 
 
-// slices of the pixel range for level l: as many as level 0 has more positions than level l, at most 64
+// slices of the pixel range for level l: twice as many as level 0 has more positions than level l, at most 128
+// (measured: with one slice per unit of positions the waves run too long for the launch to balance)
 int level_slices(const int *h2, const int *w2, int l) {
     const long n0 = (long)h2[0] * w2[0], nl = (long)h2[l] * w2[l];
-    long s = nl > 0 ? n0 / nl : 1;
-    return (int)(s < 1 ? 1 : s > 64 ? 64 : s);
+    long s = nl > 0 ? 2 * n0 / nl : 2;
+    if (s < 2) s = 2;
+    return (int)(s > 128 ? 128 : s);
 }
 
 int check_common(const void *f1, const float *const *f2_levels, const int *h2, const int *w2, const void *coords,
@@ -747,13 +765,8 @@ int sepcorr_lookup_backward(const float *f1, const float *const *f2_levels, cons
     if (int e = launch_error("lookup d_f1 kernel")) return e;
     hipLaunchKernelGGL(lookup_df2_kernel, dim3((unsigned)tiles, (C + NCH - 1) / NCH, B), dim3(64), 0, s, a);
     if (int e = launch_error("lookup d_f2 kernel")) return e;
-    for (int l = 0; l < L; ++l)
-        if (a.S[l] > 1) {
-            const size_t ne = (size_t)B * h2[l] * w2[l] * C;
-            const unsigned blocks = (unsigned)((ne + 255) / 256 < 4096 ? (ne + 255) / 256 : 4096);
-            hipLaunchKernelGGL(lookup_df2_reduce_kernel, dim3(blocks), dim3(256), 0, s, a, l);
-            if (int e = launch_error("lookup d_f2 reduction")) return e;
-        }
+    hipLaunchKernelGGL(lookup_df2_reduce_kernel, dim3(1024, L), dim3(256), 0, s, a);
+    if (int e = launch_error("lookup d_f2 reduction")) return e;
     return SEPCORR_OK;
 }
 
