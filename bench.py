@@ -3,7 +3,7 @@
 
 A step is one pass of the hot path over one synthetic batch, called through the C ABI with every
 input already resident in HBM: max/argmax/avg forward, attention-compression forward, compression
-backward, max/avg backward (the default workload, BASELINE config 4: B=2, C=256, 55x128, K'=4).
+backward, max/avg backward (the default workload, benchmark configuration 4: B=2, C=256, 55x128, K'=4).
 Prints ONE JSON line.  `value` is algorithmic TFLOP/s: (contraction passes x 2*B*N1*N2*C) / time,
 with passes = 7 for forward+backward with attention; epilogue flops are not counted.
 """

@@ -240,6 +240,26 @@ int sepcorr_lookup_backward(const float *f1, const float *const *f2_levels, cons
                             int B, int H1, int W1, int C, int L, int radius, float scale,
                             void *workspace, size_t workspace_bytes, void *stream);
 
+/*
+ * Lookup in one of the two separated 3D volumes: the reference's CorrBlock1D (core/corr.py:513-624), per volume.
+ *   corr    (B,dim,L,H1,W1)   a volume in the layout AlternateCorrBlockSepflow.separate returns (corr1: L = W2, corr2: L = H2)
+ *   coords  (B,2,H1,W1)       coord_channel 0 (x) addresses corr1, 1 (y) corr2 (core/corr.py:573, 598)
+ *   out     (B, levels*dim*n, H1, W1), n = 2*radius+1, fully overwritten:
+ *           out[b, l*dim*n + d*n + k, i, j] = linear sample of level l of corr[b,d,:,i,j] at coords/2^l + k - radius,
+ *           level l = l-fold average pooling by two along L (core/corr.py:546-550), zero outside the level
+ *           (grid_sample, align_corners=True, core/corr.py:553-560).  The pyramid is formed on the fly, not stored.
+ *   clamp_unit != 0 clamps the sampling positions to [-1, 1] first, as the reference does for its first volume
+ *           (core/corr.py:585); pass 1 for corr1 and 0 for corr2 to reproduce it.
+ * Limits: 8 levels, radius <= 16, L >> (levels-1) >= 1.
+ */
+int sepcorr_lookup1d_forward(const float *corr, const float *coords, float *out, int B, int dim, int L, int H1, int W1,
+                             int coord_channel, int clamp_unit, int levels, int radius, void *stream);
+
+/* Adjoint of the above with respect to corr: d_corr (B,dim,L,H1,W1), fully overwritten, from grad_out.  Every
+ * (b,d,i,j) column is owned by one thread: no atomics, fixed summation order.  coords get no gradient here. */
+int sepcorr_lookup1d_backward(const float *coords, const float *grad_out, float *d_corr, int B, int dim, int L, int H1,
+                              int W1, int coord_channel, int clamp_unit, int levels, int radius, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -367,6 +367,84 @@ def lookup_direct(fmap1, fmap2, coords, num_levels=4, radius=4):
     return out.permute(0, 3, 1, 2).contiguous()
 
 
+class CorrBlock1D:
+    """Restatement of the reference's CorrBlock1D (core/corr.py:513-624): lookup in the two 3D volumes.
+
+    corr1 (B,dim,W2,H1,W1) and corr2 (B,dim,H2,H1,W1) are pooled by two along the displacement axis into a pyramid
+    (avg_pool2d [1,2], core/corr.py:546-550); every level is sampled with grid_sample (bilinear, align_corners=True,
+    zero padding) at coords/2^l + dx, dx = -r..r.  coords channel 0 addresses corr1, channel 1 corr2.  For corr1 the
+    reference clamps the *pixel* positions to [-1, 1] before sampling (core/corr.py:585); that is kept.
+    Output channel = level*dim*(2r+1) + d*(2r+1) + k.
+    """
+
+    def __init__(self, corr1, corr2, num_levels=4, radius=4):
+        self.num_levels, self.radius = num_levels, radius
+        self.pyr = []
+        for corr in (corr1, corr2):
+            c = corr.permute(0, 3, 4, 1, 2)
+            b, h1, w1, dim, L = c.shape
+            c = c.reshape(b * h1 * w1, dim, 1, L)
+            levels = [c]
+            for _ in range(num_levels):
+                c = F.avg_pool2d(c, [1, 2], stride=[1, 2])
+                levels.append(c)
+            self.pyr.append(levels)
+
+    def __call__(self, coords):
+        r = self.radius
+        B, _, h1, w1 = coords.shape
+        outs = []
+        for which in (0, 1):
+            x = coords[:, which:which + 1].permute(0, 2, 3, 1).reshape(B * h1 * w1, 1, 1, 1)
+            per_level = []
+            for i in range(self.num_levels):
+                corr = self.pyr[which][i]
+                W = corr.shape[-1]
+                dx = torch.linspace(-r, r, 2 * r + 1, dtype=coords.dtype).view(1, 1, 2 * r + 1, 1)
+                x0 = dx + x / 2 ** i
+                y0 = torch.zeros_like(x0)
+                if which == 0:
+                    x0 = torch.clamp(x0, -1, 1)                       # core/corr.py:585
+                grid = torch.cat([2 * x0 / (W - 1) - 1, y0], dim=-1)   # core/corr.py:555-560: y is not normalised
+                smp = F.grid_sample(corr, grid, mode='bilinear', padding_mode='zeros', align_corners=True)
+                per_level.append(smp.view(B, h1, w1, -1))
+            outs.append(torch.cat(per_level, dim=-1).permute(0, 3, 1, 2).contiguous())
+        return outs[0], outs[1]
+
+
+def lookup1d_direct(corr, x, num_levels=4, radius=4, clamp_unit=False):
+    """One volume of the above from its definition: explicit pair means for the pyramid, explicit linear weights.
+
+    corr (B,dim,L,H1,W1), x (B,H1,W1) -> (B, levels*dim*(2r+1), H1, W1).  Independent of CorrBlock1D in everything
+    but the definition (no avg_pool2d, no grid_sample).
+    """
+    B, dim, L, h1, w1 = corr.shape
+    r = radius
+    outs = []
+    lvl = corr
+    for i in range(num_levels):
+        if i:
+            n = lvl.shape[2] // 2
+            lvl = 0.5 * (lvl[:, :, 0:2 * n:2] + lvl[:, :, 1:2 * n:2])
+        Li = lvl.shape[2]
+        vals = []
+        for k in range(2 * r + 1):
+            pos = x / 2 ** i + (k - r)
+            if clamp_unit:
+                pos = pos.clamp(-1, 1)
+            p0 = torch.floor(pos)
+            f = (pos - p0)[:, None]
+            acc = torch.zeros(B, dim, h1, w1, dtype=corr.dtype)
+            for d, wgt in ((0, 1 - f), (1, f)):
+                idx = (p0 + d).long()
+                ok = ((idx >= 0) & (idx < Li))[:, None]
+                g = torch.gather(lvl, 2, idx.clamp(0, Li - 1)[:, None, None].expand(B, dim, 1, h1, w1))[:, :, 0]
+                acc = acc + torch.where(ok, wgt * g, torch.zeros_like(g))
+            vals.append(acc)
+        outs.append(torch.stack(vals, dim=2).reshape(B, dim * (2 * r + 1), h1, w1))
+    return torch.cat(outs, dim=1)
+
+
 def make_inputs(B, H, W, C, seed=1234, dtype=torch.float32):
     """Seeded N(0,1) NCHW fmaps and the NHWC op inputs derived as core/corr.py:419-422."""
     g = torch.Generator().manual_seed(seed)

@@ -345,6 +345,42 @@ def lookup_backward(img1_features_l0, img2_features_lvls, coords, grad_out, radi
     return [d_f1, d_f2]
 
 
+def _lookup1d_dims(corr, coords):
+    _check("corr", corr, ndim=5)
+    B, dim, L, H1, W1 = corr.shape
+    _expect("coords", coords, (B, 2, H1, W1), corr.device)
+    return B, dim, L, H1, W1
+
+
+def lookup1d_forward(corr, coords, coord_channel, clamp_unit, num_levels, radius):
+    """Lookup in one separated volume corr (B,dim,L,H1,W1) at coords[:, coord_channel]:
+    -> (B, num_levels*dim*(2*radius+1), H1, W1), what CorrBlock1D.__call__ computes per volume (core/corr.py:565-624)."""
+    B, dim, L, H1, W1 = _lookup1d_dims(corr, coords)
+    n = 2 * int(radius) + 1
+    lib = _lib.load()
+    with torch.cuda.device(corr.device):
+        out = torch.empty((B, int(num_levels) * dim * n, H1, W1), dtype=corr.dtype, device=corr.device)
+        _lib.check(lib.sepcorr_lookup1d_forward(corr.data_ptr(), coords.data_ptr(), out.data_ptr(), B, dim, L, H1, W1,
+                                                int(coord_channel), int(bool(clamp_unit)), int(num_levels), int(radius),
+                                                _stream()))
+    return out
+
+
+def lookup1d_backward(coords, grad_out, shape, coord_channel, clamp_unit, num_levels, radius):
+    """Gradient of lookup1d_forward with respect to corr (of the given shape (B,dim,L,H1,W1))."""
+    B, dim, L, H1, W1 = shape
+    n = 2 * int(radius) + 1
+    _expect("coords", coords, (B, 2, H1, W1), grad_out.device)
+    _expect("grad_out", grad_out, (B, int(num_levels) * dim * n, H1, W1), coords.device)
+    lib = _lib.load()
+    with torch.cuda.device(grad_out.device):
+        d_corr = torch.empty(shape, dtype=grad_out.dtype, device=grad_out.device)
+        _lib.check(lib.sepcorr_lookup1d_backward(coords.data_ptr(), grad_out.data_ptr(), d_corr.data_ptr(), B, dim, L,
+                                                 H1, W1, int(coord_channel), int(bool(clamp_unit)), int(num_levels),
+                                                 int(radius), _stream()))
+    return d_corr
+
+
 CONTRACT_FP32, CONTRACT_BF16X3 = 0, 1
 
 

@@ -5,9 +5,9 @@ module wrapper and the caller class, backed by hand-written gfx950 kernels in li
 """
 from .functions import ComputeMaxArgmaxAvgFunction, ComputeMaxAvgFunction, ComputeSelfCompressionFunction
 from .modules import ComputeMaxAvgModule
-from .corr import AlternateCorrBlockSepflow
+from .corr import AlternateCorrBlockSepflow, CorrBlock1D
 
 __all__ = [
     "ComputeMaxAvgFunction", "ComputeMaxArgmaxAvgFunction", "ComputeSelfCompressionFunction",
-    "ComputeMaxAvgModule", "AlternateCorrBlockSepflow",
+    "ComputeMaxAvgModule", "AlternateCorrBlockSepflow", "CorrBlock1D",
 ]

@@ -34,6 +34,8 @@ SIGNATURES = {
     "sepcorr_lookup_forward": (_I, [_P] * 6 + [_I] * 6 + [ctypes.c_float, _P]),
     "sepcorr_lookup_backward_workspace_bytes": (_SZ, [_P] * 2 + [_I] * 6),
     "sepcorr_lookup_backward": (_I, [_P] * 8 + [_I] * 6 + [ctypes.c_float, _P, _SZ, _P]),
+    "sepcorr_lookup1d_forward": (_I, [_P] * 3 + [_I] * 9 + [_P]),
+    "sepcorr_lookup1d_backward": (_I, [_P] * 3 + [_I] * 9 + [_P]),
 }
 
 _lib = None

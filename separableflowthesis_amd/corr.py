@@ -11,8 +11,8 @@ import torch
 import torch.nn.functional as F
 
 from .functions import (AssembleVolumeFunction, AttentionWeightsFunction, ComputeMaxArgmaxAvgFunction,
-                        ComputeMaxAvgFunction, ComputeSelfCompressionFunction, LookupFunction,
-                        SeparateLevelFunction)
+                        ComputeMaxAvgFunction, ComputeSelfCompressionFunction, Lookup1DFunction,
+                        LookupFunction, SeparateLevelFunction)
 
 
 def _is_reference_attention(m):
@@ -114,3 +114,31 @@ class AlternateCorrBlockSepflow:
         f1, f2s = self._lookup_inputs
         scale = 1.0 / float(torch.sqrt(torch.tensor(f1.shape[3]).float()))
         return LookupFunction.apply(coords.detach().contiguous().float(), self.radius, scale, f1, *f2s)
+
+
+class CorrBlock1D:
+    """Lookup in the two separated 3D volumes: the reference's CorrBlock1D (core/corr.py:513-624).
+
+    corr1 (B,dim,W2,H1,W1) and corr2 (B,dim,H2,H1,W1) as separate() (or the cost aggregation after it) returns them.
+    `__call__(coords)` -> (out1, out2), each (B, num_levels*dim*(2*radius+1), H1, W1).  The reference stores a
+    pyramid of permuted copies per block and samples it with grid_sample once per level, volume and flow iteration;
+    here the volumes stay in the layout they arrive in, the pyramid is formed on the fly, and one kernel per volume does
+    the whole lookup.  The clamp of the sampling positions to [-1, 1] that the reference applies to its first volume only
+    (core/corr.py:585) is reproduced (`clamp_first=False` drops it).
+    """
+
+    def __init__(self, corr1, corr2, num_levels=4, radius=4, clamp_first=True):
+        assert corr1.shape[:2] == corr2.shape[:2] and corr1.shape[3:] == corr2.shape[3:]
+        # core/corr.py:536: the displacement axes must be as long as the image axes
+        assert corr1.shape[2] == corr1.shape[4] and corr2.shape[2] == corr2.shape[3]
+        self.num_levels = num_levels
+        self.radius = radius
+        self.clamp_first = clamp_first
+        self.corr1 = corr1.contiguous().float()
+        self.corr2 = corr2.contiguous().float()
+
+    def __call__(self, coords):
+        coords = coords.detach().contiguous().float()
+        out1 = Lookup1DFunction.apply(self.corr1, coords, 0, self.clamp_first, self.num_levels, self.radius)
+        out2 = Lookup1DFunction.apply(self.corr2, coords, 1, False, self.num_levels, self.radius)
+        return out1, out2

@@ -183,3 +183,30 @@ class LookupFunction(Function):
         with torch.cuda.device_of(grad_out):
             d_f1, d_f2 = MemorySaver.lookup_backward(f1, f2_levels, coords, grad_out, ctx.radius, ctx.scale)
         return (None, None, None, d_f1, *d_f2)
+
+
+class Lookup1DFunction(Function):
+    """Lookup in one separated 3D volume, the reference's CorrBlock1D per volume (core/corr.py:565-624).
+
+    apply(corr, coords, coord_channel, clamp_unit, num_levels, radius): corr (B,dim,L,H1,W1), coords (B,2,H1,W1)
+    -> (B, num_levels*dim*(2*radius+1), H1, W1).  The gradient goes to corr; coords get none (the flow iterations
+    detach them, core/sepflow.py:194).
+    """
+
+    @staticmethod
+    def forward(ctx, corr, coords, coord_channel, clamp_unit, num_levels, radius):
+        _contig(corr, coords)
+        with torch.cuda.device_of(corr):
+            out = MemorySaver.lookup1d_forward(corr, coords, coord_channel, clamp_unit, num_levels, radius)
+        ctx.save_for_backward(coords)
+        ctx.args = (tuple(corr.shape), coord_channel, clamp_unit, num_levels, radius)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        coords, = ctx.saved_tensors
+        shape, coord_channel, clamp_unit, num_levels, radius = ctx.args
+        with torch.cuda.device_of(grad_out):
+            d = MemorySaver.lookup1d_backward(coords, grad_out.contiguous(), shape, coord_channel, clamp_unit,
+                                              num_levels, radius)
+        return d, None, None, None, None, None

@@ -2,7 +2,7 @@
 
 * AlternateCorrBlockSepflow (host orchestration over the fmap2 pyramid, Conv3d+softmax attention,
   upsampling, concatenation) against the oracle's full-4D CorrBlock, forward and gradients.
-* BASELINE configs 1-4 at full size against the 4D oracle; config 5 (4.26 GB volume) on a seeded
+* benchmark configurations 1-4 at full size against the 4D oracle; config 5 (4.26 GB volume) on a seeded
   subset of image-1 pixels, which are independent units of the operator.
 """
 import copy

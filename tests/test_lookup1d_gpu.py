@@ -1,0 +1,74 @@
+"""GPU parity of the 3D-volume lookup (sepcorr_lookup1d_forward/backward through the C ABI, class CorrBlock1D) against
+the fp64 oracle (`oracle.CorrBlock1D`: pooled pyramid + grid_sample as core/corr.py:513-624).  rtol 1e-4 / atol 1e-5."""
+import pytest
+import torch
+
+from oracle import oracle as O
+from tests._util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(B, dim, H, W, spread, seed):
+    g = torch.Generator().manual_seed(seed)
+    c1 = torch.randn(B, dim, W, H, W, generator=g)
+    c2 = torch.randn(B, dim, H, H, W, generator=g)
+    yy, xx = torch.meshgrid(torch.arange(H), torch.arange(W), indexing='ij')
+    coords = (torch.stack([xx, yy]).float()[None].repeat(B, 1, 1, 1) + torch.randn(B, 2, H, W, generator=g) * spread).contiguous()
+    return c1, c2, coords, g
+
+
+@pytest.mark.parametrize("B,dim,H,W,L,r,spread", [
+    (2, 1, 55, 128, 4, 4, 6.0),       # the model's use: one aggregated channel, benchmark shape
+    (1, 24, 16, 24, 4, 4, 3.0),       # all channels of separate()'s output
+    (1, 3, 9, 11, 2, 3, 20.0),        # mostly outside, odd sizes
+    (1, 2, 40, 40, 3, 8, 2.0),
+])
+def test_block_matches_the_oracle_forward_and_backward(device, B, dim, H, W, L, r, spread):
+    from separableflowthesis_amd import CorrBlock1D
+    c1, c2, coords, g = _case(B, dim, H, W, spread, 500 + W)
+    n = 2 * r + 1
+    up1 = torch.randn(B, L * dim * n, H, W, generator=g)
+    up2 = torch.randn(B, L * dim * n, H, W, generator=g)
+    r1 = c1.double().requires_grad_()
+    r2 = c2.double().requires_grad_()
+    o1, o2 = O.CorrBlock1D(r1, r2, num_levels=L, radius=r)(coords.double())
+    ((o1 * up1.double()).sum() + (o2 * up2.double()).sum()).backward()
+    g1 = c1.to(device).requires_grad_()
+    g2 = c2.to(device).requires_grad_()
+    q1, q2 = CorrBlock1D(g1, g2, num_levels=L, radius=r)(coords.to(device))
+    assert q1.shape == o1.shape and q2.shape == o2.shape
+    assert_close(q1, o1, "out1 (clamped positions)")
+    assert_close(q2, o2, "out2")
+    ((q1 * up1.to(device)).sum() + (q2 * up2.to(device)).sum()).backward()
+    assert_close(g1.grad, r1.grad, "d_corr1", scale_atol=True)
+    assert_close(g2.grad, r2.grad, "d_corr2", scale_atol=True)
+
+
+def test_without_the_clamp_both_volumes_follow_the_plain_definition(device):
+    from separableflowthesis_amd import CorrBlock1D
+    c1, c2, coords, _ = _case(1, 2, 12, 20, 3.0, 77)
+    q1, _ = CorrBlock1D(c1.to(device), c2.to(device), num_levels=3, radius=4, clamp_first=False)(coords.to(device))
+    ref = O.lookup1d_direct(c1.double(), coords[:, 0].double(), 3, 4, clamp_unit=False)
+    assert_close(q1, ref, "out1 without clamp")
+
+
+def test_consumes_the_volumes_of_separate_and_checks_arguments(device):
+    from separableflowthesis_amd import AlternateCorrBlockSepflow, CorrBlock1D, MemorySaver
+    g = torch.Generator().manual_seed(3)
+    fmap1 = torch.randn(1, 64, 16, 24, generator=g).to(device)
+    fmap2 = torch.randn(1, 64, 16, 24, generator=g).to(device)
+    corr1, corr2 = AlternateCorrBlockSepflow(fmap1, fmap2, None)(None, sep=True)
+    coords = _case(1, 1, 16, 24, 2.0, 5)[2].to(device)
+    o1, o2 = CorrBlock1D(corr1, corr2)(coords)
+    r1, r2 = O.CorrBlock1D(corr1.double().cpu(), corr2.double().cpu())(coords.double().cpu())
+    assert_close(o1, r1, "lookup of separate()'s corr1")
+    assert_close(o2, r2, "lookup of separate()'s corr2")
+    with pytest.raises(RuntimeError):
+        MemorySaver.lookup1d_forward(corr1, coords, 2, False, 4, 4)
+    with pytest.raises(RuntimeError):
+        MemorySaver.lookup1d_forward(corr1, coords, 0, False, 9, 4)
+    with pytest.raises(RuntimeError):
+        MemorySaver.lookup1d_forward(corr1.cpu(), coords, 0, False, 4, 4)
+    with pytest.raises(RuntimeError):
+        MemorySaver.lookup1d_forward(corr1, coords[:, :1].contiguous(), 0, False, 4, 4)
