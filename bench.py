@@ -157,6 +157,24 @@ def lookup_level(B, H, W, C, torch, dev, reps=20):
 
     fwd = timed(lambda: MemorySaver.lookup_forward(f1, f2s, coords, 4, scale))
     bwd = timed(lambda: MemorySaver.lookup_backward(f1, f2s, coords, up, 4, scale))
+    # the lookup in the two separated volumes (CorrBlock1D): one aggregated channel as in the model, and all 24
+    one_d = {}
+    for dim in (1, 24):
+        c1 = torch.randn(B, dim, W, H, W, generator=g).to(dev)
+        c2 = torch.randn(B, dim, H, H, W, generator=g).to(dev)
+        u = torch.randn(B, 4 * dim * 9, H, W, generator=g).to(dev)
+
+        def f1d():
+            MemorySaver.lookup1d_forward(c1, coords, 0, True, 4, 4)
+            MemorySaver.lookup1d_forward(c2, coords, 1, False, 4, 4)
+
+        def b1d():
+            MemorySaver.lookup1d_backward(coords, u, tuple(c1.shape), 0, True, 4, 4)
+            MemorySaver.lookup1d_backward(coords, u, tuple(c2.shape), 1, False, 4, 4)
+
+        one_d[f"dim{dim}"] = {"forward_ms": round(timed(f1d), 4), "backward_ms": round(timed(b1d), 4),
+                              "volumes_mib": round((c1.numel() + c2.numel()) * 4 / 2 ** 20, 1)}
+        del c1, c2, u
     pts = B * H * W * 4 * 100                       # (pixel, level, grid point) pairs: one C-long dot product each
     alg = (f1.numel() + sum(t.numel() for t in f2s) + coords.numel() + up.numel()) * 4   # up has the output's size
     return {
@@ -165,10 +183,12 @@ def lookup_level(B, H, W, C, torch, dev, reps=20):
         "forward_gflop_s": round(pts * C * 2 / fwd / 1e6, 1),
         "forward_algorithmic_mib": round(alg / 2 ** 20, 1),
         "forward_hbm_gb_s": round(alg / fwd / 1e6, 1),
+        "volumes_1d": one_d,
         "what": f"sepcorr_lookup_forward / sepcorr_lookup_backward, B={B}, C={C}, {H}x{W}, 4 levels, radius 4; "
                 "window = bytes of the fmap2 rows under all windows (one C-long dot product each, 2 flop per 4 bytes; "
                 "the kernel fetches a row once for four neighbouring pixels, so this may exceed the vector cache's "
-                "256 CU x 64 B/clk x 2.4 GHz = 39.3 TB/s); algorithmic = f1 + pyramid + coords + out once",
+                "256 CU x 64 B/clk x 2.4 GHz = 39.3 TB/s); algorithmic = f1 + pyramid + coords + out once; "
+                "volumes_1d = CorrBlock1D on both separated volumes (sepcorr_lookup1d_forward/backward, 4 levels, radius 4)",
     }
 
 

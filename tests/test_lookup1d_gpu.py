@@ -23,6 +23,7 @@ def _case(B, dim, H, W, spread, seed):
     (1, 24, 16, 24, 4, 4, 3.0),       # all channels of separate()'s output
     (1, 3, 9, 11, 2, 3, 20.0),        # mostly outside, odd sizes
     (1, 2, 40, 40, 3, 8, 2.0),
+    (1, 40, 64, 104, 3, 2, 4.0),      # 266 240 columns: the backward takes its column-owner variant
 ])
 def test_block_matches_the_oracle_forward_and_backward(device, B, dim, H, W, L, r, spread):
     from separableflowthesis_amd import CorrBlock1D
