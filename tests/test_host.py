@@ -82,6 +82,19 @@ def test_lookup_argument_checks_precede_any_launch():
     assert b"aligned" in lib.sepcorr_last_error()
 
 
+def test_lookup1d_argument_checks_precede_any_launch():
+    lib = _lib.load()
+    one = ctypes.c_void_p(256)
+    f, b = lib.sepcorr_lookup1d_forward, lib.sepcorr_lookup1d_backward
+    assert f(None, one, one, 1, 1, 16, 4, 4, 0, 0, 4, 4, None) == -1 and b"NULL" in lib.sepcorr_last_error()
+    assert f(one, one, one, 1, 1, 16, 4, 4, 2, 0, 4, 4, None) == -1 and b"coord_channel" in lib.sepcorr_last_error()
+    assert f(one, one, one, 1, 1, 16, 4, 4, 0, 0, 9, 4, None) == -1 and b"levels" in lib.sepcorr_last_error()
+    assert f(one, one, one, 1, 1, 4, 4, 4, 0, 0, 4, 4, None) == -1 and b"too short" in lib.sepcorr_last_error()
+    assert f(one, one, one, 1, 1, 16, 4, 4, 0, 0, 4, 17, None) == -1 and b"radius" in lib.sepcorr_last_error()
+    assert f(one, one, one, 64, 64, 1024, 64, 64, 0, 0, 4, 4, None) == -1 and b"2^31" in lib.sepcorr_last_error()
+    assert b(one, None, one, 1, 1, 16, 4, 4, 0, 0, 4, 4, None) == -1 and b"NULL" in lib.sepcorr_last_error()
+
+
 def test_cpu_tensors_are_refused_like_check_cuda():
     from separableflowthesis_amd import MemorySaver
     f = torch.randn(1, 2, 2, 4)

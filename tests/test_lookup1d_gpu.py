@@ -73,3 +73,41 @@ def test_consumes_the_volumes_of_separate_and_checks_arguments(device):
         MemorySaver.lookup1d_forward(corr1.cpu(), coords, 0, False, 4, 4)
     with pytest.raises(RuntimeError):
         MemorySaver.lookup1d_forward(corr1, coords[:, :1].contiguous(), 0, False, 4, 4)
+
+
+def _ops(t):
+    from separableflowthesis_amd import MemorySaver
+    o1 = MemorySaver.lookup1d_forward(t["c1"], t["coords"], 0, True, 3, 4)
+    o2 = MemorySaver.lookup1d_forward(t["c2"], t["coords"], 1, False, 3, 4)
+    d1 = MemorySaver.lookup1d_backward(t["coords"], t["up"], tuple(t["c1"].shape), 0, True, 3, 4)
+    d2 = MemorySaver.lookup1d_backward(t["coords"], t["up"], tuple(t["c2"].shape), 1, False, 3, 4)
+    return [o1, o2, d1, d2]
+
+
+def _tensors(device, seed):
+    c1, c2, coords, g = _case(1, 2, 12, 12, 3.0, seed)
+    t = dict(c1=c1, c2=c2, coords=coords, up=torch.randn(1, 3 * 2 * 9, 12, 12, generator=g))
+    return {k: v.to(device) for k, v in t.items()}
+
+
+def test_follows_the_callers_stream_and_replays_from_a_captured_graph(device):
+    ref = _ops(_tensors(device, 31))
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        got = _ops({k: v * 1.0 for k, v in _tensors(device, 31).items()})    # inputs produced on s
+    s.synchronize()
+    assert all(torch.equal(x, y) for x, y in zip(got, ref))
+    static = _tensors(device, 32)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = _ops(static)
+    for seed in (33, 34):
+        fresh = _tensors(device, seed)
+        ref = _ops(fresh)                          # eager work between the replays
+        torch.cuda.synchronize()
+        for k in static:
+            static[k].copy_(fresh[k])
+        graph.replay()
+        torch.cuda.synchronize()
+        assert all(torch.equal(x, y) for x, y in zip(outs, ref)), f"replay with seed {seed} differs from eager"
