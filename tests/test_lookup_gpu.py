@@ -197,3 +197,30 @@ def test_lookup_follows_the_callers_stream_and_replays_from_a_captured_graph(dev
         graph.replay()
         torch.cuda.synchronize()
         assert all(torch.equal(x, y) for x, y in zip(outs, ref)), f"replay with seed {seed} differs from eager"
+
+
+def test_lookup_at_the_high_resolution_size_on_row_bands(device):
+    # B=1, C=256, 136x240 (the largest benchmark shape; its 4D volume would be 4.3 GB).  Image-1 pixels are independent
+    # units of the lookup, so the oracle evaluates three bands of rows and those rows of the full GPU result are compared,
+    # values and d_fmap1; d_fmap2 is checked through the bilinear identity <up, out> = <d_fmap2, fmap2>.
+    from separableflowthesis_amd import AlternateCorrBlockSepflow
+    B, C, H, W, L, r = 1, 256, 136, 240, 4, 4
+    g = torch.Generator().manual_seed(2024)
+    fmap1 = torch.randn(B, C, H, W, generator=g)
+    fmap2 = torch.randn(B, C, H, W, generator=g)
+    coords = _coords(B, H, W, g, 5.0)
+    up = torch.randn(B, L * 81, H, W, generator=g)
+    g1 = fmap1.to(device).requires_grad_()
+    g2 = fmap2.to(device).requires_grad_()
+    out = AlternateCorrBlockSepflow(g1, g2, None, num_levels=L, radius=r)(coords.to(device))
+    out.backward(up.to(device))
+    for i0 in (0, 67, 134):
+        rows = slice(i0, i0 + 2)
+        a = fmap1[:, :, rows].double().requires_grad_()
+        ref = O.lookup_direct(a, fmap2.double(), coords[:, :, rows].double(), L, r)
+        (ref * up[:, :, rows].double()).sum().backward()
+        assert_close(out[:, :, rows], ref, f"lookup rows {i0}..")
+        assert_close(g1.grad[:, :, rows], a.grad, f"d_fmap1 rows {i0}..", scale_atol=True)
+    lhs = float((out.detach().double().cpu() * up.double()).sum())
+    rhs = float((g2.grad.double().cpu() * fmap2.double()).sum())
+    assert abs(lhs - rhs) <= 1e-4 * abs(lhs) + 1e-2
