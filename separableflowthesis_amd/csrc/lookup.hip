@@ -758,16 +758,25 @@ int sepcorr_lookup_backward(const float *f1, const float *const *f2_levels, cons
     const size_t lds = (size_t)n * n * (TP + 1) * sizeof(float);
     hipLaunchKernelGGL(lookup_grid_grad_kernel, dim3((W1 + TP - 1) / TP, H1, B * L), dim3(256), lds, s, a);
     if (int e = launch_error("lookup grid-gradient kernel")) return e;
+    // d_f1 and d_f2 only read the window gradients: they run side by side on the library's side streams
+    void *va = nullptr, *vb = nullptr;
+    void *token = sepcorr_fork(s, &va, &vb);
+    hipStream_t sa = static_cast<hipStream_t>(va), sb = static_cast<hipStream_t>(vb);
     bool vec = C % 4 == 0 && (uintptr_t)d_f1 % 16 == 0;
     for (int l = 0; l < L; ++l) vec = vec && (uintptr_t)a.f2[l] % 16 == 0;
-    if (vec) hipLaunchKernelGGL(lookup_df1_group_kernel, dim3((W1 + TPG - 1) / TPG, H1, B), dim3(256), 0, s, a);
-    else hipLaunchKernelGGL(lookup_df1_kernel, dim3((unsigned)((size_t)B * H1 * W1)), dim3(256), 0, s, a);
-    if (int e = launch_error("lookup d_f1 kernel")) return e;
-    hipLaunchKernelGGL(lookup_df2_kernel, dim3((unsigned)tiles, (C + NCH - 1) / NCH, B), dim3(64), 0, s, a);
-    if (int e = launch_error("lookup d_f2 kernel")) return e;
-    hipLaunchKernelGGL(lookup_df2_reduce_kernel, dim3(1024, L), dim3(256), 0, s, a);
-    if (int e = launch_error("lookup d_f2 reduction")) return e;
-    return SEPCORR_OK;
+    if (vec) hipLaunchKernelGGL(lookup_df1_group_kernel, dim3((W1 + TPG - 1) / TPG, H1, B), dim3(256), 0, sa, a);
+    else hipLaunchKernelGGL(lookup_df1_kernel, dim3((unsigned)((size_t)B * H1 * W1)), dim3(256), 0, sa, a);
+    int rl = launch_error("lookup d_f1 kernel");
+    if (rl == SEPCORR_OK) {
+        hipLaunchKernelGGL(lookup_df2_kernel, dim3((unsigned)tiles, (C + NCH - 1) / NCH, B), dim3(64), 0, sb, a);
+        rl = launch_error("lookup d_f2 kernel");
+    }
+    if (rl == SEPCORR_OK) {
+        hipLaunchKernelGGL(lookup_df2_reduce_kernel, dim3(1024, L), dim3(256), 0, sb, a);
+        rl = launch_error("lookup d_f2 reduction");
+    }
+    const int rj = sepcorr_join(token);
+    return rl ? rl : rj;
 }
 
 }  // extern "C"

@@ -2306,6 +2306,20 @@ int check_workspace(const Dims &d, void *ws, size_t ws_bytes) {
 
 }  // namespace
 
+void *sepcorr_fork(void *user, void **sa, void **sb) {
+    ForkJoin *fj = new ForkJoin(static_cast<hipStream_t>(user));
+    *sa = fj->sa;
+    *sb = fj->sb;
+    return fj;
+}
+
+int sepcorr_join(void *token) {
+    ForkJoin *fj = static_cast<ForkJoin *>(token);
+    const int rc = fj->join();
+    delete fj;
+    return rc;
+}
+
 extern "C" {
 
 const char *sepcorr_last_error(void) { return g_err; }
