@@ -314,6 +314,7 @@ __global__ void __launch_bounds__(256) lookup_forward_group_kernel(const LookupA
 
 constexpr int TQX = 8, TQY = 4;                     // fmap2 positions per d_f2 wave: the 32 rows of one MFMA tile
 constexpr int NCH = 128;                            // channels per d_f2 wave
+constexpr int NPR = 2;                              // pixel pairs fetched before their MFMAs are issued
 static_assert(TQX * TQY == 32, "one tile position per MFMA row");
 
 struct LookupBwdArgs {
@@ -498,7 +499,8 @@ __global__ void __launch_bounds__(256) lookup_df1_group_kernel(const LookupBwdAr
 // runs over the pixels whose window touches the tile.  The wave scans its pixels 64 at a time (origins stay in the
 // lanes' registers), takes the touching ones in ascending order, two per v_mfma_f32_32x32x2_f32: operand A = the two
 // pixels' window entries at the tile's positions (zero outside the window), operand B = their f1 channels, fetched as
-// contiguous runs.  Eight pixels are fetched before their MFMAs are issued.  No LDS, no barrier, no atomics.
+// contiguous runs.  Four pixels are fetched before their MFMAs are issued (measured: 2 pixels 0.147, 4 0.137, 8 0.142 ms).
+// No LDS, no barrier, no atomics.
 typedef float lk_v16f __attribute__((ext_vector_type(16)));
 
 __global__ void __launch_bounds__(64) lookup_df2_kernel(const LookupBwdArgs a) {
@@ -539,11 +541,17 @@ __global__ void __launch_bounds__(64) lookup_df2_kernel(const LookupBwdArgs a) {
         const bool hit = p < p_end && ox < tx0 + TQX && ox + G > tx0 && oy < ty0 + TQY && oy + G > ty0;
         unsigned long long m = __ballot(hit);
         while (m) {
-            float wa[4], fb[4][NB];
-            bool any[4];
+            float wa[NPR], fb[NPR][NB];
+            bool any[NPR];
 #pragma unroll
-            for (int pr = 0; pr < 4; ++pr) {
+            for (int pr = 0; pr < NPR; ++pr) {
                 any[pr] = m != 0;                              // wave-uniform
+                if (!any[pr]) {                                // nothing left in these 64 pixels: skip the slot
+                    wa[pr] = 0.f;
+#pragma unroll
+                    for (int cb = 0; cb < NB; ++cb) fb[pr][cb] = 0.f;
+                    continue;
+                }
                 const int cn0 = m ? __builtin_ctzll(m) : 0;
                 m &= m - 1;
                 const bool two = m != 0;
@@ -562,7 +570,7 @@ __global__ void __launch_bounds__(64) lookup_df2_kernel(const LookupBwdArgs a) {
                 }
             }
 #pragma unroll
-            for (int pr = 0; pr < 4; ++pr)
+            for (int pr = 0; pr < NPR; ++pr)
                 if (any[pr]) {
 #pragma unroll
                     for (int cb = 0; cb < NB; ++cb)
