@@ -14,6 +14,12 @@ Every function cites the reference lines it follows.  How each one is pinned
 (closed forms, brute-force loops, invariants, fp64 gradcheck, the independent
 C loop restatement in ``sepcorr_loops.c``) is listed in tests/test_oracle.py;
 the reference stores no golden vectors for this path, so none are replayed.
+The two lookups (``CorrBlock4D.lookup`` / ``lookup_direct`` for the 4D pyramid,
+``CorrBlock1D`` / ``lookup1d_direct`` for the separated volumes) are pinned in
+tests/test_lookup_oracle.py and tests/test_lookup1d_oracle.py: entries of the
+stored volume at integer targets, affine volumes reproduced exactly at every
+level, zero padding, the reference's clamp, and agreement of two independent
+formulations in values and gradients.
 """
 import math
 
