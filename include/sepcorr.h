@@ -198,6 +198,16 @@ int sepcorr_assemble_backward(const float *grad_dst, float *grad_src, int B, int
                               int CT, int c0, int L0, void *stream);
 
 /*
+ * The same for up to 8 sources in one launch: source n (B,H1,W1,ch[n],Li[n]) fills the channels after those of the
+ * sources before it (the first starts at channel 0); ch, Li and the pointer tables are host arrays of nsrc entries.
+ * One launch per module-level volume instead of one per level and operator output.
+ */
+int sepcorr_assemble_forward_multi(const float *const *srcs, const int *ch, const int *Li, int nsrc, float *dst,
+                                   int B, int H1, int W1, int CT, int L0, void *stream);
+int sepcorr_assemble_backward_multi(const float *grad_dst, float *const *grad_srcs, const int *ch, const int *Li,
+                                    int nsrc, int B, int H1, int W1, int CT, int L0, void *stream);
+
+/*
  * Windowed bilinear lookup of the correlation pyramid without the 4D volume: what the caller's
  * corr_fn(coords) returns on the stored-volume path (CorrBlock.__call__, core/corr.py:193-248), for the block
  * that never stores the volume (AlternateCorrBlockSepflow.__call__, core/corr.py:479-510, which raises

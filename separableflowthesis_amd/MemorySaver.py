@@ -251,6 +251,13 @@ def attention_backward(sep, weight, a, grad_a, need_bias=True):
     return [d_sep, d_w, d_b]
 
 
+def _src_tables(shapes, ptrs):
+    import ctypes
+    n = len(shapes)
+    return ((ctypes.c_void_p * n)(*ptrs), (ctypes.c_int * n)(*[s[3] for s in shapes]),
+            (ctypes.c_int * n)(*[s[4] for s in shapes]))
+
+
 def assemble_forward(srcs, L0):
     """srcs: operator outputs (B,H1,W1,ch_n,L_n) in channel order -> (B, sum ch_n, L0, H1, W1), each one
     transposed and linearly interpolated along its last axis to length L0 (align_corners=True)."""
@@ -261,10 +268,16 @@ def assemble_forward(srcs, L0):
     lib = _lib.load()
     with torch.cuda.device(srcs[0].device):
         dst = torch.empty((B, CT, L0, H1, W1), dtype=srcs[0].dtype, device=srcs[0].device)
-        c0 = 0
         for t in srcs:
             if tuple(t.shape[:3]) != (B, H1, W1) or t.device != dst.device:
                 raise RuntimeError("assemble: all sources must share batch, H1, W1 and device")
+        if len(srcs) <= 8:     # one launch for the whole volume
+            ptrs, ch, li = _src_tables([t.shape for t in srcs], [t.data_ptr() for t in srcs])
+            _lib.check(lib.sepcorr_assemble_forward_multi(ptrs, ch, li, len(srcs), dst.data_ptr(), B, H1, W1, CT, L0,
+                                                          _stream()))
+            return dst
+        c0 = 0
+        for t in srcs:
             _lib.check(lib.sepcorr_assemble_forward(t.data_ptr(), dst.data_ptr(), B, H1, W1, t.shape[3], t.shape[4],
                                                     CT, c0, L0, _stream()))
             c0 += t.shape[3]
@@ -276,15 +289,18 @@ def assemble_backward(grad_dst, shapes):
     _check("grad_dst", grad_dst, ndim=5)
     B, CT, L0, H1, W1 = grad_dst.shape
     lib = _lib.load()
-    out = []
     with torch.cuda.device(grad_dst.device):
+        out = [torch.empty(shp, dtype=grad_dst.dtype, device=grad_dst.device) for shp in shapes]
+        if len(out) <= 8:
+            ptrs, ch, li = _src_tables(shapes, [g.data_ptr() for g in out])
+            _lib.check(lib.sepcorr_assemble_backward_multi(grad_dst.data_ptr(), ptrs, ch, li, len(out), B, H1, W1, CT, L0,
+                                                           _stream()))
+            return out
         c0 = 0
-        for shp in shapes:
-            g = torch.empty(shp, dtype=grad_dst.dtype, device=grad_dst.device)
+        for shp, g in zip(shapes, out):
             _lib.check(lib.sepcorr_assemble_backward(grad_dst.data_ptr(), g.data_ptr(), B, H1, W1, shp[3], shp[4],
                                                      CT, c0, L0, _stream()))
             c0 += shp[3]
-            out.append(g)
     return out
 
 

@@ -27,31 +27,47 @@ __device__ __forceinline__ void src_pos(int l0, float scale, int Li, int &x0, in
     lam = pos - (float)x0;
 }
 
+constexpr int MAXSRC = 8;   // sources per launch (4 pyramid levels x 2 operator outputs)
+
 struct AsmArgs {
-    const float *src;   // forward: (B,H1,W1,ch,Li); backward: grad of dst (B,CT,L0,H1,W1)
-    float *dst;         // forward: (B,CT,L0,H1,W1);  backward: grad of src (B,H1,W1,ch,Li)
-    int B, H1, W1, ch, Li, CT, c0, L0;
-    float scale;        // (Li-1)/(L0-1), 0 when L0 == 1
+    const float *src[MAXSRC];   // forward: (B,H1,W1,ch,Li) each; backward: unused
+    float *gsrc[MAXSRC];        // backward: gradients of the sources, (B,H1,W1,ch,Li) each
+    const float *gdst;          // backward: gradient of dst (B,CT,L0,H1,W1)
+    float *dst;                 // forward: (B,CT,L0,H1,W1)
+    int ch[MAXSRC], Li[MAXSRC], c0[MAXSRC];
+    int z0[MAXSRC + 1];         // first blockIdx.z of each source (B*ch[s] blocks each)
+    float scale[MAXSRC];        // (Li-1)/(L0-1), 0 when L0 == 1
+    int nsrc, B, H1, W1, CT, L0;
 };
+
+// source that owns blockIdx.z
+__device__ __forceinline__ int find_src(const AsmArgs &a) {
+    int s = 0;
+    while (s + 1 < a.nsrc && (int)blockIdx.z >= a.z0[s + 1]) ++s;
+    return s;
+}
 
 // grid: (ceil(W1/TJ), H1, B*ch); LDS tile [TJ][Li+1]
 __global__ void __launch_bounds__(256) assemble_forward_kernel(const AsmArgs a) {
     extern __shared__ float tile[];
-    const int Li = a.Li, L0 = a.L0, W1 = a.W1, H1 = a.H1;
+    const int sI = find_src(a), z = blockIdx.z - a.z0[sI], nch = a.ch[sI];
+    const int Li = a.Li[sI], L0 = a.L0, W1 = a.W1, H1 = a.H1;
     const int LS = Li + 1;
-    const int j0 = blockIdx.x * TJ, i = blockIdx.y, c = blockIdx.z % a.ch, b = blockIdx.z / a.ch;
+    const int j0 = blockIdx.x * TJ, i = blockIdx.y, c = z % nch, b = z / nch;
     const int nj = min(TJ, W1 - j0);
+    const float *src = a.src[sI];
+    const float scale = a.scale[sI];
     for (int t = threadIdx.x; t < nj * Li; t += blockDim.x) {
         const int jj = t / Li, l = t - jj * Li;
-        tile[jj * LS + l] = a.src[((((size_t)b * H1 + i) * W1 + j0 + jj) * a.ch + c) * Li + l];
+        tile[jj * LS + l] = src[((((size_t)b * H1 + i) * W1 + j0 + jj) * nch + c) * Li + l];
     }
     __syncthreads();
-    float *out = a.dst + (((size_t)b * a.CT + a.c0 + c) * L0) * H1 * W1 + (size_t)i * W1 + j0;
+    float *out = a.dst + (((size_t)b * a.CT + a.c0[sI] + c) * L0) * H1 * W1 + (size_t)i * W1 + j0;
     for (int t = threadIdx.x; t < L0 * TJ; t += blockDim.x) {
         const int l0 = t / TJ, jj = t % TJ;
         if (jj < nj) {
             int x0, x1; float lam;
-            src_pos(l0, a.scale, Li, x0, x1, lam);
+            src_pos(l0, scale, Li, x0, x1, lam);
             out[(size_t)l0 * H1 * W1 + jj] = (1.f - lam) * tile[jj * LS + x0] + lam * tile[jj * LS + x1];
         }
     }
@@ -60,53 +76,76 @@ __global__ void __launch_bounds__(256) assemble_forward_kernel(const AsmArgs a) 
 // grid as above; LDS tile [L0][TJ+1] of the output gradient
 __global__ void __launch_bounds__(256) assemble_backward_kernel(const AsmArgs a) {
     extern __shared__ float tile[];
-    const int Li = a.Li, L0 = a.L0, W1 = a.W1, H1 = a.H1;
+    const int sI = find_src(a), z = blockIdx.z - a.z0[sI], nch = a.ch[sI];
+    const int Li = a.Li[sI], L0 = a.L0, W1 = a.W1, H1 = a.H1;
     constexpr int GS = TJ + 1;
-    const int j0 = blockIdx.x * TJ, i = blockIdx.y, c = blockIdx.z % a.ch, b = blockIdx.z / a.ch;
+    const int j0 = blockIdx.x * TJ, i = blockIdx.y, c = z % nch, b = z / nch;
     const int nj = min(TJ, W1 - j0);
-    const float *g = a.src + (((size_t)b * a.CT + a.c0 + c) * L0) * H1 * W1 + (size_t)i * W1 + j0;
+    const float scale = a.scale[sI];
+    float *gsrc = a.gsrc[sI];
+    const float *g = a.gdst + (((size_t)b * a.CT + a.c0[sI] + c) * L0) * H1 * W1 + (size_t)i * W1 + j0;
     for (int t = threadIdx.x; t < L0 * TJ; t += blockDim.x) {
         const int l0 = t / TJ, jj = t % TJ;
         tile[l0 * GS + jj] = jj < nj ? g[(size_t)l0 * H1 * W1 + jj] : 0.f;
     }
     __syncthreads();
     // d_src[l] = sum over l0 of (1-lam)[x0==l] + lam[x1==l, x1!=x0]; candidates around l/scale
-    const float inv = a.scale > 0.f ? 1.f / a.scale : 0.f;
+    const float inv = scale > 0.f ? 1.f / scale : 0.f;
     for (int t = threadIdx.x; t < nj * Li; t += blockDim.x) {
         const int jj = t / Li, l = t - jj * Li;
         int lo = 0, hi = L0 - 1;
-        if (a.scale > 0.f) {
+        if (scale > 0.f) {
             lo = max(0, (int)floorf((float)(l - 1) * inv) - 1);
             hi = min(L0 - 1, (int)ceilf((float)(l + 1) * inv) + 1);
         }
         float s = 0.f;
         for (int l0 = lo; l0 <= hi; ++l0) {
             int x0, x1; float lam;
-            src_pos(l0, a.scale, Li, x0, x1, lam);
+            src_pos(l0, scale, Li, x0, x1, lam);
             const float gv = tile[l0 * GS + jj];
             if (x0 == l) s += (1.f - lam) * gv;
             if (x1 == l) s += lam * gv;     // when x1 == x0 the two weights add up to 1, as in the forward
         }
-        a.dst[((((size_t)b * H1 + i) * W1 + j0 + jj) * a.ch + c) * Li + l] = s;
+        gsrc[((((size_t)b * H1 + i) * W1 + j0 + jj) * nch + c) * Li + l] = s;
     }
 }
 
 int bad(const char *msg) { return sepcorr_set_error(SEPCORR_EINVAL, msg); }
 
-int run(bool backward, const float *src, float *dst, int B, int H1, int W1, int ch, int Li, int CT, int c0, int L0, void *stream) {
-    if (!src || !dst) return bad("sepcorr: assemble: NULL pointer");
-    if (B < 1 || H1 < 1 || W1 < 1 || ch < 1 || Li < 1 || CT < 1 || L0 < 1 || c0 < 0 || c0 + ch > CT)
-        return bad("sepcorr: assemble: sizes out of range");
-    if ((double)B * CT * L0 * H1 * W1 > 2147483647.0 || (double)B * H1 * W1 * ch * Li > 2147483647.0)
-        return bad("sepcorr: a tensor would have 2^31 or more elements");
-    if ((long)B * ch > 65535 || H1 > 65535) return bad("sepcorr: assemble: B*ch and H1 must be below 65536");
-    const size_t lds = backward ? (size_t)L0 * (TJ + 1) * sizeof(float) : (size_t)TJ * (Li + 1) * sizeof(float);
+// One launch for up to MAXSRC sources that share dst (forward) or grad_dst (backward); channel offsets follow the
+// order of the sources, starting at c0.
+int run(bool backward, const float *const *srcs, float *const *gsrcs, const float *gdst, float *dst, const int *ch,
+        const int *Li, int nsrc, int B, int H1, int W1, int CT, int c0, int L0, void *stream) {
+    if (nsrc < 1 || nsrc > MAXSRC) return bad("sepcorr: assemble: 1 to 8 sources per call");
+    if ((backward ? (const void *)gdst : (const void *)dst) == nullptr || !ch || !Li) return bad("sepcorr: assemble: NULL pointer");
+    if (B < 1 || H1 < 1 || W1 < 1 || CT < 1 || L0 < 1 || c0 < 0) return bad("sepcorr: assemble: sizes out of range");
+    if ((double)B * CT * L0 * H1 * W1 > 2147483647.0) return bad("sepcorr: a tensor would have 2^31 or more elements");
+    if (H1 > 65535) return bad("sepcorr: assemble: B*ch and H1 must be below 65536");
+    AsmArgs a = {};
+    a.gdst = gdst; a.dst = dst; a.nsrc = nsrc; a.B = B; a.H1 = H1; a.W1 = W1; a.CT = CT; a.L0 = L0;
+    size_t lds = 0;
+    long z = 0;
+    int c = c0;
+    for (int s = 0; s < nsrc; ++s) {
+        if (!(backward ? (const void *)gsrcs[s] : (const void *)srcs[s])) return bad("sepcorr: assemble: NULL pointer");
+        if (ch[s] < 1 || Li[s] < 1 || c + ch[s] > CT) return bad("sepcorr: assemble: sizes out of range");
+        if ((double)B * H1 * W1 * ch[s] * Li[s] > 2147483647.0) return bad("sepcorr: a tensor would have 2^31 or more elements");
+        if (backward) a.gsrc[s] = gsrcs[s]; else a.src[s] = srcs[s];
+        a.ch[s] = ch[s]; a.Li[s] = Li[s]; a.c0[s] = c;
+        a.scale[s] = L0 > 1 ? (float)(Li[s] - 1) / (float)(L0 - 1) : 0.f;
+        a.z0[s] = (int)z;
+        z += (long)B * ch[s];
+        c += ch[s];
+        const size_t need = backward ? (size_t)L0 * (TJ + 1) * sizeof(float) : (size_t)TJ * (Li[s] + 1) * sizeof(float);
+        lds = need > lds ? need : lds;
+    }
+    a.z0[nsrc] = (int)z;
+    if (z > 65535) return bad("sepcorr: assemble: B*ch and H1 must be below 65536");
     if (lds > 64 * 1024) return bad("sepcorr: assemble: displacement axis too long for the LDS tile");
-    AsmArgs a = {src, dst, B, H1, W1, ch, Li, CT, c0, L0, L0 > 1 ? (float)(Li - 1) / (float)(L0 - 1) : 0.f};
-    const dim3 grid((W1 + TJ - 1) / TJ, H1, B * ch), block(256);
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    if (backward) hipLaunchKernelGGL(assemble_backward_kernel, grid, block, lds, s, a);
-    else hipLaunchKernelGGL(assemble_forward_kernel, grid, block, lds, s, a);
+    const dim3 grid((W1 + TJ - 1) / TJ, H1, (unsigned)z), block(256);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (backward) hipLaunchKernelGGL(assemble_backward_kernel, grid, block, lds, st, a);
+    else hipLaunchKernelGGL(assemble_forward_kernel, grid, block, lds, st, a);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         char msg[160];
@@ -122,12 +161,26 @@ extern "C" {
 
 int sepcorr_assemble_forward(const float *src, float *dst, int B, int H1, int W1, int ch, int Li, int CT, int c0, int L0,
                              void *stream) {
-    return run(false, src, dst, B, H1, W1, ch, Li, CT, c0, L0, stream);
+    if (!src) return bad("sepcorr: assemble: NULL pointer");
+    return run(false, &src, nullptr, nullptr, dst, &ch, &Li, 1, B, H1, W1, CT, c0, L0, stream);
 }
 
 int sepcorr_assemble_backward(const float *grad_dst, float *grad_src, int B, int H1, int W1, int ch, int Li, int CT, int c0,
                               int L0, void *stream) {
-    return run(true, grad_dst, grad_src, B, H1, W1, ch, Li, CT, c0, L0, stream);
+    if (!grad_src) return bad("sepcorr: assemble: NULL pointer");
+    return run(true, nullptr, &grad_src, grad_dst, nullptr, &ch, &Li, 1, B, H1, W1, CT, c0, L0, stream);
+}
+
+int sepcorr_assemble_forward_multi(const float *const *srcs, const int *ch, const int *Li, int nsrc, float *dst, int B,
+                                   int H1, int W1, int CT, int L0, void *stream) {
+    if (!srcs) return bad("sepcorr: assemble: NULL pointer");
+    return run(false, srcs, nullptr, nullptr, dst, ch, Li, nsrc, B, H1, W1, CT, 0, L0, stream);
+}
+
+int sepcorr_assemble_backward_multi(const float *grad_dst, float *const *grad_srcs, const int *ch, const int *Li, int nsrc,
+                                    int B, int H1, int W1, int CT, int L0, void *stream) {
+    if (!grad_srcs) return bad("sepcorr: assemble: NULL pointer");
+    return run(true, nullptr, grad_srcs, grad_dst, nullptr, ch, Li, nsrc, B, H1, W1, CT, 0, L0, stream);
 }
 
 }  // extern "C"
