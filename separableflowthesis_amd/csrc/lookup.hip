@@ -469,7 +469,7 @@ __global__ void __launch_bounds__(256) lookup_df1_group_kernel(const LookupBwdAr
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                 __builtin_amdgcn_wave_barrier();
                 int bx = 0, by = 0;
-#pragma unroll 2
+#pragma unroll 4
                 for (int bp = 0; bp < npts; ++bp) {
                     const int yc = min(max(qy0 + by, 0), H2 - 1), xc = min(max(qx0 + bx, 0), W2 - 1);
                     const float4 v = *reinterpret_cast<const float4 *>(f2 + ((size_t)yc * W2 + xc) * C);
