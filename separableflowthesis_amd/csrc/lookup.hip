@@ -609,6 +609,7 @@ __global__ void __launch_bounds__(256) lookup_df2_reduce_kernel(const LookupBwdA
     if (n % 4 == 0 && (uintptr_t)dst % 16 == 0) {
         for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < n / 4; e += stride) {
             float4 s = reinterpret_cast<const float4 *>(part)[e];
+#pragma unroll 8
             for (int k = 1; k < S; ++k) {
                 const float4 v = reinterpret_cast<const float4 *>(part + (size_t)k * n)[e];
                 s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
