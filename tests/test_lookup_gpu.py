@@ -94,6 +94,8 @@ def test_lookup_special_coordinates_and_errors(device):
     (1, 100, 9, 20, 2, 3, 25.0),      # most windows outside, C not a multiple of 64
     (1, 37, 8, 20, 2, 1, 2.0),
     (1, 300, 8, 16, 2, 2, 2.0),       # two channel blocks in the d_f2 kernel
+    (1, 64, 10, 12, 1, 2, 2.0),       # a single level
+    (3, 32, 6, 70, 2, 4, 1.0),        # batch of three, long rows, one float4 per lane
 ])
 def test_lookup_gradients_match_autograd_through_the_oracle(device, B, C, H, W, levels, r, spread):
     from separableflowthesis_amd import AlternateCorrBlockSepflow
