@@ -1790,7 +1790,18 @@ __global__ void __launch_bounds__(64 * NW) df1_bf_kernel(const BwdArgs a, const 
 // out[i] (+)= sum_s part[s*n + i], in split order.
 __global__ void __launch_bounds__(256) reduce_splits_kernel(const float *part, float *out, size_t n, int nsplit,
                                                             int accumulate) {
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    if (n % 4 == 0 && (reinterpret_cast<uintptr_t>(part) | reinterpret_cast<uintptr_t>(out)) % 16 == 0) {
+        // four elements per thread and several splits in flight
+        for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n / 4; i += stride) {
+            v4f s = accumulate ? reinterpret_cast<const v4f *>(out)[i] : v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 8
+            for (int k = 0; k < nsplit; ++k) s += reinterpret_cast<const v4f *>(part + (size_t)k * n)[i];
+            reinterpret_cast<v4f *>(out)[i] = s;
+        }
+        return;
+    }
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
         float s = accumulate ? out[i] : 0.f;
         for (int k = 0; k < nsplit; ++k) s += part[(size_t)k * n + i];
         out[i] = s;
