@@ -259,7 +259,7 @@ int sepcorr_lookup_backward(const float *f1, const float *const *f2_levels, cons
  *           level l = l-fold average pooling by two along L (core/corr.py:546-550), zero outside the level
  *           (grid_sample, align_corners=True, core/corr.py:553-560).  The pyramid is formed on the fly, not stored.
  *   clamp_unit != 0 clamps the sampling positions to [-1, 1] first, as the reference does for its first volume
- *           (core/corr.py:585); pass 1 for corr1 and 0 for corr2 to reproduce it.
+ *           (core/corr.py:593); pass 1 for corr1 and 0 for corr2 to reproduce it.
  * Limits: 8 levels, radius <= 16, L >> (levels-1) >= 1.
  */
 int sepcorr_lookup1d_forward(const float *corr, const float *coords, float *out, int B, int dim, int L, int H1, int W1,

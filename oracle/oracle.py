@@ -276,16 +276,26 @@ class CorrBlock4D:
             corr = F.avg_pool2d(corr, 2, stride=2)
             self.pyramid.append(corr)
 
-    def separate(self, attention_weights=None):
+    def separate(self, attention_weights=None, argmax=None):
+        """`argmax` (optional, tests of near-ties): per level a pair (argmax_u (B,h1,w1,1,hl), argmax_v (B,h1,w1,1,wl))
+        in the operator's convention; the maxima are then read at these positions instead of being searched, so that
+        the gradient of a maximum flows to the entry the checked implementation selected.  The caller verifies that
+        every given index attains the true maximum to within rounding (tests/_util.py:check_argmax)."""
         B, h1, w1, h2, w2 = self.shape
         us, vs = [], []
-        for corr in self.pyramid:
+        for lvl, corr in enumerate(self.pyramid):
             hl, wl = corr.shape[2], corr.shape[3]
             s = corr.reshape(B, h1, w1, hl, wl)
+            if argmax is None:
+                max_over_u, max_over_v = s.max(dim=3)[0], s.max(dim=4)[0]
+            else:
+                am_u, am_v = argmax[lvl]
+                max_over_v = torch.gather(s, 4, am_u[:, :, :, 0, :, None].long()).squeeze(4)
+                max_over_u = torch.gather(s, 3, am_v[:, :, :, 0, None, :].long()).squeeze(3)
             # core/corr.py:77-91: reduce over dim=2 (rows u) -> keeps v: sep_u (B,2,wl,h1,w1)
-            sep_u = torch.stack((s.max(dim=3)[0], s.mean(dim=3)), dim=1).permute(0, 1, 4, 2, 3)
+            sep_u = torch.stack((max_over_u, s.mean(dim=3)), dim=1).permute(0, 1, 4, 2, 3)
             # core/corr.py:96-102: reduce over columns v -> keeps u: sep_v (B,2,hl,h1,w1)
-            sep_v = torch.stack((s.max(dim=4)[0], s.mean(dim=4)), dim=1).permute(0, 1, 4, 2, 3)
+            sep_v = torch.stack((max_over_v, s.mean(dim=4)), dim=1).permute(0, 1, 4, 2, 3)
             if attention_weights is not None:
                 att1, att2 = attention_weights
                 a_u = att1(sep_u).softmax(dim=2)          # (B,K',wl,h1,w1)  core/corr.py:116-122
@@ -379,7 +389,7 @@ class CorrBlock1D:
     corr1 (B,dim,W2,H1,W1) and corr2 (B,dim,H2,H1,W1) are pooled by two along the displacement axis into a pyramid
     (avg_pool2d [1,2], core/corr.py:546-550); every level is sampled with grid_sample (bilinear, align_corners=True,
     zero padding) at coords/2^l + dx, dx = -r..r.  coords channel 0 addresses corr1, channel 1 corr2.  For corr1 the
-    reference clamps the *pixel* positions to [-1, 1] before sampling (core/corr.py:585); that is kept.
+    reference clamps the *pixel* positions to [-1, 1] before sampling (core/corr.py:593); that is kept.
     Output channel = level*dim*(2r+1) + d*(2r+1) + k.
     """
 
@@ -410,7 +420,7 @@ class CorrBlock1D:
                 x0 = dx + x / 2 ** i
                 y0 = torch.zeros_like(x0)
                 if which == 0:
-                    x0 = torch.clamp(x0, -1, 1)                       # core/corr.py:585
+                    x0 = torch.clamp(x0, -1, 1)                       # core/corr.py:593
                 grid = torch.cat([2 * x0 / (W - 1) - 1, y0], dim=-1)   # core/corr.py:555-560: y is not normalised
                 smp = F.grid_sample(corr, grid, mode='bilinear', padding_mode='zeros', align_corners=True)
                 per_level.append(smp.view(B, h1, w1, -1))

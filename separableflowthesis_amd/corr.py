@@ -124,7 +124,7 @@ class CorrBlock1D:
     pyramid of permuted copies per block and samples it with grid_sample once per level, volume and flow iteration;
     here the volumes stay in the layout they arrive in, the pyramid is formed on the fly, and one kernel per volume does
     the whole lookup.  The clamp of the sampling positions to [-1, 1] that the reference applies to its first volume only
-    (core/corr.py:585) is reproduced (`clamp_first=False` drops it).
+    (core/corr.py:593) is reproduced (`clamp_first=False` drops it).
     """
 
     def __init__(self, corr1, corr2, num_levels=4, radius=4, clamp_first=True):

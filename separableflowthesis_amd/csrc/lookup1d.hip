@@ -6,7 +6,7 @@
 // zero padding) at x/2^l + k - r, k = 0..2r, where x = coords[b, coord_channel, i, j]:
 //   out[b, l*dim*n + d*n + k, i, j],  n = 2r+1.
 // For its first volume the reference clamps the sampling positions to [-1, 1] before sampling
-// (core/corr.py:585); `clamp_unit` reproduces that.
+// (core/corr.py:593); `clamp_unit` reproduces that.
 //
 // The pyramid is not stored: entry m of level l is the mean of level-0 entries [m*2^l, (m+1)*2^l).  One thread per (b, d, i, j): neighbouring threads are
 // neighbouring image-1 pixels, whose reads of corr[b,d,w,i,j] sit side by side whenever their w agree (smooth flow).

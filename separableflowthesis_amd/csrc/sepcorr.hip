@@ -385,7 +385,9 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                     }
                 } else {
                     float m = -INFINITY, s = 0.f;
-                    int mi = 0x7fffffff;
+                    // starts at the lane's first column: a row without any finite value above -inf (all NaN or
+                    // -inf) then ends up with index 0, as the reference's pre-zeroed argmax does
+                    int mi = vbase + 32 * vcw + 4 * h;
                     if (ragged) {   // wave-uniform: only the last column chunk of a row can be partial
 #pragma unroll
                         for (int r = 0; r < 16; ++r) {
@@ -1836,7 +1838,11 @@ struct ProfRec {
     const char *name;
     hipEvent_t e0, e1;
 };
-bool g_prof_on = false;
+std::atomic<bool> g_prof_on{false};
+// The flag as the current API call saw it on entry: fork/join and every launch bracket of one call agree even if
+// another thread toggles profiling meanwhile.
+thread_local bool t_prof_on = false;
+void api_enter() { t_prof_on = g_prof_on.load(std::memory_order_relaxed); }
 std::mutex g_prof_mu;
 std::vector<ProfRec> g_prof_recs;
 
@@ -1844,7 +1850,7 @@ struct ProfScope {
     ProfRec rec;
     hipStream_t s;
     bool on;
-    ProfScope(const char *name, hipStream_t stream) : s(stream), on(g_prof_on) {
+    ProfScope(const char *name, hipStream_t stream) : s(stream), on(t_prof_on) {
         if (!on) return;
         rec.name = name;
         if (hipEventCreate(&rec.e0) != hipSuccess || hipEventCreate(&rec.e1) != hipSuccess) { on = false; return; }
@@ -2253,7 +2259,7 @@ bool overlap_enabled() {
         const char *e = getenv("SEPCORR_SINGLE_STREAM");
         return !(e && e[0] == '1');
     }();
-    return on && !g_prof_on;   // per-kernel timing wants the kernels one after the other
+    return on && !t_prof_on;   // per-kernel timing wants the kernels one after the other
 }
 
 SideStreams *side_streams() {
@@ -2307,8 +2313,8 @@ int check_workspace(const Dims &d, void *ws, size_t ws_bytes) {
     const size_t need = sepcorr_backward_workspace_bytes(d.B, d.H1, d.W1, d.H2, d.W2, d.C);
     if (need > 0 && (ws == nullptr || ws_bytes < need))
         return fail(SEPCORR_EWORKSPACE, "sepcorr: backward needs %zu bytes of workspace, got %zu", need, ws ? ws_bytes : (size_t)0);
-    if (need > 0 && (reinterpret_cast<uintptr_t>(ws) & 15))
-        return fail(SEPCORR_EWORKSPACE, "sepcorr: workspace must be 16-byte aligned");
+    if (need > 0 && (reinterpret_cast<uintptr_t>(ws) & 255))
+        return fail(SEPCORR_EWORKSPACE, "sepcorr: workspace must be 256-byte aligned");
     return SEPCORR_OK;
 }
 
@@ -2318,6 +2324,7 @@ int check_workspace(const Dims &d, void *ws, size_t ws_bytes) {
 }  // namespace
 
 void *sepcorr_fork(void *user, void **sa, void **sb) {
+    api_enter();
     ForkJoin *fj = new ForkJoin(static_cast<hipStream_t>(user));
     *sa = fj->sa;
     *sb = fj->sb;
@@ -2342,8 +2349,7 @@ int sepcorr_set_contraction(int mode) {
 }
 
 int sepcorr_profile_enable(int on) {
-    std::lock_guard<std::mutex> lk(g_prof_mu);
-    g_prof_on = on != 0;
+    g_prof_on.store(on != 0, std::memory_order_relaxed);
     return SEPCORR_OK;
 }
 
@@ -2370,6 +2376,7 @@ int sepcorr_profile_collect(char *names, size_t names_cap, float *ms, int cap) {
 
 int sepcorr_max_avg_forward(const float *f1, const float *f2, float *out_u, float *out_v, int B, int H1, int W1, int H2,
                             int W2, int C, void *stream) {
+    api_enter();
     REQUIRE_PTR(f1); REQUIRE_PTR(f2); REQUIRE_PTR(out_u); REQUIRE_PTR(out_v);
     const Dims d = {B, H1, W1, H2, W2, C};
     if (int rc = check_dims(d, 2)) return rc;
@@ -2384,6 +2391,7 @@ int sepcorr_max_avg_forward(const float *f1, const float *f2, float *out_u, floa
 
 int sepcorr_max_argmax_avg_forward(const float *f1, const float *f2, float *out_u, float *out_v, int32_t *argmax_u,
                                    int32_t *argmax_v, int B, int H1, int W1, int H2, int W2, int C, void *stream) {
+    api_enter();
     REQUIRE_PTR(f1); REQUIRE_PTR(f2); REQUIRE_PTR(out_u); REQUIRE_PTR(out_v); REQUIRE_PTR(argmax_u); REQUIRE_PTR(argmax_v);
     const Dims d = {B, H1, W1, H2, W2, C};
     if (int rc = check_dims(d, 2)) return rc;
@@ -2398,6 +2406,7 @@ int sepcorr_max_argmax_avg_forward(const float *f1, const float *f2, float *out_
 
 int sepcorr_compression_forward(const float *f1, const float *f2, const float *a_u, const float *a_v, float *comp_u,
                                 float *comp_v, int B, int H1, int W1, int H2, int W2, int C, int K, void *stream) {
+    api_enter();
     REQUIRE_PTR(f1); REQUIRE_PTR(f2); REQUIRE_PTR(a_u); REQUIRE_PTR(a_v); REQUIRE_PTR(comp_u); REQUIRE_PTR(comp_v);
     const Dims d = {B, H1, W1, H2, W2, C};
     if (int rc = check_dims(d, K)) return rc;
@@ -2413,6 +2422,7 @@ size_t sepcorr_backward_workspace_bytes(int B, int H1, int W1, int H2, int W2, i
 int sepcorr_max_argmax_avg_backward(const float *f1, const float *f2, const int32_t *argmax_u, const int32_t *argmax_v,
                                     const float *grad_u, const float *grad_v, float *d_f1, float *d_f2, int B, int H1,
                                     int W1, int H2, int W2, int C, void *workspace, size_t workspace_bytes, void *stream) {
+    api_enter();
     REQUIRE_PTR(f1); REQUIRE_PTR(f2); REQUIRE_PTR(argmax_u); REQUIRE_PTR(argmax_v); REQUIRE_PTR(grad_u); REQUIRE_PTR(grad_v);
     REQUIRE_PTR(d_f1); REQUIRE_PTR(d_f2);
     const Dims d = {B, H1, W1, H2, W2, C};
@@ -2434,6 +2444,7 @@ int sepcorr_compression_backward(const float *f1, const float *f2, const float *
                                  const float *g_cv, float *d_f1, float *d_f2, float *d_a_u, float *d_a_v, int B, int H1,
                                  int W1, int H2, int W2, int C, int K, void *workspace, size_t workspace_bytes,
                                  void *stream) {
+    api_enter();
     REQUIRE_PTR(f1); REQUIRE_PTR(f2); REQUIRE_PTR(a_u); REQUIRE_PTR(a_v); REQUIRE_PTR(g_cu); REQUIRE_PTR(g_cv);
     REQUIRE_PTR(d_a_u); REQUIRE_PTR(d_a_v);
     const Dims d = {B, H1, W1, H2, W2, C};
@@ -2473,6 +2484,7 @@ int sepcorr_fused_backward(const float *f1, const float *f2, const int32_t *argm
                            const float *grad_u, const float *grad_v, const float *a_u, const float *a_v,
                            const float *g_cu, const float *g_cv, float *d_f1, float *d_f2, int B, int H1, int W1, int H2,
                            int W2, int C, int K, void *workspace, size_t workspace_bytes, void *stream) {
+    api_enter();
     REQUIRE_PTR(f1); REQUIRE_PTR(f2); REQUIRE_PTR(argmax_u); REQUIRE_PTR(argmax_v); REQUIRE_PTR(grad_u); REQUIRE_PTR(grad_v);
     REQUIRE_PTR(a_u); REQUIRE_PTR(a_v); REQUIRE_PTR(g_cu); REQUIRE_PTR(g_cv); REQUIRE_PTR(d_f1); REQUIRE_PTR(d_f2);
     const Dims d = {B, H1, W1, H2, W2, C};

@@ -62,3 +62,58 @@ def op_inputs(B, H1, W1, H2, W2, C, seed, scale=True):
 
 def softmax_weights(B, H1, W1, K, L, g):
     return torch.randn(B, H1, W1, K, L, generator=g).softmax(dim=-1).contiguous()
+
+
+def error_report(got, ref64, cpu32, name, max_ratio=2.0):
+    """Gradient parity made explicit: the error of the GPU result against fp64 next to the error the fp32 CPU
+    run of the same full-4D path makes against fp64.
+
+    Asserts the usual bound (assert_close with the RMS-scaled absolute term) and, so that this bound is not
+    just asserted to be fair, that the GPU's RMS error is at most `max_ratio` times the fp32 CPU path's.
+    Prints both errors and how many elements fall outside the plain rtol 1e-4 / atol 1e-5.
+    """
+    g = got.detach().double().cpu()
+    r = ref64.detach().double().cpu()
+    c = cpu32.detach().double().cpu()
+    eg, ec = (g - r).abs(), (c - r).abs()
+    plain = ATOL + RTOL * r.abs()
+    rms = lambda e: float(e.pow(2).mean().sqrt())
+    rep = {"name": name, "rms_ref": rms(r), "gpu_rms_err": rms(eg), "cpu32_rms_err": rms(ec),
+           "gpu_max_err": float(eg.max()), "cpu32_max_err": float(ec.max()),
+           "gpu_outside_plain_tol": int((eg > plain).sum()), "cpu32_outside_plain_tol": int((ec > plain).sum()),
+           "numel": r.numel()}
+    print("parity " + " ".join(f"{k}={v:.4g}" if isinstance(v, float) else f"{k}={v}" for k, v in rep.items()), flush=True)
+    assert_close(got, ref64, name, scale_atol=True)
+    floor = 1e-7 * max(1.0, rep["rms_ref"])   # both exact to the last bit or so: nothing to compare
+    assert rep["gpu_rms_err"] <= max_ratio * max(rep["cpu32_rms_err"], floor), (
+        f"{name}: GPU rms error {rep['gpu_rms_err']:.3g} exceeds {max_ratio} x the fp32 CPU path's {rep['cpu32_rms_err']:.3g}")
+    return rep
+
+
+def native_argmax_levels(fmap1, fmap2, device, num_levels=4):
+    """The argmax tensors the native block's forward pass produces at every pyramid level, for NCHW fmaps as the
+    caller holds them: same inputs, same kernels as AlternateCorrBlockSepflow.separate (core/corr.py:416-425).
+    Returns [(argmax_u, argmax_v)] on the CPU."""
+    import torch.nn.functional as F
+    from separableflowthesis_amd import MemorySaver
+    x1, x2 = fmap1.to(device), fmap2.to(device)
+    f1 = x1.permute(0, 2, 3, 1).contiguous() / torch.sqrt(torch.tensor(x1.shape[1]).float())
+    out = []
+    for _ in range(num_levels):
+        _, _, am_u, am_v = MemorySaver.max_argmax_avg_forward(f1, x2.permute(0, 2, 3, 1).contiguous())
+        out.append((am_u.cpu(), am_v.cpu()))
+        x2 = F.avg_pool2d(x2, 2, stride=2)
+    return out
+
+
+def check_argmax_levels(argmax, block64, name):
+    """Every index of `argmax` (from native_argmax_levels) against the fp64 pyramid of an oracle CorrBlock4D: equal to
+    the oracle's argmax except at near-ties.  Returns the number of near-tie mismatches over all levels."""
+    B, h1, w1, _, _ = block64.shape
+    n = 0
+    for lvl, (corr, (am_u, am_v)) in enumerate(zip(block64.pyramid, argmax)):
+        s64 = corr.detach().reshape(B, h1, w1, corr.shape[2], corr.shape[3])
+        _, _, rau, rav = O.max_argmax_avg_from_volume(s64)
+        n += check_argmax(am_u, rau, s64, 4, f"{name}: level {lvl} argmax_u")
+        n += check_argmax(am_v, rav, s64, 3, f"{name}: level {lvl} argmax_v")
+    return n

@@ -59,6 +59,13 @@ def test_argument_checks_precede_any_launch():
     assert lib.sepcorr_max_argmax_avg_backward(one, one, one, one, one, one, one, one, *args, None, 0, None) == -3
     assert lib.sepcorr_compression_backward(one, one, one, one, one, one, one, one, one, one, *args, 4, one, 16, None) == -3
     assert b"workspace" in lib.sepcorr_last_error()
+    # the documented 256-byte alignment is enforced by every backward entry point
+    big = 1 << 40
+    for ptr in (16, 128, 256 + 64):
+        assert lib.sepcorr_max_argmax_avg_backward(one, one, one, one, one, one, one, one, *args, ctypes.c_void_p(ptr), big, None) == -3
+        assert b"256-byte aligned" in lib.sepcorr_last_error()
+    assert lib.sepcorr_fused_backward(*([one] * 12), *args, 4, ctypes.c_void_p(48), big, None) == -3
+    assert lib.sepcorr_compression_backward(*([one] * 10), *args, 4, ctypes.c_void_p(48), big, None) == -3
 
 
 def test_lookup_argument_checks_precede_any_launch():

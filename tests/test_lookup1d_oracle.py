@@ -61,7 +61,7 @@ def test_affine_profile_is_reproduced_at_every_level_inside_the_volume():
 
 
 def test_first_volume_positions_are_clamped_to_the_unit_interval():
-    # core/corr.py:585: every sampling position of corr1 ends up in [-1, 1], wherever the flow points
+    # core/corr.py:593: every sampling position of corr1 ends up in [-1, 1], wherever the flow points
     B, dim, H, W, r = 1, 1, 6, 8, 2
     c1, c2, g = _volumes(B, dim, H, W, 3)
     coords = _grid(B, H, W) + 3.0

@@ -88,6 +88,37 @@ def test_forward_ties_lowest_index(device):
     f1 = torch.ones(1, 2, 3, 4); f2 = torch.ones(1, 5, 100, 4)
     ou, ov, au, av = _native().max_argmax_avg_forward(f1.to(device), f2.to(device))
     assert torch.all(au == 0) and torch.all(av == 0) and torch.all(ou == 4) and torch.all(ov == 4)
+    # the same where a row is swept in several passes of 256 columns and the last chunk is ragged
+    f1 = torch.ones(1, 2, 3, 8); f2 = torch.ones(1, 3, 300, 8)
+    ou, ov, au, av = _native().max_argmax_avg_forward(f1.to(device), f2.to(device))
+    assert torch.all(au == 0) and torch.all(av == 0) and torch.all(ou == 8) and torch.all(ov == 8)
+    # two equal maxima in different column passes: the lower column wins
+    f2 = torch.zeros(1, 2, 300, 8); f2[0, 0, 290] = 1; f2[0, 0, 17] = 1; f2[0, 1, 299] = 1; f2[0, 1, 256] = 1
+    _, _, au, av = _native().max_argmax_avg_forward(f1.to(device), f2.to(device))
+    assert torch.all(au[..., 0] == 17) and torch.all(au[..., 1] == 256)
+
+
+@pytest.mark.parametrize("shape", [(1, 2, 5, 3, 40, 16), (1, 3, 7, 9, 300, 32), (2, 4, 4, 20, 70, 256)])
+def test_argmax_stays_in_range_without_finite_values(device, shape):
+    """Rows/columns holding only NaN or -inf: the reference's kernel leaves its pre-zeroed argmax at 0
+    (MemorySaver_kernel_forward.cu:990-992 zero-fill, :498-507 strict '>' update); every index must stay a valid
+    index of its axis, so that a consumer may gather with it."""
+    B, H1, W1, H2, W2, C = shape
+    g = torch.Generator().manual_seed(8)
+    f1 = torch.randn(B, H1, W1, C, generator=g)
+    f2 = torch.randn(B, H2, W2, C, generator=g)
+    f1n = f1.clone(); f1n[0, 0, 0] = float("nan")            # pixel (0,0): the whole slice S[0,0,0,:,:] is NaN
+    f2n = f2.clone(); f2n[0, H2 - 1] = float("nan")          # last fmap2 row: NaN for every pixel
+    for a, b in ((f1n, f2), (f1, f2n), (f1n, f2n)):
+        _, _, au, av = _native().max_argmax_avg_forward(a.to(device), b.to(device))
+        assert int(au.min()) >= 0 and int(au.max()) < W2
+        assert int(av.min()) >= 0 and int(av.max()) < H2
+    _, _, au, av = _native().max_argmax_avg_forward(f1n.to(device), f2.to(device))
+    assert torch.all(au[0, 0, 0] == 0) and torch.all(av[0, 0, 0] == 0)
+    # -inf everywhere for one pixel (inf * positive features of one sign)
+    f1i = f1.abs(); f1i[0, 0, 0] = float("-inf")
+    _, _, au, av = _native().max_argmax_avg_forward(f1i.to(device), f2.abs().to(device))
+    assert torch.all(au[0, 0, 0] == 0) and torch.all(av[0, 0, 0] == 0)
 
 
 @pytest.mark.parametrize("shape", SHAPES)
