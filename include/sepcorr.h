@@ -125,6 +125,25 @@ int sepcorr_max_argmax_avg_backward(const float *f1, const float *f2,
                                     void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * The same computation and results as sepcorr_max_argmax_avg_backward, for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  The scratch memory is an array of SEPCORR_STATIC_SCRATCH_BYTES bytes inside the
+ * library's device image (one copy per GPU, held until the process ends) instead of a workspace argument; the
+ * call allocates nothing, creates no streams or events and runs all its kernels on `stream`.
+ *   - Sizes whose sepcorr_backward_workspace_bytes() exceeds SEPCORR_STATIC_SCRATCH_BYTES are refused with
+ *     SEPCORR_EWORKSPACE; use the workspace variant for them.
+ *   - All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different streams or
+ *     threads) race and give undefined results.  Calls on one stream are ordered and safe.  The array's contents
+ *     between calls are unspecified; every call overwrites what it reads.
+ */
+#define SEPCORR_STATIC_SCRATCH_BYTES (64u << 20)
+int sepcorr_max_argmax_avg_backward_static(const float *f1, const float *f2,
+                                           const int32_t *argmax_u, const int32_t *argmax_v,
+                                           const float *grad_u, const float *grad_v,
+                                           float *d_f1, float *d_f2,
+                                           int B, int H1, int W1, int H2, int W2, int C, void *stream);
+
+/*
  * Replaces MemorySaver.compression_backward (MemorySaver_cuda.cpp:80-103 ->
  * MemorySaver_kernel_compression_backward.cu:651-666).  With
  *   G = sum_k a_u[..,k,v]*g_cu[..,k,u] + a_v[..,k,u]*g_cv[..,k,v]

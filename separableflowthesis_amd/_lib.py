@@ -24,6 +24,7 @@ SIGNATURES = {
     "sepcorr_compression_forward": (_I, [_P] * 6 + [_I] * 7 + [_P]),
     "sepcorr_backward_workspace_bytes": (_SZ, [_I] * 6),
     "sepcorr_max_argmax_avg_backward": (_I, [_P] * 8 + [_I] * 6 + [_P, _SZ, _P]),
+    "sepcorr_max_argmax_avg_backward_static": (_I, [_P] * 8 + [_I] * 6 + [_P]),
     "sepcorr_compression_backward": (_I, [_P] * 10 + [_I] * 7 + [_P, _SZ, _P]),
     "sepcorr_fused_backward": (_I, [_P] * 12 + [_I] * 7 + [_P, _SZ, _P]),
     "sepcorr_attention_forward": (_I, [_P] * 4 + [_I] * 5 + [_P]),

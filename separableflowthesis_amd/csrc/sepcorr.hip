@@ -39,6 +39,11 @@
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
+// Scratch memory of sepcorr_max_argmax_avg_backward_static: part of the library's device image, one copy per GPU,
+// held until the process ends.  In host code this name is a handle, not a device address: the address on each
+// device comes from hipGetSymbolAddress (static_scratch() below), and only that pointer is handed to kernels.
+static __device__ __align__(256) unsigned char scratch[SEPCORR_STATIC_SCRATCH_BYTES];
+
 namespace {
 
 constexpr int TP = 32;        // pixels per MFMA column block
@@ -1843,6 +1848,9 @@ std::atomic<bool> g_prof_on{false};
 // another thread toggles profiling meanwhile.
 thread_local bool t_prof_on = false;
 void api_enter() { t_prof_on = g_prof_on.load(std::memory_order_relaxed); }
+// Set for the duration of a call that must not allocate: no side streams or events are created, no stream-ordered
+// memory is taken (the bf16-plane contraction is skipped), no timing events are recorded.
+thread_local bool t_no_alloc = false;
 std::mutex g_prof_mu;
 std::vector<ProfRec> g_prof_recs;
 
@@ -2124,7 +2132,7 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s
         ProfScope ps(GMODE == GMODE_COMP ? "df1_comp" : GMODE == GMODE_BOTH ? "df1_both" : "df1_maxavg", s1); \
         hipLaunchKernelGGL((df1_kernel<GMODE, KC, NCB, CV, MT>), grid, block, lds, s1, a);         \
     } while (0)
-        const bool planes = g_contraction.load(std::memory_order_relaxed) == SEPCORR_CONTRACT_BF16X3 && d.C == 256 &&
+        const bool planes = !t_no_alloc && g_contraction.load(std::memory_order_relaxed) == SEPCORR_CONTRACT_BF16X3 && d.C == 256 &&
                             wg.vpasses == 1 && cvec && (size_t)d.H1 * d.W1 * MAX_K * d.H2 * 4 <= big &&
                             (size_t)d.H2 * nvc_all * BF_CHUNK <= big && (size_t)d.H2 * (2 * MAX_K + 3) * d.H1 * d.W1 * 4 <= big;
         if (planes) {
@@ -2259,7 +2267,7 @@ bool overlap_enabled() {
         const char *e = getenv("SEPCORR_SINGLE_STREAM");
         return !(e && e[0] == '1');
     }();
-    return on && !t_prof_on;   // per-kernel timing wants the kernels one after the other
+    return on && !t_prof_on && !t_no_alloc;   // per-kernel timing wants the kernels one after the other
 }
 
 SideStreams *side_streams() {
@@ -2308,6 +2316,27 @@ struct ForkJoin {
     }
     ~ForkJoin() { (void)join(); }
 };
+
+std::mutex g_scratch_mu;
+void *g_scratch_ptr[64];
+
+// Device address of `scratch` on the current device, resolved once per device.
+int static_scratch(void **out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(SEPCORR_ELAUNCH, "sepcorr: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= 64) return fail(SEPCORR_EINVAL, "sepcorr: device index %d is not supported", dev);
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void *ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr)
+            return fail(SEPCORR_ELAUNCH, "sepcorr: address of the static scratch array on device %d: %s", dev, hipGetErrorString(e));
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return SEPCORR_OK;
+}
 
 int check_workspace(const Dims &d, void *ws, size_t ws_bytes) {
     const size_t need = sepcorr_backward_workspace_bytes(d.B, d.H1, d.W1, d.H2, d.W2, d.C);
@@ -2438,6 +2467,36 @@ int sepcorr_max_argmax_avg_backward(const float *f1, const float *f2, const int3
     const int rc = launch_bwd<GMODE_MAXAVG, 1>(a, d, workspace, fj.sa, fj.user);   // d_f1 aside, d_f2 on the caller's stream
     const int rj = fj.join();
     return rc ? rc : rj;
+}
+
+int sepcorr_max_argmax_avg_backward_static(const float *f1, const float *f2, const int32_t *argmax_u, const int32_t *argmax_v,
+                                           const float *grad_u, const float *grad_v, float *d_f1, float *d_f2, int B, int H1,
+                                           int W1, int H2, int W2, int C, void *stream) {
+    api_enter();
+    REQUIRE_PTR(f1); REQUIRE_PTR(f2); REQUIRE_PTR(argmax_u); REQUIRE_PTR(argmax_v); REQUIRE_PTR(grad_u); REQUIRE_PTR(grad_v);
+    REQUIRE_PTR(d_f1); REQUIRE_PTR(d_f2);
+    const Dims d = {B, H1, W1, H2, W2, C};
+    if (int rc = check_dims(d, 2)) return rc;
+    const size_t need = sepcorr_backward_workspace_bytes(B, H1, W1, H2, W2, C);
+    if (need > (size_t)SEPCORR_STATIC_SCRATCH_BYTES)
+        return fail(SEPCORR_EWORKSPACE,
+                    "sepcorr: these sizes need %zu bytes of scratch, the static array holds %zu: use "
+                    "sepcorr_max_argmax_avg_backward with a workspace", need, (size_t)SEPCORR_STATIC_SCRATCH_BYTES);
+    void *ws = nullptr;
+    if (int rc = static_scratch(&ws)) return rc;
+    struct NoAlloc {   // nothing below may allocate: one stream, fp32 contraction, no timing events
+        bool prof;
+        NoAlloc() : prof(t_prof_on) { t_no_alloc = true; t_prof_on = false; }
+        ~NoAlloc() { t_no_alloc = false; t_prof_on = prof; }
+    } guard;
+    BwdArgs a;
+    memset(&a, 0, sizeof(a));
+    a.xcd_order = xcd_order_enabled();
+    a.f1 = f1; a.f2 = f2; a.am_u = argmax_u; a.am_v = argmax_v; a.g_u = grad_u; a.g_v = grad_v;
+    a.d1 = d_f1; a.d2 = d_f2;
+    a.B = B; a.N1 = H1 * W1; a.H2 = H2; a.W2 = W2; a.C = C; a.KT = 1;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return launch_bwd<GMODE_MAXAVG, 1>(a, d, ws, s, s);
 }
 
 int sepcorr_compression_backward(const float *f1, const float *f2, const float *a_u, const float *a_v, const float *g_cu,

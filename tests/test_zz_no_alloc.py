@@ -1,0 +1,74 @@
+"""The backward entry point that allocates nothing: sepcorr_max_argmax_avg_backward_static.
+
+Its scratch memory is an array inside the library's device image instead of a caller-supplied workspace; results must
+equal those of sepcorr_max_argmax_avg_backward (same kernels, same plan: bit for bit) on calls in a row that share
+the array, the second with a smaller input, and stale contents of the array from the first call must not leak.
+Called through the C ABI.
+"""
+import ctypes
+
+import pytest
+import torch
+
+from separableflowthesis_amd import _lib
+from tests._util import op_inputs
+
+pytestmark = pytest.mark.gpu
+
+LIMIT = 64 << 20   # SEPCORR_STATIC_SCRATCH_BYTES (include/sepcorr.h)
+
+
+def _case(device, B, H1, W1, H2, W2, C, seed):
+    f1, f2, g = op_inputs(B, H1, W1, H2, W2, C, seed)
+    am_u = torch.randint(0, W2, (B, H1, W1, 1, H2), generator=g, dtype=torch.int32)
+    am_v = torch.randint(0, H2, (B, H1, W1, 1, W2), generator=g, dtype=torch.int32)
+    g_u = torch.randn(B, H1, W1, 2, H2, generator=g)
+    g_v = torch.randn(B, H1, W1, 2, W2, generator=g)
+    return [t.to(device) for t in (f1, f2, am_u, am_v, g_u, g_v)]
+
+
+def _both(lib, device, dims, seed):
+    B, H1, W1, H2, W2, C = dims
+    ins = _case(device, *dims, seed)
+    need = lib.sepcorr_backward_workspace_bytes(*dims)
+    assert need <= LIMIT, f"test sizes must fit the static array: {need}"
+    stream = torch.cuda.current_stream().cuda_stream
+    P = lambda t: t.data_ptr()
+    ws = torch.empty(max(need, 256), dtype=torch.uint8, device=device)
+    r1, r2 = torch.empty_like(ins[0]), torch.empty_like(ins[1])
+    _lib.check(lib.sepcorr_max_argmax_avg_backward(*map(P, ins), P(r1), P(r2), *dims, P(ws), need, stream))
+    d1 = torch.full_like(ins[0], float("nan"))
+    d2 = torch.full_like(ins[1], float("nan"))
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    _lib.check(lib.sepcorr_max_argmax_avg_backward_static(*map(P, ins), P(d1), P(d2), *dims, stream))
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before
+    return (d1, d2), (r1, r2), need
+
+
+def test_static_scratch_variant_matches_the_workspace_variant(device):
+    lib = _lib.load()
+    # first a size that uses split partial sums and the transposed weights (C == 256), then a smaller input that
+    # reuses the same array, then the first again
+    shapes = [(2, 24, 64, 24, 64, 256), (1, 11, 36, 6, 20, 64), (2, 24, 64, 24, 64, 256), (1, 9, 16, 9, 16, 256)]
+    used = []
+    for n, dims in enumerate(shapes):
+        got, ref, need = _both(lib, device, dims, seed=100 + n)
+        used.append(need)
+        for g, r, name in zip(got, ref, ("d_f1", "d_f2")):
+            assert torch.isfinite(g).all(), f"call {n} {name}: not fully written"
+            assert torch.equal(g, r), f"call {n} {dims} {name}: max diff {float((g - r).abs().max())}"
+    assert max(used) > 0 and used[1] < used[0]
+
+
+def test_static_scratch_variant_refuses_sizes_beyond_its_array(device):
+    lib = _lib.load()
+    dims = (2, 55, 128, 55, 128, 256)
+    assert lib.sepcorr_backward_workspace_bytes(*dims) > LIMIT
+    one = ctypes.c_void_p(256)   # never dereferenced: the size check comes first
+    rc = lib.sepcorr_max_argmax_avg_backward_static(one, one, one, one, one, one, one, one, *dims, None)
+    assert rc == -3
+    msg = lib.sepcorr_last_error()
+    assert b"static array" in msg and b"sepcorr_max_argmax_avg_backward" in msg
+    assert lib.sepcorr_max_argmax_avg_backward_static(None, one, one, one, one, one, one, one, *dims, None) == -1
