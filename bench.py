@@ -2,15 +2,20 @@
 """Benchmark of the memory-saving correlation separation on one MI355X.
 
 A step is one pass of the hot path over one synthetic batch, called through the C ABI with every
-input already resident in HBM: max/argmax/avg forward, attention-compression forward, compression
-backward, max/avg backward (the default workload, benchmark configuration 4: B=2, C=256, 55x128, K'=4).
+input already resident in HBM.  The headline workload is benchmark configuration 4 (B=2, C=256, 55x128,
+K'=4): max/argmax/avg forward, attention-compression forward, compression backward, max/avg backward.
 Prints ONE JSON line.  `value` is algorithmic TFLOP/s: (contraction passes x 2*B*N1*N2*C) / time,
-with passes = 7 for forward+backward with attention; epilogue flops are not counted.
+with passes = 7 for forward+backward with attention; epilogue flops are not counted.  The same line
+carries a `configs` table with all five benchmark configurations (ms/step, TFLOP/s, fraction of the
+fp32 MFMA peak, peak HBM allocated, dominant-kernel roofline), the CPU baseline (full-4D torch path on
+the host cores, one thread and all threads) and, as extras, the caller-level measurements.
 """
 import argparse
 import ctypes
+import gc
 import json
 import os
+import re
 import sys
 import time
 
@@ -19,6 +24,7 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP32_MFMA_TFLOPS = 157.3   # 256 CU x 256 flop/clk x 2.4 GHz
 METRIC = "fused corr-separation fwd+bwd ms and MFMA TFLOP/s at B=2, C=256, 55×128"
+C = 256
 
 # name -> (B, H, W, K', ops).  ops: f = max/avg(+argmax) fwd, c = compression fwd, C = compression bwd, F = max/avg bwd
 WORKLOADS = {
@@ -28,18 +34,42 @@ WORKLOADS = {
     "cfg4": (2, 55, 128, 4, "fcCF"),
     "cfg5": (1, 136, 240, 4, "fc"),
 }
+OPS_TEXT = "(f=max/argmax/avg fwd, c=compression fwd, C=compression bwd, F=max/avg bwd)"
 PASSES = {"f": 1, "c": 1, "C": 3, "F": 2}
-# contraction passes (units of W = 2*B*N1*N2*C flops) executed by one launch of each kernel
-KERNEL_PASSES = {"df1_both": 1, "df2_both": 1, "fwd_maxavg": 1, "fwd_weighted": 1, "df1_comp": 1, "df2_comp": 1, "df1_maxavg": 1, "df2_maxavg": 1}
-# HBM bytes per launch at cfg4 from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by the factors a
-# 256 MiB device copy gives in the same run (profiles/cfg4_fwd_bwd_kernels.txt); None = not measured
+# kernels that execute one contraction pass (W = 2*B*N1*N2*C flops) per launch
+SWEEP_KERNELS = ("fwd_maxavg", "fwd_weighted", "df1_comp", "df2_comp", "df1_maxavg", "df2_maxavg", "df1_both", "df2_both")
 _MIB = 2 ** 20
-TRAFFIC_BYTES_CFG4 = {"fwd_maxavg": 115.9 * _MIB, "fwd_weighted": 187.6 * _MIB, "df1_comp": 202.6 * _MIB,
-                      "df2_comp": 289.1 * _MIB, "df1_maxavg": 153.4 * _MIB, "df2_maxavg": 203.7 * _MIB,
-                      "df1_both": 232.1 * _MIB, "df2_both": 438.6 * _MIB}
 
 
-def make_inputs(B, H, W, C, Kp, torch):
+def measured_traffic(workload):
+    """HBM bytes per launch by kernel label, from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary committed
+    under profiles/ for this workload (scaled there by what a plain copy of known size reads on the same
+    counters).  Lines of the form `traffic <label> <fetch_KiB> <write_KiB> <MiB>`; {} when there is no summary."""
+    path = os.path.join(ROOT, "profiles", f"{workload}_fwd_bwd_kernels.txt")
+    out = {}
+    if os.path.exists(path):
+        for line in open(path):
+            m = re.match(r"traffic\s+(\S+)\s+([\d.]+)\s+([\d.]+)\s+([\d.]+)\s*$", line)
+            if m:
+                out[m.group(1)] = float(m.group(4)) * _MIB
+    return out
+
+
+def algorithmic_bytes(label, B, N, H, W, Kp):
+    """Bytes a launch must move at least: every input read once, every output written once (fp32/int32)."""
+    feat = B * N * C
+    per_p_u, per_p_v = B * N * H, B * N * W          # one channel of a *_u / *_v tensor
+    if label == "fwd_maxavg":
+        n = 2 * feat + 3 * (per_p_u + per_p_v)         # f1, f2; max, avg, argmax of both volumes
+    elif label == "fwd_weighted":
+        n = 2 * feat + 2 * Kp * (per_p_u + per_p_v)    # f1, f2; K' weights in, K' sums out, both volumes
+    else:
+        fields = {"maxavg": 3, "comp": 2 * Kp, "both": 3 + 2 * Kp}[label.split("_")[1]]
+        n = 2 * feat + fields * (per_p_u + per_p_v)    # one fmap in, one gradient out, the weight fields of dL/dS
+    return 4 * n
+
+
+def make_inputs(B, H, W, Kp, torch):
     """Seeded CPU tensors exactly as the caller builds them (core/corr.py:419-422)."""
     g = torch.Generator().manual_seed(1234)
     fmap1 = torch.randn(B, C, H, W, generator=g)
@@ -54,15 +84,22 @@ def make_inputs(B, H, W, C, Kp, torch):
     return f1, f2, grads, att
 
 
-def cpu_baseline(B, H, W, C, Kp, ops, torch, budget_s=20.0):
-    """The full-4D PyTorch path (oracle restatement of core/corr.py) timed on the host cores.
+# ------------------------------------------------------------------------------------------------
+# CPU baseline: the full-4D PyTorch path (oracle restatement of core/corr.py) on the host cores
+# ------------------------------------------------------------------------------------------------
 
-    Bounded sample: batch 1 of the workload, repeated until ~budget_s of CPU time is spent.
-    """
+def _cpu_step(name, torch, pixel_fraction=1):
+    """One step of workload `name` at batch 1 on the CPU; `pixel_fraction` > 1 keeps every n-th image-1 pixel row
+    (image-1 pixels are independent units of the operator).  Returns a callable and the flops it stands for."""
     from oracle import oracle as O
-    f1, f2, grads, att = make_inputs(1, H, W, C, Kp, torch)
+    _, H, W, Kp, ops = WORKLOADS[name]
+    f1, f2, grads, att = make_inputs(1, H, W, Kp, torch)
+    if pixel_fraction > 1:
+        rows = slice(0, H, pixel_fraction)
+        f1 = f1[:, rows].contiguous()
+        grads = {k: v[:, rows].contiguous() for k, v in grads.items()}
     backward = "C" in ops or "F" in ops
-    threads = torch.get_num_threads()
+    n1 = f1.shape[1] * f1.shape[2]
 
     def once():
         x1 = f1.clone().requires_grad_(backward)
@@ -81,57 +118,241 @@ def cpu_baseline(B, H, W, C, Kp, ops, torch, budget_s=20.0):
             if backward:
                 loss.backward()
 
-    once()  # warm-up (allocator, thread pool)
+    return once, sum(PASSES[o] for o in ops) * 2.0 * n1 * (H * W) * C
+
+
+def _time_cpu(fn, budget_s, max_reps, warm):
+    if warm:
+        fn()
     n, t0 = 0, time.perf_counter()
     while True:
-        once()
+        fn()
         n += 1
         dt = time.perf_counter() - t0
-        if dt >= budget_s or n >= 20:
-            break
-    ms = dt / n * 1e3
-    passes = sum(PASSES[o] for o in ops)
-    flops = passes * 2.0 * 1 * (H * W) ** 2 * C
-    return {
-        "value": round(flops / (ms * 1e-3) / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
-        "ms_per_step": round(ms, 1),
+        if dt >= budget_s or n >= max_reps:
+            return dt / n * 1e3, n
+
+
+def cpu_baseline(torch, headline="cfg4"):
+    """Bounded sample of every workload at batch 1: the headline with all host threads (warm-up + repeats, ~10 s) and
+    with one thread (one repeat), the other configurations once each with all threads; config 5 on every 8th
+    image-1 pixel row (its whole 4D volume is 4.26 GB per copy)."""
+    threads = torch.get_num_threads()
+    fn, flops = _cpu_step(headline, torch)
+    ms_all, n_all = _time_cpu(fn, 10.0, 12, warm=True)
+    torch.set_num_threads(1)
+    try:
+        ms_one, _ = _time_cpu(fn, 0.0, 1, warm=False)
+    finally:
+        torch.set_num_threads(threads)
+    _, H, W, Kp, ops = WORKLOADS[headline]
+    out = {
+        "value": round(flops / (ms_all * 1e-3) / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+        "ms_per_step": round(ms_all, 1),
+        "one_thread": {"value": round(flops / (ms_one * 1e-3) / 1e12, 4), "ms_per_step": round(ms_one, 1), "cores": 1},
+        "host_cpus": os.cpu_count(),
         "sample": f"batch 1 of the workload (B=1, {H}x{W}, C={C}, K'={Kp}), full-4D torch path "
-                  f"{'fwd+bwd via autograd' if backward else 'fwd'}, {n} repeats after 1 warm-up, same algorithmic flop count",
+                  f"{'fwd+bwd via autograd' if 'C' in ops or 'F' in ops else 'fwd'}: {n_all} repeats after 1 warm-up with "
+                  f"{threads} threads, 1 repeat with 1 thread; same algorithmic flop count as the GPU step",
+        "configs": {},
     }
+    for name in sorted(WORKLOADS):
+        if name == headline:
+            out["configs"][name] = {"ms_per_step_b1": round(ms_all, 1), "tflops": out["value"], "cores": threads}
+            continue
+        frac = 8 if name == "cfg5" else 1
+        fn, fl = _cpu_step(name, torch, frac)
+        ms, _ = _time_cpu(fn, 0.0, 1, warm=name != "cfg5")
+        ent = {"ms_per_step_b1": round(ms * frac, 1), "tflops": round(fl / (ms * 1e-3) / 1e12, 4), "cores": threads}
+        if frac > 1:
+            ent["sample"] = f"every {frac}th image-1 pixel row, time scaled by {frac}"
+        out["configs"][name] = ent
+    return out
 
 
-def module_level(B, H, W, C, Kp, torch, dev, reps=5):
-    """The caller's whole separate() over 4 pyramid levels through the drop-in classes (untimed extra):
-    NHWC copies, both operators per level, the fused attention producer and volume assembly, autograd."""
+# ------------------------------------------------------------------------------------------------
+# GPU: one workload through the C ABI
+# ------------------------------------------------------------------------------------------------
+
+class Workload:
+    def __init__(self, name, lib, torch, dev):
+        from separableflowthesis_amd import MemorySaver, _lib
+        self.name, self.lib, self.torch = name, lib, torch
+        B, H, W, Kp, ops = WORKLOADS[name]
+        self.B, self.H, self.W, self.Kp, self.ops = B, H, W, Kp, ops
+        torch.cuda.synchronize()
+        torch.cuda.reset_peak_memory_stats()
+        self.base_alloc = torch.cuda.memory_allocated()
+        f1c, f2c, gr, att = make_inputs(B, H, W, Kp, torch)
+        f1, f2 = f1c.to(dev), f2c.to(dev)
+        gr = {k: v.to(dev) for k, v in gr.items()}
+        E = lambda *s, dt=torch.float32: torch.empty(*s, dtype=dt, device=dev)
+        out_u, out_v = E(B, H, W, 2, H), E(B, H, W, 2, W)
+        am_u, am_v = E(B, H, W, 1, H, dt=torch.int32), E(B, H, W, 1, W, dt=torch.int32)
+        backward = "C" in ops or "F" in ops
+        nws = lib.sepcorr_backward_workspace_bytes(B, H, W, H, W, C) if backward else 0
+        ws = torch.empty(max(nws, 256), dtype=torch.uint8, device=dev)
+        self.workspace_bytes = nws
+        dims = (B, H, W, H, W, C)
+        stream = torch.cuda.current_stream().cuda_stream
+        P = lambda t: t.data_ptr()
+        chk = _lib.check
+
+        def op_f():
+            chk(lib.sepcorr_max_argmax_avg_forward(P(f1), P(f2), P(out_u), P(out_v), P(am_u), P(am_v), *dims, stream))
+
+        op_f()
+        table = {"f": op_f}
+        if Kp:
+            # attention weights as the caller produces them: Conv3d on the (max,avg) volumes, softmax over the
+            # kept axis, back to (B,H1,W1,K',L) (core/corr.py:437-446)
+            with torch.no_grad():
+                a_u = MemorySaver.attention_forward(out_v, att[0].weight.to(dev).contiguous(), att[0].bias.to(dev))
+                a_v = MemorySaver.attention_forward(out_u, att[1].weight.to(dev).contiguous(), att[1].bias.to(dev))
+            cu, cv = E(B, H, W, Kp, H), E(B, H, W, Kp, W)
+            table["c"] = lambda: chk(lib.sepcorr_compression_forward(P(f1), P(f2), P(a_u), P(a_v), P(cu), P(cv), *dims, Kp, stream))
+        if "C" in ops:
+            d1, d2 = E(B, H, W, C), E(B, H, W, C)
+            da_u, da_v = torch.empty_like(a_u), torch.empty_like(a_v)
+            table["C"] = lambda: chk(lib.sepcorr_compression_backward(
+                P(f1), P(f2), P(a_u), P(a_v), P(gr["g_cu"]), P(gr["g_cv"]), P(d1), P(d2), P(da_u), P(da_v), *dims, Kp,
+                P(ws), nws, stream))
+        if "F" in ops:
+            d1b, d2b = E(B, H, W, C), E(B, H, W, C)
+            table["F"] = lambda: chk(lib.sepcorr_max_argmax_avg_backward(
+                P(f1), P(f2), P(am_u), P(am_v), P(gr["g_u"]), P(gr["g_v"]), P(d1b), P(d2b), *dims, P(ws), nws, stream))
+        self.seq = [table[o] for o in ops]
+        self.fused_step = None
+        if "C" in ops and "F" in ops:
+            # The same job through the entry points that have no counterpart in the reference's two-operator API:
+            # weight gradients alone, then one contraction per feature gradient with dL/dS of both operators added
+            # (5 sweeps over the volume instead of 7).
+            def fused_step():
+                table["f"]()
+                table["c"]()
+                chk(lib.sepcorr_compression_backward(P(f1), P(f2), P(a_u), P(a_v), P(gr["g_cu"]), P(gr["g_cv"]),
+                                                     None, None, P(da_u), P(da_v), *dims, Kp, None, 0, stream))
+                chk(lib.sepcorr_fused_backward(P(f1), P(f2), P(am_u), P(am_v), P(gr["g_u"]), P(gr["g_v"]),
+                                               P(a_u), P(a_v), P(gr["g_cu"]), P(gr["g_cv"]), P(d1), P(d2),
+                                               *dims, Kp, P(ws), nws, stream))
+            self.fused_step = fused_step
+
+    def step(self):
+        for fn in self.seq:
+            fn()
+
+    def time(self, fn, steps, warmup):
+        torch = self.torch
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps * 1e3
+
+    def kernel_times(self, fn, profile_steps):
+        """Per-kernel durations: HIP events recorded by the library on the stream each kernel is launched on."""
+        lib, torch = self.lib, self.torch
+        lib.sepcorr_profile_enable(1)
+        for _ in range(profile_steps):
+            fn()
+        torch.cuda.synchronize()
+        cap = 8192
+        names = ctypes.create_string_buffer(1 << 17)
+        tms = (ctypes.c_float * cap)()
+        n = lib.sepcorr_profile_collect(names, len(names), tms, cap)
+        lib.sepcorr_profile_enable(0)
+        per = {}
+        for nm, t in zip(names.value.decode().split("\n")[:n], list(tms)[:n]):
+            per.setdefault(nm, []).append(t)
+        return per
+
+    def report(self, steps, warmup, profile_steps):
+        torch = self.torch
+        B, H, W, Kp, ops = self.B, self.H, self.W, self.Kp, self.ops
+        N = H * W
+        ms = self.time(self.step, steps, warmup)
+        peak = torch.cuda.max_memory_allocated() - self.base_alloc
+        Wf = 2.0 * B * N * N * C
+        traffic = measured_traffic(self.name)
+        kernels = {}
+        for nm, ts in self.kernel_times(self.step, max(1, profile_steps)).items():
+            avg = sum(ts) / len(ts)
+            ent = {"avg_ms": round(avg, 4), "launches_per_step": round(len(ts) / max(1, profile_steps), 2)}
+            if nm in SWEEP_KERNELS:
+                ent["tflops"] = round(Wf / (avg * 1e-3) / 1e12, 2)
+                ent["frac_of_peak"] = round(ent["tflops"] / PEAK_FP32_MFMA_TFLOPS, 4)
+            kernels[nm] = ent
+        dom = max((k for k in kernels if k in SWEEP_KERNELS),
+                  key=lambda k: kernels[k]["avg_ms"] * kernels[k]["launches_per_step"])
+        ach = kernels[dom]["tflops"]
+        passes = sum(PASSES[o] for o in ops)
+        value = passes * Wf / (ms * 1e-3) / 1e12
+        roofline = {"bound": "mfma", "kernel": dom, "achieved": ach, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(ach / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": traffic.get(dom),
+                    "algorithmic_bytes": algorithmic_bytes(dom, B, N, H, W, Kp),
+                    "algorithmic_flop": Wf, "avg_launch_ms": kernels[dom]["avg_ms"]}
+        return {
+            "workload": f"{self.name}: B={B}, C={C}, {H}x{W}, K'={Kp}, ops={ops}",
+            "ms_per_step": round(ms, 4), "tflops": round(value, 3),
+            "frac_of_fp32_mfma_peak": round(value / PEAK_FP32_MFMA_TFLOPS, 4),
+            "contraction_passes": passes, "gflop_per_step": round(passes * Wf / 1e9, 2),
+            "peak_hbm_allocated_mib": round(peak / _MIB, 1),
+            "backward_workspace_mib": round(self.workspace_bytes / _MIB, 1),
+            "volume_4d_never_allocated_mib": round(B * N * N * 4 / _MIB, 1),
+            "roofline": roofline, "kernels": kernels,
+        }
+
+
+# ------------------------------------------------------------------------------------------------
+# caller level (extras, never `value`)
+# ------------------------------------------------------------------------------------------------
+
+def module_level(name, torch, dev, reps=5, backward=True):
+    """The caller's whole separate() over 4 pyramid levels through the drop-in classes: NHWC copies, both operators
+    per level, the attention producer and volume assembly, torch autograd; with the peak memory it allocates next to
+    what the stored 4D pyramid alone would take (the comparison of scripts/test_model.py:320-382 for this block)."""
     from separableflowthesis_amd import AlternateCorrBlockSepflow
+    B, H, W, Kp, _ = WORKLOADS[name]
     g = torch.Generator().manual_seed(1234)
     fmap1 = torch.randn(B, C, H, W, generator=g).to(dev).requires_grad_()
     fmap2 = torch.randn(B, C, H, W, generator=g).to(dev).requires_grad_()
     torch.manual_seed(1234)
     att = tuple(torch.nn.Conv3d(2, Kp, 3, padding=1).to(dev) for _ in range(2)) if Kp else None
 
-    def run(backward):
-        blk = AlternateCorrBlockSepflow(fmap1, fmap2, None, 4, 4, support_backward=backward)
-        c1, c2 = blk(None, sep=True, attention_weights=att)
-        if backward:
-            (c1.sum() + c2.sum()).backward()
+    def run(bw):
+        with torch.set_grad_enabled(bw):
+            blk = AlternateCorrBlockSepflow(fmap1, fmap2, None, 4, 4, support_backward=bw)
+            c1, c2 = blk(None, sep=True, attention_weights=att)
+            if bw:
+                (c1.sum() + c2.sum()).backward()
 
     out = {}
-    for name, bw in (("forward_ms", False), ("forward_backward_ms", True)):
+    for key, bw in (("forward", False), ("forward_backward", True)):
+        if bw and not backward:
+            continue
         for _ in range(2):
             run(bw)
         torch.cuda.synchronize()
+        torch.cuda.reset_peak_memory_stats()
+        base = torch.cuda.memory_allocated()
         t0 = time.perf_counter()
         for _ in range(reps):
             run(bw)
         torch.cuda.synchronize()
-        out[name] = round((time.perf_counter() - t0) / reps * 1e3, 3)
+        out[key + "_ms"] = round((time.perf_counter() - t0) / reps * 1e3, 3)
+        out[key + "_peak_allocated_mib"] = round((torch.cuda.max_memory_allocated() - base) / _MIB, 1)
+    n = H * W
+    out["returned_volumes_mib"] = round(B * 4 * (2 + Kp) * (H + W) * n * 4 / _MIB, 1)
+    out["stored_4d_pyramid_would_take_mib"] = round(B * n * n * 4 * (1 + 1 / 4 + 1 / 16 + 1 / 64) / _MIB, 1)
     out["what"] = f"AlternateCorrBlockSepflow.separate, 4 levels, B={B}, C={C}, {H}x{W}, K'={Kp}, torch autograd around the native ops"
     return out
 
 
-def lookup_level(B, H, W, C, torch, dev, reps=20):
-    """corr_fn(coords) of the block without the 4D volume (untimed extra): 4 levels, radius 4, a smooth flow field.
+def lookup_level(B, H, W, torch, dev, reps=20):
+    """corr_fn(coords) of the block without the 4D volume: 4 levels, radius 4, a smooth flow field; and CorrBlock1D.
     Forward = one gather kernel; backward = grid gradients, d_f1 gather, d_f2 by owner tiles, slice reduction."""
     from separableflowthesis_amd import MemorySaver
     g = torch.Generator().manual_seed(1234)
@@ -157,9 +378,8 @@ def lookup_level(B, H, W, C, torch, dev, reps=20):
 
     fwd = timed(lambda: MemorySaver.lookup_forward(f1, f2s, coords, 4, scale))
     bwd = timed(lambda: MemorySaver.lookup_backward(f1, f2s, coords, up, 4, scale))
-    # the lookup in the two separated volumes (CorrBlock1D): one aggregated channel as in the model, and all 24
     one_d = {}
-    for dim in (1, 24):
+    for dim in (1, 24):   # one aggregated channel as in the model, and all 24 channels of separate()
         c1 = torch.randn(B, dim, W, H, W, generator=g).to(dev)
         c2 = torch.randn(B, dim, H, H, W, generator=g).to(dev)
         u = torch.randn(B, 4 * dim * 9, H, W, generator=g).to(dev)
@@ -173,22 +393,19 @@ def lookup_level(B, H, W, C, torch, dev, reps=20):
             MemorySaver.lookup1d_backward(coords, u, tuple(c2.shape), 1, False, 4, 4)
 
         one_d[f"dim{dim}"] = {"forward_ms": round(timed(f1d), 4), "backward_ms": round(timed(b1d), 4),
-                              "volumes_mib": round((c1.numel() + c2.numel()) * 4 / 2 ** 20, 1)}
+                              "volumes_mib": round((c1.numel() + c2.numel()) * 4 / _MIB, 1)}
         del c1, c2, u
     pts = B * H * W * 4 * 100                       # (pixel, level, grid point) pairs: one C-long dot product each
     alg = (f1.numel() + sum(t.numel() for t in f2s) + coords.numel() + up.numel()) * 4   # up has the output's size
     return {
         "forward_ms": round(fwd, 4), "backward_ms": round(bwd, 4),
         "forward_window_gb_s": round(pts * C * 4 / fwd / 1e6, 1),
-        "forward_gflop_s": round(pts * C * 2 / fwd / 1e6, 1),
-        "forward_algorithmic_mib": round(alg / 2 ** 20, 1),
+        "forward_algorithmic_mib": round(alg / _MIB, 1),
         "forward_hbm_gb_s": round(alg / fwd / 1e6, 1),
         "volumes_1d": one_d,
         "what": f"sepcorr_lookup_forward / sepcorr_lookup_backward, B={B}, C={C}, {H}x{W}, 4 levels, radius 4; "
-                "window = bytes of the fmap2 rows under all windows (one C-long dot product each, 2 flop per 4 bytes; "
-                "the kernel fetches a row once for four neighbouring pixels, so this may exceed the vector cache's "
-                "256 CU x 64 B/clk x 2.4 GHz = 39.3 TB/s); algorithmic = f1 + pyramid + coords + out once; "
-                "volumes_1d = CorrBlock1D on both separated volumes (sepcorr_lookup1d_forward/backward, 4 levels, radius 4)",
+                "window = bytes of the fmap2 rows under all windows; algorithmic = f1 + pyramid + coords + out once; "
+                "volumes_1d = CorrBlock1D on both separated volumes (sepcorr_lookup1d_forward/backward)",
     }
 
 
@@ -197,13 +414,13 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="cfg4", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="cfg4", choices=sorted(WORKLOADS),
+                    help="the workload `value` is quoted on (the headline metric is cfg4)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip the configs table and the caller-level extras")
     ap.add_argument("--profile-steps", type=int, default=5)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three 256 MiB device copies (known traffic) for scaling rocprofv3 FETCH_SIZE/WRITE_SIZE")
-    ap.add_argument("--module-level", action="store_true",
-                    help="measure the caller's whole separate() too even with --no-cpu-baseline")
     ap.add_argument("--only-module-level", action="store_true",
                     help="measure nothing but the caller's whole separate() (for kernel traces of that path)")
     ap.add_argument("--only-lookup", action="store_true", help="run only the pyramid-lookup extra (for profiling)")
@@ -225,59 +442,12 @@ def main():
     torch.cuda.set_device(dev)
 
     B, H, W, Kp, ops = WORKLOADS[args.workload]
-    C = 256
-    N = H * W
     if args.only_lookup:
-        print(json.dumps({"workload": args.workload, "lookup": lookup_level(B, H, W, C, torch, dev)}))
+        print(json.dumps({"workload": args.workload, "lookup": lookup_level(B, H, W, torch, dev)}))
         return
     if args.only_module_level:
-        print(json.dumps({"workload": args.workload, "module_level": module_level(B, H, W, C, Kp, torch, dev)}))
+        print(json.dumps({"workload": args.workload, "module_level": module_level(args.workload, torch, dev)}))
         return
-    f1c, f2c, gr, att = make_inputs(B, H, W, C, Kp, torch)
-    f1, f2 = f1c.to(dev), f2c.to(dev)
-    gr = {k: v.to(dev) for k, v in gr.items()}
-    E = lambda *s, dt=torch.float32: torch.empty(*s, dtype=dt, device=dev)
-    out_u, out_v = E(B, H, W, 2, H), E(B, H, W, 2, W)
-    am_u, am_v = E(B, H, W, 1, H, dt=torch.int32), E(B, H, W, 1, W, dt=torch.int32)
-    d1, d2, d1b, d2b = E(B, H, W, C), E(B, H, W, C), E(B, H, W, C), E(B, H, W, C)
-    nws = lib.sepcorr_backward_workspace_bytes(B, H, W, H, W, C)
-    ws = torch.empty(max(nws, 256), dtype=torch.uint8, device=dev)
-    dims = (B, H, W, H, W, C)
-    stream = torch.cuda.current_stream().cuda_stream
-    P = lambda t: t.data_ptr()
-
-    def op_f():
-        _lib.check(lib.sepcorr_max_argmax_avg_forward(P(f1), P(f2), P(out_u), P(out_v), P(am_u), P(am_v), *dims, stream))
-
-    op_f()
-    if Kp:
-        # attention weights as the caller produces them: Conv3d on the (max,avg) volumes, softmax over the
-        # kept axis, back to (B,H1,W1,K',L) (core/corr.py:437-446)
-        from separableflowthesis_amd import MemorySaver
-        with torch.no_grad():
-            a_u = MemorySaver.attention_forward(out_v, att[0].weight.to(dev).contiguous(), att[0].bias.to(dev))
-            a_v = MemorySaver.attention_forward(out_u, att[1].weight.to(dev).contiguous(), att[1].bias.to(dev))
-        cu, cv = E(B, H, W, Kp, H), E(B, H, W, Kp, W)
-        da_u, da_v = torch.empty_like(a_u), torch.empty_like(a_v)
-
-    def op_c():
-        _lib.check(lib.sepcorr_compression_forward(P(f1), P(f2), P(a_u), P(a_v), P(cu), P(cv), *dims, Kp, stream))
-
-    def op_C():
-        _lib.check(lib.sepcorr_compression_backward(P(f1), P(f2), P(a_u), P(a_v), P(gr["g_cu"]), P(gr["g_cv"]),
-                                                    P(d1), P(d2), P(da_u), P(da_v), *dims, Kp, P(ws), nws, stream))
-
-    def op_F():
-        _lib.check(lib.sepcorr_max_argmax_avg_backward(P(f1), P(f2), P(am_u), P(am_v), P(gr["g_u"]), P(gr["g_v"]),
-                                                       P(d1b), P(d2b), *dims, P(ws), nws, stream))
-
-    table = {"f": op_f, "c": op_c, "C": op_C, "F": op_F}
-    seq = [table[o] for o in ops]
-
-    def step():
-        for fn in seq:
-            fn()
-
     if args.calibrate_copy:
         src = torch.empty(64 * 2**20, dtype=torch.float32, device=dev).normal_()
         dst = torch.empty_like(src)
@@ -286,134 +456,70 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    torch.cuda.reset_peak_memory_stats()
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) / args.steps * 1e3
-
-    # per-kernel durations: HIP events recorded by the library on the launch stream
-    lib.sepcorr_profile_enable(1)
-    for _ in range(max(1, args.profile_steps)):
-        step()
-    torch.cuda.synchronize()
-    cap = 4096
-    names = ctypes.create_string_buffer(1 << 16)
-    tms = (ctypes.c_float * cap)()
-    n = lib.sepcorr_profile_collect(names, len(names), tms, cap)
-    lib.sepcorr_profile_enable(0)
-    per = {}
-    for nm, t in zip(names.value.decode().split("\n")[:n], list(tms)[:n]):
-        per.setdefault(nm, []).append(t)
-    Wf = 2.0 * B * N * N * C
-    kernels = {}
-    for nm, ts in per.items():
-        avg = sum(ts) / len(ts)
-        calls = len(ts) / max(1, args.profile_steps)
-        ent = {"avg_ms": round(avg, 4), "launches_per_step": round(calls, 2)}
-        if nm in KERNEL_PASSES:
-            ent["tflops"] = round(KERNEL_PASSES[nm] * Wf / (avg * 1e-3) / 1e12, 2)
-        kernels[nm] = ent
-    dom = max((k for k in kernels if k in KERNEL_PASSES),
-              key=lambda k: kernels[k]["avg_ms"] * kernels[k]["launches_per_step"])
-    ach = kernels[dom]["tflops"]
-    passes = sum(PASSES[o] for o in ops)
-    value = passes * Wf / (ms * 1e-3) / 1e12
-
+    wl = Workload(args.workload, lib, torch, dev)
+    head = wl.report(args.steps, args.warmup, args.profile_steps)
     out = {
-        "metric": METRIC, "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
+        "metric": METRIC, "value": head["tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": f"{args.workload}: B={B}, C={C}, {H}x{W}, K'={Kp}, ops={ops} "
-                               "(f=max/argmax/avg fwd, c=compression fwd, C=compression bwd, F=max/avg bwd)",
-                   "contraction_passes": passes, "gflop_per_step": round(passes * Wf / 1e9, 2),
-                   "frac_of_fp32_mfma_peak": round(value / PEAK_FP32_MFMA_TFLOPS, 4),
-                   "peak_hbm_allocated_mib": round(torch.cuda.max_memory_allocated() / 2**20, 1),
-                   "volume_4d_never_allocated_mib": round(B * N * N * 4 / 2**20, 1)},
-        "roofline": {"bound": "mfma", "kernel": dom, "achieved": ach, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(ach / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": TRAFFIC_BYTES_CFG4.get(dom) if args.workload == "cfg4" else None},
-        "kernels": kernels,
+        "config": {"workload": head["workload"] + " " + OPS_TEXT,
+                   "contraction_passes": head["contraction_passes"], "gflop_per_step": head["gflop_per_step"],
+                   "frac_of_fp32_mfma_peak": head["frac_of_fp32_mfma_peak"],
+                   "peak_hbm_allocated_mib": head["peak_hbm_allocated_mib"],
+                   "backward_workspace_mib": head["backward_workspace_mib"],
+                   "volume_4d_never_allocated_mib": head["volume_4d_never_allocated_mib"]},
+        "roofline": head["roofline"],
+        "kernels": head["kernels"],
     }
-    fused_step = None
-    if "C" in ops and "F" in ops:
-        # The same job through the entry points that have no counterpart in the reference's two-operator API:
-        # weight gradients alone, then one contraction per feature gradient with dL/dS of both operators added
-        # (5 sweeps over the volume instead of 7).  Reported beside the headline, never as `value`.
-        def fused_step():
-            op_f()
-            op_c()
-            _lib.check(lib.sepcorr_compression_backward(P(f1), P(f2), P(a_u), P(a_v), P(gr["g_cu"]), P(gr["g_cv"]),
-                                                        None, None, P(da_u), P(da_v), *dims, Kp, None, 0, stream))
-            _lib.check(lib.sepcorr_fused_backward(P(f1), P(f2), P(am_u), P(am_v), P(gr["g_u"]), P(gr["g_v"]),
-                                                  P(a_u), P(a_v), P(gr["g_cu"]), P(gr["g_cv"]), P(d1), P(d2),
-                                                  *dims, Kp, P(ws), nws, stream))
-        for _ in range(args.warmup):
-            fused_step()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            fused_step()
-        torch.cuda.synchronize()
-        fms = (time.perf_counter() - t0) / args.steps * 1e3
+    if wl.fused_step is not None:
+        fms = wl.time(wl.fused_step, args.steps, args.warmup)
+        Wf = head["roofline"]["algorithmic_flop"]
         out["fused_level"] = {
             "ms_per_step": round(fms, 4), "contraction_passes_executed": 5,
             "tflops_executed": round(5 * Wf / (fms * 1e-3) / 1e12, 2),
             "what": "same inputs and outputs as the headline step (d_f1, d_f2 are the sums of the two operators' "
                     "gradients), via sepcorr_compression_backward(d_f1=d_f2=NULL) + sepcorr_fused_backward"}
-    # The same headline step with the forward sweeps contracting in three bf16 planes per operand (an option of
-    # this library with the same accuracy bar, see sepcorr_set_contraction).  Reported beside the headline, never
-    # as `value`: the headline arithmetic is fp32 MFMA throughout.
-    prev_mode = lib.sepcorr_set_contraction(1)
-    try:
-        for _ in range(args.warmup):
-            step()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            step()
-        torch.cuda.synchronize()
-        pms = (time.perf_counter() - t0) / args.steps * 1e3
-        lib.sepcorr_profile_enable(1)
-        step()
-        torch.cuda.synchronize()
-        names = ctypes.create_string_buffer(1 << 16)
-        tms = (ctypes.c_float * 4096)()
-        n = lib.sepcorr_profile_collect(names, len(names), tms, 4096)
-        lib.sepcorr_profile_enable(0)
-        pk = {}
-        for nm, t in zip(names.value.decode().split("\n")[:n], list(tms)[:n]):
-            if nm.endswith("bf16x3") or nm.startswith("split_planes") or nm == "df1_reduce_chunks":
-                pk.setdefault(nm, []).append(t)
-        out["bf16_planes"] = {
-            "ms_per_step": round(pms, 4), "tflops_fp32_equivalent": round(passes * Wf / (pms * 1e-3) / 1e12, 2),
-            "kernels_ms": {k: round(sum(v) / len(v), 4) for k, v in pk.items()},
-            "what": "headline step with sepcorr_set_contraction(SEPCORR_CONTRACT_BF16X3): forward-type sweeps "
-                    "(max/argmax/avg, compression forward, attention gradients) and d_f1 in bf16 planes, d_f2 "
-                    "in fp32 MFMA"}
-        if fused_step is not None:
-            for _ in range(args.warmup):
-                fused_step()
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            for _ in range(args.steps):
-                fused_step()
-            torch.cuda.synchronize()
-            out["bf16_planes"]["fused_level_ms_per_step"] = round((time.perf_counter() - t0) / args.steps * 1e3, 4)
-        if not args.no_cpu_baseline or args.module_level:
-            ml = module_level(B, H, W, C, Kp, torch, dev)
-            out["bf16_planes"]["module_level"] = {k: v for k, v in ml.items() if k != "what"}
-    finally:
-        lib.sepcorr_set_contraction(prev_mode)
-    if not args.no_cpu_baseline or args.module_level:
-        out["module_level"] = module_level(B, H, W, C, Kp, torch, dev)
-    if not args.no_cpu_baseline or args.module_level:
-        out["lookup"] = lookup_level(B, H, W, C, torch, dev)
+        # The headline step with the forward sweeps and d_f1 contracting in three bf16 planes per operand: an option
+        # of this library (sepcorr_set_contraction), not the headline arithmetic, which is fp32 MFMA throughout.
+        prev_mode = lib.sepcorr_set_contraction(1)
+        try:
+            pms = wl.time(wl.step, args.steps, args.warmup)
+        finally:
+            lib.sepcorr_set_contraction(prev_mode)
+        out["bf16_planes"] = {"ms_per_step": round(pms, 4),
+                              "what": "optional bf16x3 contraction for the forward sweeps and d_f1 (d_f2 stays fp32 MFMA); "
+                                      "reported for information, never the headline"}
+    del wl
+    gc.collect()
+    torch.cuda.empty_cache()
+
+    if not args.no_extras:
+        # every benchmark configuration, measured in this run (fewer steps than the headline for the small ones is
+        # not needed: all of them take milliseconds)
+        table = {}
+        for name in sorted(WORKLOADS):
+            if name == args.workload:
+                row = dict(head)
+            else:
+                w = Workload(name, lib, torch, dev)
+                row = w.report(min(args.steps, 20), args.warmup, min(args.profile_steps, 3))
+                del w
+                gc.collect()
+                torch.cuda.empty_cache()
+            row["kernels"] = {k: v["avg_ms"] for k, v in row["kernels"].items()}
+            table[name] = row
+        out["configs"] = table
+        out["module_level"] = module_level(args.workload, torch, dev)
+        # peak memory of the block that never stores the volume, next to the stored 4D pyramid, per configuration
+        mem = {}
+        for name in ("cfg3", "cfg4", "cfg5"):
+            m = out["module_level"] if name == args.workload else module_level(name, torch, dev, reps=2, backward=name != "cfg5")
+            mem[name] = {k: v for k, v in m.items() if k.endswith("_mib")}
+            torch.cuda.empty_cache()
+        out["memory"] = mem
+        out["lookup"] = lookup_level(B, H, W, torch, dev)
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(B, H, W, C, Kp, ops, torch)
+        out["cpu_baseline"] = cpu_baseline(torch, args.workload)
     print(json.dumps(out))
 
 
