@@ -36,13 +36,49 @@
 
 #include "sepcorr.h"
 
+// This file is compiled once per part (see the Makefile) so that its many kernel instantiations build in parallel:
+// part 0 holds the C ABI and the state shared by all parts, every other part holds the explicit instantiations of
+// some of the launchers (launch_fwd / launch_bwd) with the kernels they start.  Without SEPCORR_PART the whole
+// library is one translation unit.
+#ifndef SEPCORR_PART
+#define SEPCORR_PART (-1)
+#endif
+#define SEPCORR_IN_PART(n) (SEPCORR_PART < 0 || SEPCORR_PART == (n))
+
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 // Scratch memory of sepcorr_max_argmax_avg_backward_static: part of the library's device image, one copy per GPU,
 // held until the process ends.  In host code this name is a handle, not a device address: the address on each
 // device comes from hipGetSymbolAddress (static_scratch() below), and only that pointer is handed to kernels.
+#if SEPCORR_IN_PART(0)
 static __device__ __align__(256) unsigned char scratch[SEPCORR_STATIC_SCRATCH_BYTES];
+#endif
+
+namespace sepcorr_impl {
+extern thread_local char g_err[256];
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+}  // namespace sepcorr_impl
+using namespace sepcorr_impl;
+
+#if SEPCORR_IN_PART(0)
+namespace sepcorr_impl {
+thread_local char g_err[256] = "";
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+}  // namespace sepcorr_impl
+
+// shared with the other translation units of the library (sepcorr_internal.h)
+int sepcorr_set_error(int code, const char *msg) {
+    snprintf(g_err, sizeof(g_err), "%s", msg);
+    return code;
+}
+#endif
 
 namespace {
 
@@ -51,26 +87,6 @@ constexpr int MAX_W2 = 2048;  // rows beyond 256 columns are swept in passes of 
 constexpr int MAX_C = 1024;
 constexpr int MAX_K = 8;
 constexpr int KCH = 4;        // attention channels handled per launch
-
-thread_local char g_err[256] = "";
-
-int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
-int fail(int code, const char *fmt, ...) {
-    va_list ap;
-    va_start(ap, fmt);
-    vsnprintf(g_err, sizeof(g_err), fmt, ap);
-    va_end(ap);
-    return code;
-}
-}  // namespace
-
-// shared with the other translation units of the library (sepcorr_internal.h)
-int sepcorr_set_error(int code, const char *msg) {
-    snprintf(g_err, sizeof(g_err), "%s", msg);
-    return code;
-}
-
-namespace {
 
 // Row of the 32x32 accumulator held in register r of a lane in half h (lane / 32).
 __device__ __forceinline__ int vmap(int r, int h) { return 8 * (r >> 2) + 4 * h + (r & 3); }
@@ -228,6 +244,8 @@ __device__ __forceinline__ int xcd_contiguous(int bid, int n) {
     return c * q + (c < r ? c : r) + slot;
 }
 
+}  // namespace
+namespace sepcorr_impl {
 struct FwdArgs {
     const float *f1, *f2;
     const char *f2_planes;   // bf16-plane variant: fmap2 split by split_planes_kernel
@@ -245,6 +263,8 @@ struct FwdArgs {
     int stage;         // collect the rows of out_u in LDS and store them coalesced at the end
     int xcd_order;     // map workgroup ids so that each XCD gets a contiguous range
 };
+}  // namespace sepcorr_impl
+namespace {
 
 // CMODE: 0 = any C (scalar loads), 1 = C % 4 == 0 (16-byte loads), 2 = C % 32 == 0 (branch-free fast path),
 //        3 = C == 256 (fast path with the channel loop unrolled: every load offset is an immediate)
@@ -841,6 +861,8 @@ enum { GMODE_MAXAVG = 0, GMODE_COMP = 1, GMODE_BOTH = 2 };
 constexpr bool g_has_comp(int gmode) { return gmode != GMODE_MAXAVG; }
 constexpr bool g_has_maxavg(int gmode) { return gmode != GMODE_COMP; }
 
+}  // namespace
+namespace sepcorr_impl {
 struct BwdArgs {
     const float *f1, *f2;
     const int *am_u, *am_v;          // GMODE_MAXAVG
@@ -859,6 +881,8 @@ struct BwdArgs {
     int accumulate;                  // add to the destination instead of overwriting
     int xcd_order;                   // map workgroup ids so that each XCD gets a contiguous range
 };
+}  // namespace sepcorr_impl
+namespace {
 
 // Weights of one lane that depend on (p, v) and on (p, u).  Members a mode does not use stay unset and
 // cost no registers.
@@ -1818,9 +1842,13 @@ __global__ void __launch_bounds__(256) reduce_splits_kernel(const float *part, f
 // ------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------
+}  // namespace
+namespace sepcorr_impl {
 struct Dims {
     int B, H1, W1, H2, W2, C;
 };
+}  // namespace sepcorr_impl
+namespace {
 
 int check_dims(const Dims &d, int K) {
     if (d.B < 1 || d.H1 < 1 || d.W1 < 1 || d.H2 < 1 || d.W2 < 1 || d.C < 1)
@@ -1839,20 +1867,32 @@ int check_dims(const Dims &d, int K) {
 
 // Optional per-kernel timing: when enabled, every kernel launch is bracketed by HIP events recorded
 // on the stream it is launched on.  Off by default (zero cost: one branch per launch).
+}  // namespace
+namespace sepcorr_impl {
 struct ProfRec {
     const char *name;
     hipEvent_t e0, e1;
 };
-std::atomic<bool> g_prof_on{false};
+extern std::atomic<bool> g_prof_on;
 // The flag as the current API call saw it on entry: fork/join and every launch bracket of one call agree even if
 // another thread toggles profiling meanwhile.
-thread_local bool t_prof_on = false;
-void api_enter() { t_prof_on = g_prof_on.load(std::memory_order_relaxed); }
+extern thread_local bool t_prof_on;
 // Set for the duration of a call that must not allocate: no side streams or events are created, no stream-ordered
 // memory is taken (the bf16-plane contraction is skipped), no timing events are recorded.
+extern thread_local bool t_no_alloc;
+extern std::mutex g_prof_mu;
+extern std::vector<ProfRec> g_prof_recs;
+extern std::atomic<int> g_contraction;
+#if SEPCORR_IN_PART(0)
+std::atomic<bool> g_prof_on{false};
+thread_local bool t_prof_on = false;
 thread_local bool t_no_alloc = false;
 std::mutex g_prof_mu;
 std::vector<ProfRec> g_prof_recs;
+#endif
+}  // namespace sepcorr_impl
+namespace {
+void api_enter() { t_prof_on = g_prof_on.load(std::memory_order_relaxed); }
 
 struct ProfScope {
     ProfRec rec;
@@ -1908,6 +1948,8 @@ WaveGrid wave_grid(int B, int tiles_per_batch, int W2, int H2) {
     return g;
 }
 
+}  // namespace
+namespace sepcorr_impl {
 template <int MODE, int KC, int UR>
 int launch_fwd(FwdArgs a, int B, hipStream_t s) {
     const WaveGrid wg = wave_grid(B, a.tiles_per_batch, a.W2, a.H2);
@@ -1970,6 +2012,29 @@ int launch_fwd(FwdArgs a, int B, hipStream_t s) {
 #undef SEPCORR_FWD
     return check_launch("forward kernel");
 }
+// instantiated in one part each; everywhere else only declared
+#define SEPCORR_FWD_DECL(MODE, KC, UR) extern template int launch_fwd<MODE, KC, UR>(FwdArgs, int, hipStream_t)
+#define SEPCORR_FWD_INST(MODE, KC, UR) template int launch_fwd<MODE, KC, UR>(FwdArgs, int, hipStream_t)
+SEPCORR_FWD_DECL(MODE_MAXAVG, 1, 2);
+SEPCORR_FWD_DECL(MODE_ARGMAX, 1, 2);
+SEPCORR_FWD_DECL(MODE_WEIGHTED, 1, 2);
+SEPCORR_FWD_DECL(MODE_WEIGHTED, 2, 2);
+SEPCORR_FWD_DECL(MODE_WEIGHTED, 3, 1);
+SEPCORR_FWD_DECL(MODE_WEIGHTED, 4, 1);
+#if SEPCORR_IN_PART(1)
+SEPCORR_FWD_INST(MODE_MAXAVG, 1, 2);
+SEPCORR_FWD_INST(MODE_ARGMAX, 1, 2);
+#endif
+#if SEPCORR_IN_PART(2)
+SEPCORR_FWD_INST(MODE_WEIGHTED, 1, 2);
+SEPCORR_FWD_INST(MODE_WEIGHTED, 2, 2);
+#endif
+#if SEPCORR_IN_PART(3)
+SEPCORR_FWD_INST(MODE_WEIGHTED, 3, 1);
+SEPCORR_FWD_INST(MODE_WEIGHTED, 4, 1);
+#endif
+}  // namespace sepcorr_impl
+namespace {
 
 template <int MODE>
 int launch_fwd_weighted_k(const FwdArgs &a, int kc, int B, hipStream_t s) {
@@ -1991,10 +2056,16 @@ int xcd_order_enabled() {
 // most 256 columns).  sepcorr_set_contraction() selects;
 // SEPCORR_BF16X3=1 in the environment makes the planes the initial choice.  fmap2 is split once per call into
 // stream-ordered memory that is released, in stream order, when the call returns.
+}  // namespace
+#if SEPCORR_IN_PART(0)
+namespace sepcorr_impl {
 std::atomic<int> g_contraction{[] {
     const char *e = getenv("SEPCORR_BF16X3");
     return e && e[0] == '1' ? SEPCORR_CONTRACT_BF16X3 : SEPCORR_CONTRACT_FP32;
 }()};
+}  // namespace sepcorr_impl
+#endif
+namespace {
 struct Bf16Planes {
     void *ptr = nullptr;
     int H2p = 0;
@@ -2109,6 +2180,8 @@ size_t df1_uwt_bytes(const Dims &d) {
     return d.C == 256 ? (size_t)d.B * d.H2 * (2 * KCH + 3) * d.H1 * d.W1 * sizeof(float) : 0;
 }
 
+}  // namespace
+namespace sepcorr_impl {
 template <int GMODE, int KC>
 int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s) {
     // s1: stream of the d_f1 kernel; s: stream of the d_f2 kernel and its split reduction
@@ -2248,6 +2321,34 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s
     }
     return SEPCORR_OK;
 }
+#define SEPCORR_BWD_DECL(GMODE, KC) extern template int launch_bwd<GMODE, KC>(BwdArgs, const Dims &, void *, hipStream_t, hipStream_t)
+#define SEPCORR_BWD_INST(GMODE, KC) template int launch_bwd<GMODE, KC>(BwdArgs, const Dims &, void *, hipStream_t, hipStream_t)
+SEPCORR_BWD_DECL(GMODE_MAXAVG, 1);
+SEPCORR_BWD_DECL(GMODE_COMP, 1);
+SEPCORR_BWD_DECL(GMODE_COMP, 2);
+SEPCORR_BWD_DECL(GMODE_COMP, 3);
+SEPCORR_BWD_DECL(GMODE_COMP, 4);
+SEPCORR_BWD_DECL(GMODE_BOTH, 2);
+SEPCORR_BWD_DECL(GMODE_BOTH, 4);
+#if SEPCORR_IN_PART(4)
+SEPCORR_BWD_INST(GMODE_MAXAVG, 1);
+SEPCORR_BWD_INST(GMODE_COMP, 1);
+#endif
+#if SEPCORR_IN_PART(5)
+SEPCORR_BWD_INST(GMODE_COMP, 2);
+SEPCORR_BWD_INST(GMODE_COMP, 3);
+#endif
+#if SEPCORR_IN_PART(6)
+SEPCORR_BWD_INST(GMODE_COMP, 4);
+#endif
+#if SEPCORR_IN_PART(7)
+SEPCORR_BWD_INST(GMODE_BOTH, 2);
+#endif
+#if SEPCORR_IN_PART(8)
+SEPCORR_BWD_INST(GMODE_BOTH, 4);
+#endif
+}  // namespace sepcorr_impl
+namespace {
 
 // The kernels of one backward call are independent of each other (they only read the inputs), so they
 // are issued on separate streams: the tail of one kernel, where part of the chip would idle, is filled
@@ -2317,6 +2418,7 @@ struct ForkJoin {
     ~ForkJoin() { (void)join(); }
 };
 
+#if SEPCORR_IN_PART(0)
 std::mutex g_scratch_mu;
 void *g_scratch_ptr[64];
 
@@ -2337,6 +2439,7 @@ int static_scratch(void **out) {
     *out = g_scratch_ptr[dev];
     return SEPCORR_OK;
 }
+#endif
 
 int check_workspace(const Dims &d, void *ws, size_t ws_bytes) {
     const size_t need = sepcorr_backward_workspace_bytes(d.B, d.H1, d.W1, d.H2, d.W2, d.C);
@@ -2352,6 +2455,7 @@ int check_workspace(const Dims &d, void *ws, size_t ws_bytes) {
 
 }  // namespace
 
+#if SEPCORR_IN_PART(0)
 void *sepcorr_fork(void *user, void **sa, void **sb) {
     api_enter();
     ForkJoin *fj = new ForkJoin(static_cast<hipStream_t>(user));
@@ -2589,3 +2693,4 @@ int sepcorr_fused_backward(const float *f1, const float *f2, const int32_t *argm
 }
 
 }  // extern "C"
+#endif  // part 0
