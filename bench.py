@@ -198,8 +198,13 @@ class Workload:
         P = lambda t: t.data_ptr()
         chk = _lib.check
 
+        nfw = lib.sepcorr_forward_workspace_bytes(*dims, max(Kp, 2))
+        fws = torch.empty(max(nfw, 256), dtype=torch.uint8, device=dev)
+        fwp = P(fws) if nfw else None
+        self.forward_workspace_bytes = nfw
+
         def op_f():
-            chk(lib.sepcorr_max_argmax_avg_forward(P(f1), P(f2), P(out_u), P(out_v), P(am_u), P(am_v), *dims, stream))
+            chk(lib.sepcorr_max_argmax_avg_forward(P(f1), P(f2), P(out_u), P(out_v), P(am_u), P(am_v), *dims, fwp, nfw, stream))
 
         op_f()
         table = {"f": op_f}
@@ -210,7 +215,7 @@ class Workload:
                 a_u = MemorySaver.attention_forward(out_v, att[0].weight.to(dev).contiguous(), att[0].bias.to(dev))
                 a_v = MemorySaver.attention_forward(out_u, att[1].weight.to(dev).contiguous(), att[1].bias.to(dev))
             cu, cv = E(B, H, W, Kp, H), E(B, H, W, Kp, W)
-            table["c"] = lambda: chk(lib.sepcorr_compression_forward(P(f1), P(f2), P(a_u), P(a_v), P(cu), P(cv), *dims, Kp, stream))
+            table["c"] = lambda: chk(lib.sepcorr_compression_forward(P(f1), P(f2), P(a_u), P(a_v), P(cu), P(cv), *dims, Kp, fwp, nfw, stream))
         if "C" in ops:
             d1, d2 = E(B, H, W, C), E(B, H, W, C)
             da_u, da_v = torch.empty_like(a_u), torch.empty_like(a_v)
@@ -231,7 +236,7 @@ class Workload:
                 table["f"]()
                 table["c"]()
                 chk(lib.sepcorr_compression_backward(P(f1), P(f2), P(a_u), P(a_v), P(gr["g_cu"]), P(gr["g_cv"]),
-                                                     None, None, P(da_u), P(da_v), *dims, Kp, None, 0, stream))
+                                                     None, None, P(da_u), P(da_v), *dims, Kp, fwp, nfw, stream))
                 chk(lib.sepcorr_fused_backward(P(f1), P(f2), P(am_u), P(am_v), P(gr["g_u"]), P(gr["g_v"]),
                                                P(a_u), P(a_v), P(gr["g_cu"]), P(gr["g_cv"]), P(d1), P(d2),
                                                *dims, Kp, P(ws), nws, stream))
@@ -301,6 +306,7 @@ class Workload:
             "contraction_passes": passes, "gflop_per_step": round(passes * Wf / 1e9, 2),
             "peak_hbm_allocated_mib": round(peak / _MIB, 1),
             "backward_workspace_mib": round(self.workspace_bytes / _MIB, 1),
+            "forward_workspace_mib": round(self.forward_workspace_bytes / _MIB, 1),
             "volume_4d_never_allocated_mib": round(B * N * N * 4 / _MIB, 1),
             "roofline": roofline, "kernels": kernels,
         }

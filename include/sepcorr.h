@@ -24,6 +24,10 @@
  *    enough that every tensor has fewer than 2^31 elements.
  *  - Backward entry points need scratch memory: query sepcorr_backward_workspace_bytes() and pass a
  *    device buffer of at least that size (256-byte aligned).  Its contents on entry are ignored.
+ *  - Forward entry points take scratch memory optionally (sepcorr_forward_workspace_bytes(), 256-byte aligned,
+ *    contents on entry ignored; NULL is allowed).  With it the sweep is dealt out to the chip in pieces smaller
+ *    than a 32-pixel tile where whole tiles would leave compute units idle (e.g. 440 tiles on 256 units); results
+ *    are deterministic either way and differ from each other only in the rounding of the sums over u.
  */
 #ifndef SEPCORR_H
 #define SEPCORR_H
@@ -82,7 +86,12 @@ int sepcorr_set_contraction(int mode);
  *   out_v[b,i,j,0,v] = max_u S   out_v[b,i,j,1,v] = (sum_u S) / H2      (B,H1,W1,2,W2)
  */
 int sepcorr_max_avg_forward(const float *f1, const float *f2, float *out_u, float *out_v,
-                            int B, int H1, int W1, int H2, int W2, int C, void *stream);
+                            int B, int H1, int W1, int H2, int W2, int C,
+                            void *workspace, size_t workspace_bytes, void *stream);
+
+/* Scratch bytes a forward entry point can make use of for these sizes (K = 2 for the max/avg entry points); 0 when
+ * whole tiles already fill the chip. */
+size_t sepcorr_forward_workspace_bytes(int B, int H1, int W1, int H2, int W2, int C, int K);
 
 /*
  * Replaces MemorySaver.max_argmax_avg_forward (MemorySaver_cuda.cpp:23-34 ->
@@ -92,7 +101,8 @@ int sepcorr_max_avg_forward(const float *f1, const float *f2, float *out_u, floa
  */
 int sepcorr_max_argmax_avg_forward(const float *f1, const float *f2, float *out_u, float *out_v,
                                    int32_t *argmax_u, int32_t *argmax_v,
-                                   int B, int H1, int W1, int H2, int W2, int C, void *stream);
+                                   int B, int H1, int W1, int H2, int W2, int C,
+                                   void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * Replaces MemorySaver.compression_forward (MemorySaver_cuda.cpp:36-53 ->
@@ -103,7 +113,8 @@ int sepcorr_max_argmax_avg_forward(const float *f1, const float *f2, float *out_
  */
 int sepcorr_compression_forward(const float *f1, const float *f2, const float *a_u, const float *a_v,
                                 float *comp_u, float *comp_v,
-                                int B, int H1, int W1, int H2, int W2, int C, int K, void *stream);
+                                int B, int H1, int W1, int H2, int W2, int C, int K,
+                                void *workspace, size_t workspace_bytes, void *stream);
 
 /* Scratch bytes needed by any of the three backward entry points for these sizes (0 is possible). */
 size_t sepcorr_backward_workspace_bytes(int B, int H1, int W1, int H2, int W2, int C);
@@ -130,8 +141,9 @@ int sepcorr_max_argmax_avg_backward(const float *f1, const float *f2,
  * counterpart in the reference.  The scratch memory is an array of SEPCORR_STATIC_SCRATCH_BYTES bytes inside the
  * library's device image (one copy per GPU, held until the process ends) instead of a workspace argument; the
  * call allocates nothing, creates no streams or events and runs all its kernels on `stream`.
- *   - Sizes whose sepcorr_backward_workspace_bytes() exceeds SEPCORR_STATIC_SCRATCH_BYTES are refused with
- *     SEPCORR_EWORKSPACE; use the workspace variant for them.
+ *   - Sizes that need more scratch than SEPCORR_STATIC_SCRATCH_BYTES are refused with SEPCORR_EWORKSPACE; use the
+ *     workspace variant for them.  (Any size whose sepcorr_backward_workspace_bytes() fits is accepted; that figure
+ *     also covers the other backward entry points, so somewhat larger sizes fit as well.)
  *   - All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different streams or
  *     threads) race and give undefined results.  Calls on one stream are ordered and safe.  The array's contents
  *     between calls are unspecified; every call overwrites what it reads.
@@ -149,7 +161,8 @@ int sepcorr_max_argmax_avg_backward_static(const float *f1, const float *f2,
  *   G = sum_k a_u[..,k,v]*g_cu[..,k,u] + a_v[..,k,u]*g_cv[..,k,v]
  *   d_f1 = sum_{u,v} G f2      d_f2 = sum_{i,j} G f1
  *   d_a_u[b,i,j,k,v] = sum_u S * g_cu[b,i,j,k,u]      d_a_v[b,i,j,k,u] = sum_v S * g_cv[b,i,j,k,v]
- * d_f1 and d_f2 may both be NULL: then only d_a_u and d_a_v are computed (one sweep, no workspace needed).
+ * d_f1 and d_f2 may both be NULL: then only d_a_u and d_a_v are computed (one sweep; workspace as for a forward
+ * entry point: optional, sepcorr_forward_workspace_bytes(..., K)).
  */
 int sepcorr_compression_backward(const float *f1, const float *f2, const float *a_u, const float *a_v,
                                  const float *g_cu, const float *g_cv,

@@ -55,6 +55,15 @@ def _workspace(lib, dims, device):
     return ws, n
 
 
+def _fwd_workspace(lib, dims, K, device):
+    """Optional scratch of the forward-type sweeps (lets them use the whole chip when tiles do not divide evenly)."""
+    n = lib.sepcorr_forward_workspace_bytes(*dims, K)
+    if n == 0:
+        return None, None, 0
+    ws = torch.empty(n, dtype=torch.uint8, device=device)
+    return ws, ws.data_ptr(), n
+
+
 def max_avg_forward(img1_features_l0, img2_features_lk):
     """-> [max_avg_output_u (B,H1,W1,2,H2), max_avg_output_v (B,H1,W1,2,W2)]"""
     f1, f2 = img1_features_l0, img2_features_lk
@@ -63,8 +72,9 @@ def max_avg_forward(img1_features_l0, img2_features_lk):
     with torch.cuda.device(f1.device):
         out_u = torch.empty((B, H1, W1, 2, H2), dtype=f1.dtype, device=f1.device)
         out_v = torch.empty((B, H1, W1, 2, W2), dtype=f1.dtype, device=f1.device)
+        ws, wptr, n = _fwd_workspace(lib, (B, H1, W1, H2, W2, C), 2, f1.device)
         _lib.check(lib.sepcorr_max_avg_forward(f1.data_ptr(), f2.data_ptr(), out_u.data_ptr(), out_v.data_ptr(),
-                                               B, H1, W1, H2, W2, C, _stream()))
+                                               B, H1, W1, H2, W2, C, wptr, n, _stream()))
     return [out_u, out_v]
 
 
@@ -78,8 +88,10 @@ def max_argmax_avg_forward(img1_features_l0, img2_features_lk):
         out_v = torch.empty((B, H1, W1, 2, W2), dtype=f1.dtype, device=f1.device)
         am_u = torch.empty((B, H1, W1, 1, H2), dtype=torch.int32, device=f1.device)
         am_v = torch.empty((B, H1, W1, 1, W2), dtype=torch.int32, device=f1.device)
+        ws, wptr, n = _fwd_workspace(lib, (B, H1, W1, H2, W2, C), 2, f1.device)
         _lib.check(lib.sepcorr_max_argmax_avg_forward(f1.data_ptr(), f2.data_ptr(), out_u.data_ptr(), out_v.data_ptr(),
-                                                      am_u.data_ptr(), am_v.data_ptr(), B, H1, W1, H2, W2, C, _stream()))
+                                                      am_u.data_ptr(), am_v.data_ptr(), B, H1, W1, H2, W2, C, wptr, n,
+                                                      _stream()))
     return [out_u, out_v, am_u, am_v]
 
 
@@ -118,9 +130,10 @@ def compression_forward(img1_features_l0, img2_features_lk, attention_weights_u,
     with torch.cuda.device(dev):
         cu = torch.empty((B, H1, W1, K, H2), dtype=f1.dtype, device=dev)
         cv = torch.empty((B, H1, W1, K, W2), dtype=f1.dtype, device=dev)
+        ws, wptr, n = _fwd_workspace(lib, (B, H1, W1, H2, W2, C), K, dev)
         _lib.check(lib.sepcorr_compression_forward(
             f1.data_ptr(), f2.data_ptr(), attention_weights_u.data_ptr(), attention_weights_v.data_ptr(),
-            cu.data_ptr(), cv.data_ptr(), B, H1, W1, H2, W2, C, K, _stream()))
+            cu.data_ptr(), cv.data_ptr(), B, H1, W1, H2, W2, C, K, wptr, n, _stream()))
     return [cu, cv]
 
 
@@ -170,10 +183,11 @@ def compression_weight_gradients(img1_features_l0, img2_features_lk, attention_w
     with torch.cuda.device(dev):
         da_u = torch.empty_like(attention_weights_u)
         da_v = torch.empty_like(attention_weights_v)
+        ws, wptr, n = _fwd_workspace(lib, (B, H1, W1, H2, W2, C), K, dev)
         _lib.check(lib.sepcorr_compression_backward(
             f1.data_ptr(), f2.data_ptr(), attention_weights_u.data_ptr(), attention_weights_v.data_ptr(),
             grad_compressed_output_u.data_ptr(), grad_compressed_output_v.data_ptr(),
-            None, None, da_u.data_ptr(), da_v.data_ptr(), B, H1, W1, H2, W2, C, K, None, 0, _stream()))
+            None, None, da_u.data_ptr(), da_v.data_ptr(), B, H1, W1, H2, W2, C, K, wptr, n, _stream()))
     return [da_u, da_v]
 
 

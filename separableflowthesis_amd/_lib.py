@@ -19,9 +19,10 @@ SIGNATURES = {
     "sepcorr_set_contraction": (_I, [_I]),
     "sepcorr_profile_enable": (_I, [_I]),
     "sepcorr_profile_collect": (_I, [ctypes.c_char_p, _SZ, ctypes.POINTER(ctypes.c_float), _I]),
-    "sepcorr_max_avg_forward": (_I, [_P, _P, _P, _P] + [_I] * 6 + [_P]),
-    "sepcorr_max_argmax_avg_forward": (_I, [_P] * 6 + [_I] * 6 + [_P]),
-    "sepcorr_compression_forward": (_I, [_P] * 6 + [_I] * 7 + [_P]),
+    "sepcorr_max_avg_forward": (_I, [_P, _P, _P, _P] + [_I] * 6 + [_P, _SZ, _P]),
+    "sepcorr_forward_workspace_bytes": (_SZ, [_I] * 7),
+    "sepcorr_max_argmax_avg_forward": (_I, [_P] * 6 + [_I] * 6 + [_P, _SZ, _P]),
+    "sepcorr_compression_forward": (_I, [_P] * 6 + [_I] * 7 + [_P, _SZ, _P]),
     "sepcorr_backward_workspace_bytes": (_SZ, [_I] * 6),
     "sepcorr_max_argmax_avg_backward": (_I, [_P] * 8 + [_I] * 6 + [_P, _SZ, _P]),
     "sepcorr_max_argmax_avg_backward_static": (_I, [_P] * 8 + [_I] * 6 + [_P]),

@@ -151,6 +151,18 @@ __device__ __forceinline__ float buf_load1s(__amdgpu_buffer_rsrc_t r, unsigned b
     return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, byte_off, uniform_off, 0));
 }
 
+// Data handed from one workgroup to another inside a kernel (pieces of a split tile).  The eight L2 caches of the
+// chip are not coherent with each other, and a device-wide fence writes back and invalidates a whole L2; these
+// 16-byte accesses carry the sc0 sc1 bits instead: they go through to the level all compute units share and leave
+// the caches alone.
+constexpr int CPOL_SC0_SC1 = 1 | 16;
+__device__ __forceinline__ void store_shared4(__amdgpu_buffer_rsrc_t r, unsigned byte_off, v4f x) {
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, x), r, byte_off, 0, CPOL_SC0_SC1);
+}
+__device__ __forceinline__ v4f load_shared4(__amdgpu_buffer_rsrc_t r, unsigned byte_off) {
+    return __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, CPOL_SC0_SC1));
+}
+
 __device__ __forceinline__ v16f mfma(float a, float b, v16f c) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
 }
@@ -262,6 +274,18 @@ struct FwdArgs {
     int vpasses;       // passes of 256 columns = ceil(W2 / 256)
     int stage;         // collect the rows of out_u in LDS and store them coalesced at the end
     int xcd_order;     // map workgroup ids so that each XCD gets a contiguous range
+    // Work split finer than a pixel tile.  A tile's sweep is a sequence of steps (one step = the rows all waves of a
+    // workgroup take in at once); the steps of all tiles, laid end to end, are dealt out evenly to the workgroups of
+    // the grid.  A workgroup whose share ends inside a tile leaves the column state of its piece (max / argmax / sum
+    // or the K sums over its rows) in a slot of sk_state; the piece that finishes a tile last adds up all pieces in
+    // row order and writes the finished columns.  sk_total == 0: one whole tile per workgroup, no scratch.
+    int sk_total;      // total steps over all tiles (0 = off)
+    int sk_steps;      // steps per tile
+    float *sk_state;   // [2 * gridDim.x] slots of sk_slot floats: first and last piece of every workgroup
+    int *sk_count;     // [tiles] pieces finished, zero at launch
+    int sk_slot;       // floats per slot
+    void *ws;          // host side only: scratch for the split (NULL: whole tiles)
+    size_t ws_bytes;
 };
 }  // namespace sepcorr_impl
 namespace {
@@ -271,9 +295,13 @@ namespace {
 // WM: 0 = one pass, one row group (both compile-time constants: the lean common case),
 //     1 = row groups enabled (narrow rows), 2 = column passes enabled (rows wider than 256).
 // BF: the experimental bf16-plane contraction (C == 256, one pass, one row group, max/avg modes)
-template <int MODE, int KC, int UR, int CMODE, int WM, bool BF = false>
+// SK: the sweep may be dealt out in pieces of tiles (FwdArgs::sk_total); without it the loop over pieces below runs
+// exactly once with compile-time bounds and costs nothing
+template <int MODE, int KC, int UR, int CMODE, int WM, bool BF = false, bool SK = false>
 __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     static_assert(!BF || (CMODE == 3 && WM <= 1), "bf16 planes: C == 256, one column pass");
+    static_assert(!(BF && SK), "the split is not built for the bf16-plane variant");
+    const int sk_total = SK ? a.sk_total : 0;
     constexpr bool CVEC = CMODE >= 1;
     constexpr int GJ = 2;  // 8-channel slices per prefetch group
     constexpr int NPART = (MODE == MODE_WEIGHTED) ? KC : 3;
@@ -288,8 +316,6 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     const int vcw = RG ? wave % nvc : wave, ug = RG ? wave / nvc : 0;
     const int vpasses = (WM == 2) ? a.vpasses : 1;
     const int wg = a.xcd_order ? xcd_contiguous(blockIdx.x, gridDim.x) : (int)blockIdx.x;
-    const int b = wg / a.tiles_per_batch;
-    const int p0 = (wg % a.tiles_per_batch) * TP;
     const int N1 = a.N1, H2 = a.H2, W2 = a.W2, C = a.C;
     const int LS = BF ? BF_LS : a.CP + 4;
     float *f1s = smem;
@@ -298,6 +324,35 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     constexpr int NCHO = (MODE == MODE_WEIGHTED) ? KC : 2;            // out_u channels of this launch
     float *ostage = part + 2 * UR * NPART * (blockDim.x >> 6) * 32;   // [32 p][NCHO][H2] when a.stage
     int *ostage_am = reinterpret_cast<int *>(ostage + TP * NCHO * a.H2);   // [32 p][H2], MODE_ARGMAX
+
+    // This workgroup's share of the steps of all tiles: [gs0, gs_end).  Without the split it is exactly one tile.
+    // A share is cut into pieces at tile boundaries.  When it ends inside a tile, that last piece (which starts at
+    // the tile's row 0) is done first and the others follow in order: every workgroup of the grid then starts at
+    // row 0 and all of them move down the rows of fmap2 together, so that a row is fetched into an L2 once.
+    const int S = sk_total ? a.sk_steps : 1;
+    const int gs0 = sk_total ? (int)(((long)wg * sk_total) / (int)gridDim.x) : wg;
+    const int gs_end = sk_total ? (int)(((long)(wg + 1) * sk_total) / (int)gridDim.x) : wg + 1;
+    int head = gs_end % S;                              // steps of the piece at the end of the share
+    if (gs_end - head <= gs0) head = 0;                 // (the share lies inside one tile: a single piece)
+    const int body_end = gs_end - head;
+    int cur = gs0;
+    for (int seg_no = 0;; ++seg_no) {
+    int pb, pe;                                         // this piece: steps [pb, pe) of all tiles laid end to end
+    if (seg_no == 0 && head) {
+        pb = body_end; pe = gs_end;
+    } else {
+        if (cur >= body_end) break;
+        pb = cur;
+        pe = min(body_end, (cur / S + 1) * S);
+        cur = pe;
+    }
+    const int tile = pb / S;
+    const int sa = pb - tile * S;                       // first step of this piece within the tile
+    const int sb = pe - tile * S;                       // one past its last step
+    const bool whole = !SK || !sk_total || (sa == 0 && sb == S);
+    const int b = tile / a.tiles_per_batch;
+    const int p0 = (tile % a.tiles_per_batch) * TP;
+    if (seg_no > 0) __syncthreads();   // the previous piece has finished with LDS
 
     {   // stage the f1 tile [TP][CP] (zero padded) into LDS
         const int c4n = a.CP >> 2;
@@ -366,7 +421,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
 
     const int NJ = a.CP >> 3;
     const int NG = (NJ + GJ - 1) / GJ;
-    const int nsteps = ((H2 + UR - 1) / UR + NUG - 1) / NUG;   // steps per wave; rows past H2 are skipped
+    const int nsteps = sk_total ? sb - sa : ((H2 + UR - 1) / UR + NUG - 1) / NUG;   // steps per wave; rows past H2 are skipped
     const int T = nsteps * NG;
 
     v16f acc[UR];
@@ -380,7 +435,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     auto issue = [&](int step, int g, v4f(&buf)[UR][GJ]) {
 #pragma unroll
         for (int r = 0; r < UR; ++r) {
-            const int u = (step * NUG + ug) * UR + r;
+            const int u = ((sa + step) * NUG + ug) * UR + r;
 #pragma unroll
             for (int jj = 0; jj < GJ; ++jj) {
                 const int j = g * GJ + jj;
@@ -394,7 +449,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         float *pb = part + (step & 1) * (UR * NPART * nW * 32);
 #pragma unroll
         for (int ru = 0; ru < UR; ++ru) {
-            const int u = (step * NUG + ug) * UR + ru;
+            const int u = ((sa + step) * NUG + ug) * UR + ru;
             if (u < H2) {
                 if constexpr (MODE == MODE_WEIGHTED) {
 #pragma unroll
@@ -454,7 +509,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         if constexpr (MODE == MODE_WEIGHTED) {
             for (int idx = tid; idx < NUG * UR * KC * 32; idx += blockDim.x) {
                 const int p = idx & 31, k = (idx >> 5) % KC, ru = (idx / (32 * KC)) % UR, g2 = idx / (32 * KC * UR);
-                const int u = (step * NUG + g2) * UR + ru;
+                const int u = ((sa + step) * NUG + g2) * UR + ru;
                 if (u < H2 && p0 + p < N1) {
                     float s = 0.f;
                     for (int w = g2 * nvc; w < (g2 + 1) * nvc; ++w) s += pb[((ru * NPART + k) * nW + w) * 32 + p];
@@ -474,7 +529,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         } else {
             for (int idx = tid; idx < NUG * UR * 32; idx += blockDim.x) {
                 const int p = idx & 31, ru = (idx >> 5) % UR, g2 = idx / (32 * UR);
-                const int u = (step * NUG + g2) * UR + ru;
+                const int u = ((sa + step) * NUG + g2) * UR + ru;
                 if (u < H2 && p0 + p < N1) {
                     const int w0 = g2 * nvc;
                     float m = pb[((ru * NPART + 0) * nW + w0) * 32 + p];
@@ -519,7 +574,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
             if (g == 0) {
 #pragma unroll
                 for (int r = 0; r < UR; ++r) {
-                    const int u = (step * NUG + ug) * UR + r;
+                    const int u = ((sa + step) * NUG + ug) * UR + r;
 #pragma unroll
                     for (int k = 0; k < KC; ++k)
                         wur[r][k] = (pok && u < H2) ? a.wu[(bp * a.KT + a.k0 + k) * H2 + u] : 0.f;
@@ -552,7 +607,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         auto issueB = [&](int step, int J, v4f(&buf)[UR][6]) {
 #pragma unroll
             for (int r = 0; r < UR; ++r) {
-                const unsigned row = (unsigned)((step * NUG + ug) * UR + r) * rowbytes;   // wave-uniform: travels in a scalar register
+                const unsigned row = (unsigned)(((sa + step) * NUG + ug) * UR + r) * rowbytes;   // wave-uniform: travels in a scalar register
 #pragma unroll
                 for (int i = 0; i < 6; ++i) buf[r][i] = buf_load4s(rsrc, lane_off, row + (unsigned)(J * 6 + i) * 1024u);   // i = 2 plane + k-step
             }
@@ -563,7 +618,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                 if (J == 0) {
 #pragma unroll
                     for (int r = 0; r < UR; ++r) {
-                        const int u = min((step * NUG + ug) * UR + r, H2 - 1);
+                        const int u = min(((sa + step) * NUG + ug) * UR + r, H2 - 1);
 #pragma unroll
                         for (int k = 0; k < KC; ++k) wur[r][k] = a.wu[(bp * a.KT + a.k0 + k) * H2 + u];
                     }
@@ -620,7 +675,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         auto issueF = [&](int step, int J, v4f(&buf)[UR][4]) {
 #pragma unroll
             for (int r = 0; r < UR; ++r) {
-                const unsigned off = lane_off + (unsigned)((step * NUG + ug) * UR + r) * rowbytes + (unsigned)J * 128u;
+                const unsigned off = lane_off + (unsigned)(((sa + step) * NUG + ug) * UR + r) * rowbytes + (unsigned)J * 128u;
 #pragma unroll
                 for (int tq = 0; tq < 4; ++tq) {
                     buf[r][tq] = buf_load4(rsrc, off + 16u * tq);
@@ -633,7 +688,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                 if (J == 0) {
 #pragma unroll
                     for (int r = 0; r < UR; ++r) {
-                        const int u = min((step * NUG + ug) * UR + r, H2 - 1);
+                        const int u = min(((sa + step) * NUG + ug) * UR + r, H2 - 1);
 #pragma unroll
                         for (int k = 0; k < KC; ++k) wur[r][k] = a.wu[(bp * a.KT + a.k0 + k) * H2 + u];
                     }
@@ -754,16 +809,31 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     // flush the staged out_u rows: per pixel a contiguous run of NCHO*H2 floats
     if (a.stage && vp == vpasses - 1) {
         __syncthreads();
-        const int runlen = NCHO * H2;
         const int cht = (MODE == MODE_WEIGHTED) ? a.KT : 2, ch0 = (MODE == MODE_WEIGHTED) ? a.k0 : 0;
-        for (int idx = tid; idx < TP * runlen; idx += blockDim.x) {
-            const int p = idx / runlen, o = idx - p * runlen;
-            if (p0 + p < N1) a.out_u[(((size_t)b * N1 + p0 + p) * cht + ch0) * H2 + o] = ostage[idx];
-        }
-        if constexpr (MODE == MODE_ARGMAX) {
-            for (int idx = tid; idx < TP * H2; idx += blockDim.x) {
-                const int p = idx / H2;
-                if (p0 + p < N1) a.am_u[((size_t)b * N1 + p0) * H2 + idx] = ostage_am[idx];
+        if (whole) {
+            const int runlen = NCHO * H2;
+            for (int idx = tid; idx < TP * runlen; idx += blockDim.x) {
+                const int p = idx / runlen, o = idx - p * runlen;
+                if (p0 + p < N1) a.out_u[(((size_t)b * N1 + p0 + p) * cht + ch0) * H2 + o] = ostage[idx];
+            }
+            if constexpr (MODE == MODE_ARGMAX) {
+                for (int idx = tid; idx < TP * H2; idx += blockDim.x) {
+                    const int p = idx / H2;
+                    if (p0 + p < N1) a.am_u[((size_t)b * N1 + p0) * H2 + idx] = ostage_am[idx];
+                }
+            }
+        } else {   // the rows of this piece only: per pixel and channel a run of u1 - u0 floats
+            const int u0 = sa * NUG * UR, nu = min(H2, sb * NUG * UR) - u0;
+            for (int idx = tid; idx < TP * NCHO * nu; idx += blockDim.x) {
+                const int p = idx / (NCHO * nu), rem = idx - p * (NCHO * nu), ch = rem / nu, u = u0 + rem - ch * nu;
+                if (p0 + p < N1)
+                    a.out_u[(((size_t)b * N1 + p0 + p) * cht + ch0 + ch) * H2 + u] = ostage[(p * NCHO + ch) * H2 + u];
+            }
+            if constexpr (MODE == MODE_ARGMAX) {
+                for (int idx = tid; idx < TP * nu; idx += blockDim.x) {
+                    const int p = idx / nu, u = u0 + idx - p * nu;
+                    if (p0 + p < N1) a.am_u[((size_t)b * N1 + p0 + p) * H2 + u] = ostage_am[p * H2 + u];
+                }
             }
         }
     }
@@ -806,6 +876,28 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         }
     }
 
+    // A piece of a tile leaves its column state in this workgroup's slot in register order, sums undivided:
+    // [column chunk][quantity][register group g4][lane][4]: every store of a wave is one contiguous KB
+    if (!whole) {
+        if (ug == 0 && vbase + 32 * vcw < W2) {
+            constexpr int NQ = (MODE == MODE_WEIGHTED) ? KC : 3;
+            const __amdgpu_buffer_rsrc_t rs_sk = make_rsrc(a.sk_state, 2u * gridDim.x * (unsigned)a.sk_slot * 4u);
+            const unsigned base = ((unsigned)(2 * wg + (pb == gs0 ? 0 : 1)) * (unsigned)a.sk_slot +
+                                   (unsigned)((vbase >> 5) + vcw) * (NQ * 1024u) + 4u * lane) * 4u;
+#pragma unroll
+            for (int q = 0; q < NQ; ++q)
+#pragma unroll
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    v4f x;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if constexpr (MODE == MODE_WEIGHTED) x[e] = rv[q][4 * g4 + e];
+                        else x[e] = q == 0 ? vmax[4 * g4 + e] : q == 1 ? __int_as_float(vidx[4 * g4 + e]) : vsum[4 * g4 + e];
+                    }
+                    store_shared4(rs_sk, base + (unsigned)(q * 4 + g4) * 1024u, x);
+                }
+        }
+    } else
     // store the state that was reduced over u: registers 4g..4g+3 hold 4 consecutive columns
     if (pok && ug == 0) {
         if ((W2 & 3) == 0) {   // 16-byte stores (rows of out_v are then 16-byte aligned)
@@ -851,6 +943,74 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         }
     }
     }   // column passes
+
+    if (!whole) {
+        // Publish this piece and find out whether it completes the tile.  The pieces of a tile belong to consecutive
+        // workgroups; a workgroup keeps the first piece of its share in its slot 0 and a later one (which can only be
+        // its last: the tiles between are whole) in its slot 1.
+        const int G = (int)gridDim.x;
+        const long t0 = (long)tile * S, t1 = t0 + S;
+        int wfirst = (int)((t0 * G) / sk_total);                       // the workgroup that holds step t0
+        while (wfirst > 0 && ((long)wfirst * sk_total) / G > t0) --wfirst;
+        while (((long)(wfirst + 1) * sk_total) / G <= t0) ++wfirst;
+        int wlast = wfirst;                                              // the workgroup that holds step t1 - 1
+        while (((long)(wlast + 1) * sk_total) / G < t1) ++wlast;
+        const int npieces = wlast - wfirst + 1;
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's words of the piece have arrived
+        __syncthreads();
+        int *flag = reinterpret_cast<int *>(smem);
+        if (tid == 0) *flag = __hip_atomic_fetch_add(a.sk_count + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        const bool last = *flag == npieces - 1;
+        __syncthreads();
+        if (last) {
+            // Add up the pieces in row order (equal maxima keep the lower row) and write the finished columns.
+            // An item = the 4 consecutive columns a lane holds in one register group of one column chunk.
+            constexpr int NQ = (MODE == MODE_WEIGHTED) ? KC : 3;
+            const __amdgpu_buffer_rsrc_t rs_sk = make_rsrc(a.sk_state, 2u * gridDim.x * (unsigned)a.sk_slot * 4u);
+            const int nchunks = (W2 + 31) >> 5;
+            for (int it = tid; it < nchunks * 256; it += blockDim.x) {
+                const int ln = it & 63, g4 = (it >> 6) & 3, chunk = it >> 8;
+                const int p = ln & 31, v = 32 * chunk + vmap(4 * g4, ln >> 5);
+                v4f acc4[NQ];
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) acc4[q] = v4f{0.f, 0.f, 0.f, 0.f};
+                if constexpr (MODE != MODE_WEIGHTED) acc4[0] = v4f{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+                for (int w = wfirst; w <= wlast; ++w) {
+                    const bool first_piece = ((long)w * sk_total) / G >= t0;   // w's share starts inside this tile
+                    const unsigned base = ((unsigned)(2 * w + (first_piece ? 0 : 1)) * (unsigned)a.sk_slot +
+                                           (unsigned)chunk * (NQ * 1024u) + 4u * ln) * 4u;
+                    v4f x[NQ];
+#pragma unroll
+                    for (int q = 0; q < NQ; ++q) x[q] = load_shared4(rs_sk, base + (unsigned)(q * 4 + g4) * 1024u);
+                    if constexpr (MODE == MODE_WEIGHTED) {
+#pragma unroll
+                        for (int q = 0; q < NQ; ++q) acc4[q] += x[q];
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (x[0][e] > acc4[0][e]) { acc4[0][e] = x[0][e]; acc4[1][e] = x[1][e]; }
+                        acc4[2] += x[2];
+                    }
+                }
+                if (p0 + p >= N1) continue;
+                const size_t o = (size_t)b * N1 + p0 + p;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (v + e >= W2) break;
+                    if constexpr (MODE == MODE_WEIGHTED) {
+#pragma unroll
+                        for (int q = 0; q < NQ; ++q) a.out_v[(o * a.KT + a.k0 + q) * W2 + v + e] = acc4[q][e];
+                    } else {
+                        a.out_v[(o * 2 + 0) * W2 + v + e] = acc4[0][e];
+                        a.out_v[(o * 2 + 1) * W2 + v + e] = acc4[2][e] / (float)H2;
+                        if constexpr (MODE == MODE_ARGMAX) a.am_v[o * W2 + v + e] = __float_as_int(acc4[1][e]);
+                    }
+                }
+            }
+        }
+    }
+    }   // pieces of this workgroup
 }
 
 // ------------------------------------------------------------------------------------------
@@ -1948,6 +2108,50 @@ WaveGrid wave_grid(int B, int tiles_per_batch, int W2, int H2) {
     return g;
 }
 
+__global__ void __launch_bounds__(256) zero_ints_kernel(int *p, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+// How a forward-type sweep is dealt out to workgroups.  Whole tiles (one workgroup each) leave part of the chip idle
+// when the tile count is not close to a multiple of the resident workgroups (440 tiles on 512 places: 86 %); then the
+// steps of all tiles are dealt out evenly instead and pieces of a tile are combined by whichever finishes last.
+struct FwdSplit {
+    bool on;
+    int G, S;          // workgroups, steps per tile
+    long T;            // steps in total
+    size_t count_bytes, slot_floats, bytes;   // scratch: counters, one slot, everything
+};
+constexpr int kCUs = 256;
+FwdSplit fwd_split(int tiles, int H2, int W2, int rows_per_step, int nq, int wgs_per_cu) {
+    FwdSplit f;
+    f.S = (H2 + rows_per_step - 1) / rows_per_step;
+    f.T = (long)tiles * f.S;
+    const long places = (long)kCUs * wgs_per_cu;
+    const double plain = (double)tiles / (double)(((tiles + places - 1) / places) * places);
+    f.G = (int)(f.T < places ? f.T : places);
+    const double split = (double)f.T / (double)(((f.T + f.G - 1) / f.G) * f.G);
+    f.on = f.S >= 2 && f.T < (1L << 30) && split > plain + 0.04;
+    f.count_bytes = ((size_t)tiles * sizeof(int) + 255) & ~(size_t)255;
+    f.slot_floats = (size_t)nq * 1024 * ((W2 + 31) / 32);   // [column chunk][quantity][4 register groups][64 lanes][4]
+    f.bytes = f.on ? f.count_bytes + 2 * (size_t)f.G * f.slot_floats * sizeof(float) : 0;
+    return f;
+}
+// Upper bound of the scratch any forward-type sweep of these sizes asks for (channels of the widest launch).
+size_t fwd_split_bytes(int B, int H1, int W1, int H2, int W2, int K) {
+    const int tpb = (H1 * W1 + TP - 1) / TP;
+    const WaveGrid wg = wave_grid(B, tpb, W2, H2);
+    const int nW = wg.nvc * wg.nug;
+    const int nq = K > 3 ? (K < KCH ? K : KCH) : 3;
+    size_t best = 0;
+    for (int ur = 1; ur <= 2; ++ur)
+        for (int per = 1; per <= (nW <= 4 ? 2 : 1); ++per) {
+            const FwdSplit f = fwd_split(B * tpb, H2, W2, ur * wg.nug, nq, per);
+            if (f.bytes > best) best = f.bytes;
+        }
+    return best;
+}
+
 }  // namespace
 namespace sepcorr_impl {
 template <int MODE, int KC, int UR>
@@ -1967,12 +2171,27 @@ int launch_fwd(FwdArgs a, int B, hipStream_t s) {
         const size_t merge = wg.nug > 1 ? (size_t)wg.nvc * NPART * 16 * 64 * sizeof(float) : 0;
         if (lds < merge) lds = merge;
     }
-    const dim3 grid(B * a.tiles_per_batch), block(64 * nW);
+    dim3 grid(B * a.tiles_per_batch);
+    const dim3 block(64 * nW);
+    a.sk_total = 0;
+    if (a.ws != nullptr && !a.f2_planes) {
+        const FwdSplit f = fwd_split(B * a.tiles_per_batch, a.H2, a.W2, UR * wg.nug, NPART, (nW <= 4 && lds <= 80 * 1024) ? 2 : 1);
+        if (f.on && f.bytes <= a.ws_bytes) {
+            a.sk_total = (int)f.T;
+            a.sk_steps = f.S;
+            a.sk_count = static_cast<int *>(a.ws);
+            a.sk_state = reinterpret_cast<float *>(static_cast<char *>(a.ws) + f.count_bytes);
+            a.sk_slot = (int)f.slot_floats;
+            grid = dim3(f.G);
+            const int n = B * a.tiles_per_batch;
+            hipLaunchKernelGGL(zero_ints_kernel, dim3((n + 255) / 256), dim3(256), 0, s, a.sk_count, n);
+        }
+    }
     const size_t f2_batch_bytes = (size_t)a.H2 * a.W2 * a.C * sizeof(float);
     const int cmode = (a.C % 32 == 0 && f2_batch_bytes <= (1u << 30)) ? (a.C == 256 ? 3 : 2) : (a.C % 4 == 0 ? 1 : 0);
 #define SEPCORR_FWD(CV, RGV)                                                      \
     do {                                                                         \
-        auto k = fwd_kernel<MODE, KC, UR, CV, RGV>;                              \
+        auto k = a.sk_total ? fwd_kernel<MODE, KC, UR, CV, RGV, false, true> : fwd_kernel<MODE, KC, UR, CV, RGV>; \
         if (int rc = set_lds(k, lds)) return rc;                                 \
         ProfScope ps(MODE == MODE_WEIGHTED ? "fwd_weighted" : "fwd_maxavg", s);  \
         hipLaunchKernelGGL(k, grid, block, lds, s, a);                           \
@@ -2023,14 +2242,20 @@ SEPCORR_FWD_DECL(MODE_WEIGHTED, 3, 1);
 SEPCORR_FWD_DECL(MODE_WEIGHTED, 4, 1);
 #if SEPCORR_IN_PART(1)
 SEPCORR_FWD_INST(MODE_MAXAVG, 1, 2);
-SEPCORR_FWD_INST(MODE_ARGMAX, 1, 2);
 #endif
 #if SEPCORR_IN_PART(2)
-SEPCORR_FWD_INST(MODE_WEIGHTED, 1, 2);
-SEPCORR_FWD_INST(MODE_WEIGHTED, 2, 2);
+SEPCORR_FWD_INST(MODE_ARGMAX, 1, 2);
 #endif
 #if SEPCORR_IN_PART(3)
+SEPCORR_FWD_INST(MODE_WEIGHTED, 1, 2);
+#endif
+#if SEPCORR_IN_PART(4)
+SEPCORR_FWD_INST(MODE_WEIGHTED, 2, 2);
+#endif
+#if SEPCORR_IN_PART(5)
 SEPCORR_FWD_INST(MODE_WEIGHTED, 3, 1);
+#endif
+#if SEPCORR_IN_PART(6)
 SEPCORR_FWD_INST(MODE_WEIGHTED, 4, 1);
 #endif
 }  // namespace sepcorr_impl
@@ -2105,10 +2330,11 @@ FwdArgs fwd_args(const Dims &d) {
 
 // sum_v S wv[k,v] -> out_u[k,u];  sum_u S wu[k,u] -> out_v[k,v]  for K channels, KCH per launch
 int weighted_forward(const Dims &d, const float *f1, const float *f2, const float *wv, const float *wu, float *out_u,
-                     float *out_v, int K, hipStream_t s) {
+                     float *out_v, int K, void *ws, size_t ws_bytes, hipStream_t s) {
     FwdArgs a = fwd_args(d);
     a.f1 = f1; a.f2 = f2; a.wv = wv; a.wu = wu; a.out_u = out_u; a.out_v = out_v;
     a.KT = K;
+    a.ws = ws; a.ws_bytes = ws_bytes;
     Bf16Planes planes;
     if (int rc = planes.make(d, f2, s)) return rc;
     a.f2_planes = static_cast<const char *>(planes.ptr);
@@ -2177,7 +2403,8 @@ size_t df2_part_bytes(const Dims &d) {
     return (bytes + 255) & ~(size_t)255;
 }
 size_t df1_uwt_bytes(const Dims &d) {
-    return d.C == 256 ? (size_t)d.B * d.H2 * (2 * KCH + 3) * d.H1 * d.W1 * sizeof(float) : 0;
+    const size_t bytes = d.C == 256 ? (size_t)d.B * d.H2 * (2 * KCH + 3) * d.H1 * d.W1 * sizeof(float) : 0;
+    return (bytes + 255) & ~(size_t)255;
 }
 
 }  // namespace
@@ -2330,21 +2557,21 @@ SEPCORR_BWD_DECL(GMODE_COMP, 3);
 SEPCORR_BWD_DECL(GMODE_COMP, 4);
 SEPCORR_BWD_DECL(GMODE_BOTH, 2);
 SEPCORR_BWD_DECL(GMODE_BOTH, 4);
-#if SEPCORR_IN_PART(4)
+#if SEPCORR_IN_PART(7)
 SEPCORR_BWD_INST(GMODE_MAXAVG, 1);
 SEPCORR_BWD_INST(GMODE_COMP, 1);
 #endif
-#if SEPCORR_IN_PART(5)
+#if SEPCORR_IN_PART(8)
 SEPCORR_BWD_INST(GMODE_COMP, 2);
 SEPCORR_BWD_INST(GMODE_COMP, 3);
 #endif
-#if SEPCORR_IN_PART(6)
+#if SEPCORR_IN_PART(9)
 SEPCORR_BWD_INST(GMODE_COMP, 4);
 #endif
-#if SEPCORR_IN_PART(7)
+#if SEPCORR_IN_PART(10)
 SEPCORR_BWD_INST(GMODE_BOTH, 2);
 #endif
-#if SEPCORR_IN_PART(8)
+#if SEPCORR_IN_PART(11)
 SEPCORR_BWD_INST(GMODE_BOTH, 4);
 #endif
 }  // namespace sepcorr_impl
@@ -2450,6 +2677,16 @@ int check_workspace(const Dims &d, void *ws, size_t ws_bytes) {
     return SEPCORR_OK;
 }
 
+// Scratch of a forward-type sweep is optional: without it every workgroup takes a whole pixel tile.
+int check_fwd_workspace(const Dims &d, int K, void *ws, size_t ws_bytes) {
+    if (ws == nullptr) return SEPCORR_OK;
+    const size_t need = fwd_split_bytes(d.B, d.H1, d.W1, d.H2, d.W2, K);
+    if (ws_bytes < need)
+        return fail(SEPCORR_EWORKSPACE, "sepcorr: forward workspace of %zu bytes given, %zu needed (or pass NULL)", ws_bytes, need);
+    if (reinterpret_cast<uintptr_t>(ws) & 255) return fail(SEPCORR_EWORKSPACE, "sepcorr: workspace must be 256-byte aligned");
+    return SEPCORR_OK;
+}
+
 #define REQUIRE_PTR(p) \
     if ((p) == nullptr) return fail(SEPCORR_EINVAL, "sepcorr: argument %s is NULL", #p)
 
@@ -2474,7 +2711,7 @@ int sepcorr_join(void *token) {
 extern "C" {
 
 const char *sepcorr_last_error(void) { return g_err; }
-int sepcorr_abi_version(void) { return 1; }
+int sepcorr_abi_version(void) { return 2; }
 
 int sepcorr_set_contraction(int mode) {
     if (mode != SEPCORR_CONTRACT_FP32 && mode != SEPCORR_CONTRACT_BF16X3) return g_contraction.load();
@@ -2507,13 +2744,20 @@ int sepcorr_profile_collect(char *names, size_t names_cap, float *ms, int cap) {
     return n;
 }
 
+size_t sepcorr_forward_workspace_bytes(int B, int H1, int W1, int H2, int W2, int C, int K) {
+    if (B < 1 || H1 < 1 || W1 < 1 || H2 < 1 || W2 < 1 || C < 1 || K < 1) return 0;
+    return fwd_split_bytes(B, H1, W1, H2, W2, K);
+}
+
 int sepcorr_max_avg_forward(const float *f1, const float *f2, float *out_u, float *out_v, int B, int H1, int W1, int H2,
-                            int W2, int C, void *stream) {
+                            int W2, int C, void *workspace, size_t workspace_bytes, void *stream) {
     api_enter();
     REQUIRE_PTR(f1); REQUIRE_PTR(f2); REQUIRE_PTR(out_u); REQUIRE_PTR(out_v);
     const Dims d = {B, H1, W1, H2, W2, C};
     if (int rc = check_dims(d, 2)) return rc;
+    if (int rc = check_fwd_workspace(d, 2, workspace, workspace_bytes)) return rc;
     FwdArgs a = fwd_args(d);
+    a.ws = workspace; a.ws_bytes = workspace_bytes;
     a.f1 = f1; a.f2 = f2; a.out_u = out_u; a.out_v = out_v;
     Bf16Planes planes;
     if (int rc = planes.make(d, f2, static_cast<hipStream_t>(stream))) return rc;
@@ -2523,12 +2767,15 @@ int sepcorr_max_avg_forward(const float *f1, const float *f2, float *out_u, floa
 }
 
 int sepcorr_max_argmax_avg_forward(const float *f1, const float *f2, float *out_u, float *out_v, int32_t *argmax_u,
-                                   int32_t *argmax_v, int B, int H1, int W1, int H2, int W2, int C, void *stream) {
+                                   int32_t *argmax_v, int B, int H1, int W1, int H2, int W2, int C, void *workspace,
+                                   size_t workspace_bytes, void *stream) {
     api_enter();
     REQUIRE_PTR(f1); REQUIRE_PTR(f2); REQUIRE_PTR(out_u); REQUIRE_PTR(out_v); REQUIRE_PTR(argmax_u); REQUIRE_PTR(argmax_v);
     const Dims d = {B, H1, W1, H2, W2, C};
     if (int rc = check_dims(d, 2)) return rc;
+    if (int rc = check_fwd_workspace(d, 2, workspace, workspace_bytes)) return rc;
     FwdArgs a = fwd_args(d);
+    a.ws = workspace; a.ws_bytes = workspace_bytes;
     a.f1 = f1; a.f2 = f2; a.out_u = out_u; a.out_v = out_v; a.am_u = argmax_u; a.am_v = argmax_v;
     Bf16Planes planes;
     if (int rc = planes.make(d, f2, static_cast<hipStream_t>(stream))) return rc;
@@ -2538,18 +2785,21 @@ int sepcorr_max_argmax_avg_forward(const float *f1, const float *f2, float *out_
 }
 
 int sepcorr_compression_forward(const float *f1, const float *f2, const float *a_u, const float *a_v, float *comp_u,
-                                float *comp_v, int B, int H1, int W1, int H2, int W2, int C, int K, void *stream) {
+                                float *comp_v, int B, int H1, int W1, int H2, int W2, int C, int K, void *workspace,
+                                size_t workspace_bytes, void *stream) {
     api_enter();
     REQUIRE_PTR(f1); REQUIRE_PTR(f2); REQUIRE_PTR(a_u); REQUIRE_PTR(a_v); REQUIRE_PTR(comp_u); REQUIRE_PTR(comp_v);
     const Dims d = {B, H1, W1, H2, W2, C};
     if (int rc = check_dims(d, K)) return rc;
-    return weighted_forward(d, f1, f2, a_u, a_v, comp_u, comp_v, K, static_cast<hipStream_t>(stream));
+    if (int rc = check_fwd_workspace(d, K, workspace, workspace_bytes)) return rc;
+    return weighted_forward(d, f1, f2, a_u, a_v, comp_u, comp_v, K, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
 size_t sepcorr_backward_workspace_bytes(int B, int H1, int W1, int H2, int W2, int C) {
     if (B < 1 || H1 < 1 || W1 < 1 || H2 < 1 || W2 < 1 || C < 1) return 0;
     const Dims d = {B, H1, W1, H2, W2, C};
-    return df2_part_bytes(d) + df1_uwt_bytes(d);
+    // split partial sums of d_f2, transposed weights of d_f1, scratch of the weight-gradient sweep
+    return df2_part_bytes(d) + df1_uwt_bytes(d) + fwd_split_bytes(B, H1, W1, H2, W2, MAX_K);
 }
 
 int sepcorr_max_argmax_avg_backward(const float *f1, const float *f2, const int32_t *argmax_u, const int32_t *argmax_v,
@@ -2581,7 +2831,7 @@ int sepcorr_max_argmax_avg_backward_static(const float *f1, const float *f2, con
     REQUIRE_PTR(d_f1); REQUIRE_PTR(d_f2);
     const Dims d = {B, H1, W1, H2, W2, C};
     if (int rc = check_dims(d, 2)) return rc;
-    const size_t need = sepcorr_backward_workspace_bytes(B, H1, W1, H2, W2, C);
+    const size_t need = df2_part_bytes(d) + df1_uwt_bytes(d);   // what this entry point itself uses of the workspace
     if (need > (size_t)SEPCORR_STATIC_SCRATCH_BYTES)
         return fail(SEPCORR_EWORKSPACE,
                     "sepcorr: these sizes need %zu bytes of scratch, the static array holds %zu: use "
@@ -2614,12 +2864,15 @@ int sepcorr_compression_backward(const float *f1, const float *f2, const float *
     if (int rc = check_dims(d, K)) return rc;
     if ((d_f1 == nullptr) != (d_f2 == nullptr))
         return fail(SEPCORR_EINVAL, "sepcorr: d_f1 and d_f2 must be given together or both be NULL");
-    if (d_f1 == nullptr)   // only the gradients of the weights: one sweep, no scratch
-        return weighted_forward(d, f1, f2, g_cv, g_cu, d_a_v, d_a_u, K, static_cast<hipStream_t>(stream));
+    if (d_f1 == nullptr) {   // only the gradients of the weights: one sweep; its scratch is optional like the forward's
+        if (int rc = check_fwd_workspace(d, K, workspace, workspace_bytes)) return rc;
+        return weighted_forward(d, f1, f2, g_cv, g_cu, d_a_v, d_a_u, K, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+    }
     if (int rc = check_workspace(d, workspace, workspace_bytes)) return rc;
     ForkJoin fj(static_cast<hipStream_t>(stream));
     // d_a_v[k,u] = sum_v S g_cv[k,v];  d_a_u[k,v] = sum_u S g_cu[k,u]: the forward's weighted sums
-    int rc = weighted_forward(d, f1, f2, g_cv, g_cu, d_a_v, d_a_u, K, fj.user);
+    char *fwd_ws = static_cast<char *>(workspace) + df2_part_bytes(d) + df1_uwt_bytes(d);
+    int rc = weighted_forward(d, f1, f2, g_cv, g_cu, d_a_v, d_a_u, K, fwd_ws, fwd_split_bytes(B, H1, W1, H2, W2, MAX_K), fj.user);
     BwdArgs a;
     memset(&a, 0, sizeof(a));
     a.xcd_order = xcd_order_enabled();

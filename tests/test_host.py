@@ -22,7 +22,7 @@ def header_symbols():
 
 def test_library_exports_every_declared_symbol():
     names = header_symbols()
-    assert len(names) == 25
+    assert len(names) == 26
     lib = ctypes.CDLL(_lib.LIB_PATH)
     for n in names:
         assert hasattr(lib, n), f"libsepcorr.so does not export {n}"
@@ -31,29 +31,39 @@ def test_library_exports_every_declared_symbol():
 
 def test_abi_version_and_workspace_query():
     lib = _lib.load()
-    assert lib.sepcorr_abi_version() == 1
+    assert lib.sepcorr_abi_version() == 2
     assert lib.sepcorr_backward_workspace_bytes(0, 1, 1, 1, 1, 1) == 0
     n = lib.sepcorr_backward_workspace_bytes(2, 55, 128, 55, 128, 256)
-    # d_f2-sized partial buffers, then (C == 256) the transposed copy of up to 11 weight fields of size B*H2*N1
+    # d_f2-sized partial buffers, then (C == 256) the transposed copy of up to 11 weight fields of size B*H2*N1,
+    # then what the weight-gradient sweep of the compression backward can use (a forward-type sweep)
     part, fields = 2 * 55 * 128 * 256 * 4, 11 * 2 * 55 * (55 * 128) * 4
-    assert n > fields and (n - fields) % part == 0
-    assert lib.sepcorr_backward_workspace_bytes(2, 55, 128, 55, 128, 64) % (2 * 55 * 128 * 64 * 4) == 0
+    fwd = lib.sepcorr_forward_workspace_bytes(2, 55, 128, 55, 128, 256, 8)
+    assert fwd > 0 and fwd % 256 == 0
+    assert n > fields + fwd and (n - fields - fwd) % part == 0
+    # whole tiles fill the chip: nothing to gain from scratch (1020 tiles of 8 waves on 256 units)
+    assert lib.sepcorr_forward_workspace_bytes(1, 136, 240, 136, 240, 256, 4) == 0
+    assert lib.sepcorr_forward_workspace_bytes(0, 1, 1, 1, 1, 1, 2) == 0
+    one = ctypes.c_void_p(256)
+    args = (2, 55, 128, 55, 128, 256)
+    assert lib.sepcorr_max_avg_forward(one, one, one, one, *args, one, 16, None) == -3          # too small
+    assert lib.sepcorr_max_avg_forward(one, one, one, one, *args, ctypes.c_void_p(260), 1 << 40, None) == -3   # misaligned
+    assert b"aligned" in lib.sepcorr_last_error()
 
 
 def test_argument_checks_precede_any_launch():
     lib = _lib.load()
     one = ctypes.c_void_p(256)   # never dereferenced: every call below must fail in the checks
-    assert lib.sepcorr_max_avg_forward(None, one, one, one, 1, 1, 1, 1, 1, 1, None) == -1
+    assert lib.sepcorr_max_avg_forward(None, one, one, one, 1, 1, 1, 1, 1, 1, None, 0, None) == -1
     assert b"NULL" in lib.sepcorr_last_error()
-    assert lib.sepcorr_max_avg_forward(one, one, one, one, 1, 1, 1, 1, 0, 1, None) == -1
-    assert lib.sepcorr_max_avg_forward(one, one, one, one, 1, 1, 1, 1, 2049, 1, None) == -1
+    assert lib.sepcorr_max_avg_forward(one, one, one, one, 1, 1, 1, 1, 0, 1, None, 0, None) == -1
+    assert lib.sepcorr_max_avg_forward(one, one, one, one, 1, 1, 1, 1, 2049, 1, None, 0, None) == -1
     assert b"W2=2049" in lib.sepcorr_last_error()
-    assert lib.sepcorr_max_argmax_avg_forward(one, one, one, one, one, one, 1, 1, 1, 1, 1, 2000, None) == -1
-    assert lib.sepcorr_compression_forward(one, one, one, one, one, one, 1, 1, 1, 1, 1, 1, 9, None) == -1
+    assert lib.sepcorr_max_argmax_avg_forward(one, one, one, one, one, one, 1, 1, 1, 1, 1, 2000, None, 0, None) == -1
+    assert lib.sepcorr_compression_forward(one, one, one, one, one, one, 1, 1, 1, 1, 1, 1, 9, None, 0, None) == -1
     assert b"K=9" in lib.sepcorr_last_error()
-    assert lib.sepcorr_compression_forward(one, one, one, one, one, one, 1, 1, 1, 1, 1, 1, 0, None) == -1
+    assert lib.sepcorr_compression_forward(one, one, one, one, one, one, 1, 1, 1, 1, 1, 1, 0, None, 0, None) == -1
     # 2^31 elements
-    assert lib.sepcorr_max_avg_forward(one, one, one, one, 64, 1024, 1024, 4, 4, 64, None) == -1
+    assert lib.sepcorr_max_avg_forward(one, one, one, one, 64, 1024, 1024, 4, 4, 64, None, 0, None) == -1
     # workspace missing / too small
     args = (2, 55, 128, 55, 128, 256)
     assert lib.sepcorr_max_argmax_avg_backward(one, one, one, one, one, one, one, one, *args, None, 0, None) == -3
