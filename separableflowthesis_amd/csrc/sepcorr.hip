@@ -1040,6 +1040,11 @@ struct BwdArgs {
     int nsplit, tiles_per_split;     // df2: split of the p range
     int accumulate;                  // add to the destination instead of overwriting
     int xcd_order;                   // map workgroup ids so that each XCD gets a contiguous range
+    // d_f1 dealt out in pieces of tiles, as the forward sweeps are (FwdArgs::sk_*): a piece leaves its partial
+    // [32 pixels][channels] sum in a slot; whichever piece of a tile finishes last adds them up in row order.
+    int sk_total, sk_steps;          // steps (rows per wave) over all tiles, per tile; 0 = whole tiles
+    float *sk_state;                 // [2 * grid.x * grid.y] slots of 32 x (128 * NCB) floats
+    int *sk_count;                   // [tiles * grid.y], zero at launch
 };
 }  // namespace sepcorr_impl
 namespace {
@@ -1155,7 +1160,7 @@ __device__ __forceinline__ float gval(const VW<GMODE, KC> &wv, const UW<GMODE, K
 // through the scalar offset and the column within the group and the channel block through the immediate.
 // (fp32 MFMA and vector instructions share the SIMD's arithmetic lanes here: every vector instruction in the
 // loop costs its issue time, nothing hides behind the matrix work.)
-template <int GMODE, int KC, int NCB, bool CVEC, int MAXT, bool FAST = false>
+template <int GMODE, int KC, int NCB, bool CVEC, int MAXT, bool FAST = false, bool SK = false>
 __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
     static_assert(!FAST || (CVEC && NCB == 2), "fast loads: 16-byte loads, 256 channels per workgroup");
     constexpr int GS = 2;            // MFMA k-steps (pairs of v) per prefetch group
@@ -1170,10 +1175,35 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
     const int nvc = a.nvc, NUG = nW / nvc;
     const int vcw = wave % nvc, ug = wave / nvc;
     const int wg = a.xcd_order ? xcd_contiguous(blockIdx.x, gridDim.x) : (int)blockIdx.x;
-    const int b = wg / a.tiles_per_batch;
-    const int p0 = (wg % a.tiles_per_batch) * TP;
     const int cb0 = blockIdx.y * CB;
     const int N1 = a.N1, H2 = a.H2, W2 = a.W2, C = a.C;
+
+    // This workgroup's share of the steps (one step = one row per wave) of all tiles, cut into pieces at tile
+    // boundaries; the piece at the end of the share starts at row 0 and is done first (see fwd_kernel).
+    const int sk_total = SK ? a.sk_total : 0;
+    const int S = sk_total ? a.sk_steps : 1;
+    const int gs0 = sk_total ? (int)(((long)wg * sk_total) / (int)gridDim.x) : wg;
+    const int gs_end = sk_total ? (int)(((long)(wg + 1) * sk_total) / (int)gridDim.x) : wg + 1;
+    int head = gs_end % S;
+    if (gs_end - head <= gs0) head = 0;
+    const int body_end = gs_end - head;
+    int cur = gs0;
+    for (int seg_no = 0;; ++seg_no) {
+    int pb, pe;
+    if (seg_no == 0 && head) {
+        pb = body_end; pe = gs_end;
+    } else {
+        if (cur >= body_end) break;
+        pb = cur;
+        pe = min(body_end, (cur / S + 1) * S);
+        cur = pe;
+    }
+    const int tile = pb / S;
+    const int sa = pb - tile * S, sb = pe - tile * S;
+    const bool whole = !SK || !sk_total || (sa == 0 && sb == S);
+    const int u_begin = sk_total ? sa * NUG : 0, u_end = sk_total ? min(H2, sb * NUG) : H2;   // this piece's rows
+    const int b = tile / a.tiles_per_batch;
+    const int p0 = (tile % a.tiles_per_batch) * TP;
     const int pix = p0 + pl;
     const bool pok = pix < N1;
     const size_t bp = (size_t)b * N1 + (pok ? pix : 0);
@@ -1282,14 +1312,15 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
             return w;
         }
     };
-    UW<GMODE, KC> wu_n = load_uw_row(min(ug, H2 - 1));
+    const int ufirst = u_begin + ug;   // this wave's first row
+    UW<GMODE, KC> wu_n = load_uw_row(min(ufirst, H2 - 1));
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
         // no mask: a column outside the image has an all-zero A operand and the column of a pixel outside the
         // image is never stored; the weights behind both are those of real entries, so G stays finite
-        G[r] = gval<GMODE, KC>(wv[r], wu_n, ug, vmap(r, 0), true);
+        G[r] = gval<GMODE, KC>(wv[r], wu_n, ufirst, vmap(r, 0), true);
     }
-    UW<GMODE, KC> wu_next = load_uw_row(min(ug + NUG, H2 - 1));
+    UW<GMODE, KC> wu_next = load_uw_row(min(ufirst + NUG, H2 - 1));
     auto compute = [&](int u, int g, v4f(&buf)[GS][NCB]) {
         static_assert(GS == 2, "two G values are produced per group");
         if (g == 0) {
@@ -1327,15 +1358,15 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
     v4f ring[NB][GS][NCB];
 #pragma unroll
     for (int k = 0; k < NB - 1; ++k) {
-        issue(min(ug, H2 - 1), k, ring[k]);
+        issue(min(ufirst, H2 - 1), k, ring[k]);
         __builtin_amdgcn_sched_barrier(0);
     }
-    for (int u = ug; u < H2; u += NUG) {
+    for (int u = ufirst; u < u_end; u += NUG) {
 #pragma unroll
         for (int g = 0; g < NG; ++g) {
             constexpr int AHEAD = NB - 1;
             if (g + AHEAD < NG) issue(u, g + AHEAD, ring[(g + AHEAD) % NB]);
-            else if (u + NUG < H2) issue(u + NUG, g + AHEAD - NG, ring[(g + AHEAD) % NB]);
+            else if (u + NUG < u_end) issue(u + NUG, g + AHEAD - NG, ring[(g + AHEAD) % NB]);
             __builtin_amdgcn_sched_barrier(0);
             compute(u, g, ring[g % NB]);
             __builtin_amdgcn_sched_barrier(0);
@@ -1344,28 +1375,68 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
 
     }   // column passes
 
-    // sum the per-wave partials in wave order through LDS, then store coalesced
-    for (int w = 0; w < nW; ++w) {
-        if (wave == w) {
+    // every wave leaves its partial [32][CB] in its own LDS region; they are added in wave order on the way out
+    {
+        float *mine = smem + wave * (TP * RS);
 #pragma unroll
-            for (int cb = 0; cb < NCB; ++cb)
+        for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    v4f x = {acc[cb][0][r], acc[cb][1][r], acc[cb][2][r], acc[cb][3][r]};
-                    v4f *d = reinterpret_cast<v4f *>(smem + pl * RS + 128 * cb + 4 * vmap(r, h));
-                    if (w > 0) x += *d;
-                    *d = x;
-                }
+            for (int r = 0; r < 16; ++r) {
+                const v4f x = {acc[cb][0][r], acc[cb][1][r], acc[cb][2][r], acc[cb][3][r]};
+                *reinterpret_cast<v4f *>(mine + pl * RS + 128 * cb + 4 * vmap(r, h)) = x;
+            }
+    }
+    __syncthreads();
+    auto tile_sum = [&](int row, int c) {
+        v4f x = *reinterpret_cast<const v4f *>(smem + row * RS + c);
+        for (int w = 1; w < nW; ++w) x += *reinterpret_cast<const v4f *>(smem + w * (TP * RS) + row * RS + c);
+        return x;
+    };
+    if (whole) {
+        for (int idx = tid; idx < TP * (CB / 4); idx += blockDim.x) {
+            const int row = idx / (CB / 4), c = (idx - row * (CB / 4)) * 4;
+            if (p0 + row < N1)
+                store4<CVEC>(a.d1 + ((size_t)b * N1 + p0 + row) * C, cb0 + c, C, tile_sum(row, c), a.accumulate != 0);
         }
+    } else {
+        // leave the piece's partial sum [32][CB] in this workgroup's slot, then see whether it completes the tile
+        constexpr unsigned SLOT = TP * CB;
+        const unsigned nslots = 2u * gridDim.x * gridDim.y;
+        const __amdgpu_buffer_rsrc_t rs_sk = make_rsrc(a.sk_state, nslots * SLOT * 4u);
+        const unsigned mine = (2u * (wg * gridDim.y + blockIdx.y) + (pb == gs0 ? 0u : 1u)) * SLOT;
+        for (int idx = tid; idx < TP * (CB / 4); idx += blockDim.x) {
+            const int row = idx / (CB / 4), c = (idx - row * (CB / 4)) * 4;
+            store_shared4(rs_sk, (mine + (unsigned)idx * 4u) * 4u, tile_sum(row, c));
+        }
+        const int G = (int)gridDim.x;
+        const long t0 = (long)tile * S, t1 = t0 + S;
+        int wfirst = (int)((t0 * G) / sk_total);                         // the workgroup that holds step t0
+        while (wfirst > 0 && ((long)wfirst * sk_total) / G > t0) --wfirst;
+        while (((long)(wfirst + 1) * sk_total) / G <= t0) ++wfirst;
+        int wlast = wfirst;                                              // the workgroup that holds step t1 - 1
+        while (((long)(wlast + 1) * sk_total) / G < t1) ++wlast;
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's part of the piece has arrived
         __syncthreads();
-    }
-    for (int idx = tid; idx < TP * (CB / 4); idx += blockDim.x) {
-        const int row = idx / (CB / 4), c = (idx - row * (CB / 4)) * 4;
-        if (p0 + row < N1) {
-            const v4f x = *reinterpret_cast<const v4f *>(smem + row * RS + c);
-            store4<CVEC>(a.d1 + ((size_t)b * N1 + p0 + row) * C, cb0 + c, C, x, a.accumulate != 0);
+        int *flag = reinterpret_cast<int *>(smem);
+        if (tid == 0)
+            *flag = __hip_atomic_fetch_add(a.sk_count + tile * gridDim.y + blockIdx.y, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        const bool last = *flag == wlast - wfirst;
+        if (last) {   // pieces in row order, after what the destination already holds when accumulating
+            for (int idx = tid; idx < TP * (CB / 4); idx += blockDim.x) {
+                const int row = idx / (CB / 4), c = (idx - row * (CB / 4)) * 4;
+                v4f x = {0.f, 0.f, 0.f, 0.f};
+                for (int w = wfirst; w <= wlast; ++w) {
+                    const bool first_piece = ((long)w * sk_total) / G >= t0;
+                    const unsigned slot = (2u * (w * gridDim.y + blockIdx.y) + (first_piece ? 0u : 1u)) * SLOT;
+                    x += load_shared4(rs_sk, (slot + (unsigned)idx * 4u) * 4u);
+                }
+                if (p0 + row < N1) store4<CVEC>(a.d1 + ((size_t)b * N1 + p0 + row) * C, cb0 + c, C, x, a.accumulate != 0);
+            }
         }
     }
+    if constexpr (SK) __syncthreads();   // the next piece reuses the LDS tile
+    }   // pieces of this workgroup
 }
 
 // d_f2[q, c] = sum_p G[p,q] f1[p,c].  Each wave is an independent task (b, split, u, v chunk);
@@ -2407,6 +2478,63 @@ size_t df1_uwt_bytes(const Dims &d) {
     return (bytes + 255) & ~(size_t)255;
 }
 
+// Launch shape of d_f1 and how it is dealt out (as fwd_split): whole tiles on one workgroup per CU, or the steps of
+// all tiles shared evenly, pieces of a tile leaving partial [32][channels] sums that the last one adds up.
+struct Df1Shape {
+    WaveGrid wg;
+    int nW, ncb, cblocks;
+    bool split;
+    int G, S;
+    long T;
+    size_t count_bytes, bytes;
+};
+Df1Shape df1_shape(const Dims &d) {
+    Df1Shape f;
+    const int tpb = (d.H1 * d.W1 + TP - 1) / TP, tiles = d.B * tpb;
+    f.wg = wave_grid(d.B, tpb, d.W2, d.H2);
+    if (f.wg.nvc * f.wg.nug > 4) f.wg.nug = 4 / f.wg.nvc > 0 ? 4 / f.wg.nvc : 1;   // d_f1 runs one wave per SIMD
+    f.nW = f.wg.nvc * f.wg.nug;
+    // more than 4 waves share the register file two to a SIMD: halve the channel block
+    f.ncb = (d.C <= 128 || f.nW > 4) ? 1 : 2;
+    f.cblocks = (d.C + 128 * f.ncb - 1) / (128 * f.ncb);
+    f.S = (d.H2 + f.wg.nug - 1) / f.wg.nug;
+    f.T = (long)tiles * f.S;
+    const long places = kCUs / f.cblocks > 0 ? kCUs / f.cblocks : 1;
+    const double plain = (double)tiles / (double)(((tiles + places - 1) / places) * places);
+    f.G = (int)(f.T < places ? f.T : places);
+    const double split = (double)f.T / (double)(((f.T + f.G - 1) / f.G) * f.G);
+    f.split = d.C % 4 == 0 && f.S >= 2 && f.T < (1L << 30) && split > plain + 0.04;
+    f.count_bytes = ((size_t)tiles * f.cblocks * sizeof(int) + 255) & ~(size_t)255;
+    f.bytes = f.split ? f.count_bytes + 2 * (size_t)f.G * f.cblocks * TP * 128 * f.ncb * sizeof(float) : 0;
+    return f;
+}
+
+// Layout of a backward call's workspace.  Regions: split partial sums of d_f2; transposed (p,u) weights of d_f1 and,
+// behind them, the pieces of a split d_f1; scratch of the weight-gradient sweep (a forward-type sweep).  When any
+// kernel is dealt out in pieces the call keeps to one stream (such kernels want the whole chip), its kernels run one
+// after the other, and the regions of different kernels share the same memory.
+struct BwdWs {
+    bool aliased;
+    size_t off_uwt, off_df1sk, fwd_bytes, own_total, total;   // own_total: without the weight-gradient sweep
+};
+BwdWs bwd_ws(const Dims &d) {
+    BwdWs w;
+    const size_t part = df2_part_bytes(d), uwt = df1_uwt_bytes(d), sk = df1_shape(d).bytes;
+    w.fwd_bytes = fwd_split_bytes(d.B, d.H1, d.W1, d.H2, d.W2, MAX_K);
+    w.aliased = sk > 0 || w.fwd_bytes > 0;
+    if (w.aliased) {
+        w.off_uwt = 0;
+        w.off_df1sk = uwt;
+        w.own_total = part > uwt + sk ? part : uwt + sk;
+        w.total = w.own_total > w.fwd_bytes ? w.own_total : w.fwd_bytes;
+    } else {
+        w.off_uwt = part;
+        w.off_df1sk = part + uwt;
+        w.own_total = w.total = part + uwt;
+    }
+    return w;
+}
+
 }  // namespace
 namespace sepcorr_impl {
 template <int GMODE, int KC>
@@ -2417,20 +2545,27 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s
     a.tiles_per_batch = (a.N1 + TP - 1) / TP;
     const int nvc_all = (d.W2 + 31) / 32;
     {
-        WaveGrid wg = wave_grid(d.B, a.tiles_per_batch, d.W2, d.H2);
-        if (wg.nvc * wg.nug > 4) wg.nug = 4 / wg.nvc > 0 ? 4 / wg.nvc : 1;   // d_f1 runs one wave per SIMD
+        const Df1Shape shp = df1_shape(d);
+        const WaveGrid wg = shp.wg;
         a.nvc = wg.nvc;
         a.vpasses = wg.vpasses;
-        const int nW = wg.nvc * wg.nug;
-        // more than 4 waves share the register file two to a SIMD: halve the channel block
-        const int ncb = (d.C <= 128 || nW > 4) ? 1 : 2;
-        const int cblocks = (d.C + 128 * ncb - 1) / (128 * ncb);
-        const dim3 grid(d.B * a.tiles_per_batch, cblocks), block(64 * nW);
-        const size_t lds = (size_t)TP * (128 * ncb + 4) * sizeof(float);
-#define SEPCORR_DF1(NCB, CV, MT)                                                                   \
+        const int nW = shp.nW, ncb = shp.ncb, cblocks = shp.cblocks;
+        dim3 grid(d.B * a.tiles_per_batch, cblocks);
+        const dim3 block(64 * nW);
+        const size_t lds = (size_t)nW * TP * (128 * ncb + 4) * sizeof(float);   // one [32][channels] region per wave
+        a.sk_total = 0;
+#define SEPCORR_DF1_K(...)                                                                         \
     do {                                                                                           \
+        auto k = df1_kernel<__VA_ARGS__>;                                                          \
+        if (int rc = set_lds(k, lds)) return rc;                                                   \
         ProfScope ps(GMODE == GMODE_COMP ? "df1_comp" : GMODE == GMODE_BOTH ? "df1_both" : "df1_maxavg", s1); \
-        hipLaunchKernelGGL((df1_kernel<GMODE, KC, NCB, CV, MT>), grid, block, lds, s1, a);         \
+        hipLaunchKernelGGL(k, grid, block, lds, s1, a);                                            \
+    } while (0)
+#define SEPCORR_DF1(NCB, CV, MT) SEPCORR_DF1_K(GMODE, KC, NCB, CV, MT)
+#define SEPCORR_DF1_SPLIT(NCB, MT)                                                                 \
+    do {                                                                                           \
+        if (a.sk_total) SEPCORR_DF1_K(GMODE, KC, NCB, true, MT, false, true);                      \
+        else SEPCORR_DF1_K(GMODE, KC, NCB, true, MT);                                              \
     } while (0)
         const bool planes = !t_no_alloc && g_contraction.load(std::memory_order_relaxed) == SEPCORR_CONTRACT_BF16X3 && d.C == 256 &&
                             wg.vpasses == 1 && cvec && (size_t)d.H1 * d.W1 * MAX_K * d.H2 * 4 <= big &&
@@ -2478,22 +2613,36 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s
             if (rc) return rc;
             if (e != hipSuccess) return fail(SEPCORR_ELAUNCH, "sepcorr: bf16 planes: %s", hipGetErrorString(e));
         }
-        else if (nW > 4) { if (cvec) SEPCORR_DF1(1, true, 512); else SEPCORR_DF1(1, false, 512); }
-        else if (ncb == 1) { if (cvec) SEPCORR_DF1(1, true, 256); else SEPCORR_DF1(1, false, 256); }
+        else {
+        if (shp.split && cvec) {   // pieces of tiles: scratch behind the d_f2 partial sums and the transposed weights
+            char *base = static_cast<char *>(ws) + bwd_ws(d).off_df1sk;
+            a.sk_total = (int)shp.T;
+            a.sk_steps = shp.S;
+            a.sk_count = reinterpret_cast<int *>(base);
+            a.sk_state = reinterpret_cast<float *>(base + shp.count_bytes);
+            grid = dim3(shp.G, cblocks);
+            const int n = d.B * a.tiles_per_batch * cblocks;
+            hipLaunchKernelGGL(zero_ints_kernel, dim3((n + 255) / 256), dim3(256), 0, s1, a.sk_count, n);
+        }
+        if (nW > 4) { if (cvec) SEPCORR_DF1_SPLIT(1, 512); else SEPCORR_DF1(1, false, 512); }
+        else if (ncb == 1) { if (cvec) SEPCORR_DF1_SPLIT(1, 256); else SEPCORR_DF1(1, false, 256); }
         // (the fast variant addresses the (p,u)-indexed tensors of one batch image with 32-bit byte offsets)
         else if (cvec && d.C == 256 && d.W2 % 4 == 0 && (size_t)d.H2 * (2 * KCH + 3) * d.H1 * d.W1 * 4 <= big) {
             constexpr int NF = (g_has_comp(GMODE) ? 2 * KC : 0) + (g_has_maxavg(GMODE) ? 3 : 0);
-            float *uwt = reinterpret_cast<float *>(static_cast<char *>(ws) + df2_part_bytes(d));
+            float *uwt = reinterpret_cast<float *>(static_cast<char *>(ws) + bwd_ws(d).off_uwt);
             {
                 ProfScope ps("transpose_uw", s1);
                 hipLaunchKernelGGL(transpose_uw_kernel<GMODE>, dim3(d.B * ((a.N1 + 63) / 64), NF), dim3(256), 0, s1, a, KC, uwt);
             }
             a.uwt = uwt;
-            ProfScope ps(GMODE == GMODE_COMP ? "df1_comp" : GMODE == GMODE_BOTH ? "df1_both" : "df1_maxavg", s1);
-            hipLaunchKernelGGL((df1_kernel<GMODE, KC, 2, true, 256, true>), grid, block, lds, s1, a);
+            if (a.sk_total) SEPCORR_DF1_K(GMODE, KC, 2, true, 256, true, true);
+            else SEPCORR_DF1_K(GMODE, KC, 2, true, 256, true);
         }
-        else { if (cvec) SEPCORR_DF1(2, true, 256); else SEPCORR_DF1(2, false, 256); }
+        else { if (cvec) SEPCORR_DF1_SPLIT(2, 256); else SEPCORR_DF1(2, false, 256); }
+        }
 #undef SEPCORR_DF1
+#undef SEPCORR_DF1_SPLIT
+#undef SEPCORR_DF1_K
         if (int rc = check_launch("d_f1 kernel")) return rc;
     }
     {
@@ -2620,8 +2769,10 @@ struct ForkJoin {
     SideStreams *ss = nullptr;
     hipStream_t user, sa, sb;
     bool failed = false;
-    explicit ForkJoin(hipStream_t u) : user(u), sa(u), sb(u) {
-        if (!overlap_enabled()) return;
+    // allow == false: everything stays on the caller's stream.  Kernels that are dealt out in pieces of tiles size
+    // their workgroups for having the whole chip at once; beside another kernel they would run in two rounds.
+    explicit ForkJoin(hipStream_t u, bool allow = true) : user(u), sa(u), sb(u) {
+        if (!allow || !overlap_enabled()) return;
         lk = std::unique_lock<std::mutex>(g_side_mu);
         ss = side_streams();
         if (!ss) return;
@@ -2798,8 +2949,7 @@ int sepcorr_compression_forward(const float *f1, const float *f2, const float *a
 size_t sepcorr_backward_workspace_bytes(int B, int H1, int W1, int H2, int W2, int C) {
     if (B < 1 || H1 < 1 || W1 < 1 || H2 < 1 || W2 < 1 || C < 1) return 0;
     const Dims d = {B, H1, W1, H2, W2, C};
-    // split partial sums of d_f2, transposed weights of d_f1, scratch of the weight-gradient sweep
-    return df2_part_bytes(d) + df1_uwt_bytes(d) + fwd_split_bytes(B, H1, W1, H2, W2, MAX_K);
+    return bwd_ws(d).total;
 }
 
 int sepcorr_max_argmax_avg_backward(const float *f1, const float *f2, const int32_t *argmax_u, const int32_t *argmax_v,
@@ -2817,7 +2967,7 @@ int sepcorr_max_argmax_avg_backward(const float *f1, const float *f2, const int3
     a.f1 = f1; a.f2 = f2; a.am_u = argmax_u; a.am_v = argmax_v; a.g_u = grad_u; a.g_v = grad_v;
     a.d1 = d_f1; a.d2 = d_f2;
     a.B = B; a.N1 = H1 * W1; a.H2 = H2; a.W2 = W2; a.C = C; a.KT = 1;
-    ForkJoin fj(static_cast<hipStream_t>(stream));
+    ForkJoin fj(static_cast<hipStream_t>(stream), !bwd_ws(d).aliased);
     const int rc = launch_bwd<GMODE_MAXAVG, 1>(a, d, workspace, fj.sa, fj.user);   // d_f1 aside, d_f2 on the caller's stream
     const int rj = fj.join();
     return rc ? rc : rj;
@@ -2831,7 +2981,7 @@ int sepcorr_max_argmax_avg_backward_static(const float *f1, const float *f2, con
     REQUIRE_PTR(d_f1); REQUIRE_PTR(d_f2);
     const Dims d = {B, H1, W1, H2, W2, C};
     if (int rc = check_dims(d, 2)) return rc;
-    const size_t need = df2_part_bytes(d) + df1_uwt_bytes(d);   // what this entry point itself uses of the workspace
+    const size_t need = bwd_ws(d).own_total;   // what this entry point itself uses of the workspace
     if (need > (size_t)SEPCORR_STATIC_SCRATCH_BYTES)
         return fail(SEPCORR_EWORKSPACE,
                     "sepcorr: these sizes need %zu bytes of scratch, the static array holds %zu: use "
@@ -2869,10 +3019,10 @@ int sepcorr_compression_backward(const float *f1, const float *f2, const float *
         return weighted_forward(d, f1, f2, g_cv, g_cu, d_a_v, d_a_u, K, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
     }
     if (int rc = check_workspace(d, workspace, workspace_bytes)) return rc;
-    ForkJoin fj(static_cast<hipStream_t>(stream));
+    const BwdWs lay = bwd_ws(d);
+    ForkJoin fj(static_cast<hipStream_t>(stream), !lay.aliased);
     // d_a_v[k,u] = sum_v S g_cv[k,v];  d_a_u[k,v] = sum_u S g_cu[k,u]: the forward's weighted sums
-    char *fwd_ws = static_cast<char *>(workspace) + df2_part_bytes(d) + df1_uwt_bytes(d);
-    int rc = weighted_forward(d, f1, f2, g_cv, g_cu, d_a_v, d_a_u, K, fwd_ws, fwd_split_bytes(B, H1, W1, H2, W2, MAX_K), fj.user);
+    int rc = weighted_forward(d, f1, f2, g_cv, g_cu, d_a_v, d_a_u, K, lay.fwd_bytes ? workspace : nullptr, lay.fwd_bytes, fj.user);
     BwdArgs a;
     memset(&a, 0, sizeof(a));
     a.xcd_order = xcd_order_enabled();
@@ -2913,7 +3063,7 @@ int sepcorr_fused_backward(const float *f1, const float *f2, const int32_t *argm
     a.a_u = a_u; a.a_v = a_v; a.g_cu = g_cu; a.g_cv = g_cv;
     a.d1 = d_f1; a.d2 = d_f2;
     a.B = B; a.N1 = H1 * W1; a.H2 = H2; a.W2 = W2; a.C = C; a.KT = K;
-    ForkJoin fj(static_cast<hipStream_t>(stream));
+    ForkJoin fj(static_cast<hipStream_t>(stream), !bwd_ws(d).aliased);
     const int kch = W2 > 128 ? 2 : KCH;
     const int kc0 = K < kch ? K : kch;
     // The first chunk of weight channels carries the max/avg terms of G along (built for 2 and 4 channels);

@@ -39,7 +39,8 @@ def test_abi_version_and_workspace_query():
     part, fields = 2 * 55 * 128 * 256 * 4, 11 * 2 * 55 * (55 * 128) * 4
     fwd = lib.sepcorr_forward_workspace_bytes(2, 55, 128, 55, 128, 256, 8)
     assert fwd > 0 and fwd % 256 == 0
-    assert n > fields + fwd and (n - fields - fwd) % part == 0
+    # (kernels dealt out in pieces run one after the other and share the memory: the largest region counts)
+    assert n >= max(fields, fwd, 2 * part) and n % 256 == 0
     # whole tiles fill the chip: nothing to gain from scratch (1020 tiles of 8 waves on 256 units)
     assert lib.sepcorr_forward_workspace_bytes(1, 136, 240, 136, 240, 256, 4) == 0
     assert lib.sepcorr_forward_workspace_bytes(0, 1, 1, 1, 1, 1, 2) == 0

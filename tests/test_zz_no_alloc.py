@@ -30,8 +30,7 @@ def _case(device, B, H1, W1, H2, W2, C, seed):
 def _both(lib, device, dims, seed):
     B, H1, W1, H2, W2, C = dims
     ins = _case(device, *dims, seed)
-    need = lib.sepcorr_backward_workspace_bytes(*dims)
-    assert need <= LIMIT, f"test sizes must fit the static array: {need}"
+    need = lib.sepcorr_backward_workspace_bytes(*dims)   # covers all backward entry points; this one uses part of it
     stream = torch.cuda.current_stream().cuda_stream
     P = lambda t: t.data_ptr()
     ws = torch.empty(max(need, 256), dtype=torch.uint8, device=device)
