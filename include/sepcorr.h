@@ -171,6 +171,54 @@ int sepcorr_compression_backward(const float *f1, const float *f2, const float *
                                  void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Attention compression straight from the logits.  The caller's
+ *   a_u = attention1(sep_u).softmax(dim=2) ...; ComputeSelfCompressionFunction.apply(fmap1, fmap2, a_u, a_v)
+ * (core/corr.py:437-448, libs/MemorySaver/functions/MemorySaver.py:107-177) with the softmax moved inside the operator:
+ *   logits_u (B,H1,W1,K,W2), logits_v (B,H1,W1,K,H2)   what the attention modules return, in the operator's layout
+ *   comp_u, comp_v                                     as sepcorr_compression_forward with a = softmax over the last axis
+ *   stats_u, stats_v (B,H1,W1,K,2)                     per row (max, sum of exp(z - max)): written here (one pass over
+ *                                                      the logits) unless stats_given != 0, in which case they are read
+ *                                                      (sepcorr_attention_logits_forward supplies them for free)
+ * The weights exp(z - max) / sum are formed where the sweep loads them; no tensor of softmax outputs exists.
+ * workspace: as for sepcorr_compression_forward (optional).
+ */
+int sepcorr_compression_forward_from_logits(const float *f1, const float *f2,
+                                            const float *logits_u, const float *logits_v,
+                                            float *comp_u, float *comp_v, float *stats_u, float *stats_v, int stats_given,
+                                            int B, int H1, int W1, int H2, int W2, int C, int K,
+                                            void *workspace, size_t workspace_bytes, void *stream);
+
+/* Scratch bytes of the call below: without (with_features = 0) or with the feature gradients. */
+size_t sepcorr_compression_backward_from_logits_workspace_bytes(int B, int H1, int W1, int H2, int W2, int C, int K,
+                                                                int with_features);
+
+/*
+ * Gradients of the above: what torch autograd computes through ComputeSelfCompressionFunction.backward
+ * (libs/MemorySaver/functions/MemorySaver.py:139-177) and the softmax in front of it (core/corr.py:441-442).
+ * Inputs are those of the forward call, its outputs comp_u, comp_v and statistics, and the upstream gradients
+ * g_cu (B,H1,W1,K,H2), g_cv (B,H1,W1,K,W2).  With a = softmax(z) and d_a as in sepcorr_compression_backward,
+ *   d_logits_u[..,k,v] = a_u (d_a_u - sum_v a_u d_a_u),   d_logits_v[..,k,u] = a_v (d_a_v - sum_u a_v d_a_v);
+ * the row sums are taken as sum_u g_cu comp_u and sum_v g_cv comp_v (the same numbers), so the gradients leave the
+ * weight-gradient sweep finished: no tensor d_a and no softmax-backward pass exist.
+ * d_f1, d_f2 as in sepcorr_compression_backward; both may be NULL (then only the logit gradients are computed).
+ */
+int sepcorr_compression_backward_from_logits(const float *f1, const float *f2,
+                                             const float *logits_u, const float *logits_v,
+                                             const float *stats_u, const float *stats_v,
+                                             const float *comp_u, const float *comp_v,
+                                             const float *g_cu, const float *g_cv,
+                                             float *d_f1, float *d_f2, float *d_logits_u, float *d_logits_v,
+                                             int B, int H1, int W1, int H2, int W2, int C, int K,
+                                             void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Row softmax helper of the two calls above for callers that need the weights themselves: for nrows rows of L logits,
+ * stats (nrows,2) = (max, sum of exp) is computed (stats_given == 0) or read, and, when a is not NULL,
+ * a = exp(z - max) / sum is written.  No counterpart in the reference (torch's softmax stands there, core/corr.py:441).
+ */
+int sepcorr_softmax_rows(const float *logits, float *stats, int stats_given, float *a, long nrows, int L, void *stream);
+
+/*
  * Feature gradients of both operators of one pyramid level in one pass; no counterpart in the reference,
  * whose two backward functions (MemorySaver_cuda.cpp:55-103) each contract their own dL/dS.  With G the sum
  * of the two expressions given above for sepcorr_max_argmax_avg_backward and sepcorr_compression_backward,
@@ -198,6 +246,22 @@ int sepcorr_fused_backward(const float *f1, const float *f2,
  */
 int sepcorr_attention_forward(const float *sep, const float *weight, const float *bias, float *a,
                               int B, int H1, int W1, int L, int K, void *stream);
+
+/*
+ * The same producer stopping at the logits: logits (B,H1,W1,K,L) = Conv3d(sep) in the operator's layout, and, when
+ * stats is not NULL, stats (B,H1,W1,K,2) = per row (max, sum of exp(z - max)), which the kernel has at hand.  Feeds
+ * sepcorr_compression_forward_from_logits (core/corr.py:437-448 with the softmax moved into the operator).
+ */
+int sepcorr_attention_logits_forward(const float *sep, const float *weight, const float *bias, float *logits, float *stats,
+                                     int B, int H1, int W1, int L, int K, void *stream);
+
+/* Its gradients from the gradient of the logits (no softmax in between): d_sep, d_weight, d_bias (or NULL) as
+ * sepcorr_attention_backward; scratch: sepcorr_attention_logits_workspace_bytes. */
+size_t sepcorr_attention_logits_workspace_bytes(int B, int H1, int W1, int L, int K);
+int sepcorr_attention_logits_backward(const float *sep, const float *weight, const float *d_logits,
+                                      float *d_sep, float *d_weight, float *d_bias,
+                                      int B, int H1, int W1, int L, int K,
+                                      void *workspace, size_t workspace_bytes, void *stream);
 
 /* Scratch bytes needed by sepcorr_attention_backward. */
 size_t sepcorr_attention_workspace_bytes(int B, int H1, int W1, int L, int K);

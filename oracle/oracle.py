@@ -170,6 +170,20 @@ def compression_backward(f1, f2, a_u, a_v, g_cu, g_cv):
     return d1, d2, da_u, da_v
 
 
+def compression_from_logits(f1, f2, z_u, z_v):
+    """The caller's softmax over the kept axis followed by the compression operator (core/corr.py:441-448):
+    logits z_u (B,H1,W1,K,W2), z_v (B,H1,W1,K,H2) -> (comp_u (B,H1,W1,K,H2), comp_v (B,H1,W1,K,W2)).  In the
+    operator's layout the kept axis is the last one.  Differentiable: torch autograd supplies the gradients of the
+    features and of the logits that the fused operator is compared with."""
+    return compression_forward(f1, f2, z_u.softmax(dim=-1), z_v.softmax(dim=-1))
+
+
+def attention_logits(sep, weight, bias):
+    """attention_weights without the softmax: the Conv3d output in the operator's layout (B,H1,W1,K,L)."""
+    x = sep.permute(0, 3, 4, 1, 2)
+    return F.conv3d(x, weight, bias, padding=1).permute(0, 3, 4, 1, 2).contiguous()
+
+
 def attention_weights(sep, weight, bias):
     """The caller's attention-weight producer, op-level layout in and out.
 

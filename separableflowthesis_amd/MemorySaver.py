@@ -191,6 +191,128 @@ def compression_weight_gradients(img1_features_l0, img2_features_lk, attention_w
     return [da_u, da_v]
 
 
+# --- attention compression with the softmax inside the operator (core/corr.py:437-448 takes the softmax in torch)
+
+def _logit_dims(f1, f2, logits_u, logits_v):
+    B, H1, W1, H2, W2, C = _dims(f1, f2)
+    _check("logits_u", logits_u, ndim=5)
+    K = logits_u.shape[3]
+    _expect("logits_u", logits_u, (B, H1, W1, K, W2), f1.device)
+    _expect("logits_v", logits_v, (B, H1, W1, K, H2), f1.device)
+    return B, H1, W1, H2, W2, C, K
+
+
+def compression_forward_from_logits(img1_features_l0, img2_features_lk, logits_u, logits_v, stats_u=None, stats_v=None):
+    """compression_forward with attention_weights = softmax(logits, dim=-1), the softmax taken inside the sweep.
+    -> [compression_output_u, compression_output_v, stats_u (B,H1,W1,K,2), stats_v]: per row (max, sum of exp).
+    Statistics a producer already has (attention_logits_forward) can be passed in; otherwise they are computed."""
+    f1, f2 = img1_features_l0, img2_features_lk
+    B, H1, W1, H2, W2, C, K = _logit_dims(f1, f2, logits_u, logits_v)
+    dev = f1.device
+    given = stats_u is not None and stats_v is not None
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        cu = torch.empty((B, H1, W1, K, H2), dtype=f1.dtype, device=dev)
+        cv = torch.empty((B, H1, W1, K, W2), dtype=f1.dtype, device=dev)
+        if given:
+            _expect("stats_u", stats_u, (B, H1, W1, K, 2), dev)
+            _expect("stats_v", stats_v, (B, H1, W1, K, 2), dev)
+        else:
+            stats_u = torch.empty((B, H1, W1, K, 2), dtype=f1.dtype, device=dev)
+            stats_v = torch.empty((B, H1, W1, K, 2), dtype=f1.dtype, device=dev)
+        ws, wptr, n = _fwd_workspace(lib, (B, H1, W1, H2, W2, C), K, dev)
+        _lib.check(lib.sepcorr_compression_forward_from_logits(
+            f1.data_ptr(), f2.data_ptr(), logits_u.data_ptr(), logits_v.data_ptr(), cu.data_ptr(), cv.data_ptr(),
+            stats_u.data_ptr(), stats_v.data_ptr(), int(given), B, H1, W1, H2, W2, C, K, wptr, n, _stream()))
+    return [cu, cv, stats_u, stats_v]
+
+
+def compression_backward_from_logits(img1_features_l0, img2_features_lk, logits_u, logits_v, stats_u, stats_v,
+                                     compression_output_u, compression_output_v,
+                                     grad_compressed_output_u, grad_compressed_output_v, need_features=True):
+    """-> [grad_fmap1_l0, grad_fmap2_lk, grad_logits_u (B,H1,W1,K,W2), grad_logits_v (B,H1,W1,K,H2)]; the feature
+    gradients are None with need_features=False (one sweep over the volume, no tensor of softmax outputs)."""
+    f1, f2 = img1_features_l0, img2_features_lk
+    B, H1, W1, H2, W2, C, K = _logit_dims(f1, f2, logits_u, logits_v)
+    dev = f1.device
+    _expect("stats_u", stats_u, (B, H1, W1, K, 2), dev)
+    _expect("stats_v", stats_v, (B, H1, W1, K, 2), dev)
+    _expect("compression_output_u", compression_output_u, (B, H1, W1, K, H2), dev)
+    _expect("compression_output_v", compression_output_v, (B, H1, W1, K, W2), dev)
+    _expect("grad_compressed_output_u", grad_compressed_output_u, (B, H1, W1, K, H2), dev)
+    _expect("grad_compressed_output_v", grad_compressed_output_v, (B, H1, W1, K, W2), dev)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        d1 = torch.empty_like(f1) if need_features else None
+        d2 = torch.empty_like(f2) if need_features else None
+        dz_u = torch.empty_like(logits_u)
+        dz_v = torch.empty_like(logits_v)
+        n = lib.sepcorr_compression_backward_from_logits_workspace_bytes(B, H1, W1, H2, W2, C, K, int(need_features))
+        ws = torch.empty(max(n, 1), dtype=torch.uint8, device=dev)
+        _lib.check(lib.sepcorr_compression_backward_from_logits(
+            f1.data_ptr(), f2.data_ptr(), logits_u.data_ptr(), logits_v.data_ptr(), stats_u.data_ptr(), stats_v.data_ptr(),
+            compression_output_u.data_ptr(), compression_output_v.data_ptr(),
+            grad_compressed_output_u.data_ptr(), grad_compressed_output_v.data_ptr(),
+            d1.data_ptr() if need_features else None, d2.data_ptr() if need_features else None,
+            dz_u.data_ptr(), dz_v.data_ptr(), B, H1, W1, H2, W2, C, K, ws.data_ptr(), n, _stream()))
+    return [d1, d2, dz_u, dz_v]
+
+
+def softmax_from_stats(logits, stats):
+    """softmax(logits, dim=-1) from the saved row statistics (max, sum of exp): (.., L), (.., 2) -> (.., L)."""
+    _check("logits", logits)
+    L = logits.shape[-1]
+    _expect("stats", stats, tuple(logits.shape[:-1]) + (2,), logits.device)
+    lib = _lib.load()
+    with torch.cuda.device(logits.device):
+        a = torch.empty_like(logits)
+        _lib.check(lib.sepcorr_softmax_rows(logits.data_ptr(), stats.data_ptr(), 1, a.data_ptr(),
+                                            logits.numel() // L, L, _stream()))
+    return a
+
+
+def attention_logits_forward(sep, weight, bias, want_stats=True):
+    """sep (B,H1,W1,2,L), Conv3d weight (K,2,3,3,3), bias (K) or None -> [logits (B,H1,W1,K,L), stats (B,H1,W1,K,2)]:
+    the convolution alone, in the operator's layout, with the row statistics of its softmax."""
+    _check("sep", sep, ndim=5)
+    B, H1, W1, ch, L = sep.shape
+    if ch != 2:
+        raise RuntimeError(f"sep must have 2 channels (max, avg), got {ch}")
+    _check("weight", weight, ndim=5)
+    K = weight.shape[0]
+    _expect("weight", weight, (K, 2, 3, 3, 3), sep.device)
+    if bias is not None:
+        _expect("bias", bias, (K,), sep.device)
+    lib = _lib.load()
+    with torch.cuda.device(sep.device):
+        z = torch.empty((B, H1, W1, K, L), dtype=sep.dtype, device=sep.device)
+        st = torch.empty((B, H1, W1, K, 2), dtype=sep.dtype, device=sep.device) if want_stats else None
+        _lib.check(lib.sepcorr_attention_logits_forward(
+            sep.data_ptr(), weight.data_ptr(), bias.data_ptr() if bias is not None else None, z.data_ptr(),
+            st.data_ptr() if want_stats else None, B, H1, W1, L, K, _stream()))
+    return [z, st]
+
+
+def attention_logits_backward(sep, weight, grad_logits, need_bias=True):
+    """-> [d_sep (B,H1,W1,2,L), d_weight (K,2,3,3,3), d_bias (K) or None] from the gradient of the logits."""
+    _check("sep", sep, ndim=5)
+    B, H1, W1, _, L = sep.shape
+    K = weight.shape[0]
+    _expect("weight", weight, (K, 2, 3, 3, 3), sep.device)
+    _expect("grad_logits", grad_logits, (B, H1, W1, K, L), sep.device)
+    lib = _lib.load()
+    with torch.cuda.device(sep.device):
+        d_sep = torch.empty_like(sep)
+        d_w = torch.empty_like(weight)
+        d_b = torch.empty(K, dtype=sep.dtype, device=sep.device) if need_bias else None
+        n = lib.sepcorr_attention_logits_workspace_bytes(B, H1, W1, L, K)
+        ws = torch.empty(max(n, 1), dtype=torch.uint8, device=sep.device)
+        _lib.check(lib.sepcorr_attention_logits_backward(
+            sep.data_ptr(), weight.data_ptr(), grad_logits.data_ptr(), d_sep.data_ptr(), d_w.data_ptr(),
+            d_b.data_ptr() if need_bias else None, B, H1, W1, L, K, ws.data_ptr(), n, _stream()))
+    return [d_sep, d_w, d_b]
+
+
 def fused_backward(img1_features_l0, img2_features_lk, argmax_output_u, argmax_output_v, grad_MaxAvg_u, grad_MaxAvg_v,
                    attention_weights_u, attention_weights_v, grad_compressed_output_u, grad_compressed_output_v):
     """-> [grad_fmap1_l0, grad_fmap2_lk]: the sum of what max_argmax_avg_backward and compression_backward return

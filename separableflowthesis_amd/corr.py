@@ -10,9 +10,9 @@ trilinearly upsampled (align_corners=True) to the level-0 displacement length.
 import torch
 import torch.nn.functional as F
 
-from .functions import (AssembleVolumeFunction, AttentionWeightsFunction, ComputeMaxArgmaxAvgFunction,
-                        ComputeMaxAvgFunction, ComputeSelfCompressionFunction, Lookup1DFunction,
-                        LookupFunction, SeparateLevelFunction)
+from .functions import (AssembleVolumeFunction, AttentionLogitsFunction, AttentionWeightsFunction,
+                        ComputeMaxArgmaxAvgFunction, ComputeMaxAvgFunction, ComputeSelfCompressionFromLogitsFunction,
+                        ComputeSelfCompressionFunction, Lookup1DFunction, LookupFunction, SeparateLevelFunction)
 
 
 def _is_reference_attention(m):
@@ -72,9 +72,10 @@ class AlternateCorrBlockSepflow:
                 parts_v.append(maxavg_u)
                 if attention_weights is not None:
                     attention1, attention2 = attention_weights
-                    a_u = AttentionWeightsFunction.apply(maxavg_v, attention1.weight.contiguous(), attention1.bias)
-                    a_v = AttentionWeightsFunction.apply(maxavg_u, attention2.weight.contiguous(), attention2.bias)
-                    adaptive_corr_u, adaptive_corr_v = ComputeSelfCompressionFunction.apply(fmap1, fmap2, a_u, a_v)
+                    z_u, st_u = AttentionLogitsFunction.apply(maxavg_v, attention1.weight.contiguous(), attention1.bias)
+                    z_v, st_v = AttentionLogitsFunction.apply(maxavg_u, attention2.weight.contiguous(), attention2.bias)
+                    adaptive_corr_u, adaptive_corr_v = ComputeSelfCompressionFromLogitsFunction.apply(
+                        fmap1, fmap2, z_u, z_v, st_u, st_v)
                     parts_v.append(adaptive_corr_u)
                     parts_u.append(adaptive_corr_v)
                 continue

@@ -52,6 +52,8 @@ struct AttArgs {
     float *dlogits;    // scratch (B,H1,W1,K,L)
     float *partial;    // scratch [nwg][K*54 + K]
     int B, H1, W1, L, K;
+    float *stats;      // forward, optional: (max, sum of exp) of every row of logits, (B,H1,W1,K,2)
+    int logits_only;   // forward: store the logits themselves instead of their softmax
 };
 
 // Forward.  NCH = ceil(L / 64) chunks per row.  A lane first gathers the 54 inputs of each of its positions (9
@@ -113,18 +115,22 @@ __global__ void __launch_bounds__(64 * WPB) att_forward_kernel(const AttArgs a) 
         for (int ch = 0; ch < NCH; ++ch)
             if (ch * 64 + lane < L) m = fmaxf(m, logit[ch]);
         m = group_max(m, lw);
-        float s = 0.f;
+        float s = 0.f, ex[NCH];
 #pragma unroll
         for (int ch = 0; ch < NCH; ++ch) {
-            logit[ch] = (ch * 64 + lane < L) ? __expf(logit[ch] - m) : 0.f;
-            s += logit[ch];
+            ex[ch] = (ch * 64 + lane < L) ? __expf(logit[ch] - m) : 0.f;
+            s += ex[ch];
         }
         s = group_sum(s, lw);
         const float inv = 1.f / s;
         float *dst = a.out + (pix * K + k) * L;
+        if (a.stats && lane == 0) {
+            a.stats[2 * (pix * K + k)] = m;
+            a.stats[2 * (pix * K + k) + 1] = s;
+        }
 #pragma unroll
         for (int ch = 0; ch < NCH; ++ch)
-            if (ch * 64 + lane < L) dst[ch * 64 + lane] = logit[ch] * inv;
+            if (ch * 64 + lane < L) dst[ch * 64 + lane] = a.logits_only ? logit[ch] : ex[ch] * inv;
     }
 }
 
@@ -166,12 +172,17 @@ __global__ void __launch_bounds__(64 * WPB) att_forward_long_kernel(const AttArg
         float s = 0.f;
         for (int l = lane; l < L; l += 64) {
             const float e = __expf(dst[l] - m);   // written by this same lane
-            dst[l] = e;
+            if (!a.logits_only) dst[l] = e;
             s += e;
         }
         s = wave_sum(s);
+        if (a.stats && lane == 0) {
+            a.stats[2 * (pix * K + k)] = m;
+            a.stats[2 * (pix * K + k) + 1] = s;
+        }
         const float inv = 1.f / s;
-        for (int l = lane; l < L; l += 64) dst[l] *= inv;
+        if (!a.logits_only)
+            for (int l = lane; l < L; l += 64) dst[l] *= inv;
     }
 }
 
@@ -392,12 +403,13 @@ size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 extern "C" {
 
-int sepcorr_attention_forward(const float *sep, const float *weight, const float *bias, float *a, int B, int H1, int W1, int L,
-                              int K, void *stream) {
+static int attention_forward(const float *sep, const float *weight, const float *bias, float *a, float *stats, int logits_only,
+                             int B, int H1, int W1, int L, int K, void *stream) {
     REQ(sep); REQ(weight); REQ(a);
     if (int rc = check_sizes(B, H1, W1, L, K)) return rc;
     AttArgs args = {};
     args.sep = sep; args.weight = weight; args.bias = bias; args.out = a;
+    args.stats = stats; args.logits_only = logits_only;
     args.B = B; args.H1 = H1; args.W1 = W1; args.L = L; args.K = K;
     const long npix = (long)B * H1 * W1;
     const long ppg = (long)WPB * (64 / lanes_per_pixel(L));   // pixels per workgroup
@@ -410,11 +422,59 @@ int sepcorr_attention_forward(const float *sep, const float *weight, const float
     return launched("attention forward kernel");
 }
 
+int sepcorr_attention_forward(const float *sep, const float *weight, const float *bias, float *a, int B, int H1, int W1, int L,
+                              int K, void *stream) {
+    return attention_forward(sep, weight, bias, a, nullptr, 0, B, H1, W1, L, K, stream);
+}
+
+int sepcorr_attention_logits_forward(const float *sep, const float *weight, const float *bias, float *logits, float *stats,
+                                     int B, int H1, int W1, int L, int K, void *stream) {
+    return attention_forward(sep, weight, bias, logits, stats, 1, B, H1, W1, L, K, stream);
+}
+
 size_t sepcorr_attention_workspace_bytes(int B, int H1, int W1, int L, int K) {
     if (B < 1 || H1 < 1 || W1 < 1 || L < 1 || K < 1 || K > MAXK) return 0;
     const size_t npix = (size_t)B * H1 * W1;
     const size_t nwg = (npix + DW_PIX - 1) / DW_PIX;
     return align256(npix * K * L * sizeof(float)) + align256(nwg * (K * 54 + K) * sizeof(float));
+}
+
+size_t sepcorr_attention_logits_workspace_bytes(int B, int H1, int W1, int L, int K) {
+    if (B < 1 || H1 < 1 || W1 < 1 || L < 1 || K < 1 || K > MAXK) return 0;
+    const size_t nwg = ((size_t)B * H1 * W1 + DW_PIX - 1) / DW_PIX;
+    return align256(nwg * (K * 54 + K) * sizeof(float));
+}
+
+int sepcorr_attention_logits_backward(const float *sep, const float *weight, const float *d_logits, float *d_sep,
+                                      float *d_weight, float *d_bias, int B, int H1, int W1, int L, int K, void *workspace,
+                                      size_t workspace_bytes, void *stream) {
+    REQ(sep); REQ(weight); REQ(d_logits); REQ(d_sep); REQ(d_weight);
+    if (int rc = check_sizes(B, H1, W1, L, K)) return rc;
+    const size_t need = sepcorr_attention_logits_workspace_bytes(B, H1, W1, L, K);
+    if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15)) {
+        char msg[160];
+        snprintf(msg, sizeof(msg), "sepcorr: attention backward needs %zu bytes of 16-byte aligned workspace, got %zu", need,
+                 workspace ? workspace_bytes : (size_t)0);
+        return sepcorr_set_error(SEPCORR_EWORKSPACE, msg);
+    }
+    const long npix = (long)B * H1 * W1;
+    const int nwg = (int)((npix + DW_PIX - 1) / DW_PIX);
+    AttArgs args = {};
+    args.sep = sep; args.weight = weight;
+    args.dlogits = const_cast<float *>(d_logits);   // read only from here on
+    args.partial = static_cast<float *>(workspace);
+    args.B = B; args.H1 = H1; args.W1 = W1; args.L = L; args.K = K;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const long ppg = (long)WPB * (64 / lanes_per_pixel(L));
+    const dim3 grid((unsigned)((npix + ppg - 1) / ppg)), block(64 * WPB);
+    args.out = d_sep;
+    hipLaunchKernelGGL(att_input_backward_kernel, grid, block, 0, s, args);
+    if (int rc = launched("attention input gradient kernel")) return rc;
+    hipLaunchKernelGGL(att_weight_backward_kernel, dim3(nwg, 2 * ((K + DW_KC - 1) / DW_KC)), dim3(256), 0, s, args);
+    if (int rc = launched("attention weight gradient kernel")) return rc;
+    const int n = K * 54 + K;
+    hipLaunchKernelGGL(att_weight_reduce_kernel, dim3((n + 3) / 4), dim3(256), 0, s, args.partial, d_weight, d_bias, nwg, K);
+    return launched("attention weight gradient reduction");
 }
 
 int sepcorr_attention_backward(const float *sep, const float *weight, const float *a, const float *grad_a, float *d_sep,

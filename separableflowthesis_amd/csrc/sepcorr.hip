@@ -246,7 +246,21 @@ __global__ void __launch_bounds__(256) split_planes_t_kernel(const float *__rest
 // ------------------------------------------------------------------------------------------
 // forward
 // ------------------------------------------------------------------------------------------
-enum { MODE_MAXAVG = 0, MODE_ARGMAX = 1, MODE_WEIGHTED = 2 };
+// MODE_SOFT: MODE_WEIGHTED with the softmax inside (FwdArgs::logits / dlog); a mode of its own so that the plain
+// weighted sweep carries none of its arguments
+enum { MODE_MAXAVG = 0, MODE_ARGMAX = 1, MODE_WEIGHTED = 2, MODE_SOFT = 3 };
+constexpr bool is_weighted(int mode) { return mode == MODE_WEIGHTED || mode == MODE_SOFT; }
+
+// Gradient of a logit from the gradient x of its softmax output: a (x - dot), a = exp(z - max) / sum.
+// row = index of the (pixel, channel) row, elem = index of the element in the row-major tensor.
+__device__ __forceinline__ float dlogit(const float *__restrict__ z, const float *__restrict__ st, const float *__restrict__ dots,
+                                        size_t row, size_t elem, float x) {
+    return __expf(z[elem] - st[2 * row]) / st[2 * row + 1] * (x - dots[row]);
+}
+// the same with the row's (max, 1 / sum, dot) at hand
+__device__ __forceinline__ float dlogit3(float z, const float *row3, float x) {
+    return __expf(z - row3[0]) * row3[1] * (x - row3[2]);
+}
 
 // Workgroups are handed to the 8 XCDs round-robin by linear id, and each XCD has its own L2.  This maps the
 // hardware id to a logical one such that every XCD works on one contiguous range of logical ids: neighbours in
@@ -286,6 +300,15 @@ struct FwdArgs {
     int sk_slot;       // floats per slot
     void *ws;          // host side only: scratch for the split (NULL: whole tiles)
     size_t ws_bytes;
+    // MODE_WEIGHTED with softmax inside.  Row statistics are (max, sum of exp) pairs per (pixel, channel) row.
+    //   logits:  wv and wu hold logits, the weights are exp(z - max) / sum with the statistics st_wv, st_wu
+    //            (attention compression straight from the logits)
+    //   dlog:    the sums are gradients of softmax outputs; what is stored is the gradient of the logits,
+    //            a (x - dot) with a = exp(z - max) / sum, for out_u rows from (z_ou, st_ou, dot_ou), for out_v
+    //            columns from (z_ov, st_ov, dot_ov); dot = sum over the row of a * x, supplied by the caller
+    int logits, dlog;
+    const float *st_wv, *st_wu;
+    const float *z_ou, *st_ou, *dot_ou, *z_ov, *st_ov, *dot_ov;
 };
 }  // namespace sepcorr_impl
 namespace {
@@ -302,9 +325,10 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     static_assert(!BF || (CMODE == 3 && WM <= 1), "bf16 planes: C == 256, one column pass");
     static_assert(!(BF && SK), "the split is not built for the bf16-plane variant");
     const int sk_total = SK ? a.sk_total : 0;
+    const bool soft_logits = MODE == MODE_SOFT && a.logits, soft_dlog = MODE == MODE_SOFT && a.dlog;
     constexpr bool CVEC = CMODE >= 1;
     constexpr int GJ = 2;  // 8-channel slices per prefetch group
-    constexpr int NPART = (MODE == MODE_WEIGHTED) ? KC : 3;
+    constexpr int NPART = (is_weighted(MODE)) ? KC : 3;
     extern __shared__ float smem[];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, pl = lane & 31, h = lane >> 5;
     const int nW = blockDim.x >> 6;
@@ -321,9 +345,12 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     float *f1s = smem;
     __bf16 *f1b = reinterpret_cast<__bf16 *>(smem);   // BF: [plane][TP][BF_LSB]
     float *part = smem + TP * LS;
-    constexpr int NCHO = (MODE == MODE_WEIGHTED) ? KC : 2;            // out_u channels of this launch
+    constexpr int NCHO = (is_weighted(MODE)) ? KC : 2;            // out_u channels of this launch
     float *ostage = part + 2 * UR * NPART * (blockDim.x >> 6) * 32;   // [32 p][NCHO][H2] when a.stage
     int *ostage_am = reinterpret_cast<int *>(ostage + TP * NCHO * a.H2);   // [32 p][H2], MODE_ARGMAX
+    // MODE_WEIGHTED with softmax inside: per (pixel, channel) row of the u-indexed tensor (max, 1 / sum) of the
+    // logits that are the weights [32 p][KC][2], or (max, 1 / sum, dot) of the logits whose gradient is stored [..][3]
+    float *cst = ostage + (a.stage ? TP * NCHO * a.H2 : 0);
 
     // This workgroup's share of the steps of all tiles: [gs0, gs_end).  Without the split it is exactly one tile.
     // A share is cut into pieces at tile boundaries.  When it ends inside a tile, that last piece (which starts at
@@ -354,6 +381,25 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     const int p0 = (tile % a.tiles_per_batch) * TP;
     if (seg_no > 0) __syncthreads();   // the previous piece has finished with LDS
 
+    if constexpr (is_weighted(MODE)) {
+        if (soft_logits) {   // (max, 1 / sum) of the rows of u-indexed logits of this tile's pixels
+            for (int idx = tid; idx < TP * KC; idx += blockDim.x) {
+                const int p = idx / KC, kk = idx - p * KC;
+                const size_t row = ((size_t)b * N1 + min(p0 + p, N1 - 1)) * a.KT + a.k0 + kk;
+                cst[2 * idx] = a.st_wu[2 * row];
+                cst[2 * idx + 1] = 1.f / a.st_wu[2 * row + 1];
+            }
+        }
+        if (soft_dlog) {
+            for (int idx = tid; idx < TP * KC; idx += blockDim.x) {
+                const int p = idx / KC, kk = idx - p * KC;
+                const size_t row = ((size_t)b * N1 + min(p0 + p, N1 - 1)) * a.KT + a.k0 + kk;
+                cst[3 * idx] = a.st_ou[2 * row];
+                cst[3 * idx + 1] = 1.f / a.st_ou[2 * row + 1];
+                cst[3 * idx + 2] = a.dot_ou[row];
+            }
+        }
+    }
     {   // stage the f1 tile [TP][CP] (zero padded) into LDS
         const int c4n = a.CP >> 2;
         for (int idx = tid; idx < TP * c4n; idx += blockDim.x) {
@@ -401,7 +447,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     float vmax[16], vsum[16];
     int vidx[16];
     float wvr[KC][16], rv[KC][16];
-    if constexpr (MODE == MODE_WEIGHTED) {
+    if constexpr (is_weighted(MODE)) {
 #pragma unroll
         for (int k = 0; k < KC; ++k)
 #pragma unroll
@@ -410,6 +456,16 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                 rv[k][r] = 0.f;
                 wvr[k][r] = (pok && v < W2) ? a.wv[(bp * a.KT + a.k0 + k) * W2 + v] : 0.f;
             }
+        if (soft_logits) {
+#pragma unroll
+            for (int k = 0; k < KC; ++k) {
+                const size_t row = bp * a.KT + a.k0 + k;
+                const float m = a.st_wv[2 * row], il = 1.f / a.st_wv[2 * row + 1];
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    wvr[k][r] = (pok && vbase + 32 * vcw + vmap(r, h) < W2) ? __expf(wvr[k][r] - m) * il : 0.f;
+            }
+        }
     } else {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -451,7 +507,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         for (int ru = 0; ru < UR; ++ru) {
             const int u = ((sa + step) * NUG + ug) * UR + ru;
             if (u < H2) {
-                if constexpr (MODE == MODE_WEIGHTED) {
+                if constexpr (is_weighted(MODE)) {
 #pragma unroll
                     for (int k = 0; k < KC; ++k) {
                         float s = 0.f;
@@ -506,7 +562,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         }
         __syncthreads();
         // combine the per-wave partials in wave order and store the finished rows
-        if constexpr (MODE == MODE_WEIGHTED) {
+        if constexpr (is_weighted(MODE)) {
             for (int idx = tid; idx < NUG * UR * KC * 32; idx += blockDim.x) {
                 const int p = idx & 31, k = (idx >> 5) % KC, ru = (idx / (32 * KC)) % UR, g2 = idx / (32 * KC * UR);
                 const int u = ((sa + step) * NUG + g2) * UR + ru;
@@ -520,8 +576,10 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                         if (vp > 0) s += *dst;   // earlier column passes, written by this same thread
                         *dst = s;
                     } else {
-                        float *dst = &a.out_u[(((size_t)b * N1 + p0 + p) * a.KT + a.k0 + k) * H2 + u];
+                        const size_t row = ((size_t)b * N1 + p0 + p) * a.KT + a.k0 + k;
+                        float *dst = &a.out_u[row * H2 + u];
                         if (vp > 0) s += *dst;
+                        if (soft_dlog && vp == vpasses - 1) s = dlogit3(a.z_ou[row * H2 + u], cst + 3 * (p * KC + k), s);
                         *dst = s;
                     }
                 }
@@ -570,14 +628,17 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     };
 
     auto compute = [&](int step, int g, v4f(&buf)[UR][GJ]) {
-        if constexpr (MODE == MODE_WEIGHTED) {
+        if constexpr (is_weighted(MODE)) {
             if (g == 0) {
 #pragma unroll
                 for (int r = 0; r < UR; ++r) {
                     const int u = ((sa + step) * NUG + ug) * UR + r;
 #pragma unroll
                     for (int k = 0; k < KC; ++k)
+                    {
                         wur[r][k] = (pok && u < H2) ? a.wu[(bp * a.KT + a.k0 + k) * H2 + u] : 0.f;
+                        if (soft_logits) wur[r][k] = __expf(wur[r][k] - cst[2 * (pl * KC + k)]) * cst[2 * (pl * KC + k) + 1];
+                    }
                 }
             }
         }
@@ -614,7 +675,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
             __builtin_amdgcn_sched_barrier(0);
         };
         auto computeB = [&](int step, int J, v4f(&buf)[UR][6]) {
-            if constexpr (MODE == MODE_WEIGHTED) {
+            if constexpr (is_weighted(MODE)) {
                 if (J == 0) {
 #pragma unroll
                     for (int r = 0; r < UR; ++r) {
@@ -662,8 +723,8 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(a.f2 + (size_t)b * H2 * W2 * C, nbytes);
         const unsigned lane_off = vrow_ok ? ((unsigned)vrow * C + 16u * h) * 4u : nbytes;
         const int NJB = (CMODE == 3) ? 8 : (C >> 5);
-        constexpr bool BPIPE = !(MODE == MODE_WEIGHTED && KC >= 3);   // needs 16 more registers
-        constexpr bool DUAL = UR == 1 && !(MODE == MODE_WEIGHTED && KC >= 3);
+        constexpr bool BPIPE = !(is_weighted(MODE) && KC >= 3);   // needs 16 more registers
+        constexpr bool DUAL = UR == 1 && !(is_weighted(MODE) && KC >= 3);
         v4f bcur[4];
         if constexpr (BPIPE) {
 #pragma unroll
@@ -684,7 +745,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
             __builtin_amdgcn_sched_barrier(0);   // keep the loads here: a full block ahead of their use
         };
         auto computeF = [&](int step, int J, v4f(&buf)[UR][4]) {
-            if constexpr (MODE == MODE_WEIGHTED) {
+            if constexpr (is_weighted(MODE)) {
                 if (J == 0) {
 #pragma unroll
                     for (int r = 0; r < UR; ++r) {
@@ -692,6 +753,13 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
 #pragma unroll
                         for (int k = 0; k < KC; ++k) wur[r][k] = a.wu[(bp * a.KT + a.k0 + k) * H2 + u];
                     }
+                }
+                if (J == (NJB > 1 ? 1 : 0) && soft_logits) {   // (a block later: the loads above have landed by now)
+#pragma unroll
+                    for (int r = 0; r < UR; ++r)
+#pragma unroll
+                        for (int k = 0; k < KC; ++k)
+                            wur[r][k] = __expf(wur[r][k] - cst[2 * (pl * KC + k)]) * cst[2 * (pl * KC + k) + 1];
                 }
             }
             // C == 256 instantiation: the first MFMA of a row takes a literal zero as its addend, which saves
@@ -806,34 +874,44 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     }
     }
 
-    // flush the staged out_u rows: per pixel a contiguous run of NCHO*H2 floats
+    // flush the staged out_u rows of this piece (all rows of a whole tile): per pixel and channel a run of floats
     if (a.stage && vp == vpasses - 1) {
         __syncthreads();
-        const int cht = (MODE == MODE_WEIGHTED) ? a.KT : 2, ch0 = (MODE == MODE_WEIGHTED) ? a.k0 : 0;
-        if (whole) {
-            const int runlen = NCHO * H2;
-            for (int idx = tid; idx < TP * runlen; idx += blockDim.x) {
-                const int p = idx / runlen, o = idx - p * runlen;
-                if (p0 + p < N1) a.out_u[(((size_t)b * N1 + p0 + p) * cht + ch0) * H2 + o] = ostage[idx];
-            }
-            if constexpr (MODE == MODE_ARGMAX) {
-                for (int idx = tid; idx < TP * H2; idx += blockDim.x) {
-                    const int p = idx / H2;
-                    if (p0 + p < N1) a.am_u[((size_t)b * N1 + p0) * H2 + idx] = ostage_am[idx];
-                }
-            }
-        } else {   // the rows of this piece only: per pixel and channel a run of u1 - u0 floats
-            const int u0 = sa * NUG * UR, nu = min(H2, sb * NUG * UR) - u0;
-            for (int idx = tid; idx < TP * NCHO * nu; idx += blockDim.x) {
+        const int cht = (is_weighted(MODE)) ? a.KT : 2, ch0 = (is_weighted(MODE)) ? a.k0 : 0;
+        const int u0 = whole ? 0 : sa * NUG * UR, nu = (whole ? H2 : min(H2, sb * NUG * UR)) - u0;
+        const int total = TP * NCHO * nu;
+        constexpr int UNR = 4;   // the logits of a batch of elements are fetched before any of them is used
+        for (int base = tid; base < total; base += UNR * blockDim.x) {
+            float zs[UNR];
+            size_t off[UNR];
+            int lds_i[UNR], pk[UNR];
+#pragma unroll
+            for (int t = 0; t < UNR; ++t) {
+                const int idx = base + t * blockDim.x;
                 const int p = idx / (NCHO * nu), rem = idx - p * (NCHO * nu), ch = rem / nu, u = u0 + rem - ch * nu;
-                if (p0 + p < N1)
-                    a.out_u[(((size_t)b * N1 + p0 + p) * cht + ch0 + ch) * H2 + u] = ostage[(p * NCHO + ch) * H2 + u];
-            }
-            if constexpr (MODE == MODE_ARGMAX) {
-                for (int idx = tid; idx < TP * nu; idx += blockDim.x) {
-                    const int p = idx / nu, u = u0 + idx - p * nu;
-                    if (p0 + p < N1) a.am_u[((size_t)b * N1 + p0 + p) * H2 + u] = ostage_am[p * H2 + u];
+                const bool ok = idx < total && p0 + p < N1;
+                off[t] = ok ? ((((size_t)b * N1 + p0 + p) * cht + ch0 + ch) * H2 + u) : (size_t)-1;
+                lds_i[t] = (p * NCHO + ch) * H2 + u;
+                pk[t] = p * KC + ch;
+                zs[t] = 0.f;
+                if constexpr (is_weighted(MODE)) {
+                    if (soft_dlog && ok) zs[t] = a.z_ou[off[t]];
                 }
+            }
+#pragma unroll
+            for (int t = 0; t < UNR; ++t) {
+                if (off[t] == (size_t)-1) continue;
+                float x = ostage[lds_i[t]];
+                if constexpr (is_weighted(MODE)) {
+                    if (soft_dlog) x = dlogit3(zs[t], cst + 3 * pk[t], x);
+                }
+                a.out_u[off[t]] = x;
+            }
+        }
+        if constexpr (MODE == MODE_ARGMAX) {
+            for (int idx = tid; idx < TP * nu; idx += blockDim.x) {
+                const int p = idx / nu, u = u0 + idx - p * nu;
+                if (p0 + p < N1) a.am_u[((size_t)b * N1 + p0 + p) * H2 + u] = ostage_am[p * H2 + u];
             }
         }
     }
@@ -841,14 +919,14 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     // merge the running state of the row groups into group 0, one group at a time, through the LDS
     // region of the f1 tile (no longer needed).  Equal maxima keep the smaller row index.
     if (NUG > 1) {
-        constexpr int NQ = (MODE == MODE_WEIGHTED) ? KC : 3;
+        constexpr int NQ = (is_weighted(MODE)) ? KC : 3;
         float *mst = smem + vcw * (NQ * 16 * 64);   // [vcw][quantity][r][lane]
         for (int g2 = 1; g2 < NUG; ++g2) {
             __syncthreads();
             if (ug == g2) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    if constexpr (MODE == MODE_WEIGHTED) {
+                    if constexpr (is_weighted(MODE)) {
 #pragma unroll
                         for (int k = 0; k < KC; ++k) mst[(k * 16 + r) * 64 + lane] = rv[k][r];
                     } else {
@@ -862,7 +940,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
             if (ug == 0) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    if constexpr (MODE == MODE_WEIGHTED) {
+                    if constexpr (is_weighted(MODE)) {
 #pragma unroll
                         for (int k = 0; k < KC; ++k) rv[k][r] += mst[(k * 16 + r) * 64 + lane];
                     } else {
@@ -880,7 +958,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     // [column chunk][quantity][register group g4][lane][4]: every store of a wave is one contiguous KB
     if (!whole) {
         if (ug == 0 && vbase + 32 * vcw < W2) {
-            constexpr int NQ = (MODE == MODE_WEIGHTED) ? KC : 3;
+            constexpr int NQ = (is_weighted(MODE)) ? KC : 3;
             const __amdgpu_buffer_rsrc_t rs_sk = make_rsrc(a.sk_state, 2u * gridDim.x * (unsigned)a.sk_slot * 4u);
             const unsigned base = ((unsigned)(2 * wg + (pb == gs0 ? 0 : 1)) * (unsigned)a.sk_slot +
                                    (unsigned)((vbase >> 5) + vcw) * (NQ * 1024u) + 4u * lane) * 4u;
@@ -891,7 +969,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                     v4f x;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        if constexpr (MODE == MODE_WEIGHTED) x[e] = rv[q][4 * g4 + e];
+                        if constexpr (is_weighted(MODE)) x[e] = rv[q][4 * g4 + e];
                         else x[e] = q == 0 ? vmax[4 * g4 + e] : q == 1 ? __int_as_float(vidx[4 * g4 + e]) : vsum[4 * g4 + e];
                     }
                     store_shared4(rs_sk, base + (unsigned)(q * 4 + g4) * 1024u, x);
@@ -906,11 +984,18 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
             for (int g4 = 0; g4 < 4; ++g4) {
                 const int v = vbase + 32 * vcw + vmap(4 * g4, h);
                 if (v < W2) {
-                    if constexpr (MODE == MODE_WEIGHTED) {
+                    if constexpr (is_weighted(MODE)) {
 #pragma unroll
                         for (int k = 0; k < KC; ++k) {
-                            const v4f x = {rv[k][4 * g4], rv[k][4 * g4 + 1], rv[k][4 * g4 + 2], rv[k][4 * g4 + 3]};
-                            *reinterpret_cast<v4f *>(a.out_v + (bp * a.KT + a.k0 + k) * W2 + v) = x;
+                            v4f x = {rv[k][4 * g4], rv[k][4 * g4 + 1], rv[k][4 * g4 + 2], rv[k][4 * g4 + 3]};
+                            const size_t row = bp * a.KT + a.k0 + k;
+                            if (soft_dlog) {
+                                const float r3[3] = {a.st_ov[2 * row], 1.f / a.st_ov[2 * row + 1], a.dot_ov[row]};
+                                const v4f z = *reinterpret_cast<const v4f *>(a.z_ov + row * W2 + v);
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) x[e] = dlogit3(z[e], r3, x[e]);
+                            }
+                            *reinterpret_cast<v4f *>(a.out_v + row * W2 + v) = x;
                         }
                     } else {
                         const v4f xm = {vmax[4 * g4], vmax[4 * g4 + 1], vmax[4 * g4 + 2], vmax[4 * g4 + 3]};
@@ -930,9 +1015,12 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
             for (int r = 0; r < 16; ++r) {
                 const int v = vbase + 32 * vcw + vmap(r, h);
                 if (v < W2) {
-                    if constexpr (MODE == MODE_WEIGHTED) {
+                    if constexpr (is_weighted(MODE)) {
 #pragma unroll
-                        for (int k = 0; k < KC; ++k) a.out_v[(bp * a.KT + a.k0 + k) * W2 + v] = rv[k][r];
+                        for (int k = 0; k < KC; ++k) {
+                            const size_t row = bp * a.KT + a.k0 + k;
+                            a.out_v[row * W2 + v] = soft_dlog ? dlogit(a.z_ov, a.st_ov, a.dot_ov, row, row * W2 + v, rv[k][r]) : rv[k][r];
+                        }
                     } else {
                         a.out_v[(bp * 2 + 0) * W2 + v] = vmax[r];
                         a.out_v[(bp * 2 + 1) * W2 + v] = vsum[r] / (float)H2;
@@ -966,7 +1054,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         if (last) {
             // Add up the pieces in row order (equal maxima keep the lower row) and write the finished columns.
             // An item = the 4 consecutive columns a lane holds in one register group of one column chunk.
-            constexpr int NQ = (MODE == MODE_WEIGHTED) ? KC : 3;
+            constexpr int NQ = (is_weighted(MODE)) ? KC : 3;
             const __amdgpu_buffer_rsrc_t rs_sk = make_rsrc(a.sk_state, 2u * gridDim.x * (unsigned)a.sk_slot * 4u);
             const int nchunks = (W2 + 31) >> 5;
             for (int it = tid; it < nchunks * 256; it += blockDim.x) {
@@ -975,7 +1063,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                 v4f acc4[NQ];
 #pragma unroll
                 for (int q = 0; q < NQ; ++q) acc4[q] = v4f{0.f, 0.f, 0.f, 0.f};
-                if constexpr (MODE != MODE_WEIGHTED) acc4[0] = v4f{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+                if constexpr (!is_weighted(MODE)) acc4[0] = v4f{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
                 for (int w = wfirst; w <= wlast; ++w) {
                     const bool first_piece = ((long)w * sk_total) / G >= t0;   // w's share starts inside this tile
                     const unsigned base = ((unsigned)(2 * w + (first_piece ? 0 : 1)) * (unsigned)a.sk_slot +
@@ -983,7 +1071,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                     v4f x[NQ];
 #pragma unroll
                     for (int q = 0; q < NQ; ++q) x[q] = load_shared4(rs_sk, base + (unsigned)(q * 4 + g4) * 1024u);
-                    if constexpr (MODE == MODE_WEIGHTED) {
+                    if constexpr (is_weighted(MODE)) {
 #pragma unroll
                         for (int q = 0; q < NQ; ++q) acc4[q] += x[q];
                     } else {
@@ -995,10 +1083,28 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                 }
                 if (p0 + p >= N1) continue;
                 const size_t o = (size_t)b * N1 + p0 + p;
+                if constexpr (is_weighted(MODE)) {
+                    if (soft_dlog) {   // sums of softmax-output gradients -> gradients of the logits
+                        float r3[NQ][3], z[NQ][4];
+#pragma unroll
+                        for (int q = 0; q < NQ; ++q) {
+                            const size_t row = o * a.KT + a.k0 + q;
+                            r3[q][0] = a.st_ov[2 * row]; r3[q][1] = a.st_ov[2 * row + 1]; r3[q][2] = a.dot_ov[row];
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) z[q][e] = v + e < W2 ? a.z_ov[row * W2 + v + e] : 0.f;
+                        }
+#pragma unroll
+                        for (int q = 0; q < NQ; ++q) {
+                            r3[q][1] = 1.f / r3[q][1];
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) acc4[q][e] = dlogit3(z[q][e], r3[q], acc4[q][e]);
+                        }
+                    }
+                }
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     if (v + e >= W2) break;
-                    if constexpr (MODE == MODE_WEIGHTED) {
+                    if constexpr (is_weighted(MODE)) {
 #pragma unroll
                         for (int q = 0; q < NQ; ++q) a.out_v[(o * a.KT + a.k0 + q) * W2 + v + e] = acc4[q][e];
                     } else {
@@ -2179,6 +2285,52 @@ WaveGrid wave_grid(int B, int tiles_per_batch, int W2, int H2) {
     return g;
 }
 
+// Row-wise helpers of the softmax inside the weighted sweeps: one wave per row of L floats, lanes along the row.
+__device__ __forceinline__ float wave_max64(float x) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) x = fmaxf(x, __shfl_xor(x, o));
+    return x;
+}
+__device__ __forceinline__ float wave_sum64(float x) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o);
+    return x;
+}
+// st[row] = (max, sum of exp(z - max))
+__global__ void __launch_bounds__(256) row_stats_kernel(const float *__restrict__ z, float *__restrict__ st, long nrows, int L) {
+    const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (row >= nrows) return;
+    const float *r = z + row * L;
+    float m = -INFINITY;
+    for (int l = lane; l < L; l += 64) m = fmaxf(m, r[l]);
+    m = wave_max64(m);
+    float sum = 0.f;
+    for (int l = lane; l < L; l += 64) sum += __expf(r[l] - m);
+    sum = wave_sum64(sum);
+    if (lane == 0) { st[2 * row] = m; st[2 * row + 1] = sum; }
+}
+// dot[row] = sum_l x[row,l] * y[row,l]
+__global__ void __launch_bounds__(256) row_dot_kernel(const float *__restrict__ x, const float *__restrict__ y, float *__restrict__ dot,
+                                                      long nrows, int L) {
+    const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (row >= nrows) return;
+    float sum = 0.f;
+    for (int l = lane; l < L; l += 64) sum += x[row * L + l] * y[row * L + l];
+    sum = wave_sum64(sum);
+    if (lane == 0) dot[row] = sum;
+}
+// a[row,l] = exp(z[row,l] - max) / sum
+__global__ void __launch_bounds__(256) softmax_apply_kernel(const float *__restrict__ z, const float *__restrict__ st, float *__restrict__ a,
+                                                            long nrows, int L) {
+    const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (row >= nrows) return;
+    const float m = st[2 * row], il = 1.f / st[2 * row + 1];
+    for (int l = lane; l < L; l += 64) a[row * L + l] = __expf(z[row * L + l] - m) * il;
+}
+
 __global__ void __launch_bounds__(256) zero_ints_kernel(int *p, int n) {
     const int i = blockIdx.x * 256 + threadIdx.x;
     if (i < n) p[i] = 0;
@@ -2231,10 +2383,10 @@ int launch_fwd(FwdArgs a, int B, hipStream_t s) {
     a.nvc = wg.nvc;
     a.vpasses = wg.vpasses;
     const int nW = wg.nvc * wg.nug;
-    constexpr int NPART = (MODE == MODE_WEIGHTED) ? KC : 3;
+    constexpr int NPART = (is_weighted(MODE)) ? KC : 3;
     size_t lds = ((size_t)TP * (a.CP + 4) + 2 * UR * NPART * nW * 32) * sizeof(float);
     {   // stage out_u in LDS when two workgroups still fit a CU's 160 KB
-        constexpr int NCHO = (MODE == MODE_WEIGHTED) ? KC : 2;
+        constexpr int NCHO = (is_weighted(MODE)) ? KC : 2;
         const size_t extra = (size_t)TP * (NCHO + (MODE == MODE_ARGMAX ? 1 : 0)) * a.H2 * sizeof(float);
         a.stage = lds + extra <= 80 * 1024;
         if (a.stage) lds += extra;
@@ -2242,6 +2394,7 @@ int launch_fwd(FwdArgs a, int B, hipStream_t s) {
         const size_t merge = wg.nug > 1 ? (size_t)wg.nvc * NPART * 16 * 64 * sizeof(float) : 0;
         if (lds < merge) lds = merge;
     }
+    if (MODE == MODE_SOFT) lds += (size_t)TP * KC * 3 * sizeof(float);   // row statistics of the tile
     dim3 grid(B * a.tiles_per_batch);
     const dim3 block(64 * nW);
     a.sk_total = 0;
@@ -2264,21 +2417,21 @@ int launch_fwd(FwdArgs a, int B, hipStream_t s) {
     do {                                                                         \
         auto k = a.sk_total ? fwd_kernel<MODE, KC, UR, CV, RGV, false, true> : fwd_kernel<MODE, KC, UR, CV, RGV>; \
         if (int rc = set_lds(k, lds)) return rc;                                 \
-        ProfScope ps(MODE == MODE_WEIGHTED ? "fwd_weighted" : "fwd_maxavg", s);  \
+        ProfScope ps(is_weighted(MODE) ? "fwd_weighted" : "fwd_maxavg", s);  \
         hipLaunchKernelGGL(k, grid, block, lds, s, a);                           \
     } while (0)
     // Always built for two waves per SIMD (256 registers): the accumulators then stay in ordinary
     // VGPRs, where the epilogue reads them without accumulator-register copies.
     if (wg.vpasses == 1 && cmode == 3 && a.f2_planes) {   // bf16-plane variant: the caller has split fmap2
         // LDS with the larger f1 tile (three bf16 planes); out_u staging only if two workgroups still fit a CU
-        constexpr int NCHO = (MODE == MODE_WEIGHTED) ? KC : 2;
+        constexpr int NCHO = (is_weighted(MODE)) ? KC : 2;
         lds = ((size_t)TP * BF_LS + 2 * UR * NPART * nW * 32) * sizeof(float);
         const size_t extra = (size_t)TP * (NCHO + (MODE == MODE_ARGMAX ? 1 : 0)) * a.H2 * sizeof(float);
         a.stage = lds + extra <= 80 * 1024;
         if (a.stage) lds += extra;
         const size_t merge = wg.nug > 1 ? (size_t)wg.nvc * NPART * 16 * 64 * sizeof(float) : 0;
         if (lds < merge) lds = merge;
-        ProfScope ps(MODE == MODE_WEIGHTED ? "fwd_weighted_bf16x3" : "fwd_maxavg_bf16x3", s);
+        ProfScope ps(is_weighted(MODE) ? "fwd_weighted_bf16x3" : "fwd_maxavg_bf16x3", s);
         if (wg.nug > 1) {
             auto k = fwd_kernel<MODE, KC, UR, 3, 1, true>;
             if (int rc = set_lds(k, lds)) return rc;
@@ -2311,6 +2464,22 @@ SEPCORR_FWD_DECL(MODE_WEIGHTED, 1, 2);
 SEPCORR_FWD_DECL(MODE_WEIGHTED, 2, 2);
 SEPCORR_FWD_DECL(MODE_WEIGHTED, 3, 1);
 SEPCORR_FWD_DECL(MODE_WEIGHTED, 4, 1);
+SEPCORR_FWD_DECL(MODE_SOFT, 1, 2);
+SEPCORR_FWD_DECL(MODE_SOFT, 2, 2);
+SEPCORR_FWD_DECL(MODE_SOFT, 3, 1);
+SEPCORR_FWD_DECL(MODE_SOFT, 4, 1);
+#if SEPCORR_IN_PART(12)
+SEPCORR_FWD_INST(MODE_SOFT, 1, 2);
+#endif
+#if SEPCORR_IN_PART(13)
+SEPCORR_FWD_INST(MODE_SOFT, 2, 2);
+#endif
+#if SEPCORR_IN_PART(14)
+SEPCORR_FWD_INST(MODE_SOFT, 3, 1);
+#endif
+#if SEPCORR_IN_PART(15)
+SEPCORR_FWD_INST(MODE_SOFT, 4, 1);
+#endif
 #if SEPCORR_IN_PART(1)
 SEPCORR_FWD_INST(MODE_MAXAVG, 1, 2);
 #endif
@@ -2400,20 +2569,27 @@ FwdArgs fwd_args(const Dims &d) {
 }
 
 // sum_v S wv[k,v] -> out_u[k,u];  sum_u S wu[k,u] -> out_v[k,v]  for K channels, KCH per launch
+// soft (optional): the softmax fields of FwdArgs (logits / dlog and what they refer to)
 int weighted_forward(const Dims &d, const float *f1, const float *f2, const float *wv, const float *wu, float *out_u,
-                     float *out_v, int K, void *ws, size_t ws_bytes, hipStream_t s) {
+                     float *out_v, int K, void *ws, size_t ws_bytes, hipStream_t s, const FwdArgs *soft = nullptr) {
     FwdArgs a = fwd_args(d);
     a.f1 = f1; a.f2 = f2; a.wv = wv; a.wu = wu; a.out_u = out_u; a.out_v = out_v;
     a.KT = K;
     a.ws = ws; a.ws_bytes = ws_bytes;
+    if (soft) {
+        a.logits = soft->logits; a.dlog = soft->dlog; a.st_wv = soft->st_wv; a.st_wu = soft->st_wu;
+        a.z_ou = soft->z_ou; a.st_ou = soft->st_ou; a.dot_ou = soft->dot_ou;
+        a.z_ov = soft->z_ov; a.st_ov = soft->st_ov; a.dot_ov = soft->dot_ov;
+    }
     Bf16Planes planes;
+    if (!soft)   // (the bf16-plane variant of the sweep has no softmax inside)
     if (int rc = planes.make(d, f2, s)) return rc;
     a.f2_planes = static_cast<const char *>(planes.ptr);
     a.H2p = planes.H2p;
     for (int k0 = 0; k0 < K; k0 += KCH) {
         a.k0 = k0;
         const int kc = K - k0 < KCH ? K - k0 : KCH;
-        if (int rc = launch_fwd_weighted_k<MODE_WEIGHTED>(a, kc, d.B, s)) return rc;
+        if (int rc = soft ? launch_fwd_weighted_k<MODE_SOFT>(a, kc, d.B, s) : launch_fwd_weighted_k<MODE_WEIGHTED>(a, kc, d.B, s)) return rc;
     }
     return SEPCORR_OK;
 }
@@ -3031,6 +3207,130 @@ int sepcorr_compression_backward(const float *f1, const float *f2, const float *
     a.B = B; a.N1 = H1 * W1; a.H2 = H2; a.W2 = W2; a.C = C; a.KT = K;
     const int kch = W2 > 128 ? 2 : KCH;  // wide workgroups have half the registers per lane
     // channel chunks accumulate into d_f1 / d_f2: each output keeps its own stream, so chunks stay ordered
+    for (int k0 = 0; k0 < K && rc == SEPCORR_OK; k0 += kch) {
+        a.k0 = k0;
+        a.accumulate = k0 > 0;
+        const int kc = K - k0 < kch ? K - k0 : kch;
+        switch (kc) {
+            case 1: rc = launch_bwd<GMODE_COMP, 1>(a, d, workspace, fj.sa, fj.sb); break;
+            case 2: rc = launch_bwd<GMODE_COMP, 2>(a, d, workspace, fj.sa, fj.sb); break;
+            case 3: rc = launch_bwd<GMODE_COMP, 3>(a, d, workspace, fj.sa, fj.sb); break;
+            default: rc = launch_bwd<GMODE_COMP, 4>(a, d, workspace, fj.sa, fj.sb); break;
+        }
+    }
+    const int rj = fj.join();
+    return rc ? rc : rj;
+}
+
+// ---- attention compression straight from the logits -------------------------------------------------------------
+
+int sepcorr_softmax_rows(const float *logits, float *stats, int stats_given, float *a, long nrows, int L, void *stream) {
+    api_enter();
+    REQUIRE_PTR(logits); REQUIRE_PTR(stats);
+    if (nrows < 1 || L < 1) return fail(SEPCORR_EINVAL, "sepcorr: softmax rows: nrows=%ld L=%d", nrows, L);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dim3 grid((unsigned)((nrows + 3) / 4)), block(256);
+    if (!stats_given) hipLaunchKernelGGL(row_stats_kernel, grid, block, 0, s, logits, stats, nrows, L);
+    if (a) hipLaunchKernelGGL(softmax_apply_kernel, grid, block, 0, s, logits, stats, a, nrows, L);
+    return check_launch("softmax rows");
+}
+
+int sepcorr_compression_forward_from_logits(const float *f1, const float *f2, const float *logits_u, const float *logits_v,
+                                            float *comp_u, float *comp_v, float *stats_u, float *stats_v, int stats_given,
+                                            int B, int H1, int W1, int H2, int W2, int C, int K, void *workspace,
+                                            size_t workspace_bytes, void *stream) {
+    api_enter();
+    REQUIRE_PTR(f1); REQUIRE_PTR(f2); REQUIRE_PTR(logits_u); REQUIRE_PTR(logits_v); REQUIRE_PTR(comp_u); REQUIRE_PTR(comp_v);
+    REQUIRE_PTR(stats_u); REQUIRE_PTR(stats_v);
+    const Dims d = {B, H1, W1, H2, W2, C};
+    if (int rc = check_dims(d, K)) return rc;
+    if (int rc = check_fwd_workspace(d, K, workspace, workspace_bytes)) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const long nrows = (long)B * H1 * W1 * K;
+    if (!stats_given) {   // (max, sum of exp) per row: one pass over the logits
+        const dim3 grid((unsigned)((nrows + 3) / 4)), block(256);
+        ProfScope ps("row_stats", s);
+        hipLaunchKernelGGL(row_stats_kernel, grid, block, 0, s, logits_u, stats_u, nrows, W2);
+        hipLaunchKernelGGL(row_stats_kernel, grid, block, 0, s, logits_v, stats_v, nrows, H2);
+        if (int rc = check_launch("row statistics")) return rc;
+    }
+    FwdArgs soft;
+    memset(&soft, 0, sizeof(soft));
+    soft.logits = 1; soft.st_wv = stats_u; soft.st_wu = stats_v;
+    return weighted_forward(d, f1, f2, logits_u, logits_v, comp_u, comp_v, K, workspace, workspace_bytes, s, &soft);
+}
+
+size_t sepcorr_compression_backward_from_logits_workspace_bytes(int B, int H1, int W1, int H2, int W2, int C, int K,
+                                                                int with_features) {
+    if (B < 1 || H1 < 1 || W1 < 1 || H2 < 1 || W2 < 1 || C < 1 || K < 1 || K > MAX_K) return 0;
+    const Dims d = {B, H1, W1, H2, W2, C};
+    const size_t rows = (size_t)B * H1 * W1 * K;
+    const size_t dots = 2 * ((rows * sizeof(float) + 255) & ~(size_t)255);
+    if (!with_features) return ((fwd_split_bytes(B, H1, W1, H2, W2, K) + 255) & ~(size_t)255) + dots;
+    const size_t a_bytes = ((rows * W2 * sizeof(float) + 255) & ~(size_t)255) + ((rows * H2 * sizeof(float) + 255) & ~(size_t)255);
+    return bwd_ws(d).total + dots + a_bytes;
+}
+
+int sepcorr_compression_backward_from_logits(const float *f1, const float *f2, const float *logits_u, const float *logits_v,
+                                             const float *stats_u, const float *stats_v, const float *comp_u,
+                                             const float *comp_v, const float *g_cu, const float *g_cv, float *d_f1,
+                                             float *d_f2, float *d_logits_u, float *d_logits_v, int B, int H1, int W1, int H2,
+                                             int W2, int C, int K, void *workspace, size_t workspace_bytes, void *stream) {
+    api_enter();
+    REQUIRE_PTR(f1); REQUIRE_PTR(f2); REQUIRE_PTR(logits_u); REQUIRE_PTR(logits_v); REQUIRE_PTR(stats_u); REQUIRE_PTR(stats_v);
+    REQUIRE_PTR(comp_u); REQUIRE_PTR(comp_v); REQUIRE_PTR(g_cu); REQUIRE_PTR(g_cv); REQUIRE_PTR(d_logits_u); REQUIRE_PTR(d_logits_v);
+    const Dims d = {B, H1, W1, H2, W2, C};
+    if (int rc = check_dims(d, K)) return rc;
+    if ((d_f1 == nullptr) != (d_f2 == nullptr))
+        return fail(SEPCORR_EINVAL, "sepcorr: d_f1 and d_f2 must be given together or both be NULL");
+    const size_t need = sepcorr_compression_backward_from_logits_workspace_bytes(B, H1, W1, H2, W2, C, K, d_f1 != nullptr);
+    if (workspace == nullptr || workspace_bytes < need)
+        return fail(SEPCORR_EWORKSPACE, "sepcorr: backward from logits needs %zu bytes of workspace, got %zu", need,
+                    workspace ? workspace_bytes : (size_t)0);
+    if (reinterpret_cast<uintptr_t>(workspace) & 255) return fail(SEPCORR_EWORKSPACE, "sepcorr: workspace must be 256-byte aligned");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t rows = (size_t)B * H1 * W1 * K;
+    const size_t dot_bytes = (rows * sizeof(float) + 255) & ~(size_t)255;
+    const size_t sweep_bytes = d_f1 ? bwd_ws(d).total : (fwd_split_bytes(B, H1, W1, H2, W2, K) + 255) & ~(size_t)255;
+    char *base = static_cast<char *>(workspace);
+    float *dot_u = reinterpret_cast<float *>(base + sweep_bytes);               // sum_u g_cu * comp_u = sum_v a_u * d_a_u
+    float *dot_v = reinterpret_cast<float *>(base + sweep_bytes + dot_bytes);   // sum_v g_cv * comp_v = sum_u a_v * d_a_v
+    {
+        const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+        ProfScope ps("row_dots", s);
+        hipLaunchKernelGGL(row_dot_kernel, grid, block, 0, s, g_cu, comp_u, dot_u, (long)rows, H2);
+        hipLaunchKernelGGL(row_dot_kernel, grid, block, 0, s, g_cv, comp_v, dot_v, (long)rows, W2);
+        if (int rc = check_launch("row dot products")) return rc;
+    }
+    // d_a_v[k,u] = sum_v S g_cv[k,v] and d_a_u[k,v] = sum_u S g_cu[k,u] as in sepcorr_compression_backward, turned into
+    // gradients of the logits where they are stored: d_z = a (d_a - sum a d_a), the sums being the dot products above
+    FwdArgs soft;
+    memset(&soft, 0, sizeof(soft));
+    soft.dlog = 1;
+    soft.z_ou = logits_v; soft.st_ou = stats_v; soft.dot_ou = dot_v;
+    soft.z_ov = logits_u; soft.st_ov = stats_u; soft.dot_ov = dot_u;
+    const size_t fwd_bytes = fwd_split_bytes(B, H1, W1, H2, W2, d_f1 ? MAX_K : K);
+    int rc = weighted_forward(d, f1, f2, g_cv, g_cu, d_logits_v, d_logits_u, K, fwd_bytes ? workspace : nullptr, fwd_bytes, s, &soft);
+    if (rc || d_f1 == nullptr) return rc;
+    // feature gradients: the weights themselves, formed once from logits and statistics behind the other scratch
+    float *a_u = reinterpret_cast<float *>(base + sweep_bytes + 2 * dot_bytes);
+    float *a_v = reinterpret_cast<float *>(base + sweep_bytes + 2 * dot_bytes + ((rows * W2 * sizeof(float) + 255) & ~(size_t)255));
+    {
+        const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+        ProfScope ps("softmax_apply", s);
+        hipLaunchKernelGGL(softmax_apply_kernel, grid, block, 0, s, logits_u, stats_u, a_u, (long)rows, W2);
+        hipLaunchKernelGGL(softmax_apply_kernel, grid, block, 0, s, logits_v, stats_v, a_v, (long)rows, H2);
+        if (int rc2 = check_launch("softmax from statistics")) return rc2;
+    }
+    const BwdWs lay = bwd_ws(d);
+    ForkJoin fj(s, !lay.aliased);
+    BwdArgs a;
+    memset(&a, 0, sizeof(a));
+    a.xcd_order = xcd_order_enabled();
+    a.f1 = f1; a.f2 = f2; a.a_u = a_u; a.a_v = a_v; a.g_cu = g_cu; a.g_cv = g_cv;
+    a.d1 = d_f1; a.d2 = d_f2;
+    a.B = B; a.N1 = H1 * W1; a.H2 = H2; a.W2 = W2; a.C = C; a.KT = K;
+    const int kch = W2 > 128 ? 2 : KCH;
     for (int k0 = 0; k0 < K && rc == SEPCORR_OK; k0 += kch) {
         a.k0 = k0;
         a.accumulate = k0 > 0;

@@ -79,6 +79,58 @@ class ComputeSelfCompressionFunction(Function):
         return d1.contiguous(), d2.contiguous(), da_u.contiguous(), da_v.contiguous()
 
 
+class ComputeSelfCompressionFromLogitsFunction(Function):
+    """ComputeSelfCompressionFunction with the softmax inside: apply(fmap1, fmap2, logits_u, logits_v) equals
+    ComputeSelfCompressionFunction.apply(fmap1, fmap2, logits_u.softmax(-1), logits_v.softmax(-1)) in values and
+    gradients (core/corr.py:441-448, functions/MemorySaver.py:107-177).  Not a class of the reference.
+
+    Saved for backward: the logits, their row statistics (max, sum of exp) and the outputs; no tensor of softmax
+    outputs or of their gradients exists in either direction.
+    """
+
+    @staticmethod
+    def forward(ctx, img1_features_l0, img2_features_lk, logits_u, logits_v, stats_u=None, stats_v=None):
+        """stats_u, stats_v (optional): row statistics (max, sum of exp) of the logits, as AttentionLogitsFunction
+        returns them; computed here when absent."""
+        _contig(img1_features_l0, img2_features_lk, logits_u, logits_v)
+        with torch.cuda.device_of(img1_features_l0):
+            cu, cv, st_u, st_v = MemorySaver.compression_forward_from_logits(img1_features_l0, img2_features_lk,
+                                                                             logits_u, logits_v, stats_u, stats_v)
+        ctx.save_for_backward(img1_features_l0, img2_features_lk, logits_u, logits_v, st_u, st_v, cu, cv)
+        return cu, cv
+
+    @staticmethod
+    def backward(ctx, grad_compressed_output_u, grad_compressed_output_v):
+        f1, f2, z_u, z_v, st_u, st_v, cu, cv = ctx.saved_tensors
+        with torch.cuda.device_of(f1):
+            d1, d2, dz_u, dz_v = MemorySaver.compression_backward_from_logits(
+                f1, f2, z_u, z_v, st_u, st_v, cu, cv,
+                grad_compressed_output_u.contiguous(), grad_compressed_output_v.contiguous())
+        return d1, d2, dz_u, dz_v, None, None
+
+
+class AttentionLogitsFunction(Function):
+    """Conv3d(2 -> K, 3, padding=1) of a max/avg volume in the operator's layout: the attention module's output
+    before the softmax (core/corr.py:441-442 applies softmax(dim=2) to it).  Not a class of the reference.
+    -> (logits (B,H1,W1,K,L), stats (B,H1,W1,K,2)); stats = per row (max, sum of exp), a by-product without gradient
+    that ComputeSelfCompressionFromLogitsFunction takes."""
+
+    @staticmethod
+    def forward(ctx, sep, weight, bias):
+        _contig(sep, weight)
+        z, st = MemorySaver.attention_logits_forward(sep, weight, bias)
+        ctx.save_for_backward(sep, weight)
+        ctx.has_bias = bias is not None
+        ctx.mark_non_differentiable(st)
+        return z, st
+
+    @staticmethod
+    def backward(ctx, grad_z, _grad_stats=None):
+        sep, weight = ctx.saved_tensors
+        d_sep, d_w, d_b = MemorySaver.attention_logits_backward(sep, weight, grad_z.contiguous(), need_bias=ctx.has_bias)
+        return d_sep, d_w, d_b
+
+
 class AttentionWeightsFunction(Function):
     """softmax over L of Conv3d(2 -> K, 3, padding=1) of a max/avg volume, in the operator's layout.
 
@@ -103,7 +155,7 @@ class AttentionWeightsFunction(Function):
 
 class SeparateLevelFunction(Function):
     """One pyramid level of the caller's loop (core/corr.py:416-457) as a single autograd node:
-    max/argmax/avg forward -> attention weights of both volumes -> compression forward.
+    max/argmax/avg forward -> attention logits of both volumes -> compression forward from the logits.
 
     Not a class of the reference.  Results equal the chain ComputeMaxArgmaxAvgFunction ->
     AttentionWeightsFunction x2 -> ComputeSelfCompressionFunction; the point is the backward pass: the
@@ -119,23 +171,32 @@ class SeparateLevelFunction(Function):
         _contig(f1, f2, weight1, weight2)
         with torch.cuda.device_of(f1):
             out_u, out_v, am_u, am_v = MemorySaver.max_argmax_avg_forward(f1, f2)
-            a_u = MemorySaver.attention_forward(out_v, weight1, bias1)
-            a_v = MemorySaver.attention_forward(out_u, weight2, bias2)
-            cu, cv = MemorySaver.compression_forward(f1, f2, a_u, a_v)
-        ctx.save_for_backward(f1, f2, am_u, am_v, out_u, out_v, a_u, a_v, weight1, weight2)
+            # the attention modules stop at the logits (and hand over the row statistics of their softmax, which
+            # they have at hand); the softmax itself happens where the compression sweep loads its weights
+            z_u, st_u = MemorySaver.attention_logits_forward(out_v, weight1, bias1)
+            z_v, st_v = MemorySaver.attention_logits_forward(out_u, weight2, bias2)
+            cu, cv, _, _ = MemorySaver.compression_forward_from_logits(f1, f2, z_u, z_v, st_u, st_v)
+        ctx.save_for_backward(f1, f2, am_u, am_v, out_u, out_v, z_u, z_v, st_u, st_v, cu, cv, weight1, weight2)
         ctx.has_bias = (bias1 is not None, bias2 is not None)
         return out_u, out_v, cu, cv
 
     @staticmethod
     def backward(ctx, g_u, g_v, g_cu, g_cv):
-        f1, f2, am_u, am_v, out_u, out_v, a_u, a_v, weight1, weight2 = ctx.saved_tensors
+        f1, f2, am_u, am_v, out_u, out_v, z_u, z_v, st_u, st_v, cu, cv, weight1, weight2 = ctx.saved_tensors
         g_u, g_v, g_cu, g_cv = (g.contiguous() for g in (g_u, g_v, g_cu, g_cv))
         with torch.cuda.device_of(f1):
-            da_u, da_v = MemorySaver.compression_weight_gradients(f1, f2, a_u, a_v, g_cu, g_cv)
-            d_out_v, d_w1, d_b1 = MemorySaver.attention_backward(out_v, weight1, a_u, da_u, need_bias=ctx.has_bias[0])
-            d_out_u, d_w2, d_b2 = MemorySaver.attention_backward(out_u, weight2, a_v, da_v, need_bias=ctx.has_bias[1])
+            # gradients of the logits straight from the weight-gradient sweep (no d_a tensors, no softmax backward)
+            _, _, dz_u, dz_v = MemorySaver.compression_backward_from_logits(f1, f2, z_u, z_v, st_u, st_v, cu, cv, g_cu, g_cv,
+                                                                            need_features=False)
+            d_out_v, d_w1, d_b1 = MemorySaver.attention_logits_backward(out_v, weight1, dz_u, need_bias=ctx.has_bias[0])
+            d_out_u, d_w2, d_b2 = MemorySaver.attention_logits_backward(out_u, weight2, dz_v, need_bias=ctx.has_bias[1])
+            del dz_u, dz_v
             d_out_u += g_u
             d_out_v += g_v
+            # the combined feature-gradient contraction reads the weights themselves: formed here from the saved
+            # statistics, for the duration of this call only
+            a_u = MemorySaver.softmax_from_stats(z_u, st_u)
+            a_v = MemorySaver.softmax_from_stats(z_v, st_v)
             d1, d2 = MemorySaver.fused_backward(f1, f2, am_u, am_v, d_out_u, d_out_v, a_u, a_v, g_cu, g_cv)
         return d1, d2, d_w1, d_b1, d_w2, d_b2
 

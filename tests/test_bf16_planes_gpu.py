@@ -185,7 +185,8 @@ def test_corr_block_with_planes(device, planes):
         return c1, c2, w1, w2
 
     (c1, c2, w1, w2), labels = _labels_of(run)
-    assert {"fwd_maxavg_bf16x3", "fwd_weighted_bf16x3", "df1_both_bf16x3"} <= labels, labels
+    # (the compression sweeps of this path take logits, which the plane variant of the sweep does not: fp32 there)
+    assert {"fwd_maxavg_bf16x3", "df1_both_bf16x3"} <= labels, labels
     assert_close(c1, rc1, "corr1")
     assert_close(c2, rc2, "corr2")
     ((rc1 * w1.double()).sum() + (rc2 * w2.double()).sum()).backward()

@@ -352,3 +352,52 @@ def test_corrblock4d_shapes_and_channel_order_with_attention():
     # a softmax-weighted sum lies between min and max of what it averages
     s = O.corr_volume(f1, f2)
     assert torch.all(cu <= s.max(dim=4)[0].unsqueeze(3) + 1e-5) and torch.all(cu >= s.min(dim=4)[0].unsqueeze(3) - 1e-5)
+
+
+def test_compression_from_logits_closed_forms_and_gradient_structure():
+    """Pins oracle.compression_from_logits (softmax over the kept axis + compression, core/corr.py:441-448):
+    constant logits give uniform weights, i.e. the avg channel of the max/avg operator; a row with one dominant
+    logit picks one slice of the volume; the gradient of the logits equals the explicit softmax-backward formula
+    applied to the operator's weight gradients, each of its rows sums to zero, and the row sums of a * d_a equal
+    the dot products of upstream gradient and output (the identity the fused backward uses)."""
+    B, H1, W1, H2, W2, C, K = 1, 3, 4, 5, 6, 8, 2
+    g = torch.Generator().manual_seed(31)
+    f1 = torch.randn(B, H1, W1, C, generator=g, dtype=torch.float64)
+    f2 = torch.randn(B, H2, W2, C, generator=g, dtype=torch.float64)
+    s = O.corr_volume(f1, f2)
+    # constant logits (any constant): comp_u = mean over v, comp_v = mean over u
+    cu, cv = O.compression_from_logits(f1, f2, torch.full((B, H1, W1, K, W2), 3.7, dtype=torch.float64),
+                                       torch.full((B, H1, W1, K, H2), -1.2, dtype=torch.float64))
+    assert torch.allclose(cu, s.mean(dim=4).unsqueeze(3).expand(-1, -1, -1, K, -1), atol=1e-12)
+    assert torch.allclose(cv, s.mean(dim=3).unsqueeze(3).expand(-1, -1, -1, K, -1), atol=1e-12)
+    # one dominant logit at column 2 / row 4: the slices S[..., :, 2] and S[..., 4, :]
+    z_u = torch.zeros(B, H1, W1, K, W2, dtype=torch.float64); z_u[..., 2] = 800.0
+    z_v = torch.zeros(B, H1, W1, K, H2, dtype=torch.float64); z_v[..., 4] = 800.0
+    cu, cv = O.compression_from_logits(f1, f2, z_u, z_v)
+    assert torch.allclose(cu[:, :, :, 0], s[..., 2], atol=1e-12) and torch.allclose(cv[:, :, :, 1], s[:, :, :, 4], atol=1e-12)
+    # gradients
+    z_u = torch.randn(B, H1, W1, K, W2, generator=g, dtype=torch.float64).requires_grad_()
+    z_v = torch.randn(B, H1, W1, K, H2, generator=g, dtype=torch.float64).requires_grad_()
+    g_cu = torch.randn(B, H1, W1, K, H2, generator=g, dtype=torch.float64)
+    g_cv = torch.randn(B, H1, W1, K, W2, generator=g, dtype=torch.float64)
+    cu, cv = O.compression_from_logits(f1, f2, z_u, z_v)
+    ((cu * g_cu).sum() + (cv * g_cv).sum()).backward()
+    a_u, a_v = z_u.detach().softmax(-1), z_v.detach().softmax(-1)
+    _, _, da_u, da_v = O.compression_backward(f1, f2, a_u, a_v, g_cu, g_cv)
+    for dz, a, da, gc, comp in ((z_u.grad, a_u, da_u, g_cu, cu.detach()), (z_v.grad, a_v, da_v, g_cv, cv.detach())):
+        dot = (a * da).sum(-1, keepdim=True)
+        assert torch.allclose(dz, a * (da - dot), atol=1e-12)
+        assert float(dz.sum(-1).abs().max()) < 1e-12
+        assert torch.allclose(dot.squeeze(-1), (gc * comp).sum(-1), atol=1e-12)
+
+
+def test_attention_logits_is_the_producer_without_softmax():
+    g = torch.Generator().manual_seed(7)
+    sep = torch.randn(2, 3, 4, 2, 9, generator=g, dtype=torch.float64)
+    w = torch.randn(3, 2, 3, 3, 3, generator=g, dtype=torch.float64)
+    b = torch.randn(3, generator=g, dtype=torch.float64)
+    z = O.attention_logits(sep, w, b)
+    assert torch.allclose(z.softmax(-1), O.attention_weights(sep, w, b), atol=1e-13)
+    # a one-tap filter at the centre copies channel 0 (plus bias)
+    w1 = torch.zeros(1, 2, 3, 3, 3, dtype=torch.float64); w1[0, 0, 1, 1, 1] = 1.0
+    assert torch.allclose(O.attention_logits(sep, w1, torch.tensor([0.5], dtype=torch.float64))[:, :, :, 0], sep[:, :, :, 0] + 0.5)
