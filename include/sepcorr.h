@@ -212,6 +212,38 @@ int sepcorr_compression_backward_from_logits(const float *f1, const float *f2,
                                              void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * The same operators for several pyramid levels of fmap2 in one call: level l is (B,h2[l],w2[l],C), all pointer tables
+ * and the size tables are host arrays of nlev <= 4 entries, outputs per level as in the single-level calls.  Replaces
+ * the loop over levels of the caller (core/corr.py:416-457): one launch covers all levels given (their work is dealt
+ * out together and the image-1 tile is shared) when every w2[l] is at most 128 and fills 1, 2 or 4 chunks of 32
+ * columns, C is a multiple of 32 and scratch is given; other shapes run level by level inside the call.
+ *   workspace: sepcorr_forward_levels_workspace_bytes(...) bytes, 256-byte aligned; optional (NULL) for the two forward
+ *   calls, required for the backward call.  The statistics of the logits are inputs here (the attention producer
+ *   supplies them); the backward call returns the logit gradients only (feature gradients: sepcorr_fused_backward or
+ *   sepcorr_compression_backward_from_logits per level).
+ */
+size_t sepcorr_forward_levels_workspace_bytes(const int *h2, const int *w2, int nlev, int B, int H1, int W1, int C, int K);
+int sepcorr_max_argmax_avg_forward_levels(const float *f1, const float *const *f2_levels, const int *h2, const int *w2, int nlev,
+                                          float *const *out_u, float *const *out_v,
+                                          int32_t *const *argmax_u, int32_t *const *argmax_v,
+                                          int B, int H1, int W1, int C,
+                                          void *workspace, size_t workspace_bytes, void *stream);
+int sepcorr_compression_forward_from_logits_levels(const float *f1, const float *const *f2_levels, const int *h2, const int *w2,
+                                                   int nlev, const float *const *logits_u, const float *const *logits_v,
+                                                   const float *const *stats_u, const float *const *stats_v,
+                                                   float *const *comp_u, float *const *comp_v,
+                                                   int B, int H1, int W1, int C, int K,
+                                                   void *workspace, size_t workspace_bytes, void *stream);
+int sepcorr_compression_backward_from_logits_levels(const float *f1, const float *const *f2_levels, const int *h2, const int *w2,
+                                                    int nlev, const float *const *logits_u, const float *const *logits_v,
+                                                    const float *const *stats_u, const float *const *stats_v,
+                                                    const float *const *comp_u, const float *const *comp_v,
+                                                    const float *const *g_cu, const float *const *g_cv,
+                                                    float *const *d_logits_u, float *const *d_logits_v,
+                                                    int B, int H1, int W1, int C, int K,
+                                                    void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * Row softmax helper of the two calls above for callers that need the weights themselves: for nrows rows of L logits,
  * stats (nrows,2) = (max, sum of exp) is computed (stats_given == 0) or read, and, when a is not NULL,
  * a = exp(z - max) / sum is written.  No counterpart in the reference (torch's softmax stands there, core/corr.py:441).

@@ -313,6 +313,95 @@ def attention_logits_backward(sep, weight, grad_logits, need_bias=True):
     return [d_sep, d_w, d_b]
 
 
+# --- several pyramid levels per call (the caller's loop over levels, core/corr.py:416-457)
+
+def _levels_setup(f1, f2_levels, K):
+    import ctypes
+    _check("img1_features_l0", f1, ndim=4)
+    B, H1, W1, C = f1.shape
+    lv = list(f2_levels)
+    if not 1 <= len(lv) <= 4:
+        raise RuntimeError("1 to 4 fmap2 levels are supported per call")
+    for n, t in enumerate(lv):
+        _check(f"img2_features_lvls[{n}]", t, ndim=4)
+        if t.shape[0] != B or t.shape[3] != C or t.device != f1.device:
+            raise RuntimeError(f"img2_features_lvls[{n}]: batch/feature size or device differs from img1_features_l0")
+    L = len(lv)
+    h2 = (ctypes.c_int * L)(*[t.shape[1] for t in lv])
+    w2 = (ctypes.c_int * L)(*[t.shape[2] for t in lv])
+    lib = _lib.load()
+    n = lib.sepcorr_forward_levels_workspace_bytes(h2, w2, L, B, H1, W1, C, K)
+    ws = torch.empty(max(n, 256), dtype=torch.uint8, device=f1.device)
+    return lib, B, H1, W1, C, L, h2, w2, ws, n
+
+
+def _ptrs(ts):
+    import ctypes
+    return (ctypes.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
+
+
+def max_argmax_avg_forward_levels(img1_features_l0, img2_features_lvls):
+    """max_argmax_avg_forward for every level of the fmap2 pyramid in one call -> list of [out_u, out_v, argmax_u, argmax_v]."""
+    f1, lv = img1_features_l0, list(img2_features_lvls)
+    lib, B, H1, W1, C, L, h2, w2, ws, n = _levels_setup(f1, lv, 2)
+    dev = f1.device
+    with torch.cuda.device(dev):
+        ou = [torch.empty((B, H1, W1, 2, t.shape[1]), dtype=f1.dtype, device=dev) for t in lv]
+        ov = [torch.empty((B, H1, W1, 2, t.shape[2]), dtype=f1.dtype, device=dev) for t in lv]
+        au = [torch.empty((B, H1, W1, 1, t.shape[1]), dtype=torch.int32, device=dev) for t in lv]
+        av = [torch.empty((B, H1, W1, 1, t.shape[2]), dtype=torch.int32, device=dev) for t in lv]
+        _lib.check(lib.sepcorr_max_argmax_avg_forward_levels(f1.data_ptr(), _ptrs(lv), h2, w2, L, _ptrs(ou), _ptrs(ov), _ptrs(au),
+                                                             _ptrs(av), B, H1, W1, C, ws.data_ptr(), n, _stream()))
+    return [list(t) for t in zip(ou, ov, au, av)]
+
+
+def _check_level_tensors(name, ts, lv, f1, K, which):
+    B, H1, W1 = f1.shape[:3]
+    for n, (t, f2) in enumerate(zip(ts, lv)):
+        last = {"u": f2.shape[1], "v": f2.shape[2], "s": 2}[which]
+        _expect(f"{name}[{n}]", t, (B, H1, W1, K, last), f1.device)
+
+
+def compression_forward_from_logits_levels(img1_features_l0, img2_features_lvls, logits_u, logits_v, stats_u, stats_v):
+    """compression_forward_from_logits (statistics given) for every level in one call -> list of [comp_u, comp_v]."""
+    f1, lv = img1_features_l0, list(img2_features_lvls)
+    K = logits_u[0].shape[3]
+    lib, B, H1, W1, C, L, h2, w2, ws, n = _levels_setup(f1, lv, K)
+    dev = f1.device
+    _check_level_tensors("logits_u", logits_u, lv, f1, K, "v"); _check_level_tensors("logits_v", logits_v, lv, f1, K, "u")
+    _check_level_tensors("stats_u", stats_u, lv, f1, K, "s"); _check_level_tensors("stats_v", stats_v, lv, f1, K, "s")
+    with torch.cuda.device(dev):
+        cu = [torch.empty((B, H1, W1, K, t.shape[1]), dtype=f1.dtype, device=dev) for t in lv]
+        cv = [torch.empty((B, H1, W1, K, t.shape[2]), dtype=f1.dtype, device=dev) for t in lv]
+        _lib.check(lib.sepcorr_compression_forward_from_logits_levels(
+            f1.data_ptr(), _ptrs(lv), h2, w2, L, _ptrs(logits_u), _ptrs(logits_v), _ptrs(stats_u), _ptrs(stats_v),
+            _ptrs(cu), _ptrs(cv), B, H1, W1, C, K, ws.data_ptr(), n, _stream()))
+    return [list(t) for t in zip(cu, cv)]
+
+
+def compression_logit_gradients_levels(img1_features_l0, img2_features_lvls, logits_u, logits_v, stats_u, stats_v,
+                                       compression_output_u, compression_output_v, grad_compressed_output_u,
+                                       grad_compressed_output_v):
+    """The logit gradients of compression_backward_from_logits for every level in one call -> list of [dz_u, dz_v]."""
+    f1, lv = img1_features_l0, list(img2_features_lvls)
+    K = logits_u[0].shape[3]
+    lib, B, H1, W1, C, L, h2, w2, ws, n = _levels_setup(f1, lv, K)
+    _check_level_tensors("logits_u", logits_u, lv, f1, K, "v"); _check_level_tensors("logits_v", logits_v, lv, f1, K, "u")
+    _check_level_tensors("stats_u", stats_u, lv, f1, K, "s"); _check_level_tensors("stats_v", stats_v, lv, f1, K, "s")
+    _check_level_tensors("compression_output_u", compression_output_u, lv, f1, K, "u")
+    _check_level_tensors("compression_output_v", compression_output_v, lv, f1, K, "v")
+    _check_level_tensors("grad_compressed_output_u", grad_compressed_output_u, lv, f1, K, "u")
+    _check_level_tensors("grad_compressed_output_v", grad_compressed_output_v, lv, f1, K, "v")
+    with torch.cuda.device(f1.device):
+        dz_u = [torch.empty_like(t) for t in logits_u]
+        dz_v = [torch.empty_like(t) for t in logits_v]
+        _lib.check(lib.sepcorr_compression_backward_from_logits_levels(
+            f1.data_ptr(), _ptrs(lv), h2, w2, L, _ptrs(logits_u), _ptrs(logits_v), _ptrs(stats_u), _ptrs(stats_v),
+            _ptrs(compression_output_u), _ptrs(compression_output_v), _ptrs(grad_compressed_output_u),
+            _ptrs(grad_compressed_output_v), _ptrs(dz_u), _ptrs(dz_v), B, H1, W1, C, K, ws.data_ptr(), n, _stream()))
+    return [list(t) for t in zip(dz_u, dz_v)]
+
+
 def fused_backward(img1_features_l0, img2_features_lk, argmax_output_u, argmax_output_v, grad_MaxAvg_u, grad_MaxAvg_v,
                    attention_weights_u, attention_weights_v, grad_compressed_output_u, grad_compressed_output_v):
     """-> [grad_fmap1_l0, grad_fmap2_lk]: the sum of what max_argmax_avg_backward and compression_backward return

@@ -30,6 +30,10 @@ SIGNATURES = {
     "sepcorr_compression_forward_from_logits": (_I, [_P] * 8 + [_I] * 8 + [_P, _SZ, _P]),
     "sepcorr_compression_backward_from_logits_workspace_bytes": (_SZ, [_I] * 8),
     "sepcorr_compression_backward_from_logits": (_I, [_P] * 14 + [_I] * 7 + [_P, _SZ, _P]),
+    "sepcorr_forward_levels_workspace_bytes": (_SZ, [_P, _P] + [_I] * 6),
+    "sepcorr_max_argmax_avg_forward_levels": (_I, [_P] * 4 + [_I] + [_P] * 4 + [_I] * 4 + [_P, _SZ, _P]),
+    "sepcorr_compression_forward_from_logits_levels": (_I, [_P] * 4 + [_I] + [_P] * 6 + [_I] * 5 + [_P, _SZ, _P]),
+    "sepcorr_compression_backward_from_logits_levels": (_I, [_P] * 4 + [_I] + [_P] * 10 + [_I] * 5 + [_P, _SZ, _P]),
     "sepcorr_softmax_rows": (_I, [_P, _P, _I, _P, ctypes.c_long, _I, _P]),
     "sepcorr_fused_backward": (_I, [_P] * 12 + [_I] * 7 + [_P, _SZ, _P]),
     "sepcorr_attention_logits_forward": (_I, [_P] * 5 + [_I] * 5 + [_P]),

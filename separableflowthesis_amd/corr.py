@@ -10,9 +10,11 @@ trilinearly upsampled (align_corners=True) to the level-0 displacement length.
 import torch
 import torch.nn.functional as F
 
+from . import MemorySaver
 from .functions import (AssembleVolumeFunction, AttentionLogitsFunction, AttentionWeightsFunction,
                         ComputeMaxArgmaxAvgFunction, ComputeMaxAvgFunction, ComputeSelfCompressionFromLogitsFunction,
-                        ComputeSelfCompressionFunction, Lookup1DFunction, LookupFunction, SeparateLevelFunction)
+                        ComputeSelfCompressionFunction, Lookup1DFunction, LookupFunction, SeparateLevelFunction,
+                        SeparatePyramidFunction)
 
 
 def _is_reference_attention(m):
@@ -40,6 +42,9 @@ class AlternateCorrBlockSepflow:
         self.radius = radius
         self.fmap1_l0 = fmap1
         self._lookup_inputs = None
+        # how the fused path runs the pyramid: "all" (every level in the same launches; fastest measured), "first_alone"
+        # (level 0 in launches of its own, the levels above it together) or "level" (one autograd node per level)
+        self.pyramid_mode = "all"
         self.pyramid = [fmap2]
         for _ in range(self.num_levels - 1):
             fmap2 = F.avg_pool2d(fmap2, 2, stride=2)
@@ -54,6 +59,21 @@ class AlternateCorrBlockSepflow:
             attention_weights is None or all(_is_reference_attention(m) for m in attention_weights))
         parts_u, parts_v = [], []      # operator outputs in final channel order (fused path)
         sep_u_lvls, sep_v_lvls = [], []
+        # (the optional bf16-plane contraction exists in the single-level sweeps only: it keeps the per-level path)
+        if (fused and attention_weights is not None and self.max_avg_function is ComputeMaxArgmaxAvgFunction
+                and 1 < self.num_levels <= 4 and self.pyramid_mode != "level"
+                and MemorySaver.set_contraction(-1) == MemorySaver.CONTRACT_FP32):
+            # the whole pyramid as one autograd node; the levels above level 0 share launches
+            attention1, attention2 = attention_weights
+            levels = [p.permute(0, 2, 3, 1).contiguous() for p in self.pyramid]
+            res = SeparatePyramidFunction.apply(fmap1, attention1.weight.contiguous(), attention1.bias,
+                                                attention2.weight.contiguous(), attention2.bias,
+                                                self.pyramid_mode == "first_alone", *levels)
+            for i in range(self.num_levels):
+                maxavg_u, maxavg_v, adaptive_corr_u, adaptive_corr_v = res[4 * i: 4 * i + 4]
+                parts_u += [maxavg_v, adaptive_corr_v]
+                parts_v += [maxavg_u, adaptive_corr_u]
+            return AssembleVolumeFunction.apply(w2, *parts_u), AssembleVolumeFunction.apply(h2, *parts_v)
         for i in range(self.num_levels):
             fmap2 = self.pyramid[i].permute(0, 2, 3, 1).contiguous()
             if fused and attention_weights is not None and self.max_avg_function is ComputeMaxArgmaxAvgFunction:

@@ -272,6 +272,17 @@ __device__ __forceinline__ int xcd_contiguous(int bid, int n) {
 
 }  // namespace
 namespace sepcorr_impl {
+// What differs between the pyramid levels of fmap2 that one launch of a forward-type sweep can cover.
+struct FwdLevel {
+    const float *f2, *wv, *wu;
+    float *out_u, *out_v;
+    int *am_u, *am_v;
+    const float *st_wv, *st_wu, *z_ou, *st_ou, *dot_ou, *z_ov, *st_ov, *dot_ov;   // softmax inside (see FwdArgs)
+    int H2, W2;
+    int nvc;           // column chunks of 32 = waves side by side; the other waves of the workgroup form row groups
+    int steps, step0;  // steps of this level per tile, and of the levels before it
+    int stage;
+};
 struct FwdArgs {
     const float *f1, *f2;
     const char *f2_planes;   // bf16-plane variant: fmap2 split by split_planes_kernel
@@ -309,6 +320,12 @@ struct FwdArgs {
     int logits, dlog;
     const float *st_wv, *st_wu;
     const float *z_ou, *st_ou, *dot_ou, *z_ov, *st_ov, *dot_ov;
+    // Several levels in one launch (split sweeps with row groups only): the steps of a tile are those of lev[0], then
+    // of lev[1], ...; pieces are cut at level boundaries as well, and the image-1 tile is shared by all of them.
+    int nlev;          // 0 or 1: one level, described by the fields above
+    int tile_steps;    // steps of all levels of one tile
+    int H2max;         // largest H2: the staged out_u rows of every level fit [32][channels][H2max]
+    FwdLevel lev[4];
 };
 }  // namespace sepcorr_impl
 namespace {
@@ -336,49 +353,84 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     // and the steps ug, ug + NUG, ... (narrow fmap2 levels have few column chunks; row groups keep the
     // workgroup at 4 or 8 waves).  NUG == 1 for rows of 97 or more columns.
     constexpr bool RG = WM == 1;
-    const int nvc = RG ? a.nvc : nW, NUG = RG ? nW / nvc : 1;
-    const int vcw = RG ? wave % nvc : wave, ug = RG ? wave / nvc : 0;
+    constexpr bool ML = SK && WM == 1;   // may cover several pyramid levels
+    const bool multi = ML && a.nlev > 1;
     const int vpasses = (WM == 2) ? a.vpasses : 1;
     const int wg = a.xcd_order ? xcd_contiguous(blockIdx.x, gridDim.x) : (int)blockIdx.x;
-    const int N1 = a.N1, H2 = a.H2, W2 = a.W2, C = a.C;
+    const int N1 = a.N1, C = a.C;
     const int LS = BF ? BF_LS : a.CP + 4;
     float *f1s = smem;
     __bf16 *f1b = reinterpret_cast<__bf16 *>(smem);   // BF: [plane][TP][BF_LSB]
     float *part = smem + TP * LS;
     constexpr int NCHO = (is_weighted(MODE)) ? KC : 2;            // out_u channels of this launch
     float *ostage = part + 2 * UR * NPART * (blockDim.x >> 6) * 32;   // [32 p][NCHO][H2] when a.stage
-    int *ostage_am = reinterpret_cast<int *>(ostage + TP * NCHO * a.H2);   // [32 p][H2], MODE_ARGMAX
+    int *ostage_am = reinterpret_cast<int *>(ostage + TP * NCHO * a.H2max);   // [32 p][H2], MODE_ARGMAX
     // MODE_WEIGHTED with softmax inside: per (pixel, channel) row of the u-indexed tensor (max, 1 / sum) of the
     // logits that are the weights [32 p][KC][2], or (max, 1 / sum, dot) of the logits whose gradient is stored [..][3]
-    float *cst = ostage + (a.stage ? TP * NCHO * a.H2 : 0);
+    float *cst = ostage + (a.stage ? TP * NCHO * a.H2max : 0);
 
     // This workgroup's share of the steps of all tiles: [gs0, gs_end).  Without the split it is exactly one tile.
     // A share is cut into pieces at tile boundaries.  When it ends inside a tile, that last piece (which starts at
     // the tile's row 0) is done first and the others follow in order: every workgroup of the grid then starts at
     // row 0 and all of them move down the rows of fmap2 together, so that a row is fetched into an L2 once.
-    const int S = sk_total ? a.sk_steps : 1;
+    // (With several levels a unit is one level of one tile, a tile's steps being those of all its levels in turn.)
+    const int S = sk_total ? (multi ? a.tile_steps : a.sk_steps) : 1;
+    // the unit that holds step g: its first step, one past its last, its level
+    auto unit_of = [&](int g, int &ubeg, int &uend) {
+        const int t = g / S;
+        int lv = 0, s0 = 0, s1 = S;
+        if (multi) {
+            const int r = g - t * S;
+            for (lv = a.nlev - 1; lv > 0 && a.lev[lv].step0 > r; --lv) {}
+            s0 = a.lev[lv].step0;
+            s1 = s0 + a.lev[lv].steps;
+        }
+        ubeg = t * S + s0;
+        uend = t * S + s1;
+        return lv;
+    };
     const int gs0 = sk_total ? (int)(((long)wg * sk_total) / (int)gridDim.x) : wg;
     const int gs_end = sk_total ? (int)(((long)(wg + 1) * sk_total) / (int)gridDim.x) : wg + 1;
-    int head = gs_end % S;                              // steps of the piece at the end of the share
-    if (gs_end - head <= gs0) head = 0;                 // (the share lies inside one tile: a single piece)
+    int head = 0;                                       // steps of the piece at the end of the share
+    {
+        int ub, ue;
+        unit_of(gs_end - 1, ub, ue);
+        if (ue != gs_end && ub > gs0) head = gs_end - ub;   // (no head: the share ends with a unit, or lies inside one)
+    }
     const int body_end = gs_end - head;
     int cur = gs0;
     for (int seg_no = 0;; ++seg_no) {
-    int pb, pe;                                         // this piece: steps [pb, pe) of all tiles laid end to end
+    int pb, pe, ubeg, uend;                             // this piece: steps [pb, pe) of all tiles laid end to end
     if (seg_no == 0 && head) {
         pb = body_end; pe = gs_end;
     } else {
         if (cur >= body_end) break;
         pb = cur;
-        pe = min(body_end, (cur / S + 1) * S);
+    }
+    const int lvl = unit_of(pb, ubeg, uend);
+    if (!(seg_no == 0 && head)) {
+        pe = min(body_end, uend);
         cur = pe;
     }
     const int tile = pb / S;
-    const int sa = pb - tile * S;                       // first step of this piece within the tile
-    const int sb = pe - tile * S;                       // one past its last step
-    const bool whole = !SK || !sk_total || (sa == 0 && sb == S);
+    const int sa = pb - ubeg;                           // first step of this piece within its unit
+    const int sb = pe - ubeg;                           // one past its last step
+    const bool whole = !SK || !sk_total || (pb == ubeg && pe == uend);
     const int b = tile / a.tiles_per_batch;
     const int p0 = (tile % a.tiles_per_batch) * TP;
+    // this piece's level
+    FwdLevel L;
+    if (multi) {
+        L = a.lev[lvl];
+    } else {
+        L.f2 = a.f2; L.wv = a.wv; L.wu = a.wu; L.out_u = a.out_u; L.out_v = a.out_v; L.am_u = a.am_u; L.am_v = a.am_v;
+        L.st_wv = a.st_wv; L.st_wu = a.st_wu; L.z_ou = a.z_ou; L.st_ou = a.st_ou; L.dot_ou = a.dot_ou;
+        L.z_ov = a.z_ov; L.st_ov = a.st_ov; L.dot_ov = a.dot_ov;
+        L.H2 = a.H2; L.W2 = a.W2; L.nvc = a.nvc; L.stage = a.stage;
+    }
+    const int H2 = L.H2, W2 = L.W2;
+    const int nvc = RG ? L.nvc : nW, NUG = RG ? nW / nvc : 1;
+    const int vcw = RG ? wave % nvc : wave, ug = RG ? wave / nvc : 0;
     if (seg_no > 0) __syncthreads();   // the previous piece has finished with LDS
 
     if constexpr (is_weighted(MODE)) {
@@ -386,17 +438,17 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
             for (int idx = tid; idx < TP * KC; idx += blockDim.x) {
                 const int p = idx / KC, kk = idx - p * KC;
                 const size_t row = ((size_t)b * N1 + min(p0 + p, N1 - 1)) * a.KT + a.k0 + kk;
-                cst[2 * idx] = a.st_wu[2 * row];
-                cst[2 * idx + 1] = 1.f / a.st_wu[2 * row + 1];
+                cst[2 * idx] = L.st_wu[2 * row];
+                cst[2 * idx + 1] = 1.f / L.st_wu[2 * row + 1];
             }
         }
         if (soft_dlog) {
             for (int idx = tid; idx < TP * KC; idx += blockDim.x) {
                 const int p = idx / KC, kk = idx - p * KC;
                 const size_t row = ((size_t)b * N1 + min(p0 + p, N1 - 1)) * a.KT + a.k0 + kk;
-                cst[3 * idx] = a.st_ou[2 * row];
-                cst[3 * idx + 1] = 1.f / a.st_ou[2 * row + 1];
-                cst[3 * idx + 2] = a.dot_ou[row];
+                cst[3 * idx] = L.st_ou[2 * row];
+                cst[3 * idx + 1] = 1.f / L.st_ou[2 * row + 1];
+                cst[3 * idx + 2] = L.dot_ou[row];
             }
         }
     }
@@ -434,7 +486,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     const int vbase = (WM == 2) ? vp * 256 : 0;
     const int vrow = vbase + 32 * vcw + pl;   // the fmap2 column this lane feeds to the A operand
     const bool vrow_ok = vrow < W2;
-    const float *f2lane = a.f2 + ((size_t)b * H2 * W2 + (vrow_ok ? vrow : 0)) * C;
+    const float *f2lane = L.f2 + ((size_t)b * H2 * W2 + (vrow_ok ? vrow : 0)) * C;
     const size_t rowstride = (size_t)W2 * C;
 
     const bool ragged = vbase + 32 * vcw + 32 > W2;
@@ -454,13 +506,13 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
             for (int r = 0; r < 16; ++r) {
                 const int v = vbase + 32 * vcw + vmap(r, h);
                 rv[k][r] = 0.f;
-                wvr[k][r] = (pok && v < W2) ? a.wv[(bp * a.KT + a.k0 + k) * W2 + v] : 0.f;
+                wvr[k][r] = (pok && v < W2) ? L.wv[(bp * a.KT + a.k0 + k) * W2 + v] : 0.f;
             }
         if (soft_logits) {
 #pragma unroll
             for (int k = 0; k < KC; ++k) {
                 const size_t row = bp * a.KT + a.k0 + k;
-                const float m = a.st_wv[2 * row], il = 1.f / a.st_wv[2 * row + 1];
+                const float m = L.st_wv[2 * row], il = 1.f / L.st_wv[2 * row + 1];
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
                     wvr[k][r] = (pok && vbase + 32 * vcw + vmap(r, h) < W2) ? __expf(wvr[k][r] - m) * il : 0.f;
@@ -571,15 +623,15 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                     for (int w = g2 * nvc; w < (g2 + 1) * nvc; ++w) s += pb[((ru * NPART + k) * nW + w) * 32 + p];
                     // (LDS and global destinations are kept in separate branches: a pointer that may be either
                     // turns into FLAT accesses, whose counters force every later wait to zero)
-                    if (a.stage) {
+                    if (L.stage) {
                         float *dst = &ostage[(p * NCHO + k) * H2 + u];
                         if (vp > 0) s += *dst;   // earlier column passes, written by this same thread
                         *dst = s;
                     } else {
                         const size_t row = ((size_t)b * N1 + p0 + p) * a.KT + a.k0 + k;
-                        float *dst = &a.out_u[row * H2 + u];
+                        float *dst = &L.out_u[row * H2 + u];
                         if (vp > 0) s += *dst;
-                        if (soft_dlog && vp == vpasses - 1) s = dlogit3(a.z_ou[row * H2 + u], cst + 3 * (p * KC + k), s);
+                        if (soft_dlog && vp == vpasses - 1) s = dlogit3(L.z_ou[row * H2 + u], cst + 3 * (p * KC + k), s);
                         *dst = s;
                     }
                 }
@@ -599,7 +651,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                         s += pb[((ru * NPART + 2) * nW + w) * 32 + p];
                     }
                     const bool last = vp == vpasses - 1;   // the running sum is kept until the last pass
-                    if (a.stage) {
+                    if (L.stage) {
                         float *dm = &ostage[(p * 2 + 0) * H2 + u], *ds = &ostage[(p * 2 + 1) * H2 + u];
                         int *di = &ostage_am[p * H2 + u];
                         if (vp > 0) {   // merge with the earlier column passes (lower v: they win ties)
@@ -612,15 +664,15 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                         if constexpr (MODE == MODE_ARGMAX) *di = mi;
                     } else {
                         const size_t o = ((size_t)b * N1 + p0 + p);
-                        float *dm = &a.out_u[(o * 2 + 0) * H2 + u], *ds = &a.out_u[(o * 2 + 1) * H2 + u];
+                        float *dm = &L.out_u[(o * 2 + 0) * H2 + u], *ds = &L.out_u[(o * 2 + 1) * H2 + u];
                         if (vp > 0) {
                             const float pm = *dm;
                             s += *ds;
-                            if (!(m > pm)) { m = pm; if constexpr (MODE == MODE_ARGMAX) mi = a.am_u[o * H2 + u]; }
+                            if (!(m > pm)) { m = pm; if constexpr (MODE == MODE_ARGMAX) mi = L.am_u[o * H2 + u]; }
                         }
                         *dm = m;
                         *ds = last ? s / (float)W2 : s;
-                        if constexpr (MODE == MODE_ARGMAX) a.am_u[o * H2 + u] = mi;
+                        if constexpr (MODE == MODE_ARGMAX) L.am_u[o * H2 + u] = mi;
                     }
                 }
             }
@@ -636,7 +688,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
 #pragma unroll
                     for (int k = 0; k < KC; ++k)
                     {
-                        wur[r][k] = (pok && u < H2) ? a.wu[(bp * a.KT + a.k0 + k) * H2 + u] : 0.f;
+                        wur[r][k] = (pok && u < H2) ? L.wu[(bp * a.KT + a.k0 + k) * H2 + u] : 0.f;
                         if (soft_logits) wur[r][k] = __expf(wur[r][k] - cst[2 * (pl * KC + k)]) * cst[2 * (pl * KC + k) + 1];
                     }
                 }
@@ -681,7 +733,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                     for (int r = 0; r < UR; ++r) {
                         const int u = min(((sa + step) * NUG + ug) * UR + r, H2 - 1);
 #pragma unroll
-                        for (int k = 0; k < KC; ++k) wur[r][k] = a.wu[(bp * a.KT + a.k0 + k) * H2 + u];
+                        for (int k = 0; k < KC; ++k) wur[r][k] = L.wu[(bp * a.KT + a.k0 + k) * H2 + u];
                     }
                 }
             }
@@ -720,7 +772,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         // 0..31) and 32J+16+4tq+t (lanes 32..63); the f1 tile in LDS is read with the same mapping.
         const unsigned rowbytes = (unsigned)W2 * C * 4u;
         const unsigned nbytes = (unsigned)H2 * rowbytes;
-        const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(a.f2 + (size_t)b * H2 * W2 * C, nbytes);
+        const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(L.f2 + (size_t)b * H2 * W2 * C, nbytes);
         const unsigned lane_off = vrow_ok ? ((unsigned)vrow * C + 16u * h) * 4u : nbytes;
         const int NJB = (CMODE == 3) ? 8 : (C >> 5);
         constexpr bool BPIPE = !(is_weighted(MODE) && KC >= 3);   // needs 16 more registers
@@ -751,7 +803,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                     for (int r = 0; r < UR; ++r) {
                         const int u = min(((sa + step) * NUG + ug) * UR + r, H2 - 1);
 #pragma unroll
-                        for (int k = 0; k < KC; ++k) wur[r][k] = a.wu[(bp * a.KT + a.k0 + k) * H2 + u];
+                        for (int k = 0; k < KC; ++k) wur[r][k] = L.wu[(bp * a.KT + a.k0 + k) * H2 + u];
                     }
                 }
                 if (J == (NJB > 1 ? 1 : 0) && soft_logits) {   // (a block later: the loads above have landed by now)
@@ -875,7 +927,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     }
 
     // flush the staged out_u rows of this piece (all rows of a whole tile): per pixel and channel a run of floats
-    if (a.stage && vp == vpasses - 1) {
+    if (L.stage && vp == vpasses - 1) {
         __syncthreads();
         const int cht = (is_weighted(MODE)) ? a.KT : 2, ch0 = (is_weighted(MODE)) ? a.k0 : 0;
         const int u0 = whole ? 0 : sa * NUG * UR, nu = (whole ? H2 : min(H2, sb * NUG * UR)) - u0;
@@ -895,7 +947,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                 pk[t] = p * KC + ch;
                 zs[t] = 0.f;
                 if constexpr (is_weighted(MODE)) {
-                    if (soft_dlog && ok) zs[t] = a.z_ou[off[t]];
+                    if (soft_dlog && ok) zs[t] = L.z_ou[off[t]];
                 }
             }
 #pragma unroll
@@ -905,13 +957,13 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                 if constexpr (is_weighted(MODE)) {
                     if (soft_dlog) x = dlogit3(zs[t], cst + 3 * pk[t], x);
                 }
-                a.out_u[off[t]] = x;
+                L.out_u[off[t]] = x;
             }
         }
         if constexpr (MODE == MODE_ARGMAX) {
             for (int idx = tid; idx < TP * nu; idx += blockDim.x) {
                 const int p = idx / nu, u = u0 + idx - p * nu;
-                if (p0 + p < N1) a.am_u[((size_t)b * N1 + p0 + p) * H2 + u] = ostage_am[p * H2 + u];
+                if (p0 + p < N1) L.am_u[((size_t)b * N1 + p0 + p) * H2 + u] = ostage_am[p * H2 + u];
             }
         }
     }
@@ -990,22 +1042,22 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                             v4f x = {rv[k][4 * g4], rv[k][4 * g4 + 1], rv[k][4 * g4 + 2], rv[k][4 * g4 + 3]};
                             const size_t row = bp * a.KT + a.k0 + k;
                             if (soft_dlog) {
-                                const float r3[3] = {a.st_ov[2 * row], 1.f / a.st_ov[2 * row + 1], a.dot_ov[row]};
-                                const v4f z = *reinterpret_cast<const v4f *>(a.z_ov + row * W2 + v);
+                                const float r3[3] = {L.st_ov[2 * row], 1.f / L.st_ov[2 * row + 1], L.dot_ov[row]};
+                                const v4f z = *reinterpret_cast<const v4f *>(L.z_ov + row * W2 + v);
 #pragma unroll
                                 for (int e = 0; e < 4; ++e) x[e] = dlogit3(z[e], r3, x[e]);
                             }
-                            *reinterpret_cast<v4f *>(a.out_v + row * W2 + v) = x;
+                            *reinterpret_cast<v4f *>(L.out_v + row * W2 + v) = x;
                         }
                     } else {
                         const v4f xm = {vmax[4 * g4], vmax[4 * g4 + 1], vmax[4 * g4 + 2], vmax[4 * g4 + 3]};
                         const v4f xs = {vsum[4 * g4] / (float)H2, vsum[4 * g4 + 1] / (float)H2, vsum[4 * g4 + 2] / (float)H2,
                                         vsum[4 * g4 + 3] / (float)H2};
-                        *reinterpret_cast<v4f *>(a.out_v + (bp * 2 + 0) * W2 + v) = xm;
-                        *reinterpret_cast<v4f *>(a.out_v + (bp * 2 + 1) * W2 + v) = xs;
+                        *reinterpret_cast<v4f *>(L.out_v + (bp * 2 + 0) * W2 + v) = xm;
+                        *reinterpret_cast<v4f *>(L.out_v + (bp * 2 + 1) * W2 + v) = xs;
                         if constexpr (MODE == MODE_ARGMAX) {
                             const v4i xi = {vidx[4 * g4], vidx[4 * g4 + 1], vidx[4 * g4 + 2], vidx[4 * g4 + 3]};
-                            *reinterpret_cast<v4i *>(a.am_v + bp * W2 + v) = xi;
+                            *reinterpret_cast<v4i *>(L.am_v + bp * W2 + v) = xi;
                         }
                     }
                 }
@@ -1019,12 +1071,12 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
 #pragma unroll
                         for (int k = 0; k < KC; ++k) {
                             const size_t row = bp * a.KT + a.k0 + k;
-                            a.out_v[row * W2 + v] = soft_dlog ? dlogit(a.z_ov, a.st_ov, a.dot_ov, row, row * W2 + v, rv[k][r]) : rv[k][r];
+                            L.out_v[row * W2 + v] = soft_dlog ? dlogit(L.z_ov, L.st_ov, L.dot_ov, row, row * W2 + v, rv[k][r]) : rv[k][r];
                         }
                     } else {
-                        a.out_v[(bp * 2 + 0) * W2 + v] = vmax[r];
-                        a.out_v[(bp * 2 + 1) * W2 + v] = vsum[r] / (float)H2;
-                        if constexpr (MODE == MODE_ARGMAX) a.am_v[bp * W2 + v] = vidx[r];
+                        L.out_v[(bp * 2 + 0) * W2 + v] = vmax[r];
+                        L.out_v[(bp * 2 + 1) * W2 + v] = vsum[r] / (float)H2;
+                        if constexpr (MODE == MODE_ARGMAX) L.am_v[bp * W2 + v] = vidx[r];
                     }
                 }
             }
@@ -1037,7 +1089,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         // workgroups; a workgroup keeps the first piece of its share in its slot 0 and a later one (which can only be
         // its last: the tiles between are whole) in its slot 1.
         const int G = (int)gridDim.x;
-        const long t0 = (long)tile * S, t1 = t0 + S;
+        const long t0 = ubeg, t1 = uend;
         int wfirst = (int)((t0 * G) / sk_total);                       // the workgroup that holds step t0
         while (wfirst > 0 && ((long)wfirst * sk_total) / G > t0) --wfirst;
         while (((long)(wfirst + 1) * sk_total) / G <= t0) ++wfirst;
@@ -1047,7 +1099,8 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's words of the piece have arrived
         __syncthreads();
         int *flag = reinterpret_cast<int *>(smem);
-        if (tid == 0) *flag = __hip_atomic_fetch_add(a.sk_count + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (tid == 0)
+            *flag = __hip_atomic_fetch_add(a.sk_count + (multi ? tile * a.nlev + lvl : tile), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         const bool last = *flag == npieces - 1;
         __syncthreads();
@@ -1089,9 +1142,9 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
 #pragma unroll
                         for (int q = 0; q < NQ; ++q) {
                             const size_t row = o * a.KT + a.k0 + q;
-                            r3[q][0] = a.st_ov[2 * row]; r3[q][1] = a.st_ov[2 * row + 1]; r3[q][2] = a.dot_ov[row];
+                            r3[q][0] = L.st_ov[2 * row]; r3[q][1] = L.st_ov[2 * row + 1]; r3[q][2] = L.dot_ov[row];
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) z[q][e] = v + e < W2 ? a.z_ov[row * W2 + v + e] : 0.f;
+                            for (int e = 0; e < 4; ++e) z[q][e] = v + e < W2 ? L.z_ov[row * W2 + v + e] : 0.f;
                         }
 #pragma unroll
                         for (int q = 0; q < NQ; ++q) {
@@ -1106,11 +1159,11 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                     if (v + e >= W2) break;
                     if constexpr (is_weighted(MODE)) {
 #pragma unroll
-                        for (int q = 0; q < NQ; ++q) a.out_v[(o * a.KT + a.k0 + q) * W2 + v + e] = acc4[q][e];
+                        for (int q = 0; q < NQ; ++q) L.out_v[(o * a.KT + a.k0 + q) * W2 + v + e] = acc4[q][e];
                     } else {
-                        a.out_v[(o * 2 + 0) * W2 + v + e] = acc4[0][e];
-                        a.out_v[(o * 2 + 1) * W2 + v + e] = acc4[2][e] / (float)H2;
-                        if constexpr (MODE == MODE_ARGMAX) a.am_v[o * W2 + v + e] = __float_as_int(acc4[1][e]);
+                        L.out_v[(o * 2 + 0) * W2 + v + e] = acc4[0][e];
+                        L.out_v[(o * 2 + 1) * W2 + v + e] = acc4[2][e] / (float)H2;
+                        if constexpr (MODE == MODE_ARGMAX) L.am_v[o * W2 + v + e] = __float_as_int(acc4[1][e]);
                     }
                 }
             }
@@ -2455,9 +2508,77 @@ int launch_fwd(FwdArgs a, int B, hipStream_t s) {
 #undef SEPCORR_FWD
     return check_launch("forward kernel");
 }
+// Several pyramid levels in one launch.  a.lev[0..nlev) carry pointers and sizes (H2, W2); everything else as for
+// launch_fwd.  Returns SEPCORR_EINVAL without launching when the shapes do not fit this path (the caller then runs
+// the levels one by one): rows of at most 128 columns in 1, 2 or 4 chunks, C a multiple of 32, scratch given.
+template <int MODE, int KC, int UR>
+int launch_fwd_levels(FwdArgs a, int B, hipStream_t s) {
+    constexpr int NPART = is_weighted(MODE) ? KC : 3;
+    constexpr int NCHO = is_weighted(MODE) ? KC : 2;
+    constexpr int nW = 4;
+    if (a.nlev < 2 || a.nlev > 4 || a.ws == nullptr || a.C % 32 != 0) return SEPCORR_EINVAL;
+    int steps = 0, h2max = 0, w2max = 0;
+    for (int l = 0; l < a.nlev; ++l) {
+        FwdLevel &L = a.lev[l];
+        L.nvc = (L.W2 + 31) / 32;
+        if (L.nvc != 1 && L.nvc != 2 && L.nvc != 4) return SEPCORR_EINVAL;
+        if ((size_t)L.H2 * L.W2 * a.C * sizeof(float) > (1u << 30)) return SEPCORR_EINVAL;
+        L.steps = (L.H2 + UR * (nW / L.nvc) - 1) / (UR * (nW / L.nvc));
+        L.step0 = steps;
+        steps += L.steps;
+        if (L.H2 > h2max) h2max = L.H2;
+        if (L.W2 > w2max) w2max = L.W2;
+    }
+    a.tile_steps = steps;
+    a.H2max = h2max;
+    a.vpasses = 1;
+    size_t lds = ((size_t)TP * (a.CP + 4) + 2 * UR * NPART * nW * 32) * sizeof(float);
+    const size_t extra = (size_t)TP * (NCHO + (MODE == MODE_ARGMAX ? 1 : 0)) * h2max * sizeof(float);
+    a.stage = lds + extra <= 80 * 1024;
+    if (a.stage) lds += extra;
+    for (int l = 0; l < a.nlev; ++l) a.lev[l].stage = a.stage;
+    const size_t merge = (size_t)2 * NPART * 16 * 64 * sizeof(float);   // row groups merge through LDS from offset 0
+    if (lds < merge) lds = merge;
+    if (MODE == MODE_SOFT) lds += (size_t)TP * KC * 3 * sizeof(float);
+    const int tiles = B * a.tiles_per_batch;
+    const long T = (long)tiles * steps;
+    const long places = (long)kCUs * (lds <= 80 * 1024 ? 2 : 1);
+    const int G = (int)(T < places ? T : places);
+    const size_t count_bytes = ((size_t)tiles * a.nlev * sizeof(int) + 255) & ~(size_t)255;
+    const size_t slot_floats = (size_t)NPART * 1024 * ((w2max + 31) / 32);
+    if (T >= (1L << 30) || count_bytes + 2 * (size_t)G * slot_floats * sizeof(float) > a.ws_bytes) return SEPCORR_EINVAL;
+    a.sk_total = (int)T;
+    a.sk_steps = steps;
+    a.sk_count = static_cast<int *>(a.ws);
+    a.sk_state = reinterpret_cast<float *>(static_cast<char *>(a.ws) + count_bytes);
+    a.sk_slot = (int)slot_floats;
+    const int n = tiles * a.nlev;
+    hipLaunchKernelGGL(zero_ints_kernel, dim3((n + 255) / 256), dim3(256), 0, s, a.sk_count, n);
+    const dim3 grid(G), block(64 * nW);
+    ProfScope ps(is_weighted(MODE) ? "fwd_weighted_levels" : "fwd_maxavg_levels", s);
+    if (a.C == 256) {
+        auto k = fwd_kernel<MODE, KC, UR, 3, 1, false, true>;
+        if (int rc = set_lds(k, lds)) return rc;
+        hipLaunchKernelGGL(k, grid, block, lds, s, a);
+    } else {
+        auto k = fwd_kernel<MODE, KC, UR, 2, 1, false, true>;
+        if (int rc = set_lds(k, lds)) return rc;
+        hipLaunchKernelGGL(k, grid, block, lds, s, a);
+    }
+    return check_launch("forward kernel (several levels)");
+}
+// Upper bound of the scratch launch_fwd_levels asks for.
+inline size_t fwd_levels_bytes(int tiles, int nlev, int w2max, int K) {
+    const int nq = K > 3 ? (K < KCH ? K : KCH) : 3;
+    return (((size_t)tiles * nlev * sizeof(int) + 255) & ~(size_t)255) + 2 * (size_t)(2 * kCUs) * nq * 1024 * ((w2max + 31) / 32) * sizeof(float);
+}
 // instantiated in one part each; everywhere else only declared
-#define SEPCORR_FWD_DECL(MODE, KC, UR) extern template int launch_fwd<MODE, KC, UR>(FwdArgs, int, hipStream_t)
-#define SEPCORR_FWD_INST(MODE, KC, UR) template int launch_fwd<MODE, KC, UR>(FwdArgs, int, hipStream_t)
+#define SEPCORR_FWD_DECL(MODE, KC, UR)                                              \
+    extern template int launch_fwd<MODE, KC, UR>(FwdArgs, int, hipStream_t);       \
+    extern template int launch_fwd_levels<MODE, KC, UR>(FwdArgs, int, hipStream_t)
+#define SEPCORR_FWD_INST(MODE, KC, UR)                                              \
+    template int launch_fwd<MODE, KC, UR>(FwdArgs, int, hipStream_t);              \
+    template int launch_fwd_levels<MODE, KC, UR>(FwdArgs, int, hipStream_t)
 SEPCORR_FWD_DECL(MODE_MAXAVG, 1, 2);
 SEPCORR_FWD_DECL(MODE_ARGMAX, 1, 2);
 SEPCORR_FWD_DECL(MODE_WEIGHTED, 1, 2);
@@ -2560,6 +2681,7 @@ FwdArgs fwd_args(const Dims &d) {
     memset(&a, 0, sizeof(a));
     a.N1 = d.H1 * d.W1;
     a.H2 = d.H2;
+    a.H2max = d.H2;
     a.W2 = d.W2;
     a.C = d.C;
     a.CP = (d.C + 7) & ~7;
@@ -3344,6 +3466,190 @@ int sepcorr_compression_backward_from_logits(const float *f1, const float *f2, c
     }
     const int rj = fj.join();
     return rc ? rc : rj;
+}
+
+// ---- several pyramid levels per call ---------------------------------------------------------------------------
+
+namespace {
+struct LevelDims {
+    int nlev, h2max, w2max;
+};
+int check_levels(const int *h2, const int *w2, int nlev, int B, int H1, int W1, int C, int K, LevelDims *out) {
+    if (h2 == nullptr || w2 == nullptr) return fail(SEPCORR_EINVAL, "sepcorr: level size tables are NULL");
+    if (nlev < 1 || nlev > 4) return fail(SEPCORR_EINVAL, "sepcorr: %d levels given, 1..4 supported", nlev);
+    out->nlev = nlev; out->h2max = 0; out->w2max = 0;
+    for (int l = 0; l < nlev; ++l) {
+        const Dims d = {B, H1, W1, h2[l], w2[l], C};
+        if (int rc = check_dims(d, K)) return rc;
+        if (h2[l] > out->h2max) out->h2max = h2[l];
+        if (w2[l] > out->w2max) out->w2max = w2[l];
+    }
+    return SEPCORR_OK;
+}
+size_t levels_sweep_bytes(const int *h2, const int *w2, int nlev, int B, int H1, int W1, int K) {
+    int w2max = 0;
+    size_t single = 0;
+    for (int l = 0; l < nlev; ++l) {
+        if (w2[l] > w2max) w2max = w2[l];
+        const size_t n = fwd_split_bytes(B, H1, W1, h2[l], w2[l], K);
+        if (n > single) single = n;
+    }
+    const size_t multi = fwd_levels_bytes(B * ((H1 * W1 + TP - 1) / TP), nlev, w2max, K);
+    return ((multi > single ? multi : single) + 255) & ~(size_t)255;
+}
+}  // namespace
+
+size_t sepcorr_forward_levels_workspace_bytes(const int *h2, const int *w2, int nlev, int B, int H1, int W1, int C, int K) {
+    if (h2 == nullptr || w2 == nullptr || nlev < 1 || nlev > 4 || B < 1 || H1 < 1 || W1 < 1 || C < 1 || K < 1) return 0;
+    for (int l = 0; l < nlev; ++l)
+        if (h2[l] < 1 || w2[l] < 1) return 0;
+    // + the row dot products of the backward call (two per level)
+    return levels_sweep_bytes(h2, w2, nlev, B, H1, W1, K) + 2 * (size_t)nlev * ((((size_t)B * H1 * W1 * K * sizeof(float)) + 255) & ~(size_t)255);
+}
+
+int sepcorr_max_argmax_avg_forward_levels(const float *f1, const float *const *f2_levels, const int *h2, const int *w2, int nlev,
+                                          float *const *out_u, float *const *out_v, int32_t *const *argmax_u,
+                                          int32_t *const *argmax_v, int B, int H1, int W1, int C, void *workspace,
+                                          size_t workspace_bytes, void *stream) {
+    api_enter();
+    REQUIRE_PTR(f1); REQUIRE_PTR(f2_levels); REQUIRE_PTR(out_u); REQUIRE_PTR(out_v); REQUIRE_PTR(argmax_u); REQUIRE_PTR(argmax_v);
+    LevelDims ld;
+    if (int rc = check_levels(h2, w2, nlev, B, H1, W1, C, 2, &ld)) return rc;
+    for (int l = 0; l < nlev; ++l)
+        if (!f2_levels[l] || !out_u[l] || !out_v[l] || !argmax_u[l] || !argmax_v[l])
+            return fail(SEPCORR_EINVAL, "sepcorr: a pointer of level %d is NULL", l);
+    const size_t need = levels_sweep_bytes(h2, w2, nlev, B, H1, W1, 2);
+    if (workspace != nullptr && (workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255)))
+        return fail(SEPCORR_EWORKSPACE, "sepcorr: %zu bytes of 256-byte aligned workspace needed (or NULL), got %zu", need, workspace_bytes);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const Dims d0 = {B, H1, W1, h2[0], w2[0], C};
+    FwdArgs a = fwd_args(d0);
+    a.f1 = f1; a.ws = workspace; a.ws_bytes = workspace_bytes;
+    a.nlev = nlev;
+    for (int l = 0; l < nlev; ++l) {
+        FwdLevel &L = a.lev[l];
+        L.f2 = f2_levels[l]; L.out_u = out_u[l]; L.out_v = out_v[l]; L.am_u = argmax_u[l]; L.am_v = argmax_v[l];
+        L.H2 = h2[l]; L.W2 = w2[l];
+    }
+    const int rc = nlev > 1 ? launch_fwd_levels<MODE_ARGMAX, 1, 2>(a, B, s) : SEPCORR_EINVAL;
+    if (rc != SEPCORR_EINVAL) return rc;
+    for (int l = 0; l < nlev; ++l)   // shapes outside the one-launch path: level by level
+        if (int r2 = sepcorr_max_argmax_avg_forward(f1, f2_levels[l], out_u[l], out_v[l], argmax_u[l], argmax_v[l], B, H1, W1,
+                                                    h2[l], w2[l], C, workspace, workspace ? workspace_bytes : 0, stream))
+            return r2;
+    return SEPCORR_OK;
+}
+
+namespace {
+// The weighted sweep of every level: logits -> sums (dlog == 0) or upstream gradients -> logit gradients (dlog == 1).
+int soft_levels(const float *f1, const float *const *f2, const int *h2, const int *w2, int nlev, const FwdLevel *lev, int dlog,
+                int B, int H1, int W1, int C, int K, void *ws, size_t ws_bytes, hipStream_t s) {
+    const Dims d0 = {B, H1, W1, h2[0], w2[0], C};
+    FwdArgs a = fwd_args(d0);
+    a.f1 = f1; a.ws = ws; a.ws_bytes = ws_bytes; a.KT = K;
+    a.logits = !dlog; a.dlog = dlog;
+    a.nlev = nlev;
+    for (int l = 0; l < nlev; ++l) {
+        a.lev[l] = lev[l];
+        a.lev[l].f2 = f2[l]; a.lev[l].H2 = h2[l]; a.lev[l].W2 = w2[l];
+    }
+    bool one_launch = nlev > 1;
+    for (int k0 = 0; k0 < K && one_launch; k0 += KCH) {
+        a.k0 = k0;
+        const int kc = K - k0 < KCH ? K - k0 : KCH;
+        int rc;
+        switch (kc) {
+            case 1: rc = launch_fwd_levels<MODE_SOFT, 1, 2>(a, B, s); break;
+            case 2: rc = launch_fwd_levels<MODE_SOFT, 2, 2>(a, B, s); break;
+            case 3: rc = launch_fwd_levels<MODE_SOFT, 3, 1>(a, B, s); break;
+            default: rc = launch_fwd_levels<MODE_SOFT, 4, 1>(a, B, s); break;
+        }
+        if (rc == SEPCORR_EINVAL && k0 == 0) one_launch = false;   // shapes outside the one-launch path
+        else if (rc) return rc;
+    }
+    if (one_launch) return SEPCORR_OK;
+    for (int l = 0; l < nlev; ++l) {
+        const Dims d = {B, H1, W1, h2[l], w2[l], C};
+        FwdArgs soft;
+        memset(&soft, 0, sizeof(soft));
+        soft.logits = !dlog; soft.dlog = dlog;
+        soft.st_wv = lev[l].st_wv; soft.st_wu = lev[l].st_wu;
+        soft.z_ou = lev[l].z_ou; soft.st_ou = lev[l].st_ou; soft.dot_ou = lev[l].dot_ou;
+        soft.z_ov = lev[l].z_ov; soft.st_ov = lev[l].st_ov; soft.dot_ov = lev[l].dot_ov;
+        const size_t n = fwd_split_bytes(B, H1, W1, h2[l], w2[l], K);
+        if (int rc = weighted_forward(d, f1, f2[l], lev[l].wv, lev[l].wu, lev[l].out_u, lev[l].out_v, K, n && ws ? ws : nullptr, n, s, &soft))
+            return rc;
+    }
+    return SEPCORR_OK;
+}
+}  // namespace
+
+int sepcorr_compression_forward_from_logits_levels(const float *f1, const float *const *f2_levels, const int *h2, const int *w2,
+                                                   int nlev, const float *const *logits_u, const float *const *logits_v,
+                                                   const float *const *stats_u, const float *const *stats_v,
+                                                   float *const *comp_u, float *const *comp_v, int B, int H1, int W1, int C,
+                                                   int K, void *workspace, size_t workspace_bytes, void *stream) {
+    api_enter();
+    REQUIRE_PTR(f1); REQUIRE_PTR(f2_levels); REQUIRE_PTR(logits_u); REQUIRE_PTR(logits_v); REQUIRE_PTR(stats_u); REQUIRE_PTR(stats_v);
+    REQUIRE_PTR(comp_u); REQUIRE_PTR(comp_v);
+    LevelDims ld;
+    if (int rc = check_levels(h2, w2, nlev, B, H1, W1, C, K, &ld)) return rc;
+    const size_t need = levels_sweep_bytes(h2, w2, nlev, B, H1, W1, K);
+    if (workspace != nullptr && (workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255)))
+        return fail(SEPCORR_EWORKSPACE, "sepcorr: %zu bytes of 256-byte aligned workspace needed (or NULL), got %zu", need, workspace_bytes);
+    FwdLevel lev[4];
+    memset(lev, 0, sizeof(lev));
+    for (int l = 0; l < nlev; ++l) {
+        if (!f2_levels[l] || !logits_u[l] || !logits_v[l] || !stats_u[l] || !stats_v[l] || !comp_u[l] || !comp_v[l])
+            return fail(SEPCORR_EINVAL, "sepcorr: a pointer of level %d is NULL", l);
+        lev[l].wv = logits_u[l]; lev[l].wu = logits_v[l]; lev[l].st_wv = stats_u[l]; lev[l].st_wu = stats_v[l];
+        lev[l].out_u = comp_u[l]; lev[l].out_v = comp_v[l];
+    }
+    return soft_levels(f1, f2_levels, h2, w2, nlev, lev, 0, B, H1, W1, C, K, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+int sepcorr_compression_backward_from_logits_levels(const float *f1, const float *const *f2_levels, const int *h2, const int *w2,
+                                                    int nlev, const float *const *logits_u, const float *const *logits_v,
+                                                    const float *const *stats_u, const float *const *stats_v,
+                                                    const float *const *comp_u, const float *const *comp_v,
+                                                    const float *const *g_cu, const float *const *g_cv,
+                                                    float *const *d_logits_u, float *const *d_logits_v, int B, int H1, int W1,
+                                                    int C, int K, void *workspace, size_t workspace_bytes, void *stream) {
+    api_enter();
+    REQUIRE_PTR(f1); REQUIRE_PTR(f2_levels); REQUIRE_PTR(logits_u); REQUIRE_PTR(logits_v); REQUIRE_PTR(stats_u); REQUIRE_PTR(stats_v);
+    REQUIRE_PTR(comp_u); REQUIRE_PTR(comp_v); REQUIRE_PTR(g_cu); REQUIRE_PTR(g_cv); REQUIRE_PTR(d_logits_u); REQUIRE_PTR(d_logits_v);
+    LevelDims ld;
+    if (int rc = check_levels(h2, w2, nlev, B, H1, W1, C, K, &ld)) return rc;
+    const size_t need = sepcorr_forward_levels_workspace_bytes(h2, w2, nlev, B, H1, W1, C, K);
+    if (workspace == nullptr || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255))
+        return fail(SEPCORR_EWORKSPACE, "sepcorr: %zu bytes of 256-byte aligned workspace needed, got %zu", need,
+                    workspace ? workspace_bytes : (size_t)0);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t sweep = levels_sweep_bytes(h2, w2, nlev, B, H1, W1, K);
+    const size_t rows = (size_t)B * H1 * W1 * K;
+    const size_t dot_bytes = (rows * sizeof(float) + 255) & ~(size_t)255;
+    char *base = static_cast<char *>(workspace) + sweep;
+    FwdLevel lev[4];
+    memset(lev, 0, sizeof(lev));
+    {
+        ProfScope ps("row_dots", s);
+        const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+        for (int l = 0; l < nlev; ++l) {
+            if (!f2_levels[l] || !logits_u[l] || !logits_v[l] || !stats_u[l] || !stats_v[l] || !comp_u[l] || !comp_v[l] ||
+                !g_cu[l] || !g_cv[l] || !d_logits_u[l] || !d_logits_v[l])
+                return fail(SEPCORR_EINVAL, "sepcorr: a pointer of level %d is NULL", l);
+            float *dot_u = reinterpret_cast<float *>(base + (2 * l) * dot_bytes);       // sum_u g_cu comp_u
+            float *dot_v = reinterpret_cast<float *>(base + (2 * l + 1) * dot_bytes);   // sum_v g_cv comp_v
+            hipLaunchKernelGGL(row_dot_kernel, grid, block, 0, s, g_cu[l], comp_u[l], dot_u, (long)rows, h2[l]);
+            hipLaunchKernelGGL(row_dot_kernel, grid, block, 0, s, g_cv[l], comp_v[l], dot_v, (long)rows, w2[l]);
+            lev[l].wv = g_cv[l]; lev[l].wu = g_cu[l];
+            lev[l].out_u = d_logits_v[l]; lev[l].out_v = d_logits_u[l];
+            lev[l].z_ou = logits_v[l]; lev[l].st_ou = stats_v[l]; lev[l].dot_ou = dot_v;
+            lev[l].z_ov = logits_u[l]; lev[l].st_ov = stats_u[l]; lev[l].dot_ov = dot_u;
+        }
+        if (int rc = check_launch("row dot products")) return rc;
+    }
+    return soft_levels(f1, f2_levels, h2, w2, nlev, lev, 1, B, H1, W1, C, K, workspace, sweep, s);
 }
 
 int sepcorr_fused_backward(const float *f1, const float *f2, const int32_t *argmax_u, const int32_t *argmax_v,

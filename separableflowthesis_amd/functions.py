@@ -201,6 +201,77 @@ class SeparateLevelFunction(Function):
         return d1, d2, d_w1, d_b1, d_w2, d_b2
 
 
+class SeparatePyramidFunction(Function):
+    """All pyramid levels of the caller's loop (core/corr.py:416-457) as one autograd node; per level the same results
+    as SeparateLevelFunction.  The forward-type sweeps of several levels share one launch where the shapes allow
+    (MemorySaver.*_levels): the small levels then fill the chip together instead of one after the other.
+
+    apply(f1, weight1, bias1, weight2, bias2, first_alone, *f2_levels)
+      -> (max_avg_u_0, max_avg_v_0, comp_u_0, comp_v_0, max_avg_u_1, ...), operator layouts.
+    first_alone: level 0 keeps launches of its own (the kernels without row groups, which wide rows run fastest in)
+    and only the levels above it share launches.  Not a class of the reference.
+    """
+
+    @staticmethod
+    def forward(ctx, f1, weight1, bias1, weight2, bias2, first_alone, *f2_levels):
+        lv = list(f2_levels)
+        _contig(f1, weight1, weight2, *lv)
+        n = len(lv)
+        split = 1 if (first_alone and n > 1) else 0
+        with torch.cuda.device_of(f1):
+            ma = [MemorySaver.max_argmax_avg_forward(f1, lv[0])] if split else []
+            ma += MemorySaver.max_argmax_avg_forward_levels(f1, lv[split:])
+            out_u, out_v, am_u, am_v = (list(t) for t in zip(*ma))
+            zs_u = [MemorySaver.attention_logits_forward(out_v[l], weight1, bias1) for l in range(n)]
+            zs_v = [MemorySaver.attention_logits_forward(out_u[l], weight2, bias2) for l in range(n)]
+            z_u, st_u = (list(t) for t in zip(*zs_u))
+            z_v, st_v = (list(t) for t in zip(*zs_v))
+            comp = [MemorySaver.compression_forward_from_logits(f1, lv[0], z_u[0], z_v[0], st_u[0], st_v[0])[:2]] if split else []
+            comp += MemorySaver.compression_forward_from_logits_levels(f1, lv[split:], z_u[split:], z_v[split:],
+                                                                       st_u[split:], st_v[split:])
+            cu, cv = (list(t) for t in zip(*comp))
+        ctx.save_for_backward(f1, weight1, weight2, *lv, *am_u, *am_v, *out_u, *out_v, *z_u, *z_v, *st_u, *st_v, *cu, *cv)
+        ctx.n, ctx.split = n, split
+        ctx.has_bias = (bias1 is not None, bias2 is not None)
+        out = []
+        for l in range(n):
+            out += [out_u[l], out_v[l], cu[l], cv[l]]
+        return tuple(out)
+
+    @staticmethod
+    def backward(ctx, *grads):
+        n, split = ctx.n, ctx.split
+        saved = ctx.saved_tensors
+        f1, weight1, weight2 = saved[:3]
+        groups = [list(saved[3 + i * n: 3 + (i + 1) * n]) for i in range(11)]
+        lv, am_u, am_v, out_u, out_v, z_u, z_v, st_u, st_v, cu, cv = groups
+        g_u = [grads[4 * l].contiguous() for l in range(n)]
+        g_v = [grads[4 * l + 1].contiguous() for l in range(n)]
+        g_cu = [grads[4 * l + 2].contiguous() for l in range(n)]
+        g_cv = [grads[4 * l + 3].contiguous() for l in range(n)]
+        with torch.cuda.device_of(f1):
+            dz = []
+            if split:
+                dz.append(MemorySaver.compression_backward_from_logits(f1, lv[0], z_u[0], z_v[0], st_u[0], st_v[0], cu[0], cv[0],
+                                                                       g_cu[0], g_cv[0], need_features=False)[2:])
+            dz += MemorySaver.compression_logit_gradients_levels(f1, lv[split:], z_u[split:], z_v[split:], st_u[split:],
+                                                                 st_v[split:], cu[split:], cv[split:], g_cu[split:], g_cv[split:])
+            d_f1 = d_w1 = d_b1 = d_w2 = d_b2 = None
+            d_f2 = []
+            acc = lambda total, x: x if total is None or x is None else total + x
+            for l in range(n):
+                d_out_v, w1g, b1g = MemorySaver.attention_logits_backward(out_v[l], weight1, dz[l][0], need_bias=ctx.has_bias[0])
+                d_out_u, w2g, b2g = MemorySaver.attention_logits_backward(out_u[l], weight2, dz[l][1], need_bias=ctx.has_bias[1])
+                d_out_u += g_u[l]
+                d_out_v += g_v[l]
+                a_u = MemorySaver.softmax_from_stats(z_u[l], st_u[l])
+                a_v = MemorySaver.softmax_from_stats(z_v[l], st_v[l])
+                d1, d2 = MemorySaver.fused_backward(f1, lv[l], am_u[l], am_v[l], d_out_u, d_out_v, a_u, a_v, g_cu[l], g_cv[l])
+                d_f1, d_w1, d_b1, d_w2, d_b2 = acc(d_f1, d1), acc(d_w1, w1g), acc(d_b1, b1g), acc(d_w2, w2g), acc(d_b2, b2g)
+                d_f2.append(d2)
+        return (d_f1, d_w1, d_b1, d_w2, d_b2, None, *d_f2)
+
+
 class AssembleVolumeFunction(Function):
     """Operator outputs of all levels -> one module-level volume (B, channels, L0, H1, W1).
 
