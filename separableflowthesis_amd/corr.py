@@ -60,7 +60,10 @@ class AlternateCorrBlockSepflow:
         parts_u, parts_v = [], []      # operator outputs in final channel order (fused path)
         sep_u_lvls, sep_v_lvls = [], []
         # (the optional bf16-plane contraction exists in the single-level sweeps only: it keeps the per-level path)
-        if (fused and attention_weights is not None and self.max_avg_function is ComputeMaxArgmaxAvgFunction
+        # (without support for the backward pass the same node serves as long as no graph is recorded: the argmax it
+        # also computes is simply dropped; with a graph the per-level path keeps the reference's NotImplementedError)
+        if (fused and attention_weights is not None
+                and (self.max_avg_function is ComputeMaxArgmaxAvgFunction or not torch.is_grad_enabled())
                 and 1 < self.num_levels <= 4 and self.pyramid_mode != "level"
                 and MemorySaver.set_contraction(-1) == MemorySaver.CONTRACT_FP32):
             # the whole pyramid as one autograd node; the levels above level 0 share launches

@@ -2748,8 +2748,11 @@ Df2Plan df2_plan(const Dims &d, bool both) {
         double best = -1.0;
         pl.nsplit = 1;
         for (int ns = 1; ns <= 16 && ns <= tiles; ++ns) {
+            // share of the chip kept busy x share of a workgroup's time spent sweeping (start-up, the partial tile it
+            // leaves and its later addition cost about as much as two pixel tiles of the sweep)
             const long wgs = base * ns;
-            const double eff = (double)wgs / (double)(((wgs + 255) / 256) * 256) - 0.004 * ns;
+            const double per = (double)tiles / ns;
+            const double eff = (double)wgs / (double)(((wgs + 255) / 256) * 256) * per / (per + 2.0);
             if (eff > best) { best = eff; pl.nsplit = ns; }
         }
     } else {
