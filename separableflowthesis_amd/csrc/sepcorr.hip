@@ -163,6 +163,14 @@ __device__ __forceinline__ v4f load_shared4(__amdgpu_buffer_rsrc_t r, unsigned b
     return __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, CPOL_SC0_SC1));
 }
 
+// The values the two halves of a wave (lanes 0-31, lanes 32-63) hold in x, handed to every lane: lo = the value of
+// lane (l & 31), hi = the value of lane (l | 32).  One vector instruction, no trip through LDS.
+__device__ __forceinline__ void wave_halves(float x, float &lo, float &hi) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    lo = __uint_as_float(r[0]);
+    hi = __uint_as_float(r[1]);
+}
+
 __device__ __forceinline__ v16f mfma(float a, float b, v16f c) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
 }
@@ -308,6 +316,9 @@ struct FwdArgs {
     int sk_steps;      // steps per tile
     float *sk_state;   // [2 * gridDim.x] slots of sk_slot floats: first and last piece of every workgroup
     int *sk_count;     // [tiles] pieces finished, zero at launch
+#ifdef SEPCORR_TIMELINE
+    long long *dbg;
+#endif
     int sk_slot;       // floats per slot
     void *ws;          // host side only: scratch for the split (NULL: whole tiles)
     size_t ws_bytes;
@@ -335,6 +346,119 @@ namespace {
 // WM: 0 = one pass, one row group (both compile-time constants: the lean common case),
 //     1 = row groups enabled (narrow rows), 2 = column passes enabled (rows wider than 256).
 // BF: the experimental bf16-plane contraction (C == 256, one pass, one row group, max/avg modes)
+// The kernel's argument block, read where the call stands: nothing loaded through the returned pointer can be moved
+// ahead of this point, so values needed late in a kernel are not kept in scalar registers from its start.
+typedef const __attribute__((address_space(4))) FwdArgs *KArgs;
+__device__ __forceinline__ KArgs kernargs_now() {
+    KArgs p = (KArgs)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(p));
+    return p;
+}
+
+// The last piece of a tile to finish adds up the column state of all its pieces in row order (equal maxima keep the
+// lower row) and writes the finished out_v columns.  A function of its own: its registers (the pieces of a batch are
+// fetched together) are then allotted apart from those of the sweep.  Arguments are the same in every lane.
+template <int MODE, int KC>
+__device__ __attribute__((noinline)) void merge_pieces(KArgs ka_in, int lvl_in, int b_in, int p0_in, int wfirst_in, int wlast_in, int t0_in,
+                                                       int tid) {
+    const uint64_t kp64 = reinterpret_cast<uint64_t>(ka_in);
+    const KArgs ka = reinterpret_cast<KArgs>(((uint64_t)(unsigned)__builtin_amdgcn_readfirstlane((int)(kp64 >> 32)) << 32) |
+                                             (unsigned)__builtin_amdgcn_readfirstlane((int)kp64));
+    const int lvl = __builtin_amdgcn_readfirstlane(lvl_in), b = __builtin_amdgcn_readfirstlane(b_in);
+    const int p0 = __builtin_amdgcn_readfirstlane(p0_in), wfirst = __builtin_amdgcn_readfirstlane(wfirst_in);
+    const int wlast = __builtin_amdgcn_readfirstlane(wlast_in);
+    const long t0 = __builtin_amdgcn_readfirstlane(t0_in);
+    const int G = (int)gridDim.x, sk_total = ka->sk_total, N1 = ka->N1;
+    const int H2 = ka->lev[lvl].H2, W2 = ka->lev[lvl].W2;
+    const bool soft_dlog = MODE == MODE_SOFT && ka->dlog;
+    (void)soft_dlog;
+    // Add up the pieces in row order (equal maxima keep the lower row) and write the finished columns.
+    // An item = the 4 consecutive columns a lane holds in one register group of one column chunk.
+    constexpr int NQ = (is_weighted(MODE)) ? KC : 3;
+    const __amdgpu_buffer_rsrc_t rs_sk = make_rsrc(ka->sk_state, 2u * gridDim.x * (unsigned)ka->sk_slot * 4u);
+    const int nchunks = (W2 + 31) >> 5;
+    for (int it = tid; it < nchunks * 256; it += blockDim.x) {
+        const int ln = it & 63, g4 = (it >> 6) & 3, chunk = it >> 8;
+        const int p = ln & 31, v = 32 * chunk + vmap(4 * g4, ln >> 5);
+        v4f acc4[NQ];
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) acc4[q] = v4f{0.f, 0.f, 0.f, 0.f};
+        if constexpr (!is_weighted(MODE)) acc4[0] = v4f{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+        constexpr int PB = 4;   // pieces fetched together (a tile rarely has more)
+        for (int w0 = wfirst; w0 <= wlast; w0 += PB) {
+            v4f x[PB][NQ];
+#pragma unroll
+            for (int j = 0; j < PB; ++j) {
+                const int w = w0 + j;
+                const bool first_piece = ((long)w * sk_total) / G >= t0;   // w's share starts inside this tile
+                const unsigned base = ((unsigned)(2 * w + (first_piece ? 0 : 1)) * (unsigned)ka->sk_slot +
+                                       (unsigned)chunk * (NQ * 1024u) + 4u * ln) * 4u;
+                if (w <= wlast) {
+#pragma unroll
+                    for (int q = 0; q < NQ; ++q) x[j][q] = load_shared4(rs_sk, base + (unsigned)(q * 4 + g4) * 1024u);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < PB; ++j) {
+                if (w0 + j > wlast) break;
+                if constexpr (is_weighted(MODE)) {
+#pragma unroll
+                    for (int q = 0; q < NQ; ++q) acc4[q] += x[j][q];
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (x[j][0][e] > acc4[0][e]) { acc4[0][e] = x[j][0][e]; acc4[1][e] = x[j][1][e]; }
+                    acc4[2] += x[j][2];
+                }
+            }
+        }
+        if (p0 + p >= N1) continue;
+        const size_t o = (size_t)b * N1 + p0 + p;
+        if constexpr (is_weighted(MODE)) {
+            if (soft_dlog) {   // sums of softmax-output gradients -> gradients of the logits
+                float r3[NQ][3], z[NQ][4];
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) {
+                    const size_t row = o * ka->KT + ka->k0 + q;
+                    r3[q][0] = ka->lev[lvl].st_ov[2 * row]; r3[q][1] = ka->lev[lvl].st_ov[2 * row + 1]; r3[q][2] = ka->lev[lvl].dot_ov[row];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) z[q][e] = v + e < W2 ? ka->lev[lvl].z_ov[row * W2 + v + e] : 0.f;
+                }
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) {
+                    r3[q][1] = 1.f / r3[q][1];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc4[q][e] = dlogit3(z[q][e], r3[q], acc4[q][e]);
+                }
+            }
+        }
+        if ((W2 & 3) == 0 && (reinterpret_cast<uintptr_t>(ka->lev[lvl].out_v) & 15) == 0 && MODE != MODE_ARGMAX) {
+            if (v < W2) {
+                if constexpr (is_weighted(MODE)) {
+#pragma unroll
+                    for (int q = 0; q < NQ; ++q) *reinterpret_cast<v4f *>(ka->lev[lvl].out_v + (o * ka->KT + ka->k0 + q) * W2 + v) = acc4[q];
+                } else {
+                    *reinterpret_cast<v4f *>(ka->lev[lvl].out_v + (o * 2 + 0) * W2 + v) = acc4[0];
+                    *reinterpret_cast<v4f *>(ka->lev[lvl].out_v + (o * 2 + 1) * W2 + v) = acc4[2] / (float)H2;
+                }
+            }
+            continue;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (v + e >= W2) break;
+            if constexpr (is_weighted(MODE)) {
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) ka->lev[lvl].out_v[(o * ka->KT + ka->k0 + q) * W2 + v + e] = acc4[q][e];
+            } else {
+                ka->lev[lvl].out_v[(o * 2 + 0) * W2 + v + e] = acc4[0][e];
+                ka->lev[lvl].out_v[(o * 2 + 1) * W2 + v + e] = acc4[2][e] / (float)H2;
+                if constexpr (MODE == MODE_ARGMAX) ka->lev[lvl].am_v[o * W2 + v + e] = __float_as_int(acc4[1][e]);
+            }
+        }
+    }
+}
+
 // SK: the sweep may be dealt out in pieces of tiles (FwdArgs::sk_total); without it the loop over pieces below runs
 // exactly once with compile-time bounds and costs nothing
 template <int MODE, int KC, int UR, int CMODE, int WM, bool BF = false, bool SK = false>
@@ -347,7 +471,6 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     constexpr int GJ = 2;  // 8-channel slices per prefetch group
     constexpr int NPART = (is_weighted(MODE)) ? KC : 3;
     extern __shared__ float smem[];
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, pl = lane & 31, h = lane >> 5;
     const int nW = blockDim.x >> 6;
     // Waves form a grid: nvc column chunks x NUG row groups.  Wave (vcw, ug) owns columns [32 vcw, 32 vcw + 32)
     // and the steps ug, ug + NUG, ... (narrow fmap2 levels have few column chunks; row groups keep the
@@ -407,57 +530,85 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         if (cur >= body_end) break;
         pb = cur;
     }
-    const int lvl = unit_of(pb, ubeg, uend);
+    const int lvl_dyn = unit_of(pb, ubeg, uend);
+    const int lvl = ML ? lvl_dyn : 0;
     if (!(seg_no == 0 && head)) {
         pe = min(body_end, uend);
         cur = pe;
     }
+    // Lane indices are derived from the thread id piece by piece (and once more behind the sweep): values that lived
+    // from the start of the kernel to its end would be the first to be moved out of registers, and the sweep uses them.
+    int tid = threadIdx.x;
+    if constexpr (SK) asm volatile("" : "+v"(tid));
+    const int wave = tid >> 6, lane = tid & 63, pl = lane & 31, h = lane >> 5;
     const int tile = pb / S;
     const int sa = pb - ubeg;                           // first step of this piece within its unit
     const int sb = pe - ubeg;                           // one past its last step
     const bool whole = !SK || !sk_total || (pb == ubeg && pe == uend);
     const int b = tile / a.tiles_per_batch;
     const int p0 = (tile % a.tiles_per_batch) * TP;
-    // this piece's level
-    FwdLevel L;
-    if (multi) {
-        L = a.lev[lvl];
-    } else {
-        L.f2 = a.f2; L.wv = a.wv; L.wu = a.wu; L.out_u = a.out_u; L.out_v = a.out_v; L.am_u = a.am_u; L.am_v = a.am_v;
-        L.st_wv = a.st_wv; L.st_wu = a.st_wu; L.z_ou = a.z_ou; L.st_ou = a.st_ou; L.dot_ou = a.dot_ou;
-        L.z_ov = a.z_ov; L.st_ov = a.st_ov; L.dot_ov = a.dot_ov;
-        L.H2 = a.H2; L.W2 = a.W2; L.nvc = a.nvc; L.stage = a.stage;
-    }
-    const int H2 = L.H2, W2 = L.W2;
-    const int nvc = RG ? L.nvc : nW, NUG = RG ? nW / nvc : 1;
+    // This piece's level: lev[lvl] (a launch of one level describes it in lev[0]).  Pointers that only the code
+    // before or only the code behind the sweep uses are read from the kernel arguments there and then
+    // (kernargs_now), so that they do not hold scalar registers during the sweep.
+    const int H2 = a.lev[lvl].H2, W2 = a.lev[lvl].W2;
+    const bool Lstage = a.lev[lvl].stage;
+    const float *Lf2 = a.lev[lvl].f2, *Lwu = a.lev[lvl].wu;
+    const int nvc = RG ? a.lev[lvl].nvc : nW, NUG = RG ? nW / nvc : 1;
     const int vcw = RG ? wave % nvc : wave, ug = RG ? wave / nvc : 0;
     if (seg_no > 0) __syncthreads();   // the previous piece has finished with LDS
+#ifdef SEPCORR_TIMELINE
+#define TL(i) if (a.dbg && tid == 0) a.dbg[((size_t)wg * 4 + min(seg_no, 3)) * 12 + (i)] = wall_clock64();
+    if (a.dbg && tid == 0) { long long *d = a.dbg + ((size_t)wg * 4 + min(seg_no, 3)) * 12; d[8] = pe - pb; d[9] = whole; d[11] = tile; d[10] = 0; }
+#else
+#define TL(i)
+#endif
+    TL(0)
+    const KArgs kp = kernargs_now();
 
     if constexpr (is_weighted(MODE)) {
         if (soft_logits) {   // (max, 1 / sum) of the rows of u-indexed logits of this tile's pixels
             for (int idx = tid; idx < TP * KC; idx += blockDim.x) {
                 const int p = idx / KC, kk = idx - p * KC;
                 const size_t row = ((size_t)b * N1 + min(p0 + p, N1 - 1)) * a.KT + a.k0 + kk;
-                cst[2 * idx] = L.st_wu[2 * row];
-                cst[2 * idx + 1] = 1.f / L.st_wu[2 * row + 1];
+                cst[2 * idx] = kp->lev[lvl].st_wu[2 * row];
+                cst[2 * idx + 1] = 1.f / kp->lev[lvl].st_wu[2 * row + 1];
             }
         }
         if (soft_dlog) {
             for (int idx = tid; idx < TP * KC; idx += blockDim.x) {
                 const int p = idx / KC, kk = idx - p * KC;
                 const size_t row = ((size_t)b * N1 + min(p0 + p, N1 - 1)) * a.KT + a.k0 + kk;
-                cst[3 * idx] = L.st_ou[2 * row];
-                cst[3 * idx + 1] = 1.f / L.st_ou[2 * row + 1];
-                cst[3 * idx + 2] = L.dot_ou[row];
+                cst[3 * idx] = kp->lev[lvl].st_ou[2 * row];
+                cst[3 * idx + 1] = 1.f / kp->lev[lvl].st_ou[2 * row + 1];
+                cst[3 * idx + 2] = kp->lev[lvl].dot_ou[row];
             }
         }
     }
     {   // stage the f1 tile [TP][CP] (zero padded) into LDS
-        const int c4n = a.CP >> 2;
-        for (int idx = tid; idx < TP * c4n; idx += blockDim.x) {
+        const int c4n = CMODE == 3 ? 64 : a.CP >> 2;
+        if constexpr (!BF) {   // all loads of a batch in flight before the first LDS write
+            constexpr int SU = 8;
+            for (int base = tid; base < TP * c4n; base += SU * blockDim.x) {
+                v4f x[SU];
+                int dst[SU];
+#pragma unroll
+                for (int t = 0; t < SU; ++t) {
+                    const int idx = base + t * blockDim.x;
+                    const int row = idx / c4n, c = (idx - row * c4n) * 4;
+                    const bool in = idx < TP * c4n, ok = in && p0 + row < N1;
+                    const float *src = kp->f1 + ((size_t)b * N1 + (ok ? p0 + row : 0)) * C;
+                    dst[t] = in ? row * LS + c : -1;
+                    x[t] = load4<CVEC>(src, c, C, ok);
+                }
+#pragma unroll
+                for (int t = 0; t < SU; ++t)
+                    if (dst[t] >= 0) *reinterpret_cast<v4f *>(f1s + dst[t]) = x[t];
+            }
+        }
+        for (int idx = tid; BF && idx < TP * c4n; idx += blockDim.x) {
             const int row = idx / c4n, c = (idx - row * c4n) * 4;
             const bool ok = p0 + row < N1;
-            const float *src = a.f1 + ((size_t)b * N1 + (ok ? p0 + row : 0)) * C;
+            const float *src = kp->f1 + ((size_t)b * N1 + (ok ? p0 + row : 0)) * C;
             const v4f x = load4<CVEC>(src, c, C, ok);
             if constexpr (BF) {
 #pragma unroll
@@ -475,6 +626,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         }
     }
     __syncthreads();
+    TL(1)
 
     const int pix = p0 + pl;           // this lane's image-1 pixel
     const bool pok = pix < N1;
@@ -486,7 +638,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     const int vbase = (WM == 2) ? vp * 256 : 0;
     const int vrow = vbase + 32 * vcw + pl;   // the fmap2 column this lane feeds to the A operand
     const bool vrow_ok = vrow < W2;
-    const float *f2lane = L.f2 + ((size_t)b * H2 * W2 + (vrow_ok ? vrow : 0)) * C;
+    const float *f2lane = Lf2 + ((size_t)b * H2 * W2 + (vrow_ok ? vrow : 0)) * C;
     const size_t rowstride = (size_t)W2 * C;
 
     const bool ragged = vbase + 32 * vcw + 32 > W2;
@@ -500,19 +652,35 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     int vidx[16];
     float wvr[KC][16], rv[KC][16];
     if constexpr (is_weighted(MODE)) {
+        // registers 4g..4g+3 hold four consecutive columns: one 16-byte load each where rows of wv are 16-byte aligned
+        const bool wv16 = (W2 & 3) == 0 && (reinterpret_cast<uintptr_t>(kp->lev[lvl].wv) & 15) == 0;
 #pragma unroll
-        for (int k = 0; k < KC; ++k)
+        for (int k = 0; k < KC; ++k) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int v = vbase + 32 * vcw + vmap(r, h);
-                rv[k][r] = 0.f;
-                wvr[k][r] = (pok && v < W2) ? L.wv[(bp * a.KT + a.k0 + k) * W2 + v] : 0.f;
+            for (int r = 0; r < 16; ++r) rv[k][r] = 0.f;
+            if (wv16) {   // one offset register per group of four columns; the channel travels in the scalar offset
+                const __amdgpu_buffer_rsrc_t rs = make_rsrc(kp->lev[lvl].wv + (size_t)b * N1 * a.KT * W2, (unsigned)N1 * a.KT * W2 * 4u);
+#pragma unroll
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    const int v = vbase + 32 * vcw + vmap(4 * g4, h);
+                    const unsigned o = (pok && v < W2) ? (unsigned)((pix * a.KT + a.k0) * W2 + v) * 4u : DMA_OOB;
+                    const v4f x = buf_load4s(rs, o, (unsigned)(k * W2) * 4u);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) wvr[k][4 * g4 + e] = x[e];
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int v = vbase + 32 * vcw + vmap(r, h);
+                    wvr[k][r] = (pok && v < W2) ? kp->lev[lvl].wv[(bp * a.KT + a.k0 + k) * W2 + v] : 0.f;
+                }
             }
+        }
         if (soft_logits) {
 #pragma unroll
             for (int k = 0; k < KC; ++k) {
                 const size_t row = bp * a.KT + a.k0 + k;
-                const float m = L.st_wv[2 * row], il = 1.f / L.st_wv[2 * row + 1];
+                const float m = kp->lev[lvl].st_wv[2 * row], il = 1.f / kp->lev[lvl].st_wv[2 * row + 1];
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
                     wvr[k][r] = (pok && vbase + 32 * vcw + vmap(r, h) < W2) ? __expf(wvr[k][r] - m) * il : 0.f;
@@ -527,6 +695,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         }
     }
 
+    TL(2)
     const int NJ = a.CP >> 3;
     const int NG = (NJ + GJ - 1) / GJ;
     const int nsteps = sk_total ? sb - sa : ((H2 + UR - 1) / UR + NUG - 1) / NUG;   // steps per wave; rows past H2 are skipped
@@ -553,20 +722,125 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         }
     };
 
-    auto epilogue = [&](int step) {
-        float *pb = part + (step & 1) * (UR * NPART * nW * 32);
+    // Cross-wave combination of a step's partial results (wave order) into the finished out_u rows.  The partials
+    // of step s lie in part[s & 1][wave][row of the step][quantity][32 pixels].
+    auto combine = [&](int step) {
+        const float *pbr = part + (step & 1) * (UR * NPART * nW * 32);
+        constexpr int WSTR = UR * NPART * 32;   // floats per wave
+        if constexpr (is_weighted(MODE)) {
+            for (int idx = tid; idx < NUG * UR * KC * 32; idx += blockDim.x) {
+                const int p = idx & 31, k = (idx >> 5) % KC, ru = (idx / (32 * KC)) % UR, g2 = idx / (32 * KC * UR);
+                const int u = ((sa + step) * NUG + g2) * UR + ru;
+                if (u < H2 && p0 + p < N1) {
+                    const float *src = pbr + (g2 * nvc) * WSTR + (ru * NPART + k) * 32 + p;
+                    float x[8];   // all reads before the first addition
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) x[j] = j < nvc ? src[j * WSTR] : 0.f;
+#pragma unroll
+                    for (int j = 4; j < 8; ++j) x[j] = 0.f;
+                    if (nvc > 4) {
+#pragma unroll
+                        for (int j = 4; j < 8; ++j) x[j] = j < nvc ? src[j * WSTR] : 0.f;
+                    }
+                    float s = 0.f;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) s += x[j];
+                    // (LDS and global destinations are kept in separate branches: a pointer that may be either
+                    // turns into FLAT accesses, whose counters force every later wait to zero)
+                    if (Lstage) {
+                        float *dst = &ostage[(p * NCHO + k) * H2 + u];
+                        if (vp > 0) s += *dst;   // earlier column passes, written by this same thread
+                        *dst = s;
+                    } else {
+                        const size_t row = ((size_t)b * N1 + p0 + p) * a.KT + a.k0 + k;
+                        float *dst = &a.lev[lvl].out_u[row * H2 + u];
+                        if (vp > 0) s += *dst;
+                        if (soft_dlog && vp == vpasses - 1) s = dlogit3(a.lev[lvl].z_ou[row * H2 + u], cst + 3 * (p * KC + k), s);
+                        *dst = s;
+                    }
+                }
+            }
+        } else {
+            for (int idx = tid; idx < NUG * UR * 32; idx += blockDim.x) {
+                const int p = idx & 31, ru = (idx >> 5) % UR, g2 = idx / (32 * UR);
+                const int u = ((sa + step) * NUG + g2) * UR + ru;
+                if (u < H2 && p0 + p < N1) {
+                    const float *src = pbr + (g2 * nvc) * WSTR + (ru * NPART) * 32 + p;
+                    float xm[8], xi[8], xs[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        xm[j] = -INFINITY; xi[j] = 0.f; xs[j] = 0.f;
+                    }
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (j < nvc) { xm[j] = src[j * WSTR]; xi[j] = src[j * WSTR + 32]; xs[j] = src[j * WSTR + 64]; }
+                    if (nvc > 4) {
+#pragma unroll
+                        for (int j = 4; j < 8; ++j)
+                            if (j < nvc) { xm[j] = src[j * WSTR]; xi[j] = src[j * WSTR + 32]; xs[j] = src[j * WSTR + 64]; }
+                    }
+                    float m = xm[0], s = xs[0];
+                    int mi = __float_as_int(xi[0]);
+#pragma unroll
+                    for (int j = 1; j < 8; ++j) {
+                        if (xm[j] > m) { m = xm[j]; mi = __float_as_int(xi[j]); }
+                        s += xs[j];
+                    }
+                    const bool last = vp == vpasses - 1;   // the running sum is kept until the last pass
+                    if (Lstage) {
+                        float *dm = &ostage[(p * 2 + 0) * H2 + u], *ds = &ostage[(p * 2 + 1) * H2 + u];
+                        int *di = &ostage_am[p * H2 + u];
+                        if (vp > 0) {   // merge with the earlier column passes (lower v: they win ties)
+                            const float pm = *dm;
+                            s += *ds;
+                            if (!(m > pm)) { m = pm; if constexpr (MODE == MODE_ARGMAX) mi = *di; }
+                        }
+                        *dm = m;
+                        *ds = last ? s / (float)W2 : s;
+                        if constexpr (MODE == MODE_ARGMAX) *di = mi;
+                    } else {
+                        const size_t o = ((size_t)b * N1 + p0 + p);
+                        float *dm = &a.lev[lvl].out_u[(o * 2 + 0) * H2 + u], *ds = &a.lev[lvl].out_u[(o * 2 + 1) * H2 + u];
+                        if (vp > 0) {
+                            const float pm = *dm;
+                            s += *ds;
+                            if (!(m > pm)) { m = pm; if constexpr (MODE == MODE_ARGMAX) mi = a.lev[lvl].am_u[o * H2 + u]; }
+                        }
+                        *dm = m;
+                        *ds = last ? s / (float)W2 : s;
+                        if constexpr (MODE == MODE_ARGMAX) a.lev[lvl].am_u[o * H2 + u] = mi;
+                    }
+                }
+            }
+        }
+    };
+
+    // The end of a step: every wave reduces its 32 columns of the step's rows and leaves the partial results in LDS
+    // (both halves of a wave hold the same values and write them to the same place), one barrier.  With `defer` the
+    // caller runs combine(step) later (during the next step, where its LDS latency hides behind matrix work).
+    auto epilogue = [&](int step, bool defer = false) {
+        float *pb = part + (step & 1) * (UR * NPART * nW * 32) + wave * (UR * NPART * 32) + pl;
 #pragma unroll
         for (int ru = 0; ru < UR; ++ru) {
             const int u = ((sa + step) * NUG + ug) * UR + ru;
             if (u < H2) {
                 if constexpr (is_weighted(MODE)) {
+                    float sk[KC];
 #pragma unroll
                     for (int k = 0; k < KC; ++k) {
                         float s = 0.f;
 #pragma unroll
                         for (int r = 0; r < 16; ++r) s += acc[ru][r] * wvr[k][r];
-                        s += __shfl_xor(s, 32);
-                        if (h == 0) pb[((ru * NPART + k) * nW + wave) * 32 + pl] = s;
+                        sk[k] = s;
+                    }
+#pragma unroll
+                    for (int k = 0; k < KC; ++k) {
+                        float lo, hi;
+                        wave_halves(sk[k], lo, hi);
+                        pb[(ru * NPART + k) * 32] = lo + hi;
+                    }
+#pragma unroll
+                    for (int k = 0; k < KC; ++k) {
                         const float w = wur[ru][k];
 #pragma unroll
                         for (int r = 0; r < 16; ++r) rv[k][r] += acc[ru][r] * w;
@@ -596,15 +870,14 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                         if (x > vmax[r]) { vmax[r] = x; vidx[r] = u; }
                         vsum[r] += x;
                     }
-                    const float m2 = __shfl_xor(m, 32);
-                    const int mi2 = __shfl_xor(mi, 32);
-                    s += __shfl_xor(s, 32);
-                    if (m2 > m || (m2 == m && mi2 < mi)) { m = m2; mi = mi2; }
-                    if (h == 0) {
-                        pb[((ru * NPART + 0) * nW + wave) * 32 + pl] = m;
-                        pb[((ru * NPART + 1) * nW + wave) * 32 + pl] = __int_as_float(mi);
-                        pb[((ru * NPART + 2) * nW + wave) * 32 + pl] = s;
-                    }
+                    float m_lo, m_hi, i_lo, i_hi, s_lo, s_hi;
+                    wave_halves(m, m_lo, m_hi);
+                    wave_halves(__int_as_float(mi), i_lo, i_hi);
+                    wave_halves(s, s_lo, s_hi);
+                    const bool take_hi = m_hi > m_lo || (m_hi == m_lo && __float_as_int(i_hi) < __float_as_int(i_lo));
+                    pb[(ru * NPART + 0) * 32] = take_hi ? m_hi : m_lo;
+                    pb[(ru * NPART + 1) * 32] = take_hi ? i_hi : i_lo;
+                    pb[(ru * NPART + 2) * 32] = s_lo + s_hi;
                 }
             }
             if constexpr (CMODE != 3) {
@@ -613,70 +886,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
             }
         }
         __syncthreads();
-        // combine the per-wave partials in wave order and store the finished rows
-        if constexpr (is_weighted(MODE)) {
-            for (int idx = tid; idx < NUG * UR * KC * 32; idx += blockDim.x) {
-                const int p = idx & 31, k = (idx >> 5) % KC, ru = (idx / (32 * KC)) % UR, g2 = idx / (32 * KC * UR);
-                const int u = ((sa + step) * NUG + g2) * UR + ru;
-                if (u < H2 && p0 + p < N1) {
-                    float s = 0.f;
-                    for (int w = g2 * nvc; w < (g2 + 1) * nvc; ++w) s += pb[((ru * NPART + k) * nW + w) * 32 + p];
-                    // (LDS and global destinations are kept in separate branches: a pointer that may be either
-                    // turns into FLAT accesses, whose counters force every later wait to zero)
-                    if (L.stage) {
-                        float *dst = &ostage[(p * NCHO + k) * H2 + u];
-                        if (vp > 0) s += *dst;   // earlier column passes, written by this same thread
-                        *dst = s;
-                    } else {
-                        const size_t row = ((size_t)b * N1 + p0 + p) * a.KT + a.k0 + k;
-                        float *dst = &L.out_u[row * H2 + u];
-                        if (vp > 0) s += *dst;
-                        if (soft_dlog && vp == vpasses - 1) s = dlogit3(L.z_ou[row * H2 + u], cst + 3 * (p * KC + k), s);
-                        *dst = s;
-                    }
-                }
-            }
-        } else {
-            for (int idx = tid; idx < NUG * UR * 32; idx += blockDim.x) {
-                const int p = idx & 31, ru = (idx >> 5) % UR, g2 = idx / (32 * UR);
-                const int u = ((sa + step) * NUG + g2) * UR + ru;
-                if (u < H2 && p0 + p < N1) {
-                    const int w0 = g2 * nvc;
-                    float m = pb[((ru * NPART + 0) * nW + w0) * 32 + p];
-                    int mi = __float_as_int(pb[((ru * NPART + 1) * nW + w0) * 32 + p]);
-                    float s = pb[((ru * NPART + 2) * nW + w0) * 32 + p];
-                    for (int w = w0 + 1; w < w0 + nvc; ++w) {
-                        const float m2 = pb[((ru * NPART + 0) * nW + w) * 32 + p];
-                        if (m2 > m) { m = m2; mi = __float_as_int(pb[((ru * NPART + 1) * nW + w) * 32 + p]); }
-                        s += pb[((ru * NPART + 2) * nW + w) * 32 + p];
-                    }
-                    const bool last = vp == vpasses - 1;   // the running sum is kept until the last pass
-                    if (L.stage) {
-                        float *dm = &ostage[(p * 2 + 0) * H2 + u], *ds = &ostage[(p * 2 + 1) * H2 + u];
-                        int *di = &ostage_am[p * H2 + u];
-                        if (vp > 0) {   // merge with the earlier column passes (lower v: they win ties)
-                            const float pm = *dm;
-                            s += *ds;
-                            if (!(m > pm)) { m = pm; if constexpr (MODE == MODE_ARGMAX) mi = *di; }
-                        }
-                        *dm = m;
-                        *ds = last ? s / (float)W2 : s;
-                        if constexpr (MODE == MODE_ARGMAX) *di = mi;
-                    } else {
-                        const size_t o = ((size_t)b * N1 + p0 + p);
-                        float *dm = &L.out_u[(o * 2 + 0) * H2 + u], *ds = &L.out_u[(o * 2 + 1) * H2 + u];
-                        if (vp > 0) {
-                            const float pm = *dm;
-                            s += *ds;
-                            if (!(m > pm)) { m = pm; if constexpr (MODE == MODE_ARGMAX) mi = L.am_u[o * H2 + u]; }
-                        }
-                        *dm = m;
-                        *ds = last ? s / (float)W2 : s;
-                        if constexpr (MODE == MODE_ARGMAX) L.am_u[o * H2 + u] = mi;
-                    }
-                }
-            }
-        }
+        if (!defer) combine(step);
     };
 
     auto compute = [&](int step, int g, v4f(&buf)[UR][GJ]) {
@@ -688,7 +898,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
 #pragma unroll
                     for (int k = 0; k < KC; ++k)
                     {
-                        wur[r][k] = (pok && u < H2) ? L.wu[(bp * a.KT + a.k0 + k) * H2 + u] : 0.f;
+                        wur[r][k] = (pok && u < H2) ? Lwu[(bp * a.KT + a.k0 + k) * H2 + u] : 0.f;
                         if (soft_logits) wur[r][k] = __expf(wur[r][k] - cst[2 * (pl * KC + k)]) * cst[2 * (pl * KC + k) + 1];
                     }
                 }
@@ -733,7 +943,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                     for (int r = 0; r < UR; ++r) {
                         const int u = min(((sa + step) * NUG + ug) * UR + r, H2 - 1);
 #pragma unroll
-                        for (int k = 0; k < KC; ++k) wur[r][k] = L.wu[(bp * a.KT + a.k0 + k) * H2 + u];
+                        for (int k = 0; k < KC; ++k) wur[r][k] = Lwu[(bp * a.KT + a.k0 + k) * H2 + u];
                     }
                 }
             }
@@ -772,7 +982,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         // 0..31) and 32J+16+4tq+t (lanes 32..63); the f1 tile in LDS is read with the same mapping.
         const unsigned rowbytes = (unsigned)W2 * C * 4u;
         const unsigned nbytes = (unsigned)H2 * rowbytes;
-        const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(L.f2 + (size_t)b * H2 * W2 * C, nbytes);
+        const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(Lf2 + (size_t)b * H2 * W2 * C, nbytes);
         const unsigned lane_off = vrow_ok ? ((unsigned)vrow * C + 16u * h) * 4u : nbytes;
         const int NJB = (CMODE == 3) ? 8 : (C >> 5);
         constexpr bool BPIPE = !(is_weighted(MODE) && KC >= 3);   // needs 16 more registers
@@ -796,14 +1006,23 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
             }
             __builtin_amdgcn_sched_barrier(0);   // keep the loads here: a full block ahead of their use
         };
+        // u-indexed weights of a row: per lane a fixed offset (its pixel), row and channel in the scalar offset
+        __amdgpu_buffer_rsrc_t rsrc_wu = rsrc;
+        unsigned wu_lane = 0;
+        if constexpr (is_weighted(MODE)) {
+            rsrc_wu = make_rsrc(Lwu + (size_t)b * N1 * a.KT * H2, (unsigned)N1 * a.KT * H2 * 4u);
+            wu_lane = (unsigned)(((pok ? pix : 0) * a.KT + a.k0) * H2) * 4u;
+        }
         auto computeF = [&](int step, int J, v4f(&buf)[UR][4]) {
+            // the cross-wave sums of the step before (its partial results have been in LDS since that step's barrier)
+            if (J == (NJB > 1 ? 1 : 0) && step > 0) combine(step - 1);
             if constexpr (is_weighted(MODE)) {
                 if (J == 0) {
 #pragma unroll
                     for (int r = 0; r < UR; ++r) {
                         const int u = min(((sa + step) * NUG + ug) * UR + r, H2 - 1);
 #pragma unroll
-                        for (int k = 0; k < KC; ++k) wur[r][k] = L.wu[(bp * a.KT + a.k0 + k) * H2 + u];
+                        for (int k = 0; k < KC; ++k) wur[r][k] = buf_load1s(rsrc_wu, wu_lane, (unsigned)(k * H2 + u) * 4u);
                     }
                 }
                 if (J == (NJB > 1 ? 1 : 0) && soft_logits) {   // (a block later: the loads above have landed by now)
@@ -866,7 +1085,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                         for (int e = 0; e < 16; ++e) acc_alt[e] = 0.f;
                     }
                 }
-                epilogue(step);
+                epilogue(step, true);
             }
         };
         // Ring of NB register buffers: the loads of block i+NB-1 are issued before the MFMAs of block i,
@@ -908,6 +1127,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                 }
             }
         }
+        if (nsteps > 0) combine(nsteps - 1);   // the last step's, still owed
     } else {
     v4f bufA[UR][GJ], bufB[UR][GJ];
     int step = 0, g = 0;  // position of iteration `it`
@@ -926,80 +1146,97 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     }
     }
 
+    TL(3)
+    // (lane indices for the code behind the sweep are derived afresh from the thread id, so that nothing of them
+    // is kept in registers during the sweep)
+    int tide = threadIdx.x;
+    asm volatile("" : "+v"(tide));
+    const int wave_e = tide >> 6, lane_e = tide & 63, pl_e = lane_e & 31, h_e = lane_e >> 5;
+    const int vcw_e = RG ? wave_e % nvc : wave_e, ug_e = RG ? wave_e / nvc : 0;
+    const int pix_e = p0 + pl_e;
+    const bool pok_e = pix_e < N1;
+    const size_t bp_e = (size_t)b * N1 + (pok_e ? pix_e : 0);
+    (void)lane_e; (void)h_e; (void)vcw_e; (void)ug_e; (void)bp_e;
+    const KArgs ke = kernargs_now();
     // flush the staged out_u rows of this piece (all rows of a whole tile): per pixel and channel a run of floats
-    if (L.stage && vp == vpasses - 1) {
+    if (Lstage && vp == vpasses - 1) {
         __syncthreads();
         const int cht = (is_weighted(MODE)) ? a.KT : 2, ch0 = (is_weighted(MODE)) ? a.k0 : 0;
         const int u0 = whole ? 0 : sa * NUG * UR, nu = (whole ? H2 : min(H2, sb * NUG * UR)) - u0;
-        const int total = TP * NCHO * nu;
+        // A (pixel, channel) row of nu floats goes to 8, 16, 32 or 64 neighbouring lanes, so that several short rows
+        // share a wave_e; the row index is the same for all lanes of a group (no division by nu anywhere).
+        const int lsh = nu > 32 ? 6 : nu > 16 ? 5 : nu > 8 ? 4 : 3;
+        const int lpr = 1 << lsh, rpi = 64 >> lsh;        // lanes per row, rows per wave_e and trip
+        const int lr = lane_e >> lsh, lu = lane_e & (lpr - 1);
         constexpr int UNR = 4;   // the logits of a batch of elements are fetched before any of them is used
-        for (int base = tid; base < total; base += UNR * blockDim.x) {
-            float zs[UNR];
-            size_t off[UNR];
-            int lds_i[UNR], pk[UNR];
+        for (int r0 = wave_e * rpi + lr; r0 < TP * NCHO; r0 += UNR * nW * rpi)
+            for (int uu = lu; uu < nu; uu += lpr) {
+                float zs[UNR];
+                size_t off[UNR];
+                int lds_i[UNR], pk[UNR];
 #pragma unroll
-            for (int t = 0; t < UNR; ++t) {
-                const int idx = base + t * blockDim.x;
-                const int p = idx / (NCHO * nu), rem = idx - p * (NCHO * nu), ch = rem / nu, u = u0 + rem - ch * nu;
-                const bool ok = idx < total && p0 + p < N1;
-                off[t] = ok ? ((((size_t)b * N1 + p0 + p) * cht + ch0 + ch) * H2 + u) : (size_t)-1;
-                lds_i[t] = (p * NCHO + ch) * H2 + u;
-                pk[t] = p * KC + ch;
-                zs[t] = 0.f;
-                if constexpr (is_weighted(MODE)) {
-                    if (soft_dlog && ok) zs[t] = L.z_ou[off[t]];
+                for (int t = 0; t < UNR; ++t) {
+                    const int r = r0 + t * nW * rpi;
+                    const int p = r / NCHO, ch = r - p * NCHO, u = u0 + uu;
+                    const bool ok = r < TP * NCHO && p0 + p < N1;
+                    off[t] = ok ? ((((size_t)b * N1 + p0 + p) * cht + ch0 + ch) * H2 + u) : (size_t)-1;
+                    lds_i[t] = r * H2 + u;
+                    pk[t] = p * KC + ch;
+                    zs[t] = 0.f;
+                    if constexpr (is_weighted(MODE)) {
+                        if (soft_dlog && ok) zs[t] = ke->lev[lvl].z_ou[off[t]];
+                    }
+                }
+#pragma unroll
+                for (int t = 0; t < UNR; ++t) {
+                    if (off[t] == (size_t)-1) continue;
+                    float x = ostage[lds_i[t]];
+                    if constexpr (is_weighted(MODE)) {
+                        if (soft_dlog) x = dlogit3(zs[t], cst + 3 * pk[t], x);
+                    }
+                    ke->lev[lvl].out_u[off[t]] = x;
                 }
             }
-#pragma unroll
-            for (int t = 0; t < UNR; ++t) {
-                if (off[t] == (size_t)-1) continue;
-                float x = ostage[lds_i[t]];
-                if constexpr (is_weighted(MODE)) {
-                    if (soft_dlog) x = dlogit3(zs[t], cst + 3 * pk[t], x);
-                }
-                L.out_u[off[t]] = x;
-            }
-        }
         if constexpr (MODE == MODE_ARGMAX) {
-            for (int idx = tid; idx < TP * nu; idx += blockDim.x) {
-                const int p = idx / nu, u = u0 + idx - p * nu;
-                if (p0 + p < N1) L.am_u[((size_t)b * N1 + p0 + p) * H2 + u] = ostage_am[p * H2 + u];
-            }
+            for (int p = wave_e * rpi + lr; p < TP; p += nW * rpi)
+                for (int uu = lu; uu < nu; uu += lpr)
+                    if (p0 + p < N1) ke->lev[lvl].am_u[((size_t)b * N1 + p0 + p) * H2 + u0 + uu] = ostage_am[p * H2 + u0 + uu];
         }
     }
 
+    TL(4)
     // merge the running state of the row groups into group 0, one group at a time, through the LDS
     // region of the f1 tile (no longer needed).  Equal maxima keep the smaller row index.
     if (NUG > 1) {
         constexpr int NQ = (is_weighted(MODE)) ? KC : 3;
-        float *mst = smem + vcw * (NQ * 16 * 64);   // [vcw][quantity][r][lane]
+        float *mst = smem + vcw_e * (NQ * 16 * 64);   // [vcw_e][quantity][r][lane_e]
         for (int g2 = 1; g2 < NUG; ++g2) {
             __syncthreads();
-            if (ug == g2) {
+            if (ug_e == g2) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     if constexpr (is_weighted(MODE)) {
 #pragma unroll
-                        for (int k = 0; k < KC; ++k) mst[(k * 16 + r) * 64 + lane] = rv[k][r];
+                        for (int k = 0; k < KC; ++k) mst[(k * 16 + r) * 64 + lane_e] = rv[k][r];
                     } else {
-                        mst[(0 * 16 + r) * 64 + lane] = vmax[r];
-                        mst[(1 * 16 + r) * 64 + lane] = __int_as_float(vidx[r]);
-                        mst[(2 * 16 + r) * 64 + lane] = vsum[r];
+                        mst[(0 * 16 + r) * 64 + lane_e] = vmax[r];
+                        mst[(1 * 16 + r) * 64 + lane_e] = __int_as_float(vidx[r]);
+                        mst[(2 * 16 + r) * 64 + lane_e] = vsum[r];
                     }
                 }
             }
             __syncthreads();
-            if (ug == 0) {
+            if (ug_e == 0) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     if constexpr (is_weighted(MODE)) {
 #pragma unroll
-                        for (int k = 0; k < KC; ++k) rv[k][r] += mst[(k * 16 + r) * 64 + lane];
+                        for (int k = 0; k < KC; ++k) rv[k][r] += mst[(k * 16 + r) * 64 + lane_e];
                     } else {
-                        const float m2 = mst[(0 * 16 + r) * 64 + lane];
-                        const int i2 = __float_as_int(mst[(1 * 16 + r) * 64 + lane]);
+                        const float m2 = mst[(0 * 16 + r) * 64 + lane_e];
+                        const int i2 = __float_as_int(mst[(1 * 16 + r) * 64 + lane_e]);
                         if (m2 > vmax[r] || (m2 == vmax[r] && i2 < vidx[r])) { vmax[r] = m2; vidx[r] = i2; }
-                        vsum[r] += mst[(2 * 16 + r) * 64 + lane];
+                        vsum[r] += mst[(2 * 16 + r) * 64 + lane_e];
                     }
                 }
             }
@@ -1007,13 +1244,13 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     }
 
     // A piece of a tile leaves its column state in this workgroup's slot in register order, sums undivided:
-    // [column chunk][quantity][register group g4][lane][4]: every store of a wave is one contiguous KB
+    // [column chunk][quantity][register group g4][lane_e][4]: every store of a wave_e is one contiguous KB
     if (!whole) {
-        if (ug == 0 && vbase + 32 * vcw < W2) {
+        if (ug_e == 0 && vbase + 32 * vcw_e < W2) {
             constexpr int NQ = (is_weighted(MODE)) ? KC : 3;
-            const __amdgpu_buffer_rsrc_t rs_sk = make_rsrc(a.sk_state, 2u * gridDim.x * (unsigned)a.sk_slot * 4u);
+            const __amdgpu_buffer_rsrc_t rs_sk = make_rsrc(ke->sk_state, 2u * gridDim.x * (unsigned)a.sk_slot * 4u);
             const unsigned base = ((unsigned)(2 * wg + (pb == gs0 ? 0 : 1)) * (unsigned)a.sk_slot +
-                                   (unsigned)((vbase >> 5) + vcw) * (NQ * 1024u) + 4u * lane) * 4u;
+                                   (unsigned)((vbase >> 5) + vcw_e) * (NQ * 1024u) + 4u * lane_e) * 4u;
 #pragma unroll
             for (int q = 0; q < NQ; ++q)
 #pragma unroll
@@ -1029,35 +1266,35 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         }
     } else
     // store the state that was reduced over u: registers 4g..4g+3 hold 4 consecutive columns
-    if (pok && ug == 0) {
+    if (pok_e && ug_e == 0) {
         if ((W2 & 3) == 0) {   // 16-byte stores (rows of out_v are then 16-byte aligned)
             typedef int v4i __attribute__((ext_vector_type(4)));
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4) {
-                const int v = vbase + 32 * vcw + vmap(4 * g4, h);
+                const int v = vbase + 32 * vcw_e + vmap(4 * g4, h_e);
                 if (v < W2) {
                     if constexpr (is_weighted(MODE)) {
 #pragma unroll
                         for (int k = 0; k < KC; ++k) {
                             v4f x = {rv[k][4 * g4], rv[k][4 * g4 + 1], rv[k][4 * g4 + 2], rv[k][4 * g4 + 3]};
-                            const size_t row = bp * a.KT + a.k0 + k;
+                            const size_t row = bp_e * a.KT + a.k0 + k;
                             if (soft_dlog) {
-                                const float r3[3] = {L.st_ov[2 * row], 1.f / L.st_ov[2 * row + 1], L.dot_ov[row]};
-                                const v4f z = *reinterpret_cast<const v4f *>(L.z_ov + row * W2 + v);
+                                const float r3[3] = {ke->lev[lvl].st_ov[2 * row], 1.f / ke->lev[lvl].st_ov[2 * row + 1], ke->lev[lvl].dot_ov[row]};
+                                const v4f z = *reinterpret_cast<const v4f *>(ke->lev[lvl].z_ov + row * W2 + v);
 #pragma unroll
                                 for (int e = 0; e < 4; ++e) x[e] = dlogit3(z[e], r3, x[e]);
                             }
-                            *reinterpret_cast<v4f *>(L.out_v + row * W2 + v) = x;
+                            *reinterpret_cast<v4f *>(ke->lev[lvl].out_v + row * W2 + v) = x;
                         }
                     } else {
                         const v4f xm = {vmax[4 * g4], vmax[4 * g4 + 1], vmax[4 * g4 + 2], vmax[4 * g4 + 3]};
                         const v4f xs = {vsum[4 * g4] / (float)H2, vsum[4 * g4 + 1] / (float)H2, vsum[4 * g4 + 2] / (float)H2,
                                         vsum[4 * g4 + 3] / (float)H2};
-                        *reinterpret_cast<v4f *>(L.out_v + (bp * 2 + 0) * W2 + v) = xm;
-                        *reinterpret_cast<v4f *>(L.out_v + (bp * 2 + 1) * W2 + v) = xs;
+                        *reinterpret_cast<v4f *>(ke->lev[lvl].out_v + (bp_e * 2 + 0) * W2 + v) = xm;
+                        *reinterpret_cast<v4f *>(ke->lev[lvl].out_v + (bp_e * 2 + 1) * W2 + v) = xs;
                         if constexpr (MODE == MODE_ARGMAX) {
                             const v4i xi = {vidx[4 * g4], vidx[4 * g4 + 1], vidx[4 * g4 + 2], vidx[4 * g4 + 3]};
-                            *reinterpret_cast<v4i *>(L.am_v + bp * W2 + v) = xi;
+                            *reinterpret_cast<v4i *>(ke->lev[lvl].am_v + bp_e * W2 + v) = xi;
                         }
                     }
                 }
@@ -1065,26 +1302,38 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         } else {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int v = vbase + 32 * vcw + vmap(r, h);
+                const int v = vbase + 32 * vcw_e + vmap(r, h_e);
                 if (v < W2) {
                     if constexpr (is_weighted(MODE)) {
 #pragma unroll
                         for (int k = 0; k < KC; ++k) {
-                            const size_t row = bp * a.KT + a.k0 + k;
-                            L.out_v[row * W2 + v] = soft_dlog ? dlogit(L.z_ov, L.st_ov, L.dot_ov, row, row * W2 + v, rv[k][r]) : rv[k][r];
+                            const size_t row = bp_e * a.KT + a.k0 + k;
+                            ke->lev[lvl].out_v[row * W2 + v] = soft_dlog ? dlogit(ke->lev[lvl].z_ov, ke->lev[lvl].st_ov, ke->lev[lvl].dot_ov, row, row * W2 + v, rv[k][r]) : rv[k][r];
                         }
                     } else {
-                        L.out_v[(bp * 2 + 0) * W2 + v] = vmax[r];
-                        L.out_v[(bp * 2 + 1) * W2 + v] = vsum[r] / (float)H2;
-                        if constexpr (MODE == MODE_ARGMAX) L.am_v[bp * W2 + v] = vidx[r];
+                        ke->lev[lvl].out_v[(bp_e * 2 + 0) * W2 + v] = vmax[r];
+                        ke->lev[lvl].out_v[(bp_e * 2 + 1) * W2 + v] = vsum[r] / (float)H2;
+                        if constexpr (MODE == MODE_ARGMAX) ke->lev[lvl].am_v[bp_e * W2 + v] = vidx[r];
                     }
                 }
             }
         }
     }
     }   // column passes
+    TL(5)
+    // (lane indices for the code behind the sweep are derived afresh from the thread id, so that nothing of them
+    // is kept in registers during the sweep)
+    int tide = threadIdx.x;
+    asm volatile("" : "+v"(tide));
+    const int wave_e = tide >> 6, lane_e = tide & 63, pl_e = lane_e & 31, h_e = lane_e >> 5;
+    const int vcw_e = RG ? wave_e % nvc : wave_e, ug_e = RG ? wave_e / nvc : 0;
+    const int pix_e = p0 + pl_e;
+    const bool pok_e = pix_e < N1;
+    const size_t bp_e = (size_t)b * N1 + (pok_e ? pix_e : 0);
+    (void)lane_e; (void)h_e; (void)vcw_e; (void)ug_e; (void)bp_e;
 
     if (!whole) {
+        const KArgs ke = kernargs_now();
         // Publish this piece and find out whether it completes the tile.  The pieces of a tile belong to consecutive
         // workgroups; a workgroup keeps the first piece of its share in its slot 0 and a later one (which can only be
         // its last: the tiles between are whole) in its slot 1.
@@ -1096,79 +1345,21 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         int wlast = wfirst;                                              // the workgroup that holds step t1 - 1
         while (((long)(wlast + 1) * sk_total) / G < t1) ++wlast;
         const int npieces = wlast - wfirst + 1;
-        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's words of the piece have arrived
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave_e's words of the piece have arrived
         __syncthreads();
         int *flag = reinterpret_cast<int *>(smem);
-        if (tid == 0)
-            *flag = __hip_atomic_fetch_add(a.sk_count + (multi ? tile * a.nlev + lvl : tile), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (tide == 0)
+            *flag = __hip_atomic_fetch_add(ke->sk_count + (multi ? tile * a.nlev + lvl : tile), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         const bool last = *flag == npieces - 1;
         __syncthreads();
-        if (last) {
-            // Add up the pieces in row order (equal maxima keep the lower row) and write the finished columns.
-            // An item = the 4 consecutive columns a lane holds in one register group of one column chunk.
-            constexpr int NQ = (is_weighted(MODE)) ? KC : 3;
-            const __amdgpu_buffer_rsrc_t rs_sk = make_rsrc(a.sk_state, 2u * gridDim.x * (unsigned)a.sk_slot * 4u);
-            const int nchunks = (W2 + 31) >> 5;
-            for (int it = tid; it < nchunks * 256; it += blockDim.x) {
-                const int ln = it & 63, g4 = (it >> 6) & 3, chunk = it >> 8;
-                const int p = ln & 31, v = 32 * chunk + vmap(4 * g4, ln >> 5);
-                v4f acc4[NQ];
-#pragma unroll
-                for (int q = 0; q < NQ; ++q) acc4[q] = v4f{0.f, 0.f, 0.f, 0.f};
-                if constexpr (!is_weighted(MODE)) acc4[0] = v4f{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
-                for (int w = wfirst; w <= wlast; ++w) {
-                    const bool first_piece = ((long)w * sk_total) / G >= t0;   // w's share starts inside this tile
-                    const unsigned base = ((unsigned)(2 * w + (first_piece ? 0 : 1)) * (unsigned)a.sk_slot +
-                                           (unsigned)chunk * (NQ * 1024u) + 4u * ln) * 4u;
-                    v4f x[NQ];
-#pragma unroll
-                    for (int q = 0; q < NQ; ++q) x[q] = load_shared4(rs_sk, base + (unsigned)(q * 4 + g4) * 1024u);
-                    if constexpr (is_weighted(MODE)) {
-#pragma unroll
-                        for (int q = 0; q < NQ; ++q) acc4[q] += x[q];
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (x[0][e] > acc4[0][e]) { acc4[0][e] = x[0][e]; acc4[1][e] = x[1][e]; }
-                        acc4[2] += x[2];
-                    }
-                }
-                if (p0 + p >= N1) continue;
-                const size_t o = (size_t)b * N1 + p0 + p;
-                if constexpr (is_weighted(MODE)) {
-                    if (soft_dlog) {   // sums of softmax-output gradients -> gradients of the logits
-                        float r3[NQ][3], z[NQ][4];
-#pragma unroll
-                        for (int q = 0; q < NQ; ++q) {
-                            const size_t row = o * a.KT + a.k0 + q;
-                            r3[q][0] = L.st_ov[2 * row]; r3[q][1] = L.st_ov[2 * row + 1]; r3[q][2] = L.dot_ov[row];
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) z[q][e] = v + e < W2 ? L.z_ov[row * W2 + v + e] : 0.f;
-                        }
-#pragma unroll
-                        for (int q = 0; q < NQ; ++q) {
-                            r3[q][1] = 1.f / r3[q][1];
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) acc4[q][e] = dlogit3(z[q][e], r3[q], acc4[q][e]);
-                        }
-                    }
-                }
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    if (v + e >= W2) break;
-                    if constexpr (is_weighted(MODE)) {
-#pragma unroll
-                        for (int q = 0; q < NQ; ++q) L.out_v[(o * a.KT + a.k0 + q) * W2 + v + e] = acc4[q][e];
-                    } else {
-                        L.out_v[(o * 2 + 0) * W2 + v + e] = acc4[0][e];
-                        L.out_v[(o * 2 + 1) * W2 + v + e] = acc4[2][e] / (float)H2;
-                        if constexpr (MODE == MODE_ARGMAX) L.am_v[o * W2 + v + e] = __float_as_int(acc4[1][e]);
-                    }
-                }
-            }
-        }
+        TL(6)
+#ifdef SEPCORR_TIMELINE
+        if (a.dbg && tide == 0) a.dbg[((size_t)wg * 4 + min(seg_no, 3)) * 12 + 10] = last;
+#endif
+        if (last) merge_pieces<MODE, KC>(ke, lvl, b, p0, wfirst, wlast, (int)t0, tide);
     }
+    TL(7)
     }   // pieces of this workgroup
 }
 
@@ -2448,9 +2639,19 @@ int launch_fwd(FwdArgs a, int B, hipStream_t s) {
         if (lds < merge) lds = merge;
     }
     if (MODE == MODE_SOFT) lds += (size_t)TP * KC * 3 * sizeof(float);   // row statistics of the tile
+    {   // the kernel reads the level's pointers and sizes from lev[0]
+        FwdLevel &L = a.lev[0];
+        L.f2 = a.f2; L.wv = a.wv; L.wu = a.wu; L.out_u = a.out_u; L.out_v = a.out_v; L.am_u = a.am_u; L.am_v = a.am_v;
+        L.st_wv = a.st_wv; L.st_wu = a.st_wu; L.z_ou = a.z_ou; L.st_ou = a.st_ou; L.dot_ou = a.dot_ou;
+        L.z_ov = a.z_ov; L.st_ov = a.st_ov; L.dot_ov = a.dot_ov;
+        L.H2 = a.H2; L.W2 = a.W2; L.nvc = a.nvc; L.stage = a.stage;
+    }
     dim3 grid(B * a.tiles_per_batch);
     const dim3 block(64 * nW);
     a.sk_total = 0;
+#ifdef SEPCORR_TIMELINE
+    { const char *e = getenv("SEPCORR_DBG_PTR"); a.dbg = e ? (long long *)strtoull(e, nullptr, 0) : nullptr; }
+#endif
     if (a.ws != nullptr && !a.f2_planes) {
         const FwdSplit f = fwd_split(B * a.tiles_per_batch, a.H2, a.W2, UR * wg.nug, NPART, (nW <= 4 && lds <= 80 * 1024) ? 2 : 1);
         if (f.on && f.bytes <= a.ws_bytes) {
