@@ -1470,6 +1470,59 @@ __device__ __forceinline__ void load_vw16(const BwdArgs &a, size_t bp, const int
         for (int r = 0; r < 16; ++r) w[r].am = ok[r] ? ram[v[r]] : -1;
     }
 }
+// The same for rows whose length is a multiple of 4: the four consecutive columns of a register group (vmap) come
+// with one 16-byte buffer load; per group one offset register, the field travels in the scalar offset.  v0 = first
+// column of the wave's chunk, h = half of the wave, pix = the lane's pixel within image b (pok: it exists).
+template <int GMODE, int KC>
+__device__ __forceinline__ void load_vw16_rows4(const BwdArgs &a, int b, int pix, bool pok, int v0, int h, VW<GMODE, KC> (&w)[16]) {
+    const unsigned W2 = (unsigned)a.W2, N1 = (unsigned)a.N1;
+    bool ok[4];
+#pragma unroll
+    for (int g4 = 0; g4 < 4; ++g4) ok[g4] = pok && v0 + vmap(4 * g4, h) < a.W2;
+    if constexpr (g_has_comp(GMODE)) {
+        const __amdgpu_buffer_rsrc_t ra = make_rsrc(a.a_u + (size_t)b * N1 * a.KT * W2, N1 * a.KT * W2 * 4u);
+        const __amdgpu_buffer_rsrc_t rg = make_rsrc(a.g_cv + (size_t)b * N1 * a.KT * W2, N1 * a.KT * W2 * 4u);
+        unsigned o[4];
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4)
+            o[g4] = ok[g4] ? (unsigned)((pix * a.KT + a.k0) * a.W2 + v0 + vmap(4 * g4, h)) * 4u : DMA_OOB;
+#pragma unroll
+        for (int k = 0; k < KC; ++k)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const v4f x = buf_load4s(ra, o[g4], (unsigned)k * W2 * 4u);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) w[4 * g4 + e].a[k] = x[e];
+            }
+#pragma unroll
+        for (int k = 0; k < KC; ++k)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const v4f x = buf_load4s(rg, o[g4], (unsigned)k * W2 * 4u);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) w[4 * g4 + e].g[k] = x[e];
+            }
+    }
+    if constexpr (g_has_maxavg(GMODE)) {
+        const float inv_h2 = 1.f / (float)a.H2;
+        const __amdgpu_buffer_rsrc_t rg = make_rsrc(a.g_v + (size_t)b * N1 * 2u * W2, N1 * 2u * W2 * 4u);
+        const __amdgpu_buffer_rsrc_t rm = make_rsrc(a.am_v + (size_t)b * N1 * W2, N1 * W2 * 4u);
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+            const int v = v0 + vmap(4 * g4, h);
+            const unsigned og = ok[g4] ? (unsigned)(pix * 2 * a.W2 + v) * 4u : DMA_OOB;
+            const unsigned om = ok[g4] ? (unsigned)(pix * a.W2 + v) * 4u : DMA_OOB;
+            const v4f xmax = buf_load4s(rg, og, 0u), xavg = buf_load4s(rg, og, W2 * 4u);
+            const v4f xam = buf_load4s(rm, om, 0u);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                w[4 * g4 + e].mg = xavg[e] * inv_h2;                       // (all zero where the group does not exist)
+                w[4 * g4 + e].ma = w[4 * g4 + e].mg + xmax[e];
+                w[4 * g4 + e].am = ok[g4] ? __float_as_int(xam[e]) : -1;
+            }
+        }
+    }
+}
 template <int GMODE, int KC>
 __device__ __forceinline__ UW<GMODE, KC> load_uw(const BwdArgs &a, size_t bp, int u, bool ok) {
     UW<GMODE, KC> w;
@@ -1570,7 +1623,9 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
     for (int vp = 0; vp < a.vpasses; ++vp) {
     const int vbase = vp * 256;
     VW<GMODE, KC> wv[16];
-    {
+    if ((W2 & 3) == 0) {
+        load_vw16_rows4<GMODE, KC>(a, b, pix, pok, vbase + 32 * vcw, h, wv);
+    } else {
         int vs[16];
         bool oks[16];
 #pragma unroll
@@ -1737,16 +1792,50 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
             }
     }
     __syncthreads();
-    auto tile_sum = [&](int row, int c) {
-        v4f x = *reinterpret_cast<const v4f *>(smem + row * RS + c);
-        for (int w = 1; w < nW; ++w) x += *reinterpret_cast<const v4f *>(smem + w * (TP * RS) + row * RS + c);
-        return x;
+    // The sum over the waves' LDS regions for MI items of this thread (item = 4 channels of a pixel; items idx0,
+    // idx0 + blockDim.x, ...): all reads of a batch are issued before the first addition, sums run in wave order.
+    constexpr int MI = 4;
+    constexpr int NIT = TP * (CB / 4);
+    auto tile_sums = [&](int idx0, v4f (&x)[MI]) {
+        v4f y[MI][4];
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+            const int idx = min(idx0 + i * (int)blockDim.x, NIT - 1);
+            const int row = idx / (CB / 4), c = (idx - row * (CB / 4)) * 4;
+#pragma unroll
+            for (int w = 0; w < 4; ++w)
+                y[i][w] = *reinterpret_cast<const v4f *>(smem + min(w, nW - 1) * (TP * RS) + row * RS + c);
+        }
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+            x[i] = y[i][0];
+#pragma unroll
+            for (int w = 1; w < 4; ++w)
+                if (w < nW) x[i] += y[i][w];
+        }
+        for (int w = 4; w < nW; ++w) {   // 5 to 8 waves (rows of more than 128 columns)
+#pragma unroll
+            for (int i = 0; i < MI; ++i) {
+                const int idx = min(idx0 + i * (int)blockDim.x, NIT - 1);
+                const int row = idx / (CB / 4), c = (idx - row * (CB / 4)) * 4;
+                x[i] += *reinterpret_cast<const v4f *>(smem + w * (TP * RS) + row * RS + c);
+            }
+        }
+    };
+    auto store_items = [&](int idx0, const v4f (&x)[MI]) {
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+            const int idx = idx0 + i * (int)blockDim.x;
+            const int row = idx / (CB / 4), c = (idx - row * (CB / 4)) * 4;
+            if (idx < NIT && p0 + row < N1)
+                store4<CVEC>(a.d1 + ((size_t)b * N1 + p0 + row) * C, cb0 + c, C, x[i], a.accumulate != 0);
+        }
     };
     if (whole) {
-        for (int idx = tid; idx < TP * (CB / 4); idx += blockDim.x) {
-            const int row = idx / (CB / 4), c = (idx - row * (CB / 4)) * 4;
-            if (p0 + row < N1)
-                store4<CVEC>(a.d1 + ((size_t)b * N1 + p0 + row) * C, cb0 + c, C, tile_sum(row, c), a.accumulate != 0);
+        for (int idx0 = tid; idx0 < NIT; idx0 += MI * blockDim.x) {
+            v4f x[MI];
+            tile_sums(idx0, x);
+            store_items(idx0, x);
         }
     } else {
         // leave the piece's partial sum [32][CB] in this workgroup's slot, then see whether it completes the tile
@@ -1754,9 +1843,14 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
         const unsigned nslots = 2u * gridDim.x * gridDim.y;
         const __amdgpu_buffer_rsrc_t rs_sk = make_rsrc(a.sk_state, nslots * SLOT * 4u);
         const unsigned mine = (2u * (wg * gridDim.y + blockIdx.y) + (pb == gs0 ? 0u : 1u)) * SLOT;
-        for (int idx = tid; idx < TP * (CB / 4); idx += blockDim.x) {
-            const int row = idx / (CB / 4), c = (idx - row * (CB / 4)) * 4;
-            store_shared4(rs_sk, (mine + (unsigned)idx * 4u) * 4u, tile_sum(row, c));
+        for (int idx0 = tid; idx0 < NIT; idx0 += MI * blockDim.x) {
+            v4f x[MI];
+            tile_sums(idx0, x);
+#pragma unroll
+            for (int i = 0; i < MI; ++i) {
+                const int idx = idx0 + i * (int)blockDim.x;
+                if (idx < NIT) store_shared4(rs_sk, (mine + (unsigned)idx * 4u) * 4u, x[i]);
+            }
         }
         const int G = (int)gridDim.x;
         const long t0 = (long)tile * S, t1 = t0 + S;
@@ -1773,15 +1867,30 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
         __syncthreads();
         const bool last = *flag == wlast - wfirst;
         if (last) {   // pieces in row order, after what the destination already holds when accumulating
-            for (int idx = tid; idx < TP * (CB / 4); idx += blockDim.x) {
-                const int row = idx / (CB / 4), c = (idx - row * (CB / 4)) * 4;
-                v4f x = {0.f, 0.f, 0.f, 0.f};
+            constexpr int MJ = 8;   // items of a thread whose fetches from one piece are in flight together
+            for (int idx0 = tid; idx0 < NIT; idx0 += MJ * blockDim.x) {
+                v4f x[MJ];
+#pragma unroll
+                for (int i = 0; i < MJ; ++i) x[i] = v4f{0.f, 0.f, 0.f, 0.f};
                 for (int w = wfirst; w <= wlast; ++w) {
                     const bool first_piece = ((long)w * sk_total) / G >= t0;
                     const unsigned slot = (2u * (w * gridDim.y + blockIdx.y) + (first_piece ? 0u : 1u)) * SLOT;
-                    x += load_shared4(rs_sk, (slot + (unsigned)idx * 4u) * 4u);
+                    v4f y[MJ];
+#pragma unroll
+                    for (int i = 0; i < MJ; ++i) {
+                        const int idx = idx0 + i * (int)blockDim.x;
+                        y[i] = load_shared4(rs_sk, idx < NIT ? (slot + (unsigned)idx * 4u) * 4u : DMA_OOB);
+                    }
+#pragma unroll
+                    for (int i = 0; i < MJ; ++i) x[i] += y[i];
                 }
-                if (p0 + row < N1) store4<CVEC>(a.d1 + ((size_t)b * N1 + p0 + row) * C, cb0 + c, C, x, a.accumulate != 0);
+#pragma unroll
+                for (int i = 0; i < MJ; ++i) {
+                    const int idx = idx0 + i * (int)blockDim.x;
+                    const int row = idx / (CB / 4), c = (idx - row * (CB / 4)) * 4;
+                    if (idx < NIT && p0 + row < N1)
+                        store4<CVEC>(a.d1 + ((size_t)b * N1 + p0 + row) * C, cb0 + c, C, x[i], a.accumulate != 0);
+                }
             }
         }
     }
