@@ -29,6 +29,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <algorithm>
 #include <atomic>
 #include <mutex>
 #include <string>
@@ -1388,6 +1389,11 @@ struct BwdArgs {
     int vpasses;                     // df1: passes of 256 columns
     int tiles_per_batch;             // df1: p tiles per batch
     int nsplit, tiles_per_split;     // df2: split of the p range
+    // df2, uneven split: the last split of every block of output rows is a short one (what tiles_per_split leaves
+    // over) and is dealt out behind all the long ones, so that the short ones share the compute units the long ones
+    // leave free.  Per XCD x (workgroup ids x, x + 8, ...): long units xl[x] .. xl[x+1], then short ones from xs[x].
+    int uneven, q_units;             // q_units = blocks of output rows (B x row groups x column chunks)
+    int xl[9], xs[9];
     int accumulate;                  // add to the destination instead of overwriting
     int xcd_order;                   // map workgroup ids so that each XCD gets a contiguous range
     // d_f1 dealt out in pieces of tiles, as the forward sweeps are (FwdArgs::sk_*): a piece leaves its partial
@@ -2027,11 +2033,30 @@ __global__ void __launch_bounds__(64 * NWV) df2_tiled_kernel(const BwdArgs a, in
     const int tid = threadIdx.x, lane = tid & 63, pl = lane & 31, h = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int N1 = a.N1, H2 = a.H2, W2 = a.W2, C = a.C;
-    int task = a.xcd_order ? xcd_contiguous(blockIdx.x, gridDim.x) : (int)blockIdx.x;
-    const int vc = task % nvc; task /= nvc;
-    const int ug = task % nug; task /= nug;
-    const int split = task % a.nsplit;
-    const int b = task / a.nsplit;
+    int vc, ug, split, b;
+    if (a.uneven) {
+        int q;
+        const int hw = blockIdx.x, nlong = a.q_units * (a.nsplit - 1);
+        if (a.xcd_order) {
+            const int x = hw & 7, slot = hw >> 3, lx = a.xl[x + 1] - a.xl[x];
+            const int unit = slot < lx ? a.xl[x] + slot : nlong + a.xs[x] + slot - lx;
+            split = unit / a.q_units;
+            q = unit - split * a.q_units;
+        } else {
+            split = hw / a.q_units;
+            q = hw - split * a.q_units;
+        }
+        (void)nlong;
+        vc = q % nvc; q /= nvc;
+        ug = q % nug;
+        b = q / nug;
+    } else {
+        int task = a.xcd_order ? xcd_contiguous(blockIdx.x, gridDim.x) : (int)blockIdx.x;
+        vc = task % nvc; task /= nvc;
+        ug = task % nug; task /= nug;
+        split = task % a.nsplit;
+        b = task / a.nsplit;
+    }
     const int cb0 = blockIdx.y * CB;
     const int u_raw = ug * NWV + wave;
     const int u = min(u_raw, H2 - 1);
@@ -3038,6 +3063,8 @@ struct Df2Plan {
     bool tiled;
     int nsplit;
     int rows;
+    int tiles_per_split;   // pixel tiles of a split (the last split takes what is left)
+    bool uneven;           // the last split is a short one, dealt out last (BwdArgs::uneven)
 };
 
 // How d_f2 is computed for these sizes.  The p range is split over workgroups so that the grid fills
@@ -3052,19 +3079,42 @@ Df2Plan df2_plan(const Dims &d, bool both) {
     const int tiles = (int)((n1 + TP - 1) / TP);
     const int nvc = (d.W2 + 31) / 32;
     const int cblocks = (d.C + 255) / 256;
+    pl.uneven = false;
     if (pl.tiled) {
+        // Estimated duration in pixel tiles of the sweep; a workgroup's start-up, the partial result it leaves and
+        // its later addition cost about as much as two tiles.  One workgroup per compute unit at a time.
         const int rows = pl.rows;
         const long base = (long)d.B * ((d.H2 + rows - 1) / rows) * nvc * (d.C <= 128 ? 1 : cblocks);
-        double best = -1.0;
-        pl.nsplit = 1;
+        struct Cand { int ns, tps; bool uneven; double t; };
+        Cand cand[32];
+        int nc = 0;
         for (int ns = 1; ns <= 16 && ns <= tiles; ++ns) {
-            // share of the chip kept busy x share of a workgroup's time spent sweeping (start-up, the partial tile it
-            // leaves and its later addition cost about as much as two pixel tiles of the sweep)
-            const long wgs = base * ns;
-            const double per = (double)tiles / ns;
-            const double eff = (double)wgs / (double)(((wgs + 255) / 256) * 256) * per / (per + 2.0);
-            if (eff > best) { best = eff; pl.nsplit = ns; }
+            const int per = (tiles + ns - 1) / ns, nsa = (tiles + per - 1) / per;   // nsa: splits that get tiles
+            const long wgs = base * nsa;
+            cand[nc++] = {nsa, per, false, (double)((wgs + 255) / 256) * (per + 2.0)};
+            // ns - 1 long splits that fill part of the chip in one round, and a short one whose workgroups follow
+            // one another on the compute units left over: r rounds of them take as long as one long split
+            const long nlong = base * (ns - 1);
+            if (ns >= 2 && cblocks == 1 && nlong < 256) {
+                const long free_cus = 256 - nlong;
+                const long r = (base + free_cus - 1) / free_cus;
+                const long a_len = (r * (tiles + 2) - 2 + (1 + r * (ns - 1)) - 1) / (1 + r * (ns - 1));
+                const long b_len = tiles - (long)(ns - 1) * a_len;
+                if (a_len >= 1 && b_len >= 1 && b_len <= a_len) {
+                    const double t = std::max((double)a_len + 2.0, (double)r * (b_len + 2.0));
+                    cand[nc++] = {ns, (int)a_len, true, t};
+                }
+            }
         }
+        double best = cand[0].t;
+        for (int i = 1; i < nc; ++i) best = std::min(best, cand[i].t);
+        int pick = -1;   // the fewest splits (least scratch) among those within 1.5 % of the best
+        for (int i = 0; i < nc; ++i)
+            if (cand[i].t <= best * 1.015 && (pick < 0 || cand[i].ns < cand[pick].ns || (cand[i].ns == cand[pick].ns && cand[i].t < cand[pick].t)))
+                pick = i;
+        pl.nsplit = cand[pick].ns;
+        pl.tiles_per_split = cand[pick].tps;
+        pl.uneven = cand[pick].uneven;
     } else {
         const long tasks = (long)d.B * d.H2 * nvc;
         long n = (2048 + tasks - 1) / tasks;  // aim at two waves per SIMD on 256 CUs
@@ -3073,6 +3123,7 @@ Df2Plan df2_plan(const Dims &d, bool both) {
         if (n < 1) n = 1;
         pl.nsplit = (int)n;
     }
+    if (!pl.tiled) pl.tiles_per_split = (tiles + pl.nsplit - 1) / pl.nsplit;
     return pl;
 }
 
@@ -3262,7 +3313,8 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s
         const int tiles = a.tiles_per_batch;
         const Df2Plan plan = df2_plan(d, GMODE == GMODE_BOTH);
         a.nsplit = plan.nsplit;
-        a.tiles_per_split = (tiles + a.nsplit - 1) / a.nsplit;
+        a.tiles_per_split = plan.tiles_per_split;
+        a.uneven = 0;
         const int nvc = nvc_all;
         float *d2 = a.d2;
         if (a.nsplit > 1) a.d2 = static_cast<float *>(ws);
@@ -3273,6 +3325,20 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s
             const int rows = plan.rows;
             const int nug = (d.H2 + rows - 1) / rows;
             const dim3 grid(d.B * a.nsplit * nug * nvc, cblocks), block(64 * rows);
+            if (plan.uneven) {   // long units first, short ones last, XCD by XCD
+                a.uneven = 1;
+                a.q_units = d.B * nug * nvc;
+                const int n = (int)grid.x, nlong = a.q_units * (a.nsplit - 1);
+                a.xl[0] = a.xs[0] = 0;
+                for (int x = 0; x < 8; ++x) {
+                    const int cx = (n - x + 7) / 8;                                   // workgroup ids x, x + 8, ...
+                    int lx = (int)((long)(x + 1) * nlong / 8 - (long)x * nlong / 8);
+                    if (lx > cx) lx = cx;
+                    a.xl[x + 1] = a.xl[x] + lx;
+                    a.xs[x + 1] = a.xs[x] + (cx - lx);
+                }
+                if (a.xl[8] != nlong || a.xs[8] != a.q_units) a.uneven = 0, a.tiles_per_split = (tiles + a.nsplit - 1) / a.nsplit;
+            }
             const size_t lds = ((size_t)2 * 32 * 128 * ncb + 2 * NV * 1024 + rows * UBUF * 32 * NUP) * sizeof(float);
 #define SEPCORR_DF2T(NCB, NWV)                                                                     \
     do {                                                                                           \
