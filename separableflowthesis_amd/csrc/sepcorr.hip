@@ -1165,9 +1165,9 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         const int cht = (is_weighted(MODE)) ? a.KT : 2, ch0 = (is_weighted(MODE)) ? a.k0 : 0;
         const int u0 = whole ? 0 : sa * NUG * UR, nu = (whole ? H2 : min(H2, sb * NUG * UR)) - u0;
         // A (pixel, channel) row of nu floats goes to 8, 16, 32 or 64 neighbouring lanes, so that several short rows
-        // share a wave_e; the row index is the same for all lanes of a group (no division by nu anywhere).
+        // share a wave; the row index is the same for all lanes of a group (no division by nu anywhere).
         const int lsh = nu > 32 ? 6 : nu > 16 ? 5 : nu > 8 ? 4 : 3;
-        const int lpr = 1 << lsh, rpi = 64 >> lsh;        // lanes per row, rows per wave_e and trip
+        const int lpr = 1 << lsh, rpi = 64 >> lsh;        // lanes per row, rows per wave and trip
         const int lr = lane_e >> lsh, lu = lane_e & (lpr - 1);
         constexpr int UNR = 4;   // the logits of a batch of elements are fetched before any of them is used
         for (int r0 = wave_e * rpi + lr; r0 < TP * NCHO; r0 += UNR * nW * rpi)
@@ -3098,10 +3098,12 @@ Df2Plan df2_plan(const Dims &d, bool both) {
             if (ns >= 2 && cblocks == 1 && nlong < 256) {
                 const long free_cus = 256 - nlong;
                 const long r = (base + free_cus - 1) / free_cus;
-                const long a_len = (r * (tiles + 2) - 2 + (1 + r * (ns - 1)) - 1) / (1 + r * (ns - 1));
+                // (a workgroup that follows another on a compute unit starts while that one drains: measured, a
+                // short split costs one tile of start-up, not two: 49 + 24 tiles beat 50 + 20 at B=2, 55x128)
+                const long a_len = (r * (tiles + 1) - 1 + (1 + r * (ns - 1)) - 1) / (1 + r * (ns - 1));
                 const long b_len = tiles - (long)(ns - 1) * a_len;
                 if (a_len >= 1 && b_len >= 1 && b_len <= a_len) {
-                    const double t = std::max((double)a_len + 2.0, (double)r * (b_len + 2.0));
+                    const double t = std::max((double)a_len + 2.0, (double)r * (b_len + 1.0) + 1.0);
                     cand[nc++] = {ns, (int)a_len, true, t};
                 }
             }

@@ -64,6 +64,14 @@ def softmax_weights(B, H1, W1, K, L, g):
     return torch.randn(B, H1, W1, K, L, generator=g).softmax(dim=-1).contiguous()
 
 
+def chain_ratio(chain):
+    """Bound for error_report's ratio where the GPU adds `chain` products one after the other in one fp32 MFMA
+    accumulator while the CPU's sgemm adds blocks of a few hundred (taken as 256) and then the block sums: rounding
+    error grows with the square root of the length of a sequential sum, so the ratio of the two errors is expected
+    near sqrt(chain / 256); 25 % on top, and never below the default 2."""
+    return max(2.0, 1.25 * (chain / 256.0) ** 0.5)
+
+
 def error_report(got, ref64, cpu32, name, max_ratio=2.0):
     """Gradient parity made explicit: the error of the GPU result against fp64 next to the error the fp32 CPU
     run of the same full-4D path makes against fp64.
