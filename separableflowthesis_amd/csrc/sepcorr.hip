@@ -3093,11 +3093,14 @@ Df2Plan df2_plan(const Dims &d, bool both) {
             const long wgs = base * nsa;
             cand[nc++] = {nsa, per, false, (double)((wgs + 255) / 256) * (per + 2.0)};
             // ns - 1 long splits that fill part of the chip in one round, and a short one whose workgroups follow
-            // one another on the compute units left over: r rounds of them take as long as one long split
+            // one another on the compute units left over: r rounds of them take as long as one long split.
+            // Workgroups are handed out in the order of their ids to 32 groups of 8 compute units in turn, and a
+            // workgroup waits for a unit of its own group: every group must keep a unit free of long workgroups
+            // (measured at B=4, 48x64: with 240 long ones the short ones ran behind them, not beside them).
             const long nlong = base * (ns - 1);
-            if (ns >= 2 && cblocks == 1 && nlong < 256) {
-                const long free_cus = 256 - nlong;
-                const long r = (base + free_cus - 1) / free_cus;
+            if (ns >= 2 && cblocks == 1 && nlong <= 224) {
+                const long free_per_group = 8 - (nlong + 31) / 32;
+                const long r = ((base + 31) / 32 + free_per_group - 1) / free_per_group;
                 // (a workgroup that follows another on a compute unit starts while that one drains: measured, a
                 // short split costs one tile of start-up, not two: 49 + 24 tiles beat 50 + 20 at B=2, 55x128)
                 const long a_len = (r * (tiles + 1) - 1 + (1 + r * (ns - 1)) - 1) / (1 + r * (ns - 1));
