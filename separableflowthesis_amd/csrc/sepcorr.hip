@@ -317,9 +317,6 @@ struct FwdArgs {
     int sk_steps;      // steps per tile
     float *sk_state;   // [2 * gridDim.x] slots of sk_slot floats: first and last piece of every workgroup
     int *sk_count;     // [tiles] pieces finished, zero at launch
-#ifdef SEPCORR_TIMELINE
-    long long *dbg;
-#endif
     int sk_slot;       // floats per slot
     void *ws;          // host side only: scratch for the split (NULL: whole tiles)
     size_t ws_bytes;
@@ -557,13 +554,6 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     const int nvc = RG ? a.lev[lvl].nvc : nW, NUG = RG ? nW / nvc : 1;
     const int vcw = RG ? wave % nvc : wave, ug = RG ? wave / nvc : 0;
     if (seg_no > 0) __syncthreads();   // the previous piece has finished with LDS
-#ifdef SEPCORR_TIMELINE
-#define TL(i) if (a.dbg && tid == 0) a.dbg[((size_t)wg * 4 + min(seg_no, 3)) * 12 + (i)] = wall_clock64();
-    if (a.dbg && tid == 0) { long long *d = a.dbg + ((size_t)wg * 4 + min(seg_no, 3)) * 12; d[8] = pe - pb; d[9] = whole; d[11] = tile; d[10] = 0; }
-#else
-#define TL(i)
-#endif
-    TL(0)
     const KArgs kp = kernargs_now();
 
     if constexpr (is_weighted(MODE)) {
@@ -627,7 +617,6 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         }
     }
     __syncthreads();
-    TL(1)
 
     const int pix = p0 + pl;           // this lane's image-1 pixel
     const bool pok = pix < N1;
@@ -695,8 +684,6 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
             vidx[r] = 0;
         }
     }
-
-    TL(2)
     const int NJ = a.CP >> 3;
     const int NG = (NJ + GJ - 1) / GJ;
     const int nsteps = sk_total ? sb - sa : ((H2 + UR - 1) / UR + NUG - 1) / NUG;   // steps per wave; rows past H2 are skipped
@@ -1146,8 +1133,6 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         g = g2;
     }
     }
-
-    TL(3)
     // (lane indices for the code behind the sweep are derived afresh from the thread id, so that nothing of them
     // is kept in registers during the sweep)
     int tide = threadIdx.x;
@@ -1204,8 +1189,6 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                     if (p0 + p < N1) ke->lev[lvl].am_u[((size_t)b * N1 + p0 + p) * H2 + u0 + uu] = ostage_am[p * H2 + u0 + uu];
         }
     }
-
-    TL(4)
     // merge the running state of the row groups into group 0, one group at a time, through the LDS
     // region of the f1 tile (no longer needed).  Equal maxima keep the smaller row index.
     if (NUG > 1) {
@@ -1321,7 +1304,6 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         }
     }
     }   // column passes
-    TL(5)
     // (lane indices for the code behind the sweep are derived afresh from the thread id, so that nothing of them
     // is kept in registers during the sweep)
     int tide = threadIdx.x;
@@ -1354,13 +1336,8 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         __syncthreads();
         const bool last = *flag == npieces - 1;
         __syncthreads();
-        TL(6)
-#ifdef SEPCORR_TIMELINE
-        if (a.dbg && tide == 0) a.dbg[((size_t)wg * 4 + min(seg_no, 3)) * 12 + 10] = last;
-#endif
         if (last) merge_pieces<MODE, KC>(ke, lvl, b, p0, wfirst, wlast, (int)t0, tide);
     }
-    TL(7)
     }   // pieces of this workgroup
 }
 
@@ -2783,9 +2760,6 @@ int launch_fwd(FwdArgs a, int B, hipStream_t s) {
     dim3 grid(B * a.tiles_per_batch);
     const dim3 block(64 * nW);
     a.sk_total = 0;
-#ifdef SEPCORR_TIMELINE
-    { const char *e = getenv("SEPCORR_DBG_PTR"); a.dbg = e ? (long long *)strtoull(e, nullptr, 0) : nullptr; }
-#endif
     if (a.ws != nullptr && !a.f2_planes) {
         const FwdSplit f = fwd_split(B * a.tiles_per_batch, a.H2, a.W2, UR * wg.nug, NPART, (nW <= 4 && lds <= 80 * 1024) ? 2 : 1);
         if (f.on && f.bytes <= a.ws_bytes) {
