@@ -3060,9 +3060,10 @@ Df2Plan df2_plan(const Dims &d, bool both) {
         const int rows = pl.rows;
         const long base = (long)d.B * ((d.H2 + rows - 1) / rows) * nvc * (d.C <= 128 ? 1 : cblocks);
         struct Cand { int ns, tps; bool uneven; double t; };
-        Cand cand[32];
+        Cand cand[128];
         int nc = 0;
-        for (int ns = 1; ns <= 16 && ns <= tiles; ++ns) {
+        // (coarse pyramid levels have few blocks of output rows: they fill the chip only with many short splits)
+        for (int ns = 1; ns <= 64 && ns <= tiles; ++ns) {
             const int per = (tiles + ns - 1) / ns, nsa = (tiles + per - 1) / per;   // nsa: splits that get tiles
             const long wgs = base * nsa;
             cand[nc++] = {nsa, per, false, (double)((wgs + 255) / 256) * (per + 2.0)};
