@@ -328,12 +328,16 @@ def module_level(name, torch, dev, reps=5, backward=True):
     torch.manual_seed(1234)
     att = tuple(torch.nn.Conv3d(2, Kp, 3, padding=1).to(dev) for _ in range(2)) if Kp else None
 
+    ups = {}   # upstream gradients: dense tensors, as the layers above the block hand them down
+
     def run(bw):
         with torch.set_grad_enabled(bw):
             blk = AlternateCorrBlockSepflow(fmap1, fmap2, None, 4, 4, support_backward=bw)
             c1, c2 = blk(None, sep=True, attention_weights=att)
             if bw:
-                (c1.sum() + c2.sum()).backward()
+                if not ups:
+                    ups["g"] = [torch.randn(c.shape, generator=g).to(dev) for c in (c1, c2)]
+                torch.autograd.backward([c1, c2], ups["g"])
 
     out = {}
     for key, bw in (("forward", False), ("forward_backward", True)):

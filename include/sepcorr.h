@@ -336,6 +336,22 @@ int sepcorr_assemble_backward_multi(const float *grad_dst, float *const *grad_sr
                                     int nsrc, int B, int H1, int W1, int CT, int L0, void *stream);
 
 /*
+ * The caller's preparation of a feature map for the operator, in one pass: the block keeps fmap1 and fmap2 as
+ * (B,C,H,W), pools fmap2 level after level with F.avg_pool2d(fmap2, 2, stride=2) (core/corr.py:376-382) and hands every
+ * level over as permute(0,2,3,1).contiguous(), fmap1 also divided by sqrt(C) (core/corr.py:419-422).
+ *   fmap     (B,C,H,W)
+ *   levels   host array of nlev device pointers: level l in (B, H >> l, W >> l, C); level 0 = the permuted map
+ *            divided by `divisor` (sqrt(C) for fmap1 with nlev = 1; 1 for fmap2), level l = 2x2 average pooling of
+ *            level l - 1 (sizes round down), fully overwritten
+ * Limits: 1 to 4 levels, none of them empty; B * ceil(C / 32) < 65536.
+ */
+int sepcorr_feature_pyramid_forward(const float *fmap, float *const *levels, int B, int C, int H, int W, int nlev,
+                                    float divisor, void *stream);
+/* Adjoint of the above: grad_fmap (B,C,H,W), fully overwritten, from the gradients of all levels (same layouts). */
+int sepcorr_feature_pyramid_backward(const float *const *grad_levels, float *grad_fmap, int B, int C, int H, int W,
+                                     int nlev, float divisor, void *stream);
+
+/*
  * Windowed bilinear lookup of the correlation pyramid without the 4D volume: what the caller's
  * corr_fn(coords) returns on the stored-volume path (CorrBlock.__call__, core/corr.py:193-248), for the block
  * that never stores the volume (AlternateCorrBlockSepflow.__call__, core/corr.py:479-510, which raises

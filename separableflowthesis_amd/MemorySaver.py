@@ -476,6 +476,39 @@ def attention_backward(sep, weight, a, grad_a, need_bias=True):
     return [d_sep, d_w, d_b]
 
 
+def feature_pyramid_forward(fmap, num_levels, divisor=1.0):
+    """fmap (B,C,H,W) -> [level 0 .. level num_levels-1], level l in (B, H >> l, W >> l, C): the permuted map divided
+    by `divisor`, and its 2x2 average poolings (core/corr.py:376-382, 419-422)."""
+    import ctypes
+    _check("fmap", fmap, ndim=4)
+    B, C, H, W = fmap.shape
+    lib = _lib.load()
+    with torch.cuda.device(fmap.device):
+        out = [torch.empty((B, H >> l, W >> l, C), dtype=fmap.dtype, device=fmap.device) for l in range(num_levels)]
+        ptrs = (ctypes.c_void_p * num_levels)(*[t.data_ptr() for t in out])
+        _lib.check(lib.sepcorr_feature_pyramid_forward(fmap.data_ptr(), ptrs, B, C, H, W, num_levels, float(divisor),
+                                                       _stream()))
+    return out
+
+
+def feature_pyramid_backward(grad_levels, divisor=1.0):
+    """Gradients of the levels (layouts as above) -> gradient of the (B,C,H,W) map."""
+    import ctypes
+    for n, g in enumerate(grad_levels):
+        _check(f"grad_levels[{n}]", g, ndim=4)
+    B, H, W, C = grad_levels[0].shape
+    for l, g in enumerate(grad_levels):
+        if tuple(g.shape) != (B, H >> l, W >> l, C) or g.device != grad_levels[0].device:
+            raise RuntimeError(f"feature pyramid: level {l} must have shape {(B, H >> l, W >> l, C)} on the same device")
+    n = len(grad_levels)
+    lib = _lib.load()
+    with torch.cuda.device(grad_levels[0].device):
+        out = torch.empty((B, C, H, W), dtype=grad_levels[0].dtype, device=grad_levels[0].device)
+        ptrs = (ctypes.c_void_p * n)(*[g.data_ptr() for g in grad_levels])
+        _lib.check(lib.sepcorr_feature_pyramid_backward(ptrs, out.data_ptr(), B, C, H, W, n, float(divisor), _stream()))
+    return out
+
+
 def _src_tables(shapes, ptrs):
     import ctypes
     n = len(shapes)

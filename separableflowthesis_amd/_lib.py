@@ -46,6 +46,8 @@ SIGNATURES = {
     "sepcorr_assemble_backward": (_I, [_P] * 2 + [_I] * 8 + [_P]),
     "sepcorr_assemble_forward_multi": (_I, [_P] * 3 + [_I] + [_P] + [_I] * 5 + [_P]),
     "sepcorr_assemble_backward_multi": (_I, [_P] * 4 + [_I] * 6 + [_P]),
+    "sepcorr_feature_pyramid_forward": (_I, [_P] * 2 + [_I] * 5 + [ctypes.c_float, _P]),
+    "sepcorr_feature_pyramid_backward": (_I, [_P] * 2 + [_I] * 5 + [ctypes.c_float, _P]),
     "sepcorr_lookup_forward": (_I, [_P] * 6 + [_I] * 6 + [ctypes.c_float, _P]),
     "sepcorr_lookup_backward_workspace_bytes": (_SZ, [_P] * 2 + [_I] * 6),
     "sepcorr_lookup_backward": (_I, [_P] * 8 + [_I] * 6 + [ctypes.c_float, _P, _SZ, _P]),

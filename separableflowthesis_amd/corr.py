@@ -12,6 +12,7 @@ import torch.nn.functional as F
 
 from . import MemorySaver
 from .functions import (AssembleVolumeFunction, AttentionLogitsFunction, AttentionWeightsFunction,
+                        FeaturePyramidFunction,
                         ComputeMaxArgmaxAvgFunction, ComputeMaxAvgFunction, ComputeSelfCompressionFromLogitsFunction,
                         ComputeSelfCompressionFunction, Lookup1DFunction, LookupFunction, SeparateLevelFunction,
                         SeparatePyramidFunction)
@@ -45,17 +46,25 @@ class AlternateCorrBlockSepflow:
         # how the fused path runs the pyramid: "all" (every level in the same launches; fastest measured), "first_alone"
         # (level 0 in launches of its own, the levels above it together) or "level" (one autograd node per level)
         self.pyramid_mode = "all"
-        self.pyramid = [fmap2]
-        for _ in range(self.num_levels - 1):
-            fmap2 = F.avg_pool2d(fmap2, 2, stride=2)
-            self.pyramid.append(fmap2)
+        self.fmap2_l0 = fmap2
+        self._pyramid = None
+
+    @property
+    def pyramid(self):
+        """fmap2 and its 2x2 average poolings in (B,C,H,W) (core/corr.py:376-382); built when first asked for: the
+        path that runs all levels in shared launches takes its levels from FeaturePyramidFunction instead."""
+        if self._pyramid is None:
+            fmap2 = self.fmap2_l0
+            self._pyramid = [fmap2]
+            for _ in range(self.num_levels - 1):
+                fmap2 = F.avg_pool2d(fmap2, 2, stride=2)
+                self._pyramid.append(fmap2)
+        return self._pyramid
 
     def separate(self, attention_weights):
         batch, fdim, h1, w1 = self.fmap1_l0.shape
         h2, w2 = h1, w1
-        # the scaled NHWC copy of fmap1 is level independent; made once (the reference redoes it per level)
-        fmap1 = self.fmap1_l0.permute(0, 2, 3, 1).contiguous() / torch.sqrt(torch.tensor(fdim).float())
-        fused = fmap1.is_cuda and max(h2, w2) <= 500 and (
+        fused = self.fmap1_l0.is_cuda and max(h2, w2) <= 500 and (
             attention_weights is None or all(_is_reference_attention(m) for m in attention_weights))
         parts_u, parts_v = [], []      # operator outputs in final channel order (fused path)
         sep_u_lvls, sep_v_lvls = [], []
@@ -68,7 +77,15 @@ class AlternateCorrBlockSepflow:
                 and MemorySaver.set_contraction(-1) == MemorySaver.CONTRACT_FP32):
             # the whole pyramid as one autograd node; the levels above level 0 share launches
             attention1, attention2 = attention_weights
-            levels = [p.permute(0, 2, 3, 1).contiguous() for p in self.pyramid]
+            if (self.fmap1_l0.dtype == torch.float32 and self.fmap2_l0.dtype == torch.float32
+                    and min(h2, w2) >> (self.num_levels - 1) >= 1 and batch * ((fdim + 31) // 32) < 65536):
+                # layout change, scaling and pooling in one pass per feature map
+                (fmap1,) = FeaturePyramidFunction.apply(self.fmap1_l0.contiguous(), 1,
+                                                        float(torch.sqrt(torch.tensor(fdim).float())))
+                levels = FeaturePyramidFunction.apply(self.fmap2_l0.contiguous(), self.num_levels, 1.0)
+            else:
+                fmap1 = self.fmap1_l0.permute(0, 2, 3, 1).contiguous() / torch.sqrt(torch.tensor(fdim).float())
+                levels = [p.permute(0, 2, 3, 1).contiguous() for p in self.pyramid]
             res = SeparatePyramidFunction.apply(fmap1, attention1.weight.contiguous(), attention1.bias,
                                                 attention2.weight.contiguous(), attention2.bias,
                                                 self.pyramid_mode == "first_alone", *levels)
@@ -77,6 +94,8 @@ class AlternateCorrBlockSepflow:
                 parts_u += [maxavg_v, adaptive_corr_v]
                 parts_v += [maxavg_u, adaptive_corr_u]
             return AssembleVolumeFunction.apply(w2, *parts_u), AssembleVolumeFunction.apply(h2, *parts_v)
+        # the scaled NHWC copy of fmap1 is level independent; made once (the reference redoes it per level)
+        fmap1 = self.fmap1_l0.permute(0, 2, 3, 1).contiguous() / torch.sqrt(torch.tensor(fdim).float())
         for i in range(self.num_levels):
             fmap2 = self.pyramid[i].permute(0, 2, 3, 1).contiguous()
             if fused and attention_weights is not None and self.max_avg_function is ComputeMaxArgmaxAvgFunction:

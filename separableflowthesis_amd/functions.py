@@ -290,6 +290,29 @@ class AssembleVolumeFunction(Function):
         return (None,) + tuple(MemorySaver.assemble_backward(grad.contiguous(), ctx.shapes))
 
 
+class FeaturePyramidFunction(Function):
+    """A (B,C,H,W) feature map -> its levels in the operator's layout: apply(fmap, num_levels, divisor) returns
+    num_levels tensors, level l in (B, H >> l, W >> l, C); level 0 = fmap.permute(0,2,3,1) / divisor, level l =
+    F.avg_pool2d of level l - 1 (2, stride 2).
+
+    Not a class of the reference: it stands for the pooling chain of the block's constructor and the
+    permute(0,2,3,1).contiguous() (/ sqrt(fdim)) in front of every operator call (core/corr.py:376-382, 419-422),
+    one kernel per direction instead of 2 to 8 torch kernels.
+    """
+
+    @staticmethod
+    def forward(ctx, fmap, num_levels, divisor):
+        _contig(fmap)
+        ctx.divisor = divisor
+        with torch.cuda.device_of(fmap):
+            return tuple(MemorySaver.feature_pyramid_forward(fmap, num_levels, divisor))
+
+    @staticmethod
+    def backward(ctx, *grads):
+        with torch.cuda.device_of(grads[0]):
+            return MemorySaver.feature_pyramid_backward([g.contiguous() for g in grads], ctx.divisor), None, None
+
+
 class LookupFunction(Function):
     """corr_fn(coords) of the block that never stores the 4D volume: windowed bilinear lookup in every pyramid level.
 
