@@ -36,7 +36,11 @@ __device__ __forceinline__ int lds_at(int l, int y, int x) {
 }
 constexpr int LDS_PIXELS = TY * TX + (TY / 2) * (TX / 2) + (TY / 4) * (TX / 4) + (TY / 8) * (TX / 8);
 
-// grid: (ceil(W/TX), ceil(H/TY), B * ceil(C/TC)), 256 threads
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// grid: (ceil(W/TX), ceil(H/TY), B * ceil(C/TC)), 256 threads.  VEC: W and C are multiples of 4 and all pointers are
+// 16-byte aligned: 16-byte accesses on both sides, all loads of a thread in flight before its first LDS write.
+template <bool VEC>
 __global__ void __launch_bounds__(256) pyramid_forward_kernel(const PyrArgs a) {
     __shared__ float t[LDS_PIXELS * CS];
     const int ncb = (a.C + TC - 1) / TC;
@@ -45,11 +49,31 @@ __global__ void __launch_bounds__(256) pyramid_forward_kernel(const PyrArgs a) {
     const int H = a.H, W = a.W, C = a.C;
     const float inv = 1.f / a.divisor;
     // read: for a channel and a row, TX consecutive floats of the source
-    for (int i = threadIdx.x; i < TC * TY * TX; i += blockDim.x) {
-        const int x = i % TX, y = (i / TX) % TY, c = i / (TX * TY);
-        float v = 0.f;
-        if (c0 + c < C && y0 + y < H && x0 + x < W) v = a.src[(((size_t)b * C + c0 + c) * H + y0 + y) * W + x0 + x];
-        t[lds_at(0, y, x) + c] = v;
+    if constexpr (VEC) {
+        constexpr int N = TC * TY * (TX / 4) / 256;
+        v4f v[N];
+#pragma unroll
+        for (int k = 0; k < N; ++k) {
+            const int i = threadIdx.x + 256 * k;
+            const int x4 = i % (TX / 4), y = (i / (TX / 4)) % TY, c = i / ((TX / 4) * TY);
+            v[k] = v4f{0.f, 0.f, 0.f, 0.f};
+            if (c0 + c < C && y0 + y < H && x0 + 4 * x4 < W)
+                v[k] = *reinterpret_cast<const v4f *>(a.src + (((size_t)b * C + c0 + c) * H + y0 + y) * W + x0 + 4 * x4);
+        }
+#pragma unroll
+        for (int k = 0; k < N; ++k) {
+            const int i = threadIdx.x + 256 * k;
+            const int x4 = i % (TX / 4), y = (i / (TX / 4)) % TY, c = i / ((TX / 4) * TY);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) t[lds_at(0, y, 4 * x4 + e) + c] = v[k][e];
+        }
+    } else {
+        for (int i = threadIdx.x; i < TC * TY * TX; i += blockDim.x) {
+            const int x = i % TX, y = (i / TX) % TY, c = i / (TX * TY);
+            float v = 0.f;
+            if (c0 + c < C && y0 + y < H && x0 + x < W) v = a.src[(((size_t)b * C + c0 + c) * H + y0 + y) * W + x0 + x];
+            t[lds_at(0, y, x) + c] = v;
+        }
     }
     __syncthreads();
     // pooled levels, each from the one below: the four values are added row by row, left to right, and the sum is
@@ -68,6 +92,18 @@ __global__ void __launch_bounds__(256) pyramid_forward_kernel(const PyrArgs a) {
     for (int l = 0; l < a.nlev; ++l) {
         const int ny = TY >> l, nx = TX >> l, Hl = H >> l, Wl = W >> l;
         const int yl0 = y0 >> l, xl0 = x0 >> l;
+        if constexpr (VEC) {
+            for (int i = threadIdx.x; i < ny * nx * (TC / 4); i += blockDim.x) {
+                const int c4 = i % (TC / 4), x = (i / (TC / 4)) % nx, y = i / ((TC / 4) * nx);
+                if (c0 + 4 * c4 < C && yl0 + y < Hl && xl0 + x < Wl) {
+                    const float *p = t + lds_at(l, y, x) + 4 * c4;
+                    v4f v = {p[0], p[1], p[2], p[3]};
+                    if (l == 0) v = v * inv;
+                    *reinterpret_cast<v4f *>(a.lev[l] + (((size_t)b * Hl + yl0 + y) * Wl + xl0 + x) * C + c0 + 4 * c4) = v;
+                }
+            }
+            continue;
+        }
         for (int i = threadIdx.x; i < ny * nx * TC; i += blockDim.x) {
             const int c = i % TC, x = (i / TC) % nx, y = i / (TC * nx);
             if (c0 + c < C && yl0 + y < Hl && xl0 + x < Wl) {
@@ -79,6 +115,7 @@ __global__ void __launch_bounds__(256) pyramid_forward_kernel(const PyrArgs a) {
     }
 }
 
+template <bool VEC>
 __global__ void __launch_bounds__(256) pyramid_backward_kernel(const PyrArgs a) {
     __shared__ float t[LDS_PIXELS * CS];
     const int ncb = (a.C + TC - 1) / TC;
@@ -89,6 +126,19 @@ __global__ void __launch_bounds__(256) pyramid_backward_kernel(const PyrArgs a) 
     for (int l = 0; l < a.nlev; ++l) {
         const int ny = TY >> l, nx = TX >> l, Hl = H >> l, Wl = W >> l;
         const int yl0 = y0 >> l, xl0 = x0 >> l;
+        if constexpr (VEC) {
+            for (int i = threadIdx.x; i < ny * nx * (TC / 4); i += blockDim.x) {
+                const int c4 = i % (TC / 4), x = (i / (TC / 4)) % nx, y = i / ((TC / 4) * nx);
+                v4f v = {0.f, 0.f, 0.f, 0.f};
+                if (c0 + 4 * c4 < C && yl0 + y < Hl && xl0 + x < Wl)
+                    v = *reinterpret_cast<const v4f *>(a.glev[l] + (((size_t)b * Hl + yl0 + y) * Wl + xl0 + x) * C + c0 + 4 * c4);
+                if (l == 0) v = v * inv;
+                float *p = t + lds_at(l, y, x) + 4 * c4;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) p[e] = v[e];
+            }
+            continue;
+        }
         for (int i = threadIdx.x; i < ny * nx * TC; i += blockDim.x) {
             const int c = i % TC, x = (i / TC) % nx, y = i / (TC * nx);
             float v = 0.f;
@@ -109,6 +159,18 @@ __global__ void __launch_bounds__(256) pyramid_backward_kernel(const PyrArgs a) 
         }
         __syncthreads();
     }
+    if constexpr (VEC) {
+        for (int i = threadIdx.x; i < TC * TY * (TX / 4); i += blockDim.x) {
+            const int x4 = i % (TX / 4), y = (i / (TX / 4)) % TY, c = i / ((TX / 4) * TY);
+            if (c0 + c < C && y0 + y < H && x0 + 4 * x4 < W) {
+                v4f v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = t[lds_at(0, y, 4 * x4 + e) + c];
+                *reinterpret_cast<v4f *>(a.dst + (((size_t)b * C + c0 + c) * H + y0 + y) * W + x0 + 4 * x4) = v;
+            }
+        }
+        return;
+    }
     for (int i = threadIdx.x; i < TC * TY * TX; i += blockDim.x) {
         const int x = i % TX, y = (i / TX) % TY, c = i / (TX * TY);
         if (c0 + c < C && y0 + y < H && x0 + x < W)
@@ -127,8 +189,16 @@ int run(bool backward, PyrArgs a, void *stream) {
     if (nz > 65535) return bad("sepcorr: feature pyramid: B * C / 32 must stay below 65536");
     const dim3 grid((a.W + TX - 1) / TX, (a.H + TY - 1) / TY, (unsigned)nz);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (backward) hipLaunchKernelGGL(pyramid_backward_kernel, grid, dim3(256), 0, s, a);
-    else hipLaunchKernelGGL(pyramid_forward_kernel, grid, dim3(256), 0, s, a);
+    uintptr_t align = reinterpret_cast<uintptr_t>(a.src) | reinterpret_cast<uintptr_t>(a.dst);
+    for (int l = 0; l < a.nlev; ++l) align |= reinterpret_cast<uintptr_t>(a.lev[l]) | reinterpret_cast<uintptr_t>(a.glev[l]);
+    const bool vec = a.W % 4 == 0 && a.C % 4 == 0 && align % 16 == 0;
+    if (backward) {
+        if (vec) hipLaunchKernelGGL(pyramid_backward_kernel<true>, grid, dim3(256), 0, s, a);
+        else hipLaunchKernelGGL(pyramid_backward_kernel<false>, grid, dim3(256), 0, s, a);
+    } else {
+        if (vec) hipLaunchKernelGGL(pyramid_forward_kernel<true>, grid, dim3(256), 0, s, a);
+        else hipLaunchKernelGGL(pyramid_forward_kernel<false>, grid, dim3(256), 0, s, a);
+    }
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         char msg[160];
