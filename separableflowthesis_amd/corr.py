@@ -152,8 +152,15 @@ class AlternateCorrBlockSepflow:
         """
         if self._lookup_inputs is None:
             # NHWC copies are made once per block and shared by all flow iterations (the draft redoes them per call)
-            f1 = self.fmap1_l0.permute(0, 2, 3, 1).contiguous().float()
-            self._lookup_inputs = (f1, [p.permute(0, 2, 3, 1).contiguous().float() for p in self.pyramid])
+            b, c, h, w = self.fmap1_l0.shape
+            if (self.fmap1_l0.is_cuda and self.fmap1_l0.dtype == torch.float32 and self.fmap2_l0.dtype == torch.float32
+                    and 1 <= self.num_levels <= 4 and min(h, w) >> (self.num_levels - 1) >= 1
+                    and b * ((c + 31) // 32) < 65536):
+                (f1,) = FeaturePyramidFunction.apply(self.fmap1_l0.contiguous(), 1, 1.0)
+                self._lookup_inputs = (f1, list(FeaturePyramidFunction.apply(self.fmap2_l0.contiguous(), self.num_levels, 1.0)))
+            else:
+                f1 = self.fmap1_l0.permute(0, 2, 3, 1).contiguous().float()
+                self._lookup_inputs = (f1, [p.permute(0, 2, 3, 1).contiguous().float() for p in self.pyramid])
         f1, f2s = self._lookup_inputs
         scale = 1.0 / float(torch.sqrt(torch.tensor(f1.shape[3]).float()))
         return LookupFunction.apply(coords.detach().contiguous().float(), self.radius, scale, f1, *f2s)
