@@ -2676,6 +2676,24 @@ __global__ void __launch_bounds__(256) row_dot_kernel(const float *__restrict__ 
     sum = wave_sum64(sum);
     if (lane == 0) dot[row] = sum;
 }
+// The same for up to 8 pairs of tensors with the same number of rows (the two outputs of every pyramid level) in one
+// launch: blockIdx.y picks the pair.
+struct RowDotJobs {
+    const float *x[8], *y[8];
+    float *dot[8];
+    int L[8];
+};
+__global__ void __launch_bounds__(256) row_dot_multi_kernel(const RowDotJobs j, long nrows) {
+    const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63, job = blockIdx.y;
+    if (row >= nrows) return;
+    const int L = j.L[job];
+    const float *x = j.x[job] + row * L, *y = j.y[job] + row * L;
+    float sum = 0.f;
+    for (int l = lane; l < L; l += 64) sum += x[l] * y[l];
+    sum = wave_sum64(sum);
+    if (lane == 0) j.dot[job][row] = sum;
+}
 // a[row,l] = exp(z[row,l] - max) / sum
 __global__ void __launch_bounds__(256) softmax_apply_kernel(const float *__restrict__ z, const float *__restrict__ st, float *__restrict__ a,
                                                             long nrows, int L) {
@@ -3992,20 +4010,22 @@ int sepcorr_compression_backward_from_logits_levels(const float *f1, const float
     memset(lev, 0, sizeof(lev));
     {
         ProfScope ps("row_dots", s);
-        const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+        RowDotJobs jobs;
+        memset(&jobs, 0, sizeof(jobs));
         for (int l = 0; l < nlev; ++l) {
             if (!f2_levels[l] || !logits_u[l] || !logits_v[l] || !stats_u[l] || !stats_v[l] || !comp_u[l] || !comp_v[l] ||
                 !g_cu[l] || !g_cv[l] || !d_logits_u[l] || !d_logits_v[l])
                 return fail(SEPCORR_EINVAL, "sepcorr: a pointer of level %d is NULL", l);
             float *dot_u = reinterpret_cast<float *>(base + (2 * l) * dot_bytes);       // sum_u g_cu comp_u
             float *dot_v = reinterpret_cast<float *>(base + (2 * l + 1) * dot_bytes);   // sum_v g_cv comp_v
-            hipLaunchKernelGGL(row_dot_kernel, grid, block, 0, s, g_cu[l], comp_u[l], dot_u, (long)rows, h2[l]);
-            hipLaunchKernelGGL(row_dot_kernel, grid, block, 0, s, g_cv[l], comp_v[l], dot_v, (long)rows, w2[l]);
+            jobs.x[2 * l] = g_cu[l]; jobs.y[2 * l] = comp_u[l]; jobs.dot[2 * l] = dot_u; jobs.L[2 * l] = h2[l];
+            jobs.x[2 * l + 1] = g_cv[l]; jobs.y[2 * l + 1] = comp_v[l]; jobs.dot[2 * l + 1] = dot_v; jobs.L[2 * l + 1] = w2[l];
             lev[l].wv = g_cv[l]; lev[l].wu = g_cu[l];
             lev[l].out_u = d_logits_v[l]; lev[l].out_v = d_logits_u[l];
             lev[l].z_ou = logits_v[l]; lev[l].st_ou = stats_v[l]; lev[l].dot_ou = dot_v;
             lev[l].z_ov = logits_u[l]; lev[l].st_ov = stats_u[l]; lev[l].dot_ov = dot_u;
         }
+        hipLaunchKernelGGL(row_dot_multi_kernel, dim3((unsigned)((rows + 3) / 4), 2 * nlev), dim3(256), 0, s, jobs, (long)rows);
         if (int rc = check_launch("row dot products")) return rc;
     }
     return soft_levels(f1, f2_levels, h2, w2, nlev, lev, 1, B, H1, W1, C, K, workspace, sweep, s);
