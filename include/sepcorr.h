@@ -295,6 +295,22 @@ int sepcorr_attention_logits_backward(const float *sep, const float *weight, con
                                       int B, int H1, int W1, int L, int K,
                                       void *workspace, size_t workspace_bytes, void *stream);
 
+/*
+ * The two calls above for several pyramid levels of one attention module in one set of launches (the module is
+ * applied to the max/avg volume of every level, core/corr.py:416-446): host arrays of nlev (1 to 4) device pointers
+ * and row lengths L[l]; weight, bias, B, H1, W1, K are shared.  The backward call returns d_weight and d_bias summed
+ * over the levels and, when d_sep_init is not NULL, d_sep[l] = d_sep_init[l] + (gradient through the convolution):
+ * the gradient that reaches the max/avg volume directly, added in the same pass.
+ */
+int sepcorr_attention_logits_forward_levels(const float *const *sep, const float *weight, const float *bias,
+                                            float *const *logits, float *const *stats, const int *L, int nlev,
+                                            int B, int H1, int W1, int K, void *stream);
+size_t sepcorr_attention_logits_levels_workspace_bytes(const int *L, int nlev, int B, int H1, int W1, int K);
+int sepcorr_attention_logits_backward_levels(const float *const *sep, const float *weight, const float *const *d_logits,
+                                             const float *const *d_sep_init, float *const *d_sep, float *d_weight,
+                                             float *d_bias, const int *L, int nlev, int B, int H1, int W1, int K,
+                                             void *workspace, size_t workspace_bytes, void *stream);
+
 /* Scratch bytes needed by sepcorr_attention_backward. */
 size_t sepcorr_attention_workspace_bytes(int B, int H1, int W1, int L, int K);
 

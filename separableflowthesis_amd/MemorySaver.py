@@ -313,6 +313,71 @@ def attention_logits_backward(sep, weight, grad_logits, need_bias=True):
     return [d_sep, d_w, d_b]
 
 
+def _att_levels_check(seps, weight, bias):
+    for n, t in enumerate(seps):
+        _check(f"seps[{n}]", t, ndim=5)
+    B, H1, W1, ch, _ = seps[0].shape
+    dev = seps[0].device
+    for n, t in enumerate(seps):
+        if tuple(t.shape[:4]) != (B, H1, W1, 2) or t.device != dev:
+            raise RuntimeError(f"seps[{n}] must have shape ({B},{H1},{W1},2,L) on the same device")
+    if not 1 <= len(seps) <= 4:
+        raise RuntimeError("attention: 1 to 4 levels per call")
+    _check("weight", weight, ndim=5)
+    K = weight.shape[0]
+    _expect("weight", weight, (K, 2, 3, 3, 3), dev)
+    if bias is not None:
+        _expect("bias", bias, (K,), dev)
+    return B, H1, W1, K, dev
+
+
+def attention_logits_forward_levels(seps, weight, bias):
+    """attention_logits_forward for the max/avg volumes of several pyramid levels (same module: same weight and bias)
+    in shared launches -> ([logits per level], [stats per level])."""
+    import ctypes
+    seps = list(seps)
+    B, H1, W1, K, dev = _att_levels_check(seps, weight, bias)
+    n = len(seps)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        zs = [torch.empty((B, H1, W1, K, t.shape[4]), dtype=t.dtype, device=dev) for t in seps]
+        sts = [torch.empty((B, H1, W1, K, 2), dtype=t.dtype, device=dev) for t in seps]
+        P = ctypes.c_void_p * n
+        _lib.check(lib.sepcorr_attention_logits_forward_levels(
+            P(*[t.data_ptr() for t in seps]), weight.data_ptr(), bias.data_ptr() if bias is not None else None,
+            P(*[t.data_ptr() for t in zs]), P(*[t.data_ptr() for t in sts]), (ctypes.c_int * n)(*[t.shape[4] for t in seps]),
+            n, B, H1, W1, K, _stream()))
+    return zs, sts
+
+
+def attention_logits_backward_levels(seps, weight, grad_logits, d_sep_init=None, need_bias=True):
+    """attention_logits_backward for several levels of one module in shared launches -> ([d_sep per level], d_weight,
+    d_bias or None), the weight and bias gradients summed over the levels; d_sep_init (optional, one tensor per level,
+    shaped like seps) is added to the d_sep returned."""
+    import ctypes
+    seps, grad_logits = list(seps), list(grad_logits)
+    B, H1, W1, K, dev = _att_levels_check(seps, weight, None)
+    n = len(seps)
+    for l in range(n):
+        _expect(f"grad_logits[{l}]", grad_logits[l], (B, H1, W1, K, seps[l].shape[4]), dev)
+        if d_sep_init is not None:
+            _expect(f"d_sep_init[{l}]", d_sep_init[l], tuple(seps[l].shape), dev)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        d_seps = [torch.empty_like(t) for t in seps]
+        d_w = torch.empty_like(weight)
+        d_b = torch.empty(K, dtype=weight.dtype, device=dev) if need_bias else None
+        Ls = (ctypes.c_int * n)(*[t.shape[4] for t in seps])
+        nws = lib.sepcorr_attention_logits_levels_workspace_bytes(Ls, n, B, H1, W1, K)
+        ws = torch.empty(max(nws, 1), dtype=torch.uint8, device=dev)
+        P = ctypes.c_void_p * n
+        _lib.check(lib.sepcorr_attention_logits_backward_levels(
+            P(*[t.data_ptr() for t in seps]), weight.data_ptr(), P(*[t.data_ptr() for t in grad_logits]),
+            P(*[t.data_ptr() for t in d_sep_init]) if d_sep_init is not None else None, P(*[t.data_ptr() for t in d_seps]),
+            d_w.data_ptr(), d_b.data_ptr() if need_bias else None, Ls, n, B, H1, W1, K, ws.data_ptr(), nws, _stream()))
+    return d_seps, d_w, d_b
+
+
 # --- several pyramid levels per call (the caller's loop over levels, core/corr.py:416-457)
 
 def _levels_setup(f1, f2_levels, K):

@@ -39,6 +39,9 @@ SIGNATURES = {
     "sepcorr_attention_logits_forward": (_I, [_P] * 5 + [_I] * 5 + [_P]),
     "sepcorr_attention_logits_workspace_bytes": (_SZ, [_I] * 5),
     "sepcorr_attention_logits_backward": (_I, [_P] * 6 + [_I] * 5 + [_P, _SZ, _P]),
+    "sepcorr_attention_logits_forward_levels": (_I, [_P] * 6 + [_I] * 5 + [_P]),
+    "sepcorr_attention_logits_levels_workspace_bytes": (_SZ, [_P] + [_I] * 5),
+    "sepcorr_attention_logits_backward_levels": (_I, [_P] * 8 + [_I] * 5 + [_P, _SZ, _P]),
     "sepcorr_attention_forward": (_I, [_P] * 4 + [_I] * 5 + [_P]),
     "sepcorr_attention_workspace_bytes": (_SZ, [_I] * 5),
     "sepcorr_attention_backward": (_I, [_P] * 7 + [_I] * 5 + [_P, _SZ, _P]),

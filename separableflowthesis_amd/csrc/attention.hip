@@ -54,14 +54,32 @@ struct AttArgs {
     int B, H1, W1, L, K;
     float *stats;      // forward, optional: (max, sum of exp) of every row of logits, (B,H1,W1,K,2)
     int logits_only;   // forward: store the logits themselves instead of their softmax
+    const float *init; // conv backward, optional: added to d_sep (a gradient that reaches sep by another path)
 };
+
+// Up to MAXJOBS calls of the same kind (the pyramid levels of one attention module) in one launch: workgroups
+// [first[j], first[j + 1]) of the grid's x range work on job[j].
+constexpr int MAXJOBS = 4;
+struct AttJobs {
+    AttArgs job[MAXJOBS];
+    int first[MAXJOBS + 1];
+    int njobs;
+};
+// the job of this workgroup; bx = its index within the job
+#define ATT_JOB(m)                                                   \
+    int bx = blockIdx.x, jobno = 0;                                  \
+    while (jobno + 1 < (m).njobs && bx >= (m).first[jobno + 1]) ++jobno; \
+    bx -= (m).first[jobno];                                          \
+    const AttArgs &a = (m).job[jobno]
+
 
 // Forward.  NCH = ceil(L / 64) chunks per row.  A lane first gathers the 54 inputs of each of its positions (9
 // neighbouring pixels x 2 channels x 3 shifts along L, zero outside the volume) into registers, then runs the K
 // filters over them with the weights read from LDS four at a time: 54 FMAs per position and filter, no load in
 // the filter loop.
 template <int NCH>
-__global__ void __launch_bounds__(64 * WPB) att_forward_kernel(const AttArgs a) {
+__global__ void __launch_bounds__(64 * WPB) att_forward_kernel(const AttJobs m) {
+    ATT_JOB(m);
     __shared__ __attribute__((aligned(16))) float ws[MAXK * 56 + MAXK];   // [k][56]: 54 weights (c, dl, di, dj) + 2 pad
     const int K = a.K, L = a.L, H1 = a.H1, W1 = a.W1;
     for (int t = threadIdx.x; t < K * 54; t += blockDim.x) ws[(t / 54) * 56 + t % 54] = a.weight[t];
@@ -70,7 +88,7 @@ __global__ void __launch_bounds__(64 * WPB) att_forward_kernel(const AttArgs a) 
     // rows of up to 32 (16) entries: 2 (4) pixels per wave, a group of lw lanes each
     const int lw = NCH == 1 ? lanes_per_pixel(L) : 64;
     const int lane = threadIdx.x & (lw - 1), wave = threadIdx.x >> 6, sub = (threadIdx.x & 63) / lw;
-    const long pix = ((long)blockIdx.x * WPB + wave) * (64 / lw) + sub;       // flattened (b,i,j)
+    const long pix = ((long)bx * WPB + wave) * (64 / lw) + sub;       // flattened (b,i,j)
     const long npix = (long)a.B * H1 * W1;
     if (pix >= npix) return;   // whole groups leave: the reductions below stay inside a group
     const int j = (int)(pix % W1), i = (int)((pix / W1) % H1);
@@ -135,14 +153,15 @@ __global__ void __launch_bounds__(64 * WPB) att_forward_kernel(const AttArgs a) 
 }
 
 // Forward for long rows: logits go to the output buffer first, then are normalised in place.
-__global__ void __launch_bounds__(64 * WPB) att_forward_long_kernel(const AttArgs a) {
+__global__ void __launch_bounds__(64 * WPB) att_forward_long_kernel(const AttJobs m) {
+    ATT_JOB(m);
     __shared__ float ws[MAXK * 54 + MAXK];
     const int K = a.K, L = a.L, H1 = a.H1, W1 = a.W1;
     for (int t = threadIdx.x; t < K * 54; t += blockDim.x) ws[t] = a.weight[t];
     for (int t = threadIdx.x; t < K; t += blockDim.x) ws[MAXK * 54 + t] = a.bias ? a.bias[t] : 0.f;
     __syncthreads();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const long pix = (long)blockIdx.x * WPB + wave;
+    const long pix = (long)bx * WPB + wave;
     const long npix = (long)a.B * H1 * W1;
     if (pix >= npix) return;
     const int j = (int)(pix % W1), i = (int)((pix / W1) % H1);
@@ -187,11 +206,12 @@ __global__ void __launch_bounds__(64 * WPB) att_forward_long_kernel(const AttArg
 }
 
 // dlogits = a * (grad_a - sum_l a * grad_a), one wave per pixel.
-__global__ void __launch_bounds__(64 * WPB) att_softmax_backward_kernel(const AttArgs a) {
+__global__ void __launch_bounds__(64 * WPB) att_softmax_backward_kernel(const AttJobs m) {
+    ATT_JOB(m);
     const int K = a.K, L = a.L;
     const int lw = lanes_per_pixel(L);
     const int lane = threadIdx.x & (lw - 1), wave = threadIdx.x >> 6, sub = (threadIdx.x & 63) / lw;
-    const long pix = ((long)blockIdx.x * WPB + wave) * (64 / lw) + sub;
+    const long pix = ((long)bx * WPB + wave) * (64 / lw) + sub;
     if (pix >= (long)a.B * a.H1 * a.W1) return;
     for (int k = 0; k < K; ++k) {
         const float *pa = a.a + (pix * K + k) * L, *pg = a.grad_a + (pix * K + k) * L;
@@ -206,14 +226,15 @@ __global__ void __launch_bounds__(64 * WPB) att_softmax_backward_kernel(const At
 // d_sep[(i,j),c,l] = sum_{k,dl,di,dj} w[k][c][dl][di][dj] * dlogits[(i-di+1, j-dj+1), k, l-dl+1]
 // Per filter k a lane gathers the 27 logit gradients it needs (9 neighbouring pixels x 3 shifts, zero outside the
 // volume), then applies the two 27-tap rows of the filter, read from LDS four weights at a time.
-__global__ void __launch_bounds__(64 * WPB) att_input_backward_kernel(const AttArgs a) {
+__global__ void __launch_bounds__(64 * WPB) att_input_backward_kernel(const AttJobs m) {
+    ATT_JOB(m);
     __shared__ __attribute__((aligned(16))) float ws[MAXK * 2 * 28];   // [k][c][28]: 27 weights (dl, di, dj) + 1 pad
     const int K = a.K, L = a.L, H1 = a.H1, W1 = a.W1;
     for (int t = threadIdx.x; t < K * 54; t += blockDim.x) ws[(t / 27) * 28 + t % 27] = a.weight[t];
     __syncthreads();
     const int lw = lanes_per_pixel(L);
     const int lane = threadIdx.x & (lw - 1), wave = threadIdx.x >> 6, sub = (threadIdx.x & 63) / lw;
-    const long pix = ((long)blockIdx.x * WPB + wave) * (64 / lw) + sub;
+    const long pix = ((long)bx * WPB + wave) * (64 / lw) + sub;
     if (pix >= (long)a.B * H1 * W1) return;
     const int j = (int)(pix % W1), i = (int)((pix / W1) % H1);
     for (int l = lane; l < L; l += lw) {
@@ -244,6 +265,10 @@ __global__ void __launch_bounds__(64 * WPB) att_input_backward_kernel(const AttA
                     }
             }
         }
+        if (a.init) {
+            d0 += a.init[(pix * 2 + 0) * L + l];
+            d1 += a.init[(pix * 2 + 1) * L + l];
+        }
         a.out[(pix * 2 + 0) * L + l] = d0;
         a.out[(pix * 2 + 1) * L + l] = d1;
     }
@@ -269,14 +294,15 @@ __device__ __forceinline__ float wave_sum_dpp(float x) {
 // gradients, then updates 27 x 4 accumulators (108 registers: two waves fit a SIMD); these are reduced over lanes
 // and waves in a fixed order and written as partial[x][...].
 constexpr int DW_KC = 4;
-__global__ void __launch_bounds__(256) att_weight_backward_kernel(const AttArgs a) {
+__global__ void __launch_bounds__(256) att_weight_backward_kernel(const AttJobs m) {
+    ATT_JOB(m);
     __shared__ float red[4][27 * DW_KC + DW_KC];
     const int K = a.K, L = a.L, H1 = a.H1, W1 = a.W1;
     const int lw = lanes_per_pixel(L), ppw = 64 / lw;   // short rows: ppw pixels per wave and iteration
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, sub = lane / lw, ll0 = lane & (lw - 1);
     const int c = blockIdx.y & 1, k0 = (blockIdx.y >> 1) * DW_KC;
     const long npix = (long)a.B * H1 * W1;
-    const long p0 = (long)blockIdx.x * DW_PIX;
+    const long p0 = (long)bx * DW_PIX;
     float acc[27][DW_KC], accb[DW_KC];
 #pragma unroll
     for (int t = 0; t < 27; ++t)
@@ -342,7 +368,7 @@ __global__ void __launch_bounds__(256) att_weight_backward_kernel(const AttArgs 
     }
     __syncthreads();
     // partial layout per workgroup x: [K*54 weights in weight order (k, c, dl, di, dj)][K biases]
-    float *dst = a.partial + (long)blockIdx.x * (K * 54 + K);
+    float *dst = a.partial + (long)bx * (K * 54 + K);
     for (int t = threadIdx.x; t < 27 * DW_KC; t += blockDim.x) {
         const int k = t % DW_KC, tap = t / DW_KC;
         if (k0 + k < K) dst[(k0 + k) * 54 + c * 27 + tap] = red[0][t] + red[1][t] + red[2][t] + red[3][t];
@@ -403,6 +429,72 @@ size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 extern "C" {
 
+static unsigned pixel_groups(long npix, int L);
+
+// Input, weight and bias gradients of n jobs (levels) that share the weights: one launch each for the input
+// gradients, the partial weight gradients and their reduction; d_weight / d_bias are the sums over all jobs.
+// jobs[i].dlogits, .sep, .out (d_sep), .init are set by the caller; `partial` holds the partial sums of all jobs.
+static int attention_conv_backward_jobs(const AttArgs *jobs, int n, float *partial, float *d_weight, float *d_bias, void *stream) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int K = jobs[0].K;
+    AttJobs mi = {}, mw = {};
+    unsigned gi = 0, gw = 0;
+    for (int j = 0; j < n; ++j) {
+        const long npix = (long)jobs[j].B * jobs[j].H1 * jobs[j].W1;
+        mi.job[j] = jobs[j];
+        mi.first[j] = (int)gi;
+        gi += pixel_groups(npix, jobs[j].L);
+        mw.job[j] = jobs[j];
+        mw.job[j].partial = partial + (size_t)gw * (K * 54 + K);
+        mw.first[j] = (int)gw;
+        gw += (unsigned)((npix + DW_PIX - 1) / DW_PIX);
+    }
+    mi.first[n] = (int)gi; mw.first[n] = (int)gw;
+    mi.njobs = mw.njobs = n;
+    hipLaunchKernelGGL(att_input_backward_kernel, dim3(gi), dim3(64 * WPB), 0, s, mi);
+    if (int rc = launched("attention input gradient kernel")) return rc;
+    hipLaunchKernelGGL(att_weight_backward_kernel, dim3(gw, 2 * ((K + DW_KC - 1) / DW_KC)), dim3(256), 0, s, mw);
+    if (int rc = launched("attention weight gradient kernel")) return rc;
+    const int nw = K * 54 + K;
+    hipLaunchKernelGGL(att_weight_reduce_kernel, dim3((nw + 3) / 4), dim3(256), 0, s, partial, d_weight, d_bias, (int)gw, K);
+    return launched("attention weight gradient reduction");
+}
+
+// workgroups of a forward / softmax backward / input gradient launch for rows of L entries
+static unsigned pixel_groups(long npix, int L) {
+    const long ppg = (long)WPB * (64 / lanes_per_pixel(L));   // pixels per workgroup
+    return (unsigned)((npix + ppg - 1) / ppg);
+}
+// kernel variant of the forward pass for rows of L entries: 1, 2, 4 chunks of 64, or 0 for the long-row kernel
+static int forward_variant(int L) { return L <= 64 ? 1 : L <= 128 ? 2 : L <= 256 ? 4 : 0; }
+
+// Forward pass of n jobs (levels) that share weight and bias: one launch per kernel variant among them.
+static int attention_forward_jobs(const AttArgs *jobs, int n, void *stream) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    bool done[MAXJOBS] = {};
+    for (int i = 0; i < n; ++i) {
+        if (done[i]) continue;
+        const int var = forward_variant(jobs[i].L);
+        AttJobs m = {};
+        unsigned nwg = 0;
+        for (int j = i; j < n; ++j) {
+            if (done[j] || forward_variant(jobs[j].L) != var) continue;
+            done[j] = true;
+            m.job[m.njobs] = jobs[j];
+            m.first[m.njobs] = (int)nwg;
+            nwg += pixel_groups((long)jobs[j].B * jobs[j].H1 * jobs[j].W1, jobs[j].L);
+            m.first[++m.njobs] = (int)nwg;
+        }
+        const dim3 grid(nwg), block(64 * WPB);
+        if (var == 1) hipLaunchKernelGGL(att_forward_kernel<1>, grid, block, 0, s, m);
+        else if (var == 2) hipLaunchKernelGGL(att_forward_kernel<2>, grid, block, 0, s, m);
+        else if (var == 4) hipLaunchKernelGGL(att_forward_kernel<4>, grid, block, 0, s, m);
+        else hipLaunchKernelGGL(att_forward_long_kernel, grid, block, 0, s, m);
+        if (int rc = launched("attention forward kernel")) return rc;
+    }
+    return 0;
+}
+
 static int attention_forward(const float *sep, const float *weight, const float *bias, float *a, float *stats, int logits_only,
                              int B, int H1, int W1, int L, int K, void *stream) {
     REQ(sep); REQ(weight); REQ(a);
@@ -411,15 +503,23 @@ static int attention_forward(const float *sep, const float *weight, const float 
     args.sep = sep; args.weight = weight; args.bias = bias; args.out = a;
     args.stats = stats; args.logits_only = logits_only;
     args.B = B; args.H1 = H1; args.W1 = W1; args.L = L; args.K = K;
-    const long npix = (long)B * H1 * W1;
-    const long ppg = (long)WPB * (64 / lanes_per_pixel(L));   // pixels per workgroup
-    const dim3 grid((unsigned)((npix + ppg - 1) / ppg)), block(64 * WPB);
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    if (L <= 64) hipLaunchKernelGGL(att_forward_kernel<1>, grid, block, 0, s, args);
-    else if (L <= 128) hipLaunchKernelGGL(att_forward_kernel<2>, grid, block, 0, s, args);
-    else if (L <= 256) hipLaunchKernelGGL(att_forward_kernel<4>, grid, block, 0, s, args);
-    else hipLaunchKernelGGL(att_forward_long_kernel, grid, block, 0, s, args);
-    return launched("attention forward kernel");
+    return attention_forward_jobs(&args, 1, stream);
+}
+
+int sepcorr_attention_logits_forward_levels(const float *const *sep, const float *weight, const float *bias,
+                                            float *const *logits, float *const *stats, const int *L, int nlev, int B, int H1,
+                                            int W1, int K, void *stream) {
+    REQ(sep); REQ(weight); REQ(logits); REQ(L);
+    if (nlev < 1 || nlev > MAXJOBS) return sepcorr_set_error(SEPCORR_EINVAL, "sepcorr: attention: 1 to 4 levels per call");
+    AttArgs jobs[MAXJOBS] = {};
+    for (int l = 0; l < nlev; ++l) {
+        REQ(sep[l]); REQ(logits[l]);
+        if (int rc = check_sizes(B, H1, W1, L[l], K)) return rc;
+        jobs[l].sep = sep[l]; jobs[l].weight = weight; jobs[l].bias = bias; jobs[l].out = logits[l];
+        jobs[l].stats = stats ? stats[l] : nullptr; jobs[l].logits_only = 1;
+        jobs[l].B = B; jobs[l].H1 = H1; jobs[l].W1 = W1; jobs[l].L = L[l]; jobs[l].K = K;
+    }
+    return attention_forward_jobs(jobs, nlev, stream);
 }
 
 int sepcorr_attention_forward(const float *sep, const float *weight, const float *bias, float *a, int B, int H1, int W1, int L,
@@ -457,24 +557,45 @@ int sepcorr_attention_logits_backward(const float *sep, const float *weight, con
                  workspace ? workspace_bytes : (size_t)0);
         return sepcorr_set_error(SEPCORR_EWORKSPACE, msg);
     }
-    const long npix = (long)B * H1 * W1;
-    const int nwg = (int)((npix + DW_PIX - 1) / DW_PIX);
     AttArgs args = {};
     args.sep = sep; args.weight = weight;
     args.dlogits = const_cast<float *>(d_logits);   // read only from here on
-    args.partial = static_cast<float *>(workspace);
     args.B = B; args.H1 = H1; args.W1 = W1; args.L = L; args.K = K;
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    const long ppg = (long)WPB * (64 / lanes_per_pixel(L));
-    const dim3 grid((unsigned)((npix + ppg - 1) / ppg)), block(64 * WPB);
     args.out = d_sep;
-    hipLaunchKernelGGL(att_input_backward_kernel, grid, block, 0, s, args);
-    if (int rc = launched("attention input gradient kernel")) return rc;
-    hipLaunchKernelGGL(att_weight_backward_kernel, dim3(nwg, 2 * ((K + DW_KC - 1) / DW_KC)), dim3(256), 0, s, args);
-    if (int rc = launched("attention weight gradient kernel")) return rc;
-    const int n = K * 54 + K;
-    hipLaunchKernelGGL(att_weight_reduce_kernel, dim3((n + 3) / 4), dim3(256), 0, s, args.partial, d_weight, d_bias, nwg, K);
-    return launched("attention weight gradient reduction");
+    return attention_conv_backward_jobs(&args, 1, static_cast<float *>(workspace), d_weight, d_bias, stream);
+}
+
+size_t sepcorr_attention_logits_levels_workspace_bytes(const int *L, int nlev, int B, int H1, int W1, int K) {
+    if (!L || nlev < 1 || nlev > MAXJOBS) return 0;
+    size_t total = 0;
+    for (int l = 0; l < nlev; ++l) total += sepcorr_attention_logits_workspace_bytes(B, H1, W1, L[l], K);
+    return total;
+}
+
+int sepcorr_attention_logits_backward_levels(const float *const *sep, const float *weight, const float *const *d_logits,
+                                             const float *const *d_sep_init, float *const *d_sep, float *d_weight,
+                                             float *d_bias, const int *L, int nlev, int B, int H1, int W1, int K,
+                                             void *workspace, size_t workspace_bytes, void *stream) {
+    REQ(sep); REQ(weight); REQ(d_logits); REQ(d_sep); REQ(d_weight); REQ(L);
+    if (nlev < 1 || nlev > MAXJOBS) return sepcorr_set_error(SEPCORR_EINVAL, "sepcorr: attention: 1 to 4 levels per call");
+    AttArgs jobs[MAXJOBS] = {};
+    for (int l = 0; l < nlev; ++l) {
+        REQ(sep[l]); REQ(d_logits[l]); REQ(d_sep[l]);
+        if (int rc = check_sizes(B, H1, W1, L[l], K)) return rc;
+        jobs[l].sep = sep[l]; jobs[l].weight = weight;
+        jobs[l].dlogits = const_cast<float *>(d_logits[l]);
+        jobs[l].init = d_sep_init ? d_sep_init[l] : nullptr;
+        jobs[l].out = d_sep[l];
+        jobs[l].B = B; jobs[l].H1 = H1; jobs[l].W1 = W1; jobs[l].L = L[l]; jobs[l].K = K;
+    }
+    const size_t need = sepcorr_attention_logits_levels_workspace_bytes(L, nlev, B, H1, W1, K);
+    if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15)) {
+        char msg[160];
+        snprintf(msg, sizeof(msg), "sepcorr: attention backward needs %zu bytes of 16-byte aligned workspace, got %zu", need,
+                 workspace ? workspace_bytes : (size_t)0);
+        return sepcorr_set_error(SEPCORR_EWORKSPACE, msg);
+    }
+    return attention_conv_backward_jobs(jobs, nlev, static_cast<float *>(workspace), d_weight, d_bias, stream);
 }
 
 int sepcorr_attention_backward(const float *sep, const float *weight, const float *a, const float *grad_a, float *d_sep,
@@ -490,25 +611,22 @@ int sepcorr_attention_backward(const float *sep, const float *weight, const floa
         return sepcorr_set_error(SEPCORR_EWORKSPACE, msg);
     }
     const long npix = (long)B * H1 * W1;
-    const int nwg = (int)((npix + DW_PIX - 1) / DW_PIX);
     AttArgs args = {};
     args.sep = sep; args.weight = weight; args.a = a; args.grad_a = grad_a;
     args.dlogits = static_cast<float *>(workspace);
-    args.partial = reinterpret_cast<float *>(static_cast<char *>(workspace) + align256((size_t)npix * K * L * sizeof(float)));
+    float *partial = reinterpret_cast<float *>(static_cast<char *>(workspace) + align256((size_t)npix * K * L * sizeof(float)));
     args.B = B; args.H1 = H1; args.W1 = W1; args.L = L; args.K = K;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const long ppg = (long)WPB * (64 / lanes_per_pixel(L));   // pixels per workgroup
-    const dim3 grid((unsigned)((npix + ppg - 1) / ppg)), block(64 * WPB);
-    hipLaunchKernelGGL(att_softmax_backward_kernel, grid, block, 0, s, args);
-    if (int rc = launched("attention softmax backward kernel")) return rc;
+    {
+        AttJobs m = {};
+        m.job[0] = args;
+        m.njobs = 1;
+        m.first[1] = (int)pixel_groups(npix, L);
+        hipLaunchKernelGGL(att_softmax_backward_kernel, dim3(m.first[1]), dim3(64 * WPB), 0, s, m);
+        if (int rc = launched("attention softmax backward kernel")) return rc;
+    }
     args.out = d_sep;
-    hipLaunchKernelGGL(att_input_backward_kernel, grid, block, 0, s, args);
-    if (int rc = launched("attention input gradient kernel")) return rc;
-    hipLaunchKernelGGL(att_weight_backward_kernel, dim3(nwg, 2 * ((K + DW_KC - 1) / DW_KC)), dim3(256), 0, s, args);
-    if (int rc = launched("attention weight gradient kernel")) return rc;
-    const int n = K * 54 + K;
-    hipLaunchKernelGGL(att_weight_reduce_kernel, dim3((n + 3) / 4), dim3(256), 0, s, args.partial, d_weight, d_bias, nwg, K);
-    return launched("attention weight gradient reduction");
+    return attention_conv_backward_jobs(&args, 1, partial, d_weight, d_bias, stream);
 }
 
 }  // extern "C"

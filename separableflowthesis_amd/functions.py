@@ -222,10 +222,9 @@ class SeparatePyramidFunction(Function):
             ma = [MemorySaver.max_argmax_avg_forward(f1, lv[0])] if split else []
             ma += MemorySaver.max_argmax_avg_forward_levels(f1, lv[split:])
             out_u, out_v, am_u, am_v = (list(t) for t in zip(*ma))
-            zs_u = [MemorySaver.attention_logits_forward(out_v[l], weight1, bias1) for l in range(n)]
-            zs_v = [MemorySaver.attention_logits_forward(out_u[l], weight2, bias2) for l in range(n)]
-            z_u, st_u = (list(t) for t in zip(*zs_u))
-            z_v, st_v = (list(t) for t in zip(*zs_v))
+            # each attention module on the volumes of all levels in shared launches
+            z_u, st_u = MemorySaver.attention_logits_forward_levels(out_v, weight1, bias1)
+            z_v, st_v = MemorySaver.attention_logits_forward_levels(out_u, weight2, bias2)
             comp = [MemorySaver.compression_forward_from_logits(f1, lv[0], z_u[0], z_v[0], st_u[0], st_v[0])[:2]] if split else []
             comp += MemorySaver.compression_forward_from_logits_levels(f1, lv[split:], z_u[split:], z_v[split:],
                                                                        st_u[split:], st_v[split:])
@@ -256,18 +255,19 @@ class SeparatePyramidFunction(Function):
                                                                        g_cu[0], g_cv[0], need_features=False)[2:])
             dz += MemorySaver.compression_logit_gradients_levels(f1, lv[split:], z_u[split:], z_v[split:], st_u[split:],
                                                                  st_v[split:], cu[split:], cv[split:], g_cu[split:], g_cv[split:])
-            d_f1 = d_w1 = d_b1 = d_w2 = d_b2 = None
+            # both attention modules backwards over all levels in shared launches: weight and bias gradients come out
+            # summed over the levels, the gradients of the max/avg volumes with the upstream ones already added
+            d_out_v, d_w1, d_b1 = MemorySaver.attention_logits_backward_levels(out_v, weight1, [z[0] for z in dz], g_v,
+                                                                               need_bias=ctx.has_bias[0])
+            d_out_u, d_w2, d_b2 = MemorySaver.attention_logits_backward_levels(out_u, weight2, [z[1] for z in dz], g_u,
+                                                                               need_bias=ctx.has_bias[1])
+            d_f1 = None
             d_f2 = []
-            acc = lambda total, x: x if total is None or x is None else total + x
             for l in range(n):
-                d_out_v, w1g, b1g = MemorySaver.attention_logits_backward(out_v[l], weight1, dz[l][0], need_bias=ctx.has_bias[0])
-                d_out_u, w2g, b2g = MemorySaver.attention_logits_backward(out_u[l], weight2, dz[l][1], need_bias=ctx.has_bias[1])
-                d_out_u += g_u[l]
-                d_out_v += g_v[l]
                 a_u = MemorySaver.softmax_from_stats(z_u[l], st_u[l])
                 a_v = MemorySaver.softmax_from_stats(z_v[l], st_v[l])
-                d1, d2 = MemorySaver.fused_backward(f1, lv[l], am_u[l], am_v[l], d_out_u, d_out_v, a_u, a_v, g_cu[l], g_cv[l])
-                d_f1, d_w1, d_b1, d_w2, d_b2 = acc(d_f1, d1), acc(d_w1, w1g), acc(d_b1, b1g), acc(d_w2, w2g), acc(d_b2, b2g)
+                d1, d2 = MemorySaver.fused_backward(f1, lv[l], am_u[l], am_v[l], d_out_u[l], d_out_v[l], a_u, a_v, g_cu[l], g_cv[l])
+                d_f1 = d1 if d_f1 is None else d_f1 + d1
                 d_f2.append(d2)
         return (d_f1, d_w1, d_b1, d_w2, d_b2, None, *d_f2)
 

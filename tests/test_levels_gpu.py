@@ -81,3 +81,52 @@ def test_compression_from_logits_levels(device, case, K):
         assert_close(comp[l][1], rcv, f"level {l} compression_output_v")
         assert_close(grads[l][0], r[0].grad, f"level {l} d_logits_u", scale_atol=True)
         assert_close(grads[l][1], r[1].grad, f"level {l} d_logits_v", scale_atol=True)
+
+
+@pytest.mark.parametrize("B,H1,W1,K,Ls", [
+    (2, 55, 128, 4, (128, 64, 32, 16)),     # attention1 over the four levels of the headline size
+    (2, 55, 128, 4, (55, 27, 13, 6)),       # attention2
+    (1, 9, 21, 2, (70, 7)),                 # rows of more than 64 and of fewer than 16 entries in one call
+    (1, 6, 10, 5, (300, 20, 5)),            # the long-row kernel beside the short ones, K = 5
+])
+def test_attention_modules_over_several_levels(device, B, H1, W1, K, Ls):
+    """One attention module on the max/avg volumes of several levels in shared launches = the single-level calls:
+    logits, statistics and input gradients bit for bit (same kernels, same order of operations), weight and bias
+    gradients as the sum over the levels; the upstream gradient of the volumes is added in the same pass."""
+    from separableflowthesis_amd import MemorySaver as ms
+    g = torch.Generator().manual_seed(sum(Ls) + K)
+    seps = [torch.randn(B, H1, W1, 2, L, generator=g).to(device) for L in Ls]
+    w = (torch.randn(K, 2, 3, 3, 3, generator=g) / 4).to(device)
+    b = torch.randn(K, generator=g).to(device)
+    dzs = [torch.randn(B, H1, W1, K, L, generator=g).to(device) for L in Ls]
+    inits = [torch.randn(B, H1, W1, 2, L, generator=g).to(device) for L in Ls]
+
+    zs, sts = ms.attention_logits_forward_levels(seps, w, b)
+    d_seps, d_w, d_b = ms.attention_logits_backward_levels(seps, w, dzs, inits)
+    d_seps0, d_w0, none_b = ms.attention_logits_backward_levels(seps, w, dzs, None, need_bias=False)
+    assert none_b is None
+    sum_w, sum_b = torch.zeros_like(w, dtype=torch.float64), torch.zeros_like(b, dtype=torch.float64)
+    for l, L in enumerate(Ls):
+        z1, st1 = ms.attention_logits_forward(seps[l], w, b)
+        assert torch.equal(zs[l], z1) and torch.equal(sts[l], st1)
+        ds1, dw1, db1 = ms.attention_logits_backward(seps[l], w, dzs[l])
+        assert torch.equal(d_seps0[l], ds1)
+        assert torch.equal(d_seps[l], ds1 + inits[l])
+        sum_w += dw1.double()
+        sum_b += db1.double()
+    torch.testing.assert_close(d_w.double(), sum_w, rtol=1e-5, atol=1e-5 * float(sum_w.abs().max()))
+    torch.testing.assert_close(d_w0.double(), sum_w, rtol=1e-5, atol=1e-5 * float(sum_w.abs().max()))
+    torch.testing.assert_close(d_b.double(), sum_b, rtol=1e-5, atol=1e-5 * float(sum_b.abs().max()))
+
+
+def test_attention_levels_argument_errors(device):
+    from separableflowthesis_amd import MemorySaver as ms
+    w = torch.randn(2, 2, 3, 3, 3, device=device)
+    seps = [torch.randn(1, 4, 4, 2, 8, device=device) for _ in range(5)]
+    with pytest.raises(RuntimeError):
+        ms.attention_logits_forward_levels(seps, w, None)                      # more than 4 levels
+    with pytest.raises(RuntimeError):
+        ms.attention_logits_forward_levels([seps[0], torch.randn(1, 4, 5, 2, 8, device=device)], w, None)
+    with pytest.raises(RuntimeError):
+        ms.attention_logits_backward_levels(seps[:2], w, [torch.randn(1, 4, 4, 2, 8, device=device)] * 2,
+                                            [torch.randn(1, 4, 4, 2, 9, device=device)] * 2)
