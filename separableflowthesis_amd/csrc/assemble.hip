@@ -99,6 +99,10 @@ __global__ void __launch_bounds__(256) assemble_backward_kernel(const AsmArgs a)
             hi = min(L0 - 1, (int)ceilf((float)(l + 1) * inv) + 1);
         }
         float s = 0.f;
+        if (Li == L0) {   // the finest level: the interpolation is the identity (scale 1, every weight 1 or 0)
+            gsrc[((((size_t)b * H1 + i) * W1 + j0 + jj) * nch + c) * Li + l] = tile[l * GS + jj];
+            continue;
+        }
         for (int l0 = lo; l0 <= hi; ++l0) {
             int x0, x1; float lam;
             src_pos(l0, scale, Li, x0, x1, lam);
