@@ -261,6 +261,7 @@ class SeparatePyramidFunction(Function):
                                                                                need_bias=ctx.has_bias[0])
             d_out_u, d_w2, d_b2 = MemorySaver.attention_logits_backward_levels(out_u, weight2, [z[1] for z in dz], g_u,
                                                                                need_bias=ctx.has_bias[1])
+            del dz   # (157 MiB at B=2, 55x128, K=4: not needed by the feature-gradient kernels below)
             d_f1 = None
             d_f2 = []
             for l in range(n):
