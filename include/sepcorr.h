@@ -80,6 +80,25 @@ int sepcorr_profile_collect(char *names, size_t names_cap, float *ms, int cap);
 int sepcorr_set_contraction(int mode);
 
 /*
+ * How sepcorr_max_argmax_avg_backward (and its _static variant) computes the two feature gradients; no counterpart
+ * in the reference, whose kernel visits every (pixel, position) pair.
+ *   SEPCORR_MAXAVG_AUTO    by gathers where the sizes allow and that is the faster way on MI355X: fmap2 has at
+ *                          least 16 positions per line (H2*W2 >= 16*(H2+W2)) and B*N1*N2 >= 2^23, or at least 8
+ *                          positions per line and B*N1 >= 16384; dense otherwise (the initial choice).
+ *   SEPCORR_MAXAVG_DENSE   recompute the correlation tile by tile on fp32 MFMA and multiply by the gradient it
+ *                          implies: 4*N1*N2*C flops per gradient.
+ *   SEPCORR_MAXAVG_GATHER  the gradient of a maximum selects one feature row, the gradient of an average multiplies
+ *                          a line mean: B*N1*(H2+W2) rows of C floats fetched per gradient plus two small products.
+ *                          Needs C % 4 == 0 and C <= 256; other sizes take the dense path silently.
+ * Both give the same gradients up to fp32 rounding, and each is reproducible from run to run.  The setting is
+ * process-wide and read when a call is enqueued.  Returns the previous mode; an unknown mode changes nothing.
+ */
+#define SEPCORR_MAXAVG_AUTO 0
+#define SEPCORR_MAXAVG_DENSE 1
+#define SEPCORR_MAXAVG_GATHER 2
+int sepcorr_set_max_avg_backward(int mode);
+
+/*
  * Replaces MemorySaver.max_avg_forward (MemorySaver_cuda.cpp:10-21 -> max_avg_cuda_forward,
  * MemorySaver_kernel_forward.cu:901-949).
  *   out_u[b,i,j,0,u] = max_v S   out_u[b,i,j,1,u] = (sum_v S) / W2      (B,H1,W1,2,H2)

@@ -721,6 +721,15 @@ def lookup1d_backward(coords, grad_out, shape, coord_channel, clamp_unit, num_le
 
 
 CONTRACT_FP32, CONTRACT_BF16X3 = 0, 1
+MAXAVG_AUTO, MAXAVG_DENSE, MAXAVG_GATHER = 0, 1, 2
+
+
+def set_max_avg_backward(mode):
+    """How max_argmax_avg_backward computes its gradients: MAXAVG_DENSE (recompute the correlation tile by tile),
+    MAXAVG_GATHER (fetch the feature rows the maxima chose and multiply the averages' gradients by line means; needs
+    C % 4 == 0 and C <= 256, dense elsewhere) or MAXAVG_AUTO (whichever is faster for the sizes of the call).
+    Process-wide; returns the previous mode.  Not a function of the reference."""
+    return _lib.load().sepcorr_set_max_avg_backward(int(mode))
 
 
 def set_contraction(mode):

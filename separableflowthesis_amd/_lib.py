@@ -17,6 +17,7 @@ SIGNATURES = {
     "sepcorr_last_error": (ctypes.c_char_p, []),
     "sepcorr_abi_version": (_I, []),
     "sepcorr_set_contraction": (_I, [_I]),
+    "sepcorr_set_max_avg_backward": (_I, [_I]),
     "sepcorr_profile_enable": (_I, [_I]),
     "sepcorr_profile_collect": (_I, [ctypes.c_char_p, _SZ, ctypes.POINTER(ctypes.c_float), _I]),
     "sepcorr_max_avg_forward": (_I, [_P, _P, _P, _P] + [_I] * 6 + [_P, _SZ, _P]),

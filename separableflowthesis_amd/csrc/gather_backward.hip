@@ -1,0 +1,422 @@
+// Backward of the max/avg separation without the correlation volume and without recomputing it: the gradient of a
+// maximum reaches one entry of S per output element, and the gradient of an average reaches a whole line of S with
+// one weight, so both feature gradients are sums of a few feature rows per output element.
+//
+// With S[p,(u,v)] = <f1[p,:], f2[(u,v),:]>, out_u[p,0,u] = max_v S, out_u[p,1,u] = mean_v S, out_v likewise over u
+// (max_avg_forward_kernel and its backward in libs/MemorySaver/MemorySaver_cuda_kernel.cu of the reference define
+// these outputs; the reference's backward visits every (p, u, v)):
+//
+//   d_f1[p,:]     = sum_u g_u[p,0,u] f2[(u, am_u[p,u]),:] + sum_v g_v[p,0,v] f2[(am_v[p,v], v),:]           (gather)
+//                 + sum_u g_u[p,1,u] R[u,:] + sum_v g_v[p,1,v] Q[v,:]                                         (product)
+//                   with R[u,:] = mean_v f2[(u,v),:], Q[v,:] = mean_u f2[(u,v),:]
+//   d_f2[(u,v),:] = sum_{p: am_u[p,u]=v} g_u[p,0,u] f1[p,:] + sum_{p: am_v[p,v]=u} g_v[p,0,v] f1[p,:]           (gather)
+//                 + A_u[u,:] / W2 + A_v[v,:] / H2
+//                   with A_u[u,:] = sum_p g_u[p,1,u] f1[p,:], A_v[v,:] = sum_p g_v[p,1,v] f1[p,:]              (product)
+//
+// The two products are small matrix products (H2 + W2 lines) on fp32 MFMA; the gathers move one feature row per
+// (p, u) and per (p, v) through the caches, B * N1 * (H2 + W2) * C * 4 bytes for each of the two gradients, which is
+// what bounds this path.  d_f2 has no list of the pixels that chose a given (u, v): the wave that owns (u, v) scans
+// column u of the transposed argmax_u and column v of the transposed argmax_v, collects the hits in a small queue in
+// LDS and fetches their rows eight at a time.  Every sum has a fixed order, so results do not change from run to run.
+//
+// An argmax entry outside its range contributes nothing, as in the dense kernels (no column matches it).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "sepcorr.h"
+#include "sepcorr_internal.h"
+
+namespace {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int SCAN = 256;      // pixels per step of the column scan (one 16-byte load per lane)
+constexpr int QCAP = SCAN + 64;
+static_assert(SCAN == 256, "one block of argmax_columns_kernel and one 16-byte load per lane cover a scan step");
+constexpr int NB = 8;          // feature rows in flight per wave
+constexpr int JCHUNK = 256;    // lines of the gradient tile staged in LDS at a time (df1_avg_rows_kernel)
+
+// Row of the 32x32 accumulator held in register r of a lane in half h (lane / 32).
+__device__ __forceinline__ int acc_row(int r, int h) { return (r >> 2) * 8 + h * 4 + (r & 3); }
+
+__device__ __forceinline__ void wave_sync_lds() {
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
+struct GatherArgs {
+    const float *f1, *f2, *g_u, *g_v;
+    const int *am_u, *am_v;
+    float *d1, *d2;
+    int *amT_u, *amT_v;     // [B][H2][N1p], [B][W2][N1p]; pad -1
+    float *lines;           // [B][H2+W2][C]: R then Q
+    float *table;           // [B][H2+W2][C]: A_u / W2 then A_v / H2
+    float *table_part;      // [B][S][H2+W2][C]
+    int B, N1, N1p, H2, W2, C, S;
+};
+
+// amT[b][j][p] = am[b][p][j]; entries beyond N1 are -1 (no hit).  grid (N1p / 256, L, B)
+__global__ void __launch_bounds__(256) argmax_columns_kernel(const int *am, int *amT, int N1, int N1p, int L) {
+    const int p = blockIdx.x * 256 + threadIdx.x, j = blockIdx.y, b = blockIdx.z;
+    amT[((size_t)b * L + j) * N1p + p] = p < N1 ? am[((size_t)b * N1 + p) * L + j] : -1;
+}
+
+// lines[b][j][:]: j < H2: mean_v f2[(j,v),:]; else mean_u f2[(u,j-H2),:].  grid (H2+W2, B); the four waves take every
+// fourth term, lane = 4 channels.
+__global__ void __launch_bounds__(256) fmap2_line_means_kernel(const GatherArgs a) {
+    __shared__ v4f part[4][64];
+    const int j = blockIdx.x, b = blockIdx.y, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int H2 = a.H2, W2 = a.W2, C = a.C;
+    const bool on = 4 * lane < C;
+    const float *f2b = a.f2 + (size_t)b * H2 * W2 * C + 4 * lane;
+    const bool row = j < H2;
+    const int n = row ? W2 : H2;
+    const size_t base = row ? (size_t)j * W2 * C : (size_t)(j - H2) * C, step = row ? (size_t)C : (size_t)W2 * C;
+    v4f s0 = {0.f, 0.f, 0.f, 0.f}, s1 = s0;
+    if (on) {
+        int i = wave;
+        for (; i + 4 < n; i += 8) {
+            s0 += *reinterpret_cast<const v4f *>(f2b + base + i * step);
+            s1 += *reinterpret_cast<const v4f *>(f2b + base + (i + 4) * step);
+        }
+        if (i < n) s0 += *reinterpret_cast<const v4f *>(f2b + base + i * step);
+    }
+    part[wave][lane] = s0 + s1;
+    __syncthreads();
+    if (wave == 0 && on) {
+        const v4f t = ((part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane])) * (1.f / n);
+        *reinterpret_cast<v4f *>(a.lines + ((size_t)b * (H2 + W2) + j) * C + 4 * lane) = t;
+    }
+}
+
+// table_part[b][s][j][c] = sum over the pixels of split s of g_avg[p,j] f1[p,c].  grid (ceil(L/32), S, B); the
+// product has rows j, columns c and runs over pixels two at a time; wave w owns channels [64w, 64w+64).
+__global__ void __launch_bounds__(256) avg_table_partial_kernel(const GatherArgs a) {
+    const int jt = blockIdx.x, s = blockIdx.y, b = blockIdx.z;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
+    const int N1 = a.N1, H2 = a.H2, W2 = a.W2, C = a.C, S = a.S;
+    const int c0 = wave * 64;
+    if (c0 >= C) return;
+    const int L = H2 + W2, j = jt * 32 + l32;
+    int per = (N1 + S - 1) / S;
+    per += per & 1;
+    const int pa = s * per, pb = min(N1, pa + per);
+    const bool jok = j < L;
+    const bool ju = j < H2;
+    const float *gp = ju ? a.g_u + (size_t)b * N1 * 2 * H2 + H2 + j : a.g_v + (size_t)b * N1 * 2 * W2 + W2 + (j - H2);
+    const size_t gs = ju ? 2 * (size_t)H2 : 2 * (size_t)W2;
+    const bool ok0 = c0 + l32 < C, ok1 = c0 + 32 + l32 < C;
+    const float *fp0 = a.f1 + (size_t)b * N1 * C + (ok0 ? c0 + l32 : 0);
+    const float *fp1 = a.f1 + (size_t)b * N1 * C + (ok1 ? c0 + 32 + l32 : 0);
+    v16f acc0, acc1;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { acc0[r] = 0.f; acc1[r] = 0.f; }
+    for (int p0 = pa; p0 < pb; p0 += 8) {
+        float ga[4], x0[4], x1[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int p = p0 + 2 * i + h;
+            const bool ok = p < pb;
+            const int pc = ok ? p : pa;            // pa < N1 whenever the loop runs
+            ga[i] = (ok && jok) ? gp[(size_t)pc * gs] : 0.f;
+            x0[i] = fp0[(size_t)pc * C];
+            x1[i] = fp1[(size_t)pc * C];
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(ga[i], x0[i], acc0, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(ga[i], x1[i], acc1, 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int jj = jt * 32 + acc_row(r, h);
+        if (jj < L) {
+            float *dst = a.table_part + (((size_t)b * S + s) * L + jj) * C + c0 + l32;
+            if (ok0) dst[0] = acc0[r];
+            if (ok1) dst[32] = acc1[r];
+        }
+    }
+}
+
+// table[b][j][:] = (sum over splits, in order) / (W2 for j < H2, H2 otherwise).  grid (H2+W2, B)
+__global__ void __launch_bounds__(256) avg_table_reduce_kernel(const GatherArgs a) {
+    const int j = blockIdx.x, b = blockIdx.y, L = a.H2 + a.W2, C = a.C, S = a.S;
+    const float scale = j < a.H2 ? 1.f / a.W2 : 1.f / a.H2;
+    for (int c = threadIdx.x; c < C; c += 256) {
+        float s = 0.f;
+        for (int i = 0; i < S; ++i) s += a.table_part[(((size_t)b * S + i) * L + j) * C + c];
+        a.table[((size_t)b * L + j) * C + c] = s * scale;
+    }
+}
+
+// d1[p][c] = sum_j g_avg[p,j] lines[j][c]: rows p, columns c, over the H2 + W2 lines two at a time.  grid
+// (ceil(N1/32), B); the tile of gradients goes through LDS, JCHUNK lines at a time.
+__global__ void __launch_bounds__(256) df1_avg_rows_kernel(const GatherArgs a) {
+    __shared__ float gsm[32][JCHUNK + 1];
+    const int p0 = blockIdx.x * 32, b = blockIdx.y;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
+    const int N1 = a.N1, H2 = a.H2, W2 = a.W2, C = a.C, L = H2 + W2;
+    const int c0 = wave * 64;
+    const bool wave_on = c0 < C;
+    const bool ok0 = c0 + l32 < C, ok1 = c0 + 32 + l32 < C;
+    const float *rp0 = a.lines + (size_t)b * L * C + (ok0 ? c0 + l32 : 0);
+    const float *rp1 = a.lines + (size_t)b * L * C + (ok1 ? c0 + 32 + l32 : 0);
+    v16f acc0, acc1;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { acc0[r] = 0.f; acc1[r] = 0.f; }
+    for (int jc = 0; jc < L; jc += JCHUNK) {
+        const int nj = min(JCHUNK, L - jc);
+        if (jc) __syncthreads();
+        for (int i = threadIdx.x; i < 32 * JCHUNK; i += 256) {
+            const int px = i / JCHUNK, jl = i - px * JCHUNK, p = p0 + px, j = jc + jl;
+            float g = 0.f;
+            if (p < N1 && jl < nj)
+                g = j < H2 ? a.g_u[(((size_t)b * N1 + p) * 2 + 1) * H2 + j] : a.g_v[(((size_t)b * N1 + p) * 2 + 1) * W2 + (j - H2)];
+            gsm[px][jl] = g;
+        }
+        __syncthreads();
+        if (wave_on) {
+            for (int j0 = 0; j0 < nj; j0 += 8) {
+                float ga[4], x0[4], x1[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int jl = j0 + 2 * i + h;               // < JCHUNK; entries from nj on are zero
+                    const int jr = jl < nj ? jc + jl : 0;
+                    ga[i] = gsm[l32][jl];
+                    x0[i] = rp0[(size_t)jr * C];
+                    x1[i] = rp1[(size_t)jr * C];
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(ga[i], x0[i], acc0, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(ga[i], x1[i], acc1, 0, 0, 0);
+                }
+            }
+        }
+    }
+    if (!wave_on) return;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int p = p0 + acc_row(r, h);
+        if (p < N1) {
+            float *dst = a.d1 + ((size_t)b * N1 + p) * C + c0 + l32;
+            if (ok0) dst[0] = acc0[r];
+            if (ok1) dst[32] = acc1[r];
+        }
+    }
+}
+
+// d1[p][:] += sum_u g_u[p,0,u] f2[(u, am_u[p,u]),:] + sum_v g_v[p,0,v] f2[(am_v[p,v], v),:].  One wave per pixel,
+// lane = 4 channels; grid (ceil(N1/4), B).  Runs after df1_avg_rows_kernel on the same stream.
+__global__ void __launch_bounds__(256) df1_max_gather_kernel(const GatherArgs a) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int N1 = a.N1, H2 = a.H2, W2 = a.W2, C = a.C;
+    const int p = blockIdx.x * 4 + wave, b = blockIdx.y;
+    if (p >= N1) return;
+    const size_t pp = (size_t)b * N1 + p;
+    const bool on = 4 * lane < C;
+    const float *f2b = a.f2 + (size_t)b * H2 * W2 * C + (on ? 4 * lane : 0);
+    v4f acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] = (v4f){0.f, 0.f, 0.f, 0.f};
+    for (int part = 0; part < 2; ++part) {
+        const int L = part ? W2 : H2, R = part ? H2 : W2;   // R: range of a valid index
+        const int *am = part ? a.am_v + pp * W2 : a.am_u + pp * H2;
+        const float *g = part ? a.g_v + pp * 2 * W2 : a.g_u + pp * 2 * H2;
+        for (int j0 = 0; j0 < L; j0 += 64) {
+            const int j = j0 + lane;
+            const int idx = j < L ? am[j] : -1;
+            const bool ok = (unsigned)idx < (unsigned)R;
+            const float gm = ok ? g[j] : 0.f;
+            const int off = ok ? (part ? idx * W2 + j : j * W2 + idx) * C : 0;   // N2 * C < 2^31 is checked on the host
+            const int n = min(64, L - j0);
+            for (int i0 = 0; i0 < n; i0 += NB) {
+                v4f r[NB];
+                int gi[NB];
+#pragma unroll
+                for (int i = 0; i < NB; ++i) {
+                    const int ii = (i0 + i) & 63;     // lanes beyond n hold offset 0 and gradient 0
+                    const int o = __builtin_amdgcn_readlane(off, ii);
+                    gi[i] = __builtin_amdgcn_readlane(__float_as_int(gm), ii);
+                    r[i] = *reinterpret_cast<const v4f *>(f2b + o);
+                }
+#pragma unroll
+                for (int i = 0; i < NB; ++i) acc[i & 3] += __int_as_float(gi[i]) * r[i];
+            }
+        }
+    }
+    if (on) {
+        v4f *dst = reinterpret_cast<v4f *>(a.d1 + pp * C + 4 * lane);
+        *dst = *dst + ((acc[0] + acc[1]) + (acc[2] + acc[3]));
+    }
+}
+
+// d2[(u,v)][:] = sum over the pixels that chose (u,v) in either direction + the two table lines.  One wave per
+// (u,v), lane = 4 channels; grid (ceil(N2/4), B).
+__global__ void __launch_bounds__(256) df2_gather_kernel(const GatherArgs a) {
+    __shared__ int queue[4][QCAP];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int N1 = a.N1, N1p = a.N1p, H2 = a.H2, W2 = a.W2, C = a.C;
+    const int N2 = H2 * W2;
+    const int q = blockIdx.x * 4 + wave, b = blockIdx.y;
+    if (q >= N2) return;
+    const int u = q / W2, v = q - u * W2;
+    const bool on = 4 * lane < C;
+    const float *f1b = a.f1 + (size_t)b * N1 * C + (on ? 4 * lane : 0);
+    int *qu = queue[wave];
+    v4f acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] = (v4f){0.f, 0.f, 0.f, 0.f};
+    for (int part = 0; part < 2; ++part) {
+        const int *col = part ? a.amT_v + ((size_t)b * W2 + v) * N1p : a.amT_u + ((size_t)b * H2 + u) * N1p;
+        const int tgt = part ? u : v;
+        const float *g = part ? a.g_v + (size_t)b * N1 * 2 * W2 + v : a.g_u + (size_t)b * N1 * 2 * H2 + u;
+        const size_t gs = part ? 2 * (size_t)W2 : 2 * (size_t)H2;
+        int qn = 0;
+        auto drain = [&](int at, int n) {   // n (<= 64) entries of the queue from position at
+            const int pl = lane < n ? qu[at + lane] : 0;
+            const float gl = lane < n ? g[(size_t)pl * gs] : 0.f;
+            for (int i0 = 0; i0 < n; i0 += NB) {
+                v4f r[NB];
+                int gi[NB];
+#pragma unroll
+                for (int i = 0; i < NB; ++i) {
+                    const int ii = (i0 + i) & 63;     // lanes beyond n hold pixel 0 and gradient 0
+                    const int pi = __builtin_amdgcn_readlane(pl, ii);
+                    gi[i] = __builtin_amdgcn_readlane(__float_as_int(gl), ii);
+                    r[i] = *reinterpret_cast<const v4f *>(f1b + (size_t)pi * C);
+                }
+#pragma unroll
+                for (int i = 0; i < NB; ++i) acc[i & 3] += __int_as_float(gi[i]) * r[i];
+            }
+        };
+        v4i nxt = *reinterpret_cast<const v4i *>(col + 4 * lane);
+        for (int p0 = 0; p0 < N1p; p0 += SCAN) {
+            const v4i idx = nxt;
+            if (p0 + SCAN < N1p) nxt = *reinterpret_cast<const v4i *>(col + p0 + SCAN + 4 * lane);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const bool hit = idx[i] == tgt;
+                const unsigned long long mask = __ballot(hit);
+                if (mask) {
+                    const int rank = __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0));
+                    if (hit) qu[qn + rank] = p0 + 4 * lane + i;
+                    qn += __builtin_popcountll(mask);
+                }
+            }
+            if (qn >= 64) {   // qn < 64 before the step, at most 63 + SCAN after it
+                wave_sync_lds();
+                int done = 0;
+                while (qn - done >= 64) {
+                    drain(done, 64);
+                    done += 64;
+                }
+                const int rest = qn - done;
+                const int t = lane < rest ? qu[done + lane] : 0;
+                wave_sync_lds();
+                if (lane < rest) qu[lane] = t;
+                qn = rest;
+            }
+        }
+        wave_sync_lds();
+        if (qn > 0) drain(0, qn);
+        wave_sync_lds();
+    }
+    if (on) {
+        const float *tb = a.table + (size_t)b * (H2 + W2) * C + 4 * lane;
+        v4f r = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+        r += *reinterpret_cast<const v4f *>(tb + (size_t)u * C) + *reinterpret_cast<const v4f *>(tb + (size_t)(H2 + v) * C);
+        *reinterpret_cast<v4f *>(a.d2 + ((size_t)b * N2 + q) * C + 4 * lane) = r;
+    }
+}
+
+size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
+
+int table_splits(int B, int N1, int H2, int W2) {
+    const int jt = (H2 + W2 + 31) / 32;
+    int S = (512 + jt * B - 1) / (jt * B);
+    const int cap = N1 / 64 > 1 ? N1 / 64 : 1;
+    if (S > cap) S = cap;
+    if (S > 64) S = 64;
+    return S < 1 ? 1 : S;
+}
+
+struct Layout {
+    size_t off_amT_u, off_amT_v, off_lines, off_table, off_part, total;
+    int N1p, S;
+};
+Layout layout(int B, int N1, int H2, int W2, int C) {
+    Layout l;
+    l.N1p = (N1 + SCAN - 1) / SCAN * SCAN;
+    l.S = table_splits(B, N1, H2, W2);
+    const size_t L = (size_t)H2 + W2;
+    size_t o = 0;
+    l.off_amT_u = o; o += align256((size_t)B * H2 * l.N1p * 4);
+    l.off_amT_v = o; o += align256((size_t)B * W2 * l.N1p * 4);
+    l.off_lines = o; o += align256((size_t)B * L * C * 4);
+    l.off_table = o; o += align256((size_t)B * L * C * 4);
+    l.off_part = o; o += align256((size_t)B * l.S * L * C * 4);
+    l.total = o;
+    return l;
+}
+
+struct Prof {
+    void *t;
+    Prof(const char *name, hipStream_t s) : t(sepcorr_prof_begin(name, s)) {}
+    ~Prof() { sepcorr_prof_end(t); }
+};
+
+}  // namespace
+
+int sepcorr_gather_backward_eligible(int B, int H1, int W1, int H2, int W2, int C) {
+    const size_t lim = (size_t)1 << 31;
+    return C % 4 == 0 && C <= 256 && B <= 65535 && H2 + W2 <= 65535 && (size_t)H2 * W2 * C < lim && (size_t)H1 * W1 * C < lim &&
+           (size_t)H1 * W1 + SCAN < lim;
+}
+
+size_t sepcorr_gather_backward_bytes(int B, int H1, int W1, int H2, int W2, int C) {
+    return layout(B, H1 * W1, H2, W2, C).total;
+}
+
+int sepcorr_gather_backward(const float *f1, const float *f2, const int32_t *am_u, const int32_t *am_v, const float *g_u,
+                            const float *g_v, float *d_f1, float *d_f2, int B, int H1, int W1, int H2, int W2, int C, void *ws,
+                            void *stream_f1, void *stream_f2) {
+    const Layout l = layout(B, H1 * W1, H2, W2, C);
+    char *w = static_cast<char *>(ws);
+    GatherArgs a;
+    a.f1 = f1; a.f2 = f2; a.g_u = g_u; a.g_v = g_v; a.am_u = am_u; a.am_v = am_v; a.d1 = d_f1; a.d2 = d_f2;
+    a.amT_u = reinterpret_cast<int *>(w + l.off_amT_u);
+    a.amT_v = reinterpret_cast<int *>(w + l.off_amT_v);
+    a.lines = reinterpret_cast<float *>(w + l.off_lines);
+    a.table = reinterpret_cast<float *>(w + l.off_table);
+    a.table_part = reinterpret_cast<float *>(w + l.off_part);
+    a.B = B; a.N1 = H1 * W1; a.N1p = l.N1p; a.H2 = H2; a.W2 = W2; a.C = C; a.S = l.S;
+    const int L = H2 + W2, N1 = a.N1, N2 = H2 * W2;
+    hipStream_t s1 = static_cast<hipStream_t>(stream_f1), s2 = static_cast<hipStream_t>(stream_f2);
+    const dim3 blk(256);
+    {   // d_f1: line means of fmap2, the product with the average gradients, then the rows the maxima chose
+        Prof ps("df1_maxavg_gather", s1);
+        hipLaunchKernelGGL(fmap2_line_means_kernel, dim3(L, B), blk, 0, s1, a);
+        hipLaunchKernelGGL(df1_avg_rows_kernel, dim3((N1 + 31) / 32, B), blk, 0, s1, a);
+        hipLaunchKernelGGL(df1_max_gather_kernel, dim3((N1 + 3) / 4, B), blk, 0, s1, a);
+    }
+    {   // d_f2: transposed argmax, the table of the average gradients, then the scan
+        Prof ps("df2_maxavg_gather", s2);
+        hipLaunchKernelGGL(argmax_columns_kernel, dim3(l.N1p / 256, H2, B), blk, 0, s2, am_u, a.amT_u, N1, l.N1p, H2);
+        hipLaunchKernelGGL(argmax_columns_kernel, dim3(l.N1p / 256, W2, B), blk, 0, s2, am_v, a.amT_v, N1, l.N1p, W2);
+        hipLaunchKernelGGL(avg_table_partial_kernel, dim3((L + 31) / 32, l.S, B), blk, 0, s2, a);
+        hipLaunchKernelGGL(avg_table_reduce_kernel, dim3(L, B), blk, 0, s2, a);
+        hipLaunchKernelGGL(df2_gather_kernel, dim3((N2 + 3) / 4, B), blk, 0, s2, a);
+    }
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        char msg[200];
+        snprintf(msg, sizeof(msg), "sepcorr: max/avg backward (gather): %s", hipGetErrorString(e));
+        return sepcorr_set_error(SEPCORR_ELAUNCH, msg);
+    }
+    return SEPCORR_OK;
+}

@@ -36,6 +36,7 @@
 #include <vector>
 
 #include "sepcorr.h"
+#include "sepcorr_internal.h"
 
 // This file is compiled once per part (see the Makefile) so that its many kernel instantiations build in parallel:
 // part 0 holds the C ABI and the state shared by all parts, every other part holds the explicit instantiations of
@@ -2575,6 +2576,7 @@ extern thread_local bool t_no_alloc;
 extern std::mutex g_prof_mu;
 extern std::vector<ProfRec> g_prof_recs;
 extern std::atomic<int> g_contraction;
+extern std::atomic<int> g_maxavg_backward;
 #if SEPCORR_IN_PART(0)
 std::atomic<bool> g_prof_on{false};
 thread_local bool t_prof_on = false;
@@ -2972,6 +2974,7 @@ int xcd_order_enabled() {
 }  // namespace
 #if SEPCORR_IN_PART(0)
 namespace sepcorr_impl {
+std::atomic<int> g_maxavg_backward{SEPCORR_MAXAVG_AUTO};
 std::atomic<int> g_contraction{[] {
     const char *e = getenv("SEPCORR_BF16X3");
     return e && e[0] == '1' ? SEPCORR_CONTRACT_BF16X3 : SEPCORR_CONTRACT_FP32;
@@ -3191,6 +3194,10 @@ BwdWs bwd_ws(const Dims &d) {
         w.off_uwt = part;
         w.off_df1sk = part + uwt;
         w.own_total = w.total = part + uwt;
+    }
+    if (sepcorr_gather_backward_eligible(d.B, d.H1, d.W1, d.H2, d.W2, d.C)) {   // the max/avg backward may take this path
+        const size_t g = sepcorr_gather_backward_bytes(d.B, d.H1, d.W1, d.H2, d.W2, d.C);
+        if (g > w.total) w.total = g;
     }
     return w;
 }
@@ -3513,12 +3520,47 @@ int check_fwd_workspace(const Dims &d, int K, void *ws, size_t ws_bytes) {
     return SEPCORR_OK;
 }
 
+// Max/avg backward: by gathers of feature rows where the sizes allow and sepcorr_set_max_avg_backward() does not say
+// otherwise, else by the dense recomputing kernels.  The gather path moves B*N1*(H2+W2) rows per gradient, the dense one
+// multiplies N1 x N2 x C twice per gradient: with few positions per line of fmap2, or little work altogether, the dense
+// kernels are as fast.
+bool maxavg_by_gather(const Dims &d) {
+    const int mode = g_maxavg_backward.load(std::memory_order_relaxed);
+    if (mode == SEPCORR_MAXAVG_DENSE) return false;
+    if (!sepcorr_gather_backward_eligible(d.B, d.H1, d.W1, d.H2, d.W2, d.C)) return false;
+    if (mode == SEPCORR_MAXAVG_GATHER) return true;
+    // Measured on MI355X (C = 256): the dense kernels take about 9 us per million (pixel, position) pairs plus 0.04 ms,
+    // the gather path about 0.09 ms of launches plus its row traffic; it wins from 16 positions per line on once the
+    // dense work passes 8 million pairs, and from 8 positions per line on when there are many pixels.
+    const size_t n1 = (size_t)d.B * d.H1 * d.W1, n2 = (size_t)d.H2 * d.W2, lines = (size_t)d.H2 + d.W2;
+    return (n2 >= 16 * lines && n1 * n2 >= ((size_t)8 << 20)) || (n2 >= 8 * lines && n1 >= 16384);
+}
+
+int maxavg_backward(const Dims &d, bool gather, const float *f1, const float *f2, const int32_t *am_u, const int32_t *am_v,
+                    const float *g_u, const float *g_v, float *d_f1, float *d_f2, void *ws, hipStream_t s1, hipStream_t s) {
+    if (gather)
+        return sepcorr_gather_backward(f1, f2, am_u, am_v, g_u, g_v, d_f1, d_f2, d.B, d.H1, d.W1, d.H2, d.W2, d.C, ws, s1, s);
+    BwdArgs a;
+    memset(&a, 0, sizeof(a));
+    a.xcd_order = xcd_order_enabled();
+    a.f1 = f1; a.f2 = f2; a.am_u = am_u; a.am_v = am_v; a.g_u = g_u; a.g_v = g_v;
+    a.d1 = d_f1; a.d2 = d_f2;
+    a.B = d.B; a.N1 = d.H1 * d.W1; a.H2 = d.H2; a.W2 = d.W2; a.C = d.C; a.KT = 1;
+    return launch_bwd<GMODE_MAXAVG, 1>(a, d, ws, s1, s);
+}
+
 #define REQUIRE_PTR(p) \
     if ((p) == nullptr) return fail(SEPCORR_EINVAL, "sepcorr: argument %s is NULL", #p)
 
 }  // namespace
 
 #if SEPCORR_IN_PART(0)
+void *sepcorr_prof_begin(const char *name, void *stream) {
+    return t_prof_on ? new ProfScope(name, static_cast<hipStream_t>(stream)) : nullptr;
+}
+
+void sepcorr_prof_end(void *token) { delete static_cast<ProfScope *>(token); }
+
 void *sepcorr_fork(void *user, void **sa, void **sb) {
     api_enter();
     ForkJoin *fj = new ForkJoin(static_cast<hipStream_t>(user));
@@ -3538,6 +3580,11 @@ extern "C" {
 
 const char *sepcorr_last_error(void) { return g_err; }
 int sepcorr_abi_version(void) { return 2; }
+
+int sepcorr_set_max_avg_backward(int mode) {
+    if (mode != SEPCORR_MAXAVG_AUTO && mode != SEPCORR_MAXAVG_DENSE && mode != SEPCORR_MAXAVG_GATHER) return g_maxavg_backward.load();
+    return g_maxavg_backward.exchange(mode);
+}
 
 int sepcorr_set_contraction(int mode) {
     if (mode != SEPCORR_CONTRACT_FP32 && mode != SEPCORR_CONTRACT_BF16X3) return g_contraction.load();
@@ -3636,14 +3683,10 @@ int sepcorr_max_argmax_avg_backward(const float *f1, const float *f2, const int3
     const Dims d = {B, H1, W1, H2, W2, C};
     if (int rc = check_dims(d, 2)) return rc;
     if (int rc = check_workspace(d, workspace, workspace_bytes)) return rc;
-    BwdArgs a;
-    memset(&a, 0, sizeof(a));
-    a.xcd_order = xcd_order_enabled();
-    a.f1 = f1; a.f2 = f2; a.am_u = argmax_u; a.am_v = argmax_v; a.g_u = grad_u; a.g_v = grad_v;
-    a.d1 = d_f1; a.d2 = d_f2;
-    a.B = B; a.N1 = H1 * W1; a.H2 = H2; a.W2 = W2; a.C = C; a.KT = 1;
-    ForkJoin fj(static_cast<hipStream_t>(stream), !bwd_ws(d).aliased);
-    const int rc = launch_bwd<GMODE_MAXAVG, 1>(a, d, workspace, fj.sa, fj.user);   // d_f1 aside, d_f2 on the caller's stream
+    const bool gather = maxavg_by_gather(d);
+    ForkJoin fj(static_cast<hipStream_t>(stream), gather || !bwd_ws(d).aliased);
+    // d_f1 aside, d_f2 on the caller's stream
+    const int rc = maxavg_backward(d, gather, f1, f2, argmax_u, argmax_v, grad_u, grad_v, d_f1, d_f2, workspace, fj.sa, fj.user);
     const int rj = fj.join();
     return rc ? rc : rj;
 }
@@ -3656,7 +3699,9 @@ int sepcorr_max_argmax_avg_backward_static(const float *f1, const float *f2, con
     REQUIRE_PTR(d_f1); REQUIRE_PTR(d_f2);
     const Dims d = {B, H1, W1, H2, W2, C};
     if (int rc = check_dims(d, 2)) return rc;
-    const size_t need = bwd_ws(d).own_total;   // what this entry point itself uses of the workspace
+    const bool gather = maxavg_by_gather(d);   // the same choice as sepcorr_max_argmax_avg_backward makes
+    // what this entry point itself uses of the workspace
+    const size_t need = gather ? sepcorr_gather_backward_bytes(B, H1, W1, H2, W2, C) : bwd_ws(d).own_total;
     if (need > (size_t)SEPCORR_STATIC_SCRATCH_BYTES)
         return fail(SEPCORR_EWORKSPACE,
                     "sepcorr: these sizes need %zu bytes of scratch, the static array holds %zu: use "
@@ -3668,14 +3713,8 @@ int sepcorr_max_argmax_avg_backward_static(const float *f1, const float *f2, con
         NoAlloc() : prof(t_prof_on) { t_no_alloc = true; t_prof_on = false; }
         ~NoAlloc() { t_no_alloc = false; t_prof_on = prof; }
     } guard;
-    BwdArgs a;
-    memset(&a, 0, sizeof(a));
-    a.xcd_order = xcd_order_enabled();
-    a.f1 = f1; a.f2 = f2; a.am_u = argmax_u; a.am_v = argmax_v; a.g_u = grad_u; a.g_v = grad_v;
-    a.d1 = d_f1; a.d2 = d_f2;
-    a.B = B; a.N1 = H1 * W1; a.H2 = H2; a.W2 = W2; a.C = C; a.KT = 1;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    return launch_bwd<GMODE_MAXAVG, 1>(a, d, ws, s, s);
+    return maxavg_backward(d, gather, f1, f2, argmax_u, argmax_v, grad_u, grad_v, d_f1, d_f2, ws, s, s);
 }
 
 int sepcorr_compression_backward(const float *f1, const float *f2, const float *a_u, const float *a_v, const float *g_cu,

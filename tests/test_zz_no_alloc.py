@@ -3,7 +3,7 @@
 Its scratch memory is an array inside the library's device image instead of a caller-supplied workspace; results must
 equal those of sepcorr_max_argmax_avg_backward (same kernels, same plan: bit for bit) on calls in a row that share
 the array, the second with a smaller input, and stale contents of the array from the first call must not leak.
-Called through the C ABI.
+Both ways of computing the gradients (sepcorr_set_max_avg_backward) are covered.  Called through the C ABI.
 """
 import ctypes
 
@@ -46,10 +46,19 @@ def _both(lib, device, dims, seed):
     return (d1, d2), (r1, r2), need
 
 
-def test_static_scratch_variant_matches_the_workspace_variant(device):
+@pytest.mark.parametrize("mode", [2, 1], ids=["gather", "dense"])   # SEPCORR_MAXAVG_GATHER, SEPCORR_MAXAVG_DENSE
+def test_static_scratch_variant_matches_the_workspace_variant(device, mode):
     lib = _lib.load()
-    # first a size that uses split partial sums and the transposed weights (C == 256), then a smaller input that
-    # reuses the same array, then the first again
+    prev = lib.sepcorr_set_max_avg_backward(mode)
+    try:
+        _calls_in_a_row(lib, device)
+    finally:
+        lib.sepcorr_set_max_avg_backward(prev)
+
+
+def _calls_in_a_row(lib, device):
+    # first a size that uses split partial sums and the transposed weights (dense, C == 256) or 17 positions per line
+    # (gather), then a smaller input that reuses the same array, then the first again
     shapes = [(2, 24, 64, 24, 64, 256), (1, 11, 36, 6, 20, 64), (2, 24, 64, 24, 64, 256), (1, 9, 16, 9, 16, 256)]
     used = []
     for n, dims in enumerate(shapes):
@@ -63,7 +72,7 @@ def test_static_scratch_variant_matches_the_workspace_variant(device):
 
 def test_static_scratch_variant_refuses_sizes_beyond_its_array(device):
     lib = _lib.load()
-    dims = (2, 55, 128, 55, 128, 256)
+    dims = (2, 136, 240, 136, 240, 256)   # 94 MiB of transposed argmax alone
     assert lib.sepcorr_backward_workspace_bytes(*dims) > LIMIT
     one = ctypes.c_void_p(256)   # never dereferenced: the size check comes first
     rc = lib.sepcorr_max_argmax_avg_backward_static(one, one, one, one, one, one, one, one, *dims, None)
