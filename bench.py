@@ -5,7 +5,9 @@ A step is one pass of the hot path over one synthetic batch, called through the 
 input already resident in HBM.  The headline workload is benchmark configuration 4 (B=2, C=256, 55x128,
 K'=4): max/argmax/avg forward, attention-compression forward, compression backward, max/avg backward.
 Prints ONE JSON line.  `value` is algorithmic TFLOP/s: (contraction passes x 2*B*N1*N2*C) / time,
-with passes = 7 for forward+backward with attention; epilogue flops are not counted.  The same line
+with passes = 7 for forward+backward with attention; epilogue flops are not counted.  Where the library runs
+the max/avg backward as gathers instead of its two contractions, the passes actually executed on the matrix
+cores and the timing of the all-dense step are reported beside it (`contraction_passes_executed`, `all_dense`).  The same line
 carries a `configs` table with all five benchmark configurations (ms/step, TFLOP/s, fraction of the
 fp32 MFMA peak, peak HBM allocated, dominant-kernel roofline), the CPU baseline (full-4D torch path on
 the host cores, one thread and all threads) and, as extras, the caller-level measurements.
@@ -295,6 +297,22 @@ class Workload:
         ach = kernels[dom]["tflops"]
         passes = sum(PASSES[o] for o in ops)
         value = passes * Wf / (ms * 1e-3) / 1e12
+        # The max/avg backward may run as gathers of feature rows instead of its two contractions (the library picks
+        # the faster way for the sizes): `value` keeps the algorithmic work of the step, 2*B*N1*N2*C per pass of the
+        # reference's formulation, and the passes that actually ran on the matrix cores are reported next to it,
+        # together with the same step timed with the dense max/avg backward.
+        gathered = any(k.endswith("_gather") for k in kernels)
+        executed = passes - (PASSES["F"] if gathered else 0)
+        dense = None
+        if gathered:
+            prev_mode = self.lib.sepcorr_set_max_avg_backward(1)
+            try:
+                dms = self.time(self.step, steps, warmup)
+            finally:
+                self.lib.sepcorr_set_max_avg_backward(prev_mode)
+            dense = {"ms_per_step": round(dms, 4), "tflops": round(passes * Wf / (dms * 1e-3) / 1e12, 3),
+                     "frac_of_fp32_mfma_peak": round(passes * Wf / (dms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4),
+                     "what": "the same step with sepcorr_set_max_avg_backward(SEPCORR_MAXAVG_DENSE): every pass a contraction"}
         roofline = {"bound": "mfma", "kernel": dom, "achieved": ach, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(ach / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": traffic.get(dom),
                     "algorithmic_bytes": algorithmic_bytes(dom, B, N, H, W, Kp),
@@ -304,6 +322,10 @@ class Workload:
             "ms_per_step": round(ms, 4), "tflops": round(value, 3),
             "frac_of_fp32_mfma_peak": round(value / PEAK_FP32_MFMA_TFLOPS, 4),
             "contraction_passes": passes, "gflop_per_step": round(passes * Wf / 1e9, 2),
+            "contraction_passes_executed": executed,
+            "tflops_executed": round(executed * Wf / (ms * 1e-3) / 1e12, 3),
+            "max_avg_backward": ("gather" if gathered else "dense") if "F" in ops else None,
+            "all_dense": dense,
             "peak_hbm_allocated_mib": round(peak / _MIB, 1),
             "backward_workspace_mib": round(self.workspace_bytes / _MIB, 1),
             "forward_workspace_mib": round(self.forward_workspace_bytes / _MIB, 1),
@@ -474,6 +496,9 @@ def main():
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": head["workload"] + " " + OPS_TEXT,
                    "contraction_passes": head["contraction_passes"], "gflop_per_step": head["gflop_per_step"],
+                   "contraction_passes_executed": head["contraction_passes_executed"],
+                   "tflops_executed": head["tflops_executed"], "max_avg_backward": head["max_avg_backward"],
+                   "all_dense": head["all_dense"],
                    "frac_of_fp32_mfma_peak": head["frac_of_fp32_mfma_peak"],
                    "peak_hbm_allocated_mib": head["peak_hbm_allocated_mib"],
                    "backward_workspace_mib": head["backward_workspace_mib"],

@@ -29,7 +29,9 @@ SHAPES = [
 def planes():
     from separableflowthesis_amd import MemorySaver as ms
     prev = ms.set_contraction(ms.CONTRACT_BF16X3)
+    prev_bwd = ms.set_max_avg_backward(ms.MAXAVG_DENSE)   # the planes belong to the dense kernels; gathers contract nothing
     yield ms
+    ms.set_max_avg_backward(prev_bwd)
     ms.set_contraction(prev)
 
 
