@@ -83,8 +83,8 @@ int sepcorr_set_contraction(int mode);
  * How sepcorr_max_argmax_avg_backward (and its _static variant) computes the two feature gradients; no counterpart
  * in the reference, whose kernel visits every (pixel, position) pair.
  *   SEPCORR_MAXAVG_AUTO    by gathers where the sizes allow and that is the faster way on MI355X: fmap2 has at
- *                          least 16 positions per line (H2*W2 >= 16*(H2+W2)) and B*N1*N2 >= 2^23, or at least 8
- *                          positions per line and B*N1 >= 16384; dense otherwise (the initial choice).
+ *                          least 12 positions per line (H2*W2 >= 12*(H2+W2)), or at least 8 and B*N1 >= 16384;
+ *                          dense otherwise (the initial choice).
  *   SEPCORR_MAXAVG_DENSE   recompute the correlation tile by tile on fp32 MFMA and multiply by the gradient it
  *                          implies: 4*N1*N2*C flops per gradient.
  *   SEPCORR_MAXAVG_GATHER  the gradient of a maximum selects one feature row, the gradient of an average multiplies

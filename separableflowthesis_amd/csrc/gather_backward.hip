@@ -256,8 +256,8 @@ __global__ void __launch_bounds__(256) df1_max_gather_kernel(const GatherArgs a)
 }
 
 // d2[(u,v)][:] = sum over the pixels that chose (u,v) in either direction + the two table lines.  One wave per
-// (u,v), lane = 4 channels; grid (ceil(N2/4), B).  One launch covers the pixels [pa, pb) (multiples of SCAN): the
-// first adds the table lines, the later ones add to what d2 holds.  The launches follow each other on one stream, so
+// (u,v), lane = 4 channels; grid (ceil(N2/4), B).  One launch covers the pixels [pa, pb) (multiples of SCAN): all but
+// the first add to what d2 holds, the last adds the table lines (which may come from another stream in the meantime).  The launches follow each other on one stream, so
 // the rows of fmap1 that the whole grid fetches at any time come from one slice of a few MB, which the L2 caches hold;
 // over all pixels at once they do not (measured at B=2, 55x128: 1.7 GB of L2 misses for 2.6 GB of rows, at 7 TB/s).
 __global__ void __launch_bounds__(256) df2_gather_kernel(const GatherArgs a, int pa, int pb) {
@@ -333,8 +333,8 @@ __global__ void __launch_bounds__(256) df2_gather_kernel(const GatherArgs a, int
         const float *tb = a.table + (size_t)b * (H2 + W2) * C + 4 * lane;
         v4f r = (acc[0] + acc[1]) + (acc[2] + acc[3]);
         v4f *dst = reinterpret_cast<v4f *>(a.d2 + ((size_t)b * N2 + q) * C + 4 * lane);
-        if (pa == 0) r += *reinterpret_cast<const v4f *>(tb + (size_t)u * C) + *reinterpret_cast<const v4f *>(tb + (size_t)(H2 + v) * C);
-        else r += *dst;
+        if (pa != 0) r += *dst;
+        if (pb == N1p) r += *reinterpret_cast<const v4f *>(tb + (size_t)u * C) + *reinterpret_cast<const v4f *>(tb + (size_t)(H2 + v) * C);
         *dst = r;
     }
 }
@@ -389,7 +389,7 @@ size_t sepcorr_gather_backward_bytes(int B, int H1, int W1, int H2, int W2, int 
 
 int sepcorr_gather_backward(const float *f1, const float *f2, const int32_t *am_u, const int32_t *am_v, const float *g_u,
                             const float *g_v, float *d_f1, float *d_f2, int B, int H1, int W1, int H2, int W2, int C, void *ws,
-                            void *stream_f1, void *stream_f2) {
+                            void *stream_f1, void *stream_f2, void *stream_table, void *table_event) {
     const Layout l = layout(B, H1 * W1, H2, W2, C);
     char *w = static_cast<char *>(ws);
     GatherArgs a;
@@ -402,6 +402,9 @@ int sepcorr_gather_backward(const float *f1, const float *f2, const int32_t *am_
     a.B = B; a.N1 = H1 * W1; a.N1p = l.N1p; a.H2 = H2; a.W2 = W2; a.C = C; a.S = l.S;
     const int L = H2 + W2, N1 = a.N1, N2 = H2 * W2;
     hipStream_t s1 = static_cast<hipStream_t>(stream_f1), s2 = static_cast<hipStream_t>(stream_f2);
+    hipStream_t s3 = static_cast<hipStream_t>(stream_table);
+    hipEvent_t ev = static_cast<hipEvent_t>(table_event);
+    if (ev == nullptr) s3 = s2;   // no way to order the table before the last slice across streams
     const dim3 blk(256);
     {   // d_f1: line means of fmap2, the product with the average gradients, then the rows the maxima chose
         Prof ps("df1_maxavg_gather", s1);
@@ -409,19 +412,27 @@ int sepcorr_gather_backward(const float *f1, const float *f2, const int32_t *am_
         hipLaunchKernelGGL(df1_avg_rows_kernel, dim3((N1 + 31) / 32, B), blk, 0, s1, a);
         hipLaunchKernelGGL(df1_max_gather_kernel, dim3((N1 + 3) / 4, B), blk, 0, s1, a);
     }
-    {   // d_f2: transposed argmax, the table of the average gradients, then the scan
+    {   // the table of the average gradients: needed by the last slice of the scan only
+        Prof ps("df2_maxavg_table", s3);
+        hipLaunchKernelGGL(avg_table_partial_kernel, dim3((L + 31) / 32, l.S, B), blk, 0, s3, a);
+        hipLaunchKernelGGL(avg_table_reduce_kernel, dim3(L, B), blk, 0, s3, a);
+    }
+    if (s3 != s2 && hipEventRecord(ev, s3) != hipSuccess) return sepcorr_set_error(SEPCORR_ELAUNCH, "sepcorr: max/avg backward (gather): event record failed");
+    {   // d_f2: transposed argmax, then the scan slice by slice
         Prof ps("df2_maxavg_gather", s2);
         hipLaunchKernelGGL(argmax_columns_kernel, dim3(l.N1p / 256, H2, B), blk, 0, s2, am_u, a.amT_u, N1, l.N1p, H2);
         hipLaunchKernelGGL(argmax_columns_kernel, dim3(l.N1p / 256, W2, B), blk, 0, s2, am_v, a.amT_v, N1, l.N1p, W2);
-        hipLaunchKernelGGL(avg_table_partial_kernel, dim3((L + 31) / 32, l.S, B), blk, 0, s2, a);
-        hipLaunchKernelGGL(avg_table_reduce_kernel, dim3(L, B), blk, 0, s2, a);
         // slices of about 1.75 MB of fmap1 per batch entry (measured best at 3 MB and 7 MB of features per entry)
         const int steps = l.N1p / SCAN;
         int slices = (int)(((size_t)N1 * C * 4 + (7u << 17)) / (7u << 18));
         slices = slices < 1 ? 1 : slices > steps ? steps : slices;
         const int per = (steps + slices - 1) / slices * SCAN;
-        for (int pa = 0; pa < l.N1p; pa += per)
-            hipLaunchKernelGGL(df2_gather_kernel, dim3((N2 + 3) / 4, B), blk, 0, s2, a, pa, pa + per < l.N1p ? pa + per : l.N1p);
+        for (int pa = 0; pa < l.N1p; pa += per) {
+            const bool last = pa + per >= l.N1p;
+            if (last && s3 != s2 && hipStreamWaitEvent(s2, ev, 0) != hipSuccess)
+                return sepcorr_set_error(SEPCORR_ELAUNCH, "sepcorr: max/avg backward (gather): event wait failed");
+            hipLaunchKernelGGL(df2_gather_kernel, dim3((N2 + 3) / 4, B), blk, 0, s2, a, pa, last ? l.N1p : pa + per);
+        }
     }
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) {

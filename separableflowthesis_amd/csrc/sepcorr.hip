@@ -3530,16 +3530,28 @@ bool maxavg_by_gather(const Dims &d) {
     if (!sepcorr_gather_backward_eligible(d.B, d.H1, d.W1, d.H2, d.W2, d.C)) return false;
     if (mode == SEPCORR_MAXAVG_GATHER) return true;
     // Measured on MI355X (C = 256): the dense kernels take about 9 us per million (pixel, position) pairs plus 0.04 ms,
-    // the gather path about 0.09 ms of launches plus its row traffic; it wins from 16 positions per line on once the
-    // dense work passes 8 million pairs, and from 8 positions per line on when there are many pixels.
+    // the gather path its row traffic plus 0.03 ms of launches; it wins from 12 positions per line of fmap2 on, and from
+    // 8 on when there are many pixels (the dense d_f2 then has few tiles and long sums).
     const size_t n1 = (size_t)d.B * d.H1 * d.W1, n2 = (size_t)d.H2 * d.W2, lines = (size_t)d.H2 + d.W2;
-    return (n2 >= 16 * lines && n1 * n2 >= ((size_t)8 << 20)) || (n2 >= 8 * lines && n1 >= 16384);
+    return n2 >= 12 * lines || (n2 >= 8 * lines && n1 >= 16384);
+}
+
+// Whether the gather path's three chains of kernels run beside each other: they fetch single rows of both feature maps
+// through the L2 caches, and once fmap2 of one batch entry is larger than an L2 (4 MB) they evict each other's rows
+// (B=2, 55x128: 0.41 ms beside each other, 0.375 ms one after the other; B=4, 48x64: 0.19 against 0.22 ms); below
+// 300 000 rows per gradient the fork and join cost more than the overlap gains.
+bool gather_overlap(const Dims &d) {
+    const size_t rows = (size_t)d.B * d.H1 * d.W1 * ((size_t)d.H2 + d.W2);
+    return rows >= 300000 && (size_t)d.H2 * d.W2 * d.C * 4 <= ((size_t)4 << 20);
 }
 
 int maxavg_backward(const Dims &d, bool gather, const float *f1, const float *f2, const int32_t *am_u, const int32_t *am_v,
-                    const float *g_u, const float *g_v, float *d_f1, float *d_f2, void *ws, hipStream_t s1, hipStream_t s) {
+                    const float *g_u, const float *g_v, float *d_f1, float *d_f2, void *ws, hipStream_t s1, hipStream_t s,
+                    hipStream_t s2 = nullptr, hipEvent_t s2_done = nullptr) {
+    // s2 with s2_done: a third stream for work that s waits for through that event (the gather path's table)
     if (gather)
-        return sepcorr_gather_backward(f1, f2, am_u, am_v, g_u, g_v, d_f1, d_f2, d.B, d.H1, d.W1, d.H2, d.W2, d.C, ws, s1, s);
+        return sepcorr_gather_backward(f1, f2, am_u, am_v, g_u, g_v, d_f1, d_f2, d.B, d.H1, d.W1, d.H2, d.W2, d.C, ws, s1, s,
+                                       s2_done ? s2 : s, s2_done);
     BwdArgs a;
     memset(&a, 0, sizeof(a));
     a.xcd_order = xcd_order_enabled();
@@ -3684,9 +3696,11 @@ int sepcorr_max_argmax_avg_backward(const float *f1, const float *f2, const int3
     if (int rc = check_dims(d, 2)) return rc;
     if (int rc = check_workspace(d, workspace, workspace_bytes)) return rc;
     const bool gather = maxavg_by_gather(d);
-    ForkJoin fj(static_cast<hipStream_t>(stream), gather || !bwd_ws(d).aliased);
+    ForkJoin fj(static_cast<hipStream_t>(stream), gather ? gather_overlap(d) : !bwd_ws(d).aliased);
     // d_f1 aside, d_f2 on the caller's stream
-    const int rc = maxavg_backward(d, gather, f1, f2, argmax_u, argmax_v, grad_u, grad_v, d_f1, d_f2, workspace, fj.sa, fj.user);
+    // the join event of side stream b serves as "table ready" in between: nothing else is recorded on b before the join
+    const int rc = maxavg_backward(d, gather, f1, f2, argmax_u, argmax_v, grad_u, grad_v, d_f1, d_f2, workspace, fj.sa, fj.user,
+                                   fj.sb, fj.ss ? fj.ss->jb : nullptr);
     const int rj = fj.join();
     return rc ? rc : rj;
 }

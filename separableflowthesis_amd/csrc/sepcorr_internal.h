@@ -19,11 +19,13 @@ void *sepcorr_prof_begin(const char *name, void *stream);
 void sepcorr_prof_end(void *token);
 
 // Max/avg backward as gathers of feature rows (gather_backward.hip).  Eligible sizes only; `ws` holds
-// sepcorr_gather_backward_bytes() bytes, 256-byte aligned.  d_f1 is enqueued on stream_f1, d_f2 on stream_f2; the two
-// use disjoint parts of `ws`.
+// sepcorr_gather_backward_bytes() bytes, 256-byte aligned.  d_f1 is enqueued on stream_f1, d_f2 on stream_f2 and the
+// table of average gradients that d_f2 adds at its end on stream_table, which d_f2's last launch waits for through
+// table_event (an event of the caller, recorded here; NULL keeps the table on stream_f2).  The three use disjoint
+// parts of `ws`.
 int sepcorr_gather_backward_eligible(int B, int H1, int W1, int H2, int W2, int C);
 size_t sepcorr_gather_backward_bytes(int B, int H1, int W1, int H2, int W2, int C);
 int sepcorr_gather_backward(const float *f1, const float *f2, const int32_t *am_u, const int32_t *am_v, const float *g_u,
                             const float *g_v, float *d_f1, float *d_f2, int B, int H1, int W1, int H2, int W2, int C, void *ws,
-                            void *stream_f1, void *stream_f2);
+                            void *stream_f1, void *stream_f2, void *stream_table, void *table_event);
 #endif
