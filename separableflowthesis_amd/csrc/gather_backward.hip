@@ -58,10 +58,28 @@ struct GatherArgs {
     int B, N1, N1p, H2, W2, C, S;
 };
 
-// amT[b][j][p] = am[b][p][j]; entries beyond N1 are -1 (no hit).  grid (N1p / 256, L, B)
-__global__ void __launch_bounds__(256) argmax_columns_kernel(const int *am, int *amT, int N1, int N1p, int L) {
-    const int p = blockIdx.x * 256 + threadIdx.x, j = blockIdx.y, b = blockIdx.z;
-    amT[((size_t)b * L + j) * N1p + p] = p < N1 ? am[((size_t)b * N1 + p) * L + j] : -1;
+// amT[b][j][p] = am[b][p][j] for both argmax tensors; entries beyond N1 are -1 (no hit).  grid (N1p / 64, 2, B):
+// 64 pixels of argmax_u (blockIdx.y == 0) or argmax_v go through LDS, TCHUNK lines at a time, so that the reads run
+// along a pixel's lines and the writes along the pixels of a line.
+constexpr int TCHUNK = 128;
+__global__ void __launch_bounds__(256) argmax_columns_kernel(const GatherArgs a) {
+    __shared__ int tile[64][TCHUNK + 1];
+    const int p0 = blockIdx.x * 64, b = blockIdx.z;
+    const bool second = blockIdx.y != 0;
+    const int L = second ? a.W2 : a.H2, N1 = a.N1, N1p = a.N1p;
+    const int *am = (second ? a.am_v : a.am_u) + (size_t)b * N1 * L;
+    int *amT = (second ? a.amT_v : a.amT_u) + (size_t)b * L * N1p;
+    for (int jc = 0; jc < L; jc += TCHUNK) {
+        const int nj = min(TCHUNK, L - jc);
+        if (jc) __syncthreads();
+        for (int i = threadIdx.x; i < 64 * TCHUNK; i += 256) {
+            const int px = i / TCHUNK, jl = i - px * TCHUNK, p = p0 + px;
+            if (jl < nj) tile[px][jl] = p < N1 ? am[(size_t)p * L + jc + jl] : -1;
+        }
+        __syncthreads();
+        const int px = threadIdx.x & 63;
+        for (int jl = threadIdx.x >> 6; jl < nj; jl += 4) amT[(size_t)(jc + jl) * N1p + p0 + px] = tile[px][jl];
+    }
 }
 
 // lines[b][j][:]: j < H2: mean_v f2[(j,v),:]; else mean_u f2[(u,j-H2),:].  grid (H2+W2, B); the four waves take every
@@ -92,64 +110,88 @@ __global__ void __launch_bounds__(256) fmap2_line_means_kernel(const GatherArgs 
     }
 }
 
-// table_part[b][s][j][c] = sum over the pixels of split s of g_avg[p,j] f1[p,c].  grid (ceil(L/32), S, B); the
-// product has rows j, columns c and runs over pixels two at a time; wave w owns channels [64w, 64w+64).
+// One 32x32x2 product per channel of a 16-byte operand load: lane (l32, h) holds B[k = h][4 l32 .. 4 l32 + 3], product
+// number i takes component i, so column l32 of accumulator i is channel 4 l32 + i and a lane's four accumulators
+// hold four neighbouring channels of the same rows.
+__device__ __forceinline__ void mfma4(float av, v4f x, v16f (&acc)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, x[i], acc[i], 0, 0, 0);
+}
+
+// table_part[b][s][j][c] = sum over the pixels of split s of g_avg[p,j] f1[p,c].  grid (ceil(L/32), S/2, B); the
+// product has rows j, columns c and runs over pixels two at a time.  Wave w owns channels [128 (w & 1), +128) and
+// the split 2 blockIdx.y + (w >> 1); the operands of the next eight pixels are in flight during the products.
 __global__ void __launch_bounds__(256) avg_table_partial_kernel(const GatherArgs a) {
-    const int jt = blockIdx.x, s = blockIdx.y, b = blockIdx.z;
+    const int jt = blockIdx.x, b = blockIdx.z;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
     const int N1 = a.N1, H2 = a.H2, W2 = a.W2, C = a.C, S = a.S;
-    const int c0 = wave * 64;
-    if (c0 >= C) return;
+    const int c0 = (wave & 1) * 128, s = 2 * blockIdx.y + (wave >> 1);
+    if (c0 >= C || s >= S) return;
     const int L = H2 + W2, j = jt * 32 + l32;
     int per = (N1 + S - 1) / S;
     per += per & 1;
     const int pa = s * per, pb = min(N1, pa + per);
-    const bool jok = j < L;
-    const bool ju = j < H2;
+    const bool jok = j < L, ju = j < H2;
+    const bool cok = c0 + 4 * l32 < C;
     const float *gp = ju ? a.g_u + (size_t)b * N1 * 2 * H2 + H2 + j : a.g_v + (size_t)b * N1 * 2 * W2 + W2 + (j - H2);
     const size_t gs = ju ? 2 * (size_t)H2 : 2 * (size_t)W2;
-    const bool ok0 = c0 + l32 < C, ok1 = c0 + 32 + l32 < C;
-    const float *fp0 = a.f1 + (size_t)b * N1 * C + (ok0 ? c0 + l32 : 0);
-    const float *fp1 = a.f1 + (size_t)b * N1 * C + (ok1 ? c0 + 32 + l32 : 0);
-    v16f acc0, acc1;
+    const float *fp = a.f1 + (size_t)b * N1 * C + (cok ? c0 + 4 * l32 : 0);
+    v16f acc[4];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { acc0[r] = 0.f; acc1[r] = 0.f; }
-    for (int p0 = pa; p0 < pb; p0 += 8) {
-        float ga[4], x0[4], x1[4];
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
+    struct Ops { float g[4]; v4f x[4]; };
+    auto load = [&](int p0, Ops &o) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int p = p0 + 2 * i + h;
             const bool ok = p < pb;
-            const int pc = ok ? p : pa;            // pa < N1 whenever the loop runs
-            ga[i] = (ok && jok) ? gp[(size_t)pc * gs] : 0.f;
-            x0[i] = fp0[(size_t)pc * C];
-            x1[i] = fp1[(size_t)pc * C];
+            const int pc = ok ? p : pa;            // pa < N1 whenever a load is issued
+            o.g[i] = (ok && jok) ? gp[(size_t)pc * gs] : 0.f;
+            o.x[i] = *reinterpret_cast<const v4f *>(fp + (size_t)pc * C);
         }
+    };
+    auto products = [&](const Ops &o) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(ga[i], x0[i], acc0, 0, 0, 0);
-            acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(ga[i], x1[i], acc1, 0, 0, 0);
+        for (int i = 0; i < 4; ++i) mfma4(o.g[i], o.x[i], acc);
+    };
+    Ops A, B;
+    if (pa < pb) load(pa, A);
+    for (int p0 = pa; p0 < pb; p0 += 16) {
+        if (p0 + 8 < pb) load(p0 + 8, B);
+        products(A);
+        if (p0 + 8 < pb) {
+            if (p0 + 16 < pb) load(p0 + 16, A);
+            products(B);
         }
     }
+    if (!cok) return;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
         const int jj = jt * 32 + acc_row(r, h);
-        if (jj < L) {
-            float *dst = a.table_part + (((size_t)b * S + s) * L + jj) * C + c0 + l32;
-            if (ok0) dst[0] = acc0[r];
-            if (ok1) dst[32] = acc1[r];
-        }
+        if (jj < L)
+            *reinterpret_cast<v4f *>(a.table_part + (((size_t)b * S + s) * L + jj) * C + c0 + 4 * l32) =
+                (v4f){acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
     }
 }
 
-// table[b][j][:] = (sum over splits, in order) / (W2 for j < H2, H2 otherwise).  grid (H2+W2, B)
+// table[b][j][:] = (sum over the splits) / (W2 for j < H2, H2 otherwise).  grid (H2+W2, B); wave w adds the splits
+// w, w + 4, ... in order, lane = 4 channels, and the four sums are added in wave order.
 __global__ void __launch_bounds__(256) avg_table_reduce_kernel(const GatherArgs a) {
+    __shared__ v4f part[4][64];
     const int j = blockIdx.x, b = blockIdx.y, L = a.H2 + a.W2, C = a.C, S = a.S;
-    const float scale = j < a.H2 ? 1.f / a.W2 : 1.f / a.H2;
-    for (int c = threadIdx.x; c < C; c += 256) {
-        float s = 0.f;
-        for (int i = 0; i < S; ++i) s += a.table_part[(((size_t)b * S + i) * L + j) * C + c];
-        a.table[((size_t)b * L + j) * C + c] = s * scale;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const bool on = 4 * lane < C;
+    v4f s0 = {0.f, 0.f, 0.f, 0.f};
+    if (on)
+        for (int i = wave; i < S; i += 4) s0 += *reinterpret_cast<const v4f *>(a.table_part + (((size_t)b * S + i) * L + j) * C + 4 * lane);
+    part[wave][lane] = s0;
+    __syncthreads();
+    if (wave == 0 && on) {
+        const float scale = j < a.H2 ? 1.f / a.W2 : 1.f / a.H2;
+        *reinterpret_cast<v4f *>(a.table + ((size_t)b * L + j) * C + 4 * lane) =
+            ((part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane])) * scale;
     }
 }
 
@@ -257,9 +299,10 @@ __global__ void __launch_bounds__(256) df1_max_gather_kernel(const GatherArgs a)
 
 // d2[(u,v)][:] = sum over the pixels that chose (u,v) in either direction + the two table lines.  One wave per
 // (u,v), lane = 4 channels; grid (ceil(N2/4), B).  One launch covers the pixels [pa, pb) (multiples of SCAN): all but
-// the first add to what d2 holds, the last adds the table lines (which may come from another stream in the meantime).  The launches follow each other on one stream, so
-// the rows of fmap1 that the whole grid fetches at any time come from one slice of a few MB, which the L2 caches hold;
-// over all pixels at once they do not (measured at B=2, 55x128: 1.7 GB of L2 misses for 2.6 GB of rows, at 7 TB/s).
+// the first add to what d2 holds, the last adds the table lines (which may come from another stream in the meantime).
+// The launches follow each other on one stream, so the rows of fmap1 that the whole grid fetches at any time come
+// from one slice of a few MB, which the L2 caches hold; over all pixels at once they do not (measured at B=2, 55x128:
+// 1.7 GB of L2 misses for 2.6 GB of rows, at 7 TB/s).
 __global__ void __launch_bounds__(256) df2_gather_kernel(const GatherArgs a, int pa, int pb) {
     __shared__ int queue[4][QCAP];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -347,7 +390,7 @@ int table_splits(int B, int N1, int H2, int W2) {
     const int cap = N1 / 64 > 1 ? N1 / 64 : 1;
     if (S > cap) S = cap;
     if (S > 64) S = 64;
-    return S < 1 ? 1 : S;
+    return S < 2 ? 2 : (S + 1) & ~1;   // two splits per workgroup of avg_table_partial_kernel
 }
 
 struct Layout {
@@ -414,14 +457,13 @@ int sepcorr_gather_backward(const float *f1, const float *f2, const int32_t *am_
     }
     {   // the table of the average gradients: needed by the last slice of the scan only
         Prof ps("df2_maxavg_table", s3);
-        hipLaunchKernelGGL(avg_table_partial_kernel, dim3((L + 31) / 32, l.S, B), blk, 0, s3, a);
+        hipLaunchKernelGGL(avg_table_partial_kernel, dim3((L + 31) / 32, l.S / 2, B), blk, 0, s3, a);
         hipLaunchKernelGGL(avg_table_reduce_kernel, dim3(L, B), blk, 0, s3, a);
     }
     if (s3 != s2 && hipEventRecord(ev, s3) != hipSuccess) return sepcorr_set_error(SEPCORR_ELAUNCH, "sepcorr: max/avg backward (gather): event record failed");
     {   // d_f2: transposed argmax, then the scan slice by slice
         Prof ps("df2_maxavg_gather", s2);
-        hipLaunchKernelGGL(argmax_columns_kernel, dim3(l.N1p / 256, H2, B), blk, 0, s2, am_u, a.amT_u, N1, l.N1p, H2);
-        hipLaunchKernelGGL(argmax_columns_kernel, dim3(l.N1p / 256, W2, B), blk, 0, s2, am_v, a.amT_v, N1, l.N1p, W2);
+        hipLaunchKernelGGL(argmax_columns_kernel, dim3(l.N1p / 64, 2, B), blk, 0, s2, a);
         // slices of about 1.75 MB of fmap1 per batch entry (measured best at 3 MB and 7 MB of features per entry)
         const int steps = l.N1p / SCAN;
         int slices = (int)(((size_t)N1 * C * 4 + (7u << 17)) / (7u << 18));
