@@ -137,3 +137,48 @@ def test_gather_at_the_reference_resolution(device, modes):
     for x, y, n in ((a1, b1, "grad_fmap1_l0"), (a2, b2, "grad_fmap2_lk")):
         err = float((x - y).abs().max()) / float(y.abs().max())
         assert err < 2e-5, f"{n}: gather and dense differ by {err:.2e} of the largest entry"
+
+
+def _inputs(device, seed, B=2, H=32, W=64, C=64):
+    """A size whose three chains of kernels run on three streams (>= 300 000 rows, fmap2 below 4 MB per batch entry)."""
+    f1, f2, g = op_inputs(B, H, W, H, W, C, seed=seed)
+    t = dict(f1=f1, f2=f2,
+             am_u=torch.randint(0, W, (B, H, W, 1, H), generator=g, dtype=torch.int32),
+             am_v=torch.randint(0, H, (B, H, W, 1, W), generator=g, dtype=torch.int32),
+             g_u=torch.randn(B, H, W, 2, H, generator=g), g_v=torch.randn(B, H, W, 2, W, generator=g))
+    return {k: v.to(device) for k, v in t.items()}
+
+
+def _bwd(t):
+    return ms.max_argmax_avg_backward(t["f1"], t["f2"], t["am_u"], t["am_v"], t["g_u"], t["g_v"])
+
+
+def test_gather_follows_the_callers_stream_and_replays_from_a_captured_graph(device, modes):
+    """The gather path forks onto the library's two side streams and orders its last scan slice behind the table of
+    average gradients with an event: under capture these become graph dependencies.  Every replay is checked against
+    the eager result for the inputs of that replay, with eager work between the replays."""
+    ms.set_max_avg_backward(ms.MAXAVG_GATHER)
+    ref = _bwd(_inputs(device, seed=91))
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        t = {k: v.clone() for k, v in _inputs(device, seed=91).items()}   # produced on s: the op must wait for it
+        got = _bwd(t)
+    s.synchronize()
+    assert all(torch.equal(x, y) for x, y in zip(got, ref))
+
+    static = _inputs(device, seed=92)
+    _bwd(static)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = _bwd(static)
+    for seed in (93, 94, 95):
+        fresh = _inputs(device, seed=seed)
+        ref = _bwd(fresh)
+        torch.cuda.synchronize()
+        for k in static:
+            static[k].copy_(fresh[k])
+        graph.replay()
+        torch.cuda.synchronize()
+        assert all(torch.equal(x, y) for x, y in zip(outs, ref)), f"replay with seed {seed} differs from eager"
