@@ -326,6 +326,10 @@ class Workload:
             "tflops_executed": round(executed * Wf / (ms * 1e-3) / 1e12, 3),
             "max_avg_backward": ("gather" if gathered else "dense") if "F" in ops else None,
             "all_dense": dense,
+            "note": ("tflops / frac_of_fp32_mfma_peak count the algorithmic work of the step (contraction_passes x 2*B*N1*N2*C); "
+                     "the max/avg backward ran as gathers of feature rows, so contraction_passes_executed of them ran on the "
+                     "matrix cores (tflops_executed); all_dense is the same step with every pass a contraction")
+                    if gathered else None,
             "peak_hbm_allocated_mib": round(peak / _MIB, 1),
             "backward_workspace_mib": round(self.workspace_bytes / _MIB, 1),
             "forward_workspace_mib": round(self.forward_workspace_bytes / _MIB, 1),
@@ -498,7 +502,7 @@ def main():
                    "contraction_passes": head["contraction_passes"], "gflop_per_step": head["gflop_per_step"],
                    "contraction_passes_executed": head["contraction_passes_executed"],
                    "tflops_executed": head["tflops_executed"], "max_avg_backward": head["max_avg_backward"],
-                   "all_dense": head["all_dense"],
+                   "all_dense": head["all_dense"], "note": head["note"],
                    "frac_of_fp32_mfma_peak": head["frac_of_fp32_mfma_peak"],
                    "peak_hbm_allocated_mib": head["peak_hbm_allocated_mib"],
                    "backward_workspace_mib": head["backward_workspace_mib"],
