@@ -184,3 +184,24 @@ def test_gather_follows_the_callers_stream_and_replays_from_a_captured_graph(dev
         graph.replay()
         torch.cuda.synchronize()
         assert all(torch.equal(x, y) for x, y in zip(outs, ref)), f"replay with seed {seed} differs from eager"
+
+
+def test_gather_equals_dense_on_seeded_random_shapes(device, modes):
+    """60 seeded shapes (all sizes 1..40, C a multiple of 4 up to 256, random argmax with a few entries outside the
+    range): the two paths agree to fp32 rounding everywhere."""
+    rng = torch.Generator().manual_seed(2024)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=rng))
+    for n in range(60):
+        B, H1, W1, H2, W2, C = r(1, 3), r(1, 40), r(1, 40), r(1, 40), r(1, 40), 4 * r(1, 64)
+        f1, f2, g = op_inputs(B, H1, W1, H2, W2, C, seed=300 + n)
+        au = torch.randint(-1, W2 + 1, (B, H1, W1, 1, H2), generator=g, dtype=torch.int32)
+        av = torch.randint(-1, H2 + 1, (B, H1, W1, 1, W2), generator=g, dtype=torch.int32)
+        g_u = torch.randn(B, H1, W1, 2, H2, generator=g)
+        g_v = torch.randn(B, H1, W1, 2, W2, generator=g)
+        args = tuple(t.to(device) for t in (f1, f2, au, av, g_u, g_v))
+        a1, a2 = _run(ms.MAXAVG_GATHER, *args)
+        b1, b2 = _run(ms.MAXAVG_DENSE, *args)
+        for x, y, name in ((a1, b1, "grad_fmap1_l0"), (a2, b2, "grad_fmap2_lk")):
+            scale = max(float(y.abs().max()), 1e-6)
+            err = float((x - y).abs().max()) / scale
+            assert err < 2e-5, f"shape {(B, H1, W1, H2, W2, C)} {name}: gather and dense differ by {err:.2e} of the largest entry"
