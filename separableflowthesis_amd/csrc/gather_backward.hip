@@ -56,6 +56,7 @@ struct GatherArgs {
     float *table;           // [B][H2+W2][C]: A_u / W2 then A_v / H2
     float *table_part;      // [B][S][H2+W2][C]
     int B, N1, N1p, H2, W2, C, S;
+    int line0;              // the tables hold the lines [line0, H2+W2) only (0: all; H2: those of g_v)
 };
 
 // amT[b][j][p] = am[b][p][j] for both argmax tensors; entries beyond N1 are -1 (no hit).  grid (N1p / 64, 2, B):
@@ -127,7 +128,7 @@ __global__ void __launch_bounds__(256) avg_table_partial_kernel(const GatherArgs
     const int N1 = a.N1, H2 = a.H2, W2 = a.W2, C = a.C, S = a.S;
     const int c0 = (wave & 1) * 128, s = 2 * blockIdx.y + (wave >> 1);
     if (c0 >= C || s >= S) return;
-    const int L = H2 + W2, j = jt * 32 + l32;
+    const int L = H2 + W2, NL = L - a.line0, j = a.line0 + jt * 32 + l32;
     int per = (N1 + S - 1) / S;
     per += per & 1;
     const int pa = s * per, pb = min(N1, pa + per);
@@ -169,9 +170,9 @@ __global__ void __launch_bounds__(256) avg_table_partial_kernel(const GatherArgs
     if (!cok) return;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-        const int jj = jt * 32 + acc_row(r, h);
-        if (jj < L)
-            *reinterpret_cast<v4f *>(a.table_part + (((size_t)b * S + s) * L + jj) * C + c0 + 4 * l32) =
+        const int jj = jt * 32 + acc_row(r, h);   // line within the table
+        if (jj < NL)
+            *reinterpret_cast<v4f *>(a.table_part + (((size_t)b * S + s) * NL + jj) * C + c0 + 4 * l32) =
                 (v4f){acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
     }
 }
@@ -180,7 +181,7 @@ __global__ void __launch_bounds__(256) avg_table_partial_kernel(const GatherArgs
 // w, w + 4, ... in order, lane = 4 channels, and the four sums are added in wave order.
 __global__ void __launch_bounds__(256) avg_table_reduce_kernel(const GatherArgs a) {
     __shared__ v4f part[4][64];
-    const int j = blockIdx.x, b = blockIdx.y, L = a.H2 + a.W2, C = a.C, S = a.S;
+    const int j = blockIdx.x, b = blockIdx.y, L = a.H2 + a.W2 - a.line0, C = a.C, S = a.S;   // j: line within the table
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const bool on = 4 * lane < C;
     v4f s0 = {0.f, 0.f, 0.f, 0.f};
@@ -189,7 +190,7 @@ __global__ void __launch_bounds__(256) avg_table_reduce_kernel(const GatherArgs 
     part[wave][lane] = s0;
     __syncthreads();
     if (wave == 0 && on) {
-        const float scale = j < a.H2 ? 1.f / a.W2 : 1.f / a.H2;
+        const float scale = a.line0 + j < a.H2 ? 1.f / a.W2 : 1.f / a.H2;
         *reinterpret_cast<v4f *>(a.table + ((size_t)b * L + j) * C + 4 * lane) =
             ((part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane])) * scale;
     }
@@ -384,8 +385,8 @@ __global__ void __launch_bounds__(256) df2_gather_kernel(const GatherArgs a, int
 
 size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 
-int table_splits(int B, int N1, int H2, int W2) {
-    const int jt = (H2 + W2 + 31) / 32;
+int table_splits(int B, int N1, int lines) {
+    const int jt = (lines + 31) / 32;
     int S = (512 + jt * B - 1) / (jt * B);
     const int cap = N1 / 64 > 1 ? N1 / 64 : 1;
     if (S > cap) S = cap;
@@ -400,7 +401,7 @@ struct Layout {
 Layout layout(int B, int N1, int H2, int W2, int C) {
     Layout l;
     l.N1p = (N1 + SCAN - 1) / SCAN * SCAN;
-    l.S = table_splits(B, N1, H2, W2);
+    l.S = table_splits(B, N1, H2 + W2);
     const size_t L = (size_t)H2 + W2;
     size_t o = 0;
     l.off_amT_u = o; o += align256((size_t)B * H2 * l.N1p * 4);
@@ -443,6 +444,7 @@ int sepcorr_gather_backward(const float *f1, const float *f2, const int32_t *am_
     a.table = reinterpret_cast<float *>(w + l.off_table);
     a.table_part = reinterpret_cast<float *>(w + l.off_part);
     a.B = B; a.N1 = H1 * W1; a.N1p = l.N1p; a.H2 = H2; a.W2 = W2; a.C = C; a.S = l.S;
+    a.line0 = 0;
     const int L = H2 + W2, N1 = a.N1, N2 = H2 * W2;
     hipStream_t s1 = static_cast<hipStream_t>(stream_f1), s2 = static_cast<hipStream_t>(stream_f2);
     hipStream_t s3 = static_cast<hipStream_t>(stream_table);
@@ -480,6 +482,37 @@ int sepcorr_gather_backward(const float *f1, const float *f2, const int32_t *am_
     if (e != hipSuccess) {
         char msg[200];
         snprintf(msg, sizeof(msg), "sepcorr: max/avg backward (gather): %s", hipGetErrorString(e));
+        return sepcorr_set_error(SEPCORR_ELAUNCH, msg);
+    }
+    return SEPCORR_OK;
+}
+
+// The table of the average gradients of g_v alone, for a d_f2 kernel that leaves that term out:
+//   table[b][v][c] = (1 / H2) sum_p g_v[p,1,v] f1[p,c]
+// `part` holds sepcorr_avg_table_v_part_bytes() bytes of split sums.
+int sepcorr_avg_table_v_eligible(int B, int H1, int W1, int H2, int W2, int C) {
+    return sepcorr_gather_backward_eligible(B, H1, W1, H2, W2, C);
+}
+
+size_t sepcorr_avg_table_v_part_bytes(int B, int H1, int W1, int W2, int C) {
+    return align256((size_t)B * table_splits(B, H1 * W1, W2) * W2 * C * 4);
+}
+
+int sepcorr_avg_table_v(const float *f1, const float *g_v, float *table, float *part, int B, int H1, int W1, int H2, int W2, int C,
+                        void *stream) {
+    GatherArgs a = {};
+    a.f1 = f1; a.g_u = g_v; a.g_v = g_v;   // (lines below H2 are not computed: g_u is never read)
+    a.table = table; a.table_part = part;
+    a.B = B; a.N1 = H1 * W1; a.H2 = H2; a.W2 = W2; a.C = C; a.S = table_splits(B, H1 * W1, W2);
+    a.line0 = H2;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    Prof ps("df2_avg_table", s);
+    hipLaunchKernelGGL(avg_table_partial_kernel, dim3((W2 + 31) / 32, a.S / 2, B), dim3(256), 0, s, a);
+    hipLaunchKernelGGL(avg_table_reduce_kernel, dim3(W2, B), dim3(256), 0, s, a);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        char msg[200];
+        snprintf(msg, sizeof(msg), "sepcorr: table of average gradients: %s", hipGetErrorString(e));
         return sepcorr_set_error(SEPCORR_ELAUNCH, msg);
     }
     return SEPCORR_OK;

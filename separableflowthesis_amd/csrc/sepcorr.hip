@@ -1359,6 +1359,7 @@ struct BwdArgs {
     const float *a_u, *a_v;          // GMODE_COMP:   (B,N1,KT,W2), (B,N1,KT,H2)
     const float *g_cu, *g_cv;        // GMODE_COMP:   (B,N1,KT,H2), (B,N1,KT,W2)
     const float *uwt;                // fast d_f1: the (p,u)-indexed weights transposed to [b][u][field][p]
+    const float *vtable;             // tiled d_f2 without the average term of g_v: (B,W2,C) table that stands for it
     float *d1;                       // (B,N1,C)
     float *d2;                       // (B,N2,C) or scratch [nsplit][B,N2,C]
     int B, N1, H2, W2, C;
@@ -1996,11 +1997,15 @@ __device__ __forceinline__ void dma16(__amdgpu_buffer_rsrc_t r, float *lds_chunk
 // buffers of the (p,u)-indexed weights per wave: the combined mode has LDS for one only
 constexpr int df2_tiled_ubuf(int gmode) { return gmode == GMODE_BOTH ? 1 : 2; }
 
-template <int GMODE, int KC, int NCB, int NWV>
+// NOAVGV: the term g_v[avg] / H2 of G does not depend on the row u, so its contribution to d_f2[(u,v),:] is the same
+// for every u: the line v of a small table (BwdArgs::vtable, gather_backward.hip) that the workgroups of the first
+// split add to their sums.  Without that weight tile in LDS the combined mode has room for 8 rows per workgroup.
+template <int GMODE, int KC, int NCB, int NWV, bool NOAVGV = false>
 __global__ void __launch_bounds__(64 * NWV) df2_tiled_kernel(const BwdArgs a, int nvc, int nug) {
     constexpr bool HC = g_has_comp(GMODE), HM = g_has_maxavg(GMODE);
+    static_assert(!NOAVGV || HM, "only the max/avg part has an average term");
     constexpr int NVC = HC ? 2 * KC : 0;       // weight tensors of the compression part: a_u[k].., g_cv[k]..
-    constexpr int NV = NVC + (HM ? 3 : 0);     // then g_v[max], g_v[avg], argmax_v
+    constexpr int NV = NVC + (HM ? (NOAVGV ? 2 : 3) : 0);     // then g_v[max], g_v[avg] (unless NOAVGV), argmax_v
     constexpr int NUP = (NV + 3) & ~3;
     constexpr int UBUF = df2_tiled_ubuf(GMODE);
     constexpr int CB = 128 * NCB;
@@ -2101,7 +2106,7 @@ __global__ void __launch_bounds__(64 * NWV) df2_tiled_kernel(const BwdArgs a, in
                     if constexpr (HC) dma16(kk < KC ? rs_va : rs_vb, dst, wl_c + uni);
                 } else if constexpr (HM) {
                     const int m = kk - NVC;
-                    if (m < 2) dma16(rs_vc, dst, wl_2 + (p8 * 2u * W2 + (unsigned)m * W2) * 4u);
+                    if (m < (NOAVGV ? 1 : 2)) dma16(rs_vc, dst, wl_2 + (p8 * 2u * W2 + (unsigned)m * W2) * 4u);
                     else dma16(rs_vd, dst, wl_1 + p8 * W2 * 4u);
                 }
             }
@@ -2200,8 +2205,12 @@ __global__ void __launch_bounds__(64 * NWV) df2_tiled_kernel(const BwdArgs a, in
                 }
                 if constexpr (HM) {
                     G += __float_as_int(o.uw[NVC + 2]) == v ? o.uw[NVC] : o.uw[NVC + 1];
-                    G = fmaf(o.vw[NVC + 1], inv_h2, G);
-                    if (__float_as_int(o.vw[NVC + 2]) == u) G += o.vw[NVC];
+                    if constexpr (NOAVGV) {
+                        if (__float_as_int(o.vw[NVC + 1]) == u) G += o.vw[NVC];
+                    } else {
+                        G = fmaf(o.vw[NVC + 1], inv_h2, G);
+                        if (__float_as_int(o.vw[NVC + 2]) == u) G += o.vw[NVC];
+                    }
                 }
                 // No mask needed: pixels at or beyond `pend` have all-zero f1 rows and (p,v) weights (DMA
                 // bounds), so whatever finite G they get multiplies zeros; columns beyond W2 are not stored.
@@ -2235,12 +2244,19 @@ __global__ void __launch_bounds__(64 * NWV) df2_tiled_kernel(const BwdArgs a, in
     if (vok && u_raw < H2) {
         float *dst = a.d2 + ((size_t)split * a.B + b) * H2 * W2 * C + ((size_t)u * W2 + v) * C;
         const bool accum = a.accumulate != 0 && a.nsplit == 1;
+        const bool add_line = NOAVGV && split == 0;   // the average term of g_v, once per output element
+        const float *line = a.vtable + ((size_t)b * W2 + v) * C;
+        (void)inv_h2;
 #pragma unroll
         for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const v4f x = {acc[cb][0][r], acc[cb][1][r], acc[cb][2][r], acc[cb][3][r]};
-                store4<true>(dst, cb0 + 128 * cb + 4 * vmap(r, h), C, x, accum);
+                v4f x = {acc[cb][0][r], acc[cb][1][r], acc[cb][2][r], acc[cb][3][r]};
+                const int c = cb0 + 128 * cb + 4 * vmap(r, h);
+                if constexpr (NOAVGV) {
+                    if (add_line && c < C) x += *reinterpret_cast<const v4f *>(line + c);
+                }
+                store4<true>(dst, c, C, x, accum);
             }
     }
 }
@@ -3060,13 +3076,30 @@ struct Df2Plan {
     int rows;
     int tiles_per_split;   // pixel tiles of a split (the last split takes what is left)
     bool uneven;           // the last split is a short one, dealt out last (BwdArgs::uneven)
+    bool noavgv;           // combined mode: the average term of g_v comes from a table (df2_tiled_kernel<..., NOAVGV>)
 };
+Df2Plan df2_plan_rows(const Dims &d, int rows);
 
 // How d_f2 is computed for these sizes.  The p range is split over workgroups so that the grid fills
 // the 256 CUs evenly; each split writes a partial d_f2 to scratch, summed in split order afterwards.
 Df2Plan df2_plan(const Dims &d, bool both) {
+    if (both && sepcorr_avg_table_v_eligible(d.B, d.H1, d.W1, d.H2, d.W2, d.C) && df2_rows_per_wg(d, false) == 8) {
+        // eight rows per workgroup when the table's split sums fit into the region of d_f2's own (unused until the
+        // kernel stores) and there are at least two splits
+        Df2Plan p8 = df2_plan_rows(d, 8);
+        const size_t part = (size_t)p8.nsplit * d.B * d.H2 * d.W2 * d.C * sizeof(float);
+        if (p8.tiled && p8.nsplit >= 2 && sepcorr_avg_table_v_part_bytes(d.B, d.H1, d.W1, d.W2, d.C) <= part) {
+            p8.noavgv = true;
+            return p8;
+        }
+    }
+    return df2_plan_rows(d, df2_rows_per_wg(d, both));
+}
+
+Df2Plan df2_plan_rows(const Dims &d, int rows_per_wg) {
     Df2Plan pl;
-    pl.rows = df2_rows_per_wg(d, both);
+    pl.noavgv = false;
+    pl.rows = rows_per_wg;
     const size_t big = (size_t)1 << 30;
     const size_t n1 = (size_t)d.H1 * d.W1;
     pl.tiled = d.C % 4 == 0 && d.W2 % 4 == 0 && n1 * d.C * 4 <= big && n1 * MAX_K * d.W2 * 4 <= big &&
@@ -3179,6 +3212,7 @@ Df1Shape df1_shape(const Dims &d) {
 struct BwdWs {
     bool aliased;
     size_t off_uwt, off_df1sk, fwd_bytes, own_total, total;   // own_total: without the weight-gradient sweep
+    size_t off_vtable;                                        // (B,W2,C) table of the combined d_f2 (Df2Plan::noavgv)
 };
 BwdWs bwd_ws(const Dims &d) {
     BwdWs w;
@@ -3199,6 +3233,8 @@ BwdWs bwd_ws(const Dims &d) {
         const size_t g = sepcorr_gather_backward_bytes(d.B, d.H1, d.W1, d.H2, d.W2, d.C);
         if (g > w.total) w.total = g;
     }
+    w.off_vtable = w.total;
+    if (df2_plan(d, true).noavgv) w.total += ((size_t)d.B * d.W2 * d.C * sizeof(float) + 255) & ~(size_t)255;
     return w;
 }
 
@@ -3324,9 +3360,16 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s
         float *d2 = a.d2;
         if (a.nsplit > 1) a.d2 = static_cast<float *>(ws);
         if (plan.tiled) {
-            constexpr int NV = (g_has_comp(GMODE) ? 2 * KC : 0) + (g_has_maxavg(GMODE) ? 3 : 0);
-            constexpr int NUP = (NV + 3) & ~3;
+            constexpr int NV3 = (g_has_comp(GMODE) ? 2 * KC : 0) + (g_has_maxavg(GMODE) ? 3 : 0);
+            constexpr int NUP = (NV3 + 3) & ~3;
             constexpr int UBUF = df2_tiled_ubuf(GMODE);
+            const bool noavgv = GMODE == GMODE_BOTH && plan.noavgv;
+            const int NV = noavgv ? NV3 - 1 : NV3;
+            if (noavgv) {   // the table first; its split sums use the start of d_f2's partial sums, written later
+                float *vt = reinterpret_cast<float *>(static_cast<char *>(ws) + bwd_ws(d).off_vtable);
+                if (int rc = sepcorr_avg_table_v(a.f1, a.g_v, vt, static_cast<float *>(ws), d.B, d.H1, d.W1, d.H2, d.W2, d.C, s)) return rc;
+                a.vtable = vt;
+            }
             const int rows = plan.rows;
             const int nug = (d.H2 + rows - 1) / rows;
             const dim3 grid(d.B * a.nsplit * nug * nvc, cblocks), block(64 * rows);
@@ -3352,7 +3395,20 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s
         ProfScope ps(GMODE == GMODE_COMP ? "df2_comp" : GMODE == GMODE_BOTH ? "df2_both" : "df2_maxavg", s); \
         hipLaunchKernelGGL(k, grid, block, lds, s, a, nvc, nug);                                   \
     } while (0)
-            if (rows == 8) { if (ncb == 1) SEPCORR_DF2T(1, 8); else SEPCORR_DF2T(2, 8); }
+            if (noavgv) {
+                if constexpr (GMODE == GMODE_BOTH) {
+#define SEPCORR_DF2T8(NCB)                                                                          \
+    do {                                                                                           \
+        auto k = df2_tiled_kernel<GMODE, KC, NCB, 8, true>;                                        \
+        if (int rc = set_lds(k, lds)) return rc;                                                   \
+        ProfScope ps("df2_both", s);                                                               \
+        hipLaunchKernelGGL(k, grid, block, lds, s, a, nvc, nug);                                   \
+    } while (0)
+                    if (ncb == 1) SEPCORR_DF2T8(1); else SEPCORR_DF2T8(2);
+#undef SEPCORR_DF2T8
+                }
+            }
+            else if (rows == 8) { if (ncb == 1) SEPCORR_DF2T(1, 8); else SEPCORR_DF2T(2, 8); }
             else           { if (ncb == 1) SEPCORR_DF2T(1, 4); else SEPCORR_DF2T(2, 4); }
 #undef SEPCORR_DF2T
         } else {

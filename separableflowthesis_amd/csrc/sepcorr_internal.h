@@ -28,4 +28,10 @@ size_t sepcorr_gather_backward_bytes(int B, int H1, int W1, int H2, int W2, int 
 int sepcorr_gather_backward(const float *f1, const float *f2, const int32_t *am_u, const int32_t *am_v, const float *g_u,
                             const float *g_v, float *d_f1, float *d_f2, int B, int H1, int W1, int H2, int W2, int C, void *ws,
                             void *stream_f1, void *stream_f2, void *stream_table, void *table_event);
+// table[b][v][c] = (1 / H2) sum_p g_v[p,1,v] f1[p,c] (gather_backward.hip), for the combined d_f2 kernel that leaves
+// the average term of g_v to it.  Same sizes as the gather path; `part`: sepcorr_avg_table_v_part_bytes() of scratch.
+int sepcorr_avg_table_v_eligible(int B, int H1, int W1, int H2, int W2, int C);
+size_t sepcorr_avg_table_v_part_bytes(int B, int H1, int W1, int W2, int C);
+int sepcorr_avg_table_v(const float *f1, const float *g_v, float *table, float *part, int B, int H1, int W1, int H2, int W2, int C,
+                        void *stream);
 #endif
