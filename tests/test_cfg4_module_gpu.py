@@ -112,10 +112,10 @@ def test_fused_backward_at_headline_size_matches_the_oracle(device):
         r64, r32 = ref[torch.float64], ref[torch.float32]
         # d_f1: a wave adds its 55 x 32 = 1760 products per output one after the other in the MFMA accumulator
         # (4 such partial sums per output).  d_f2: the pixel range is cut into few long splits to keep the scratch
-        # small; a split adds up to 49 tiles of 32 pixels (the two reference calls) or 99 tiles (the fused call, whose
-        # workgroups hold 4 rows) in one accumulator.  chain_ratio turns these lengths into the expected ratio.
+        # small; a split adds up to 49 tiles of 32 pixels in one accumulator (the max/avg call gathers rows instead:
+        # sums of a few hundred).  chain_ratio turns these lengths into the expected ratio.
         error_report(d1[sl], r64[0], r32[0], f"fused d_f1 [b={b}]", max_ratio=chain_ratio(1760))
-        error_report(d2[sl], r64[1], r32[1], f"fused d_f2 [b={b}]", max_ratio=chain_ratio(99 * 32))
+        error_report(d2[sl], r64[1], r32[1], f"fused d_f2 [b={b}]", max_ratio=chain_ratio(49 * 32))
         error_report(c1[sl], r64[2], r32[2], f"compression d_f1 [b={b}]", max_ratio=chain_ratio(1760))
         error_report(c2[sl], r64[3], r32[3], f"compression d_f2 [b={b}]", max_ratio=chain_ratio(49 * 32))
         error_report(m1[sl], r64[4], r32[4], f"max/avg d_f1 [b={b}]", max_ratio=chain_ratio(1760))
