@@ -3083,7 +3083,11 @@ Df2Plan df2_plan_rows(const Dims &d, int rows);
 // How d_f2 is computed for these sizes.  The p range is split over workgroups so that the grid fills
 // the 256 CUs evenly; each split writes a partial d_f2 to scratch, summed in split order afterwards.
 Df2Plan df2_plan(const Dims &d, bool both) {
-    if (both && sepcorr_avg_table_v_eligible(d.B, d.H1, d.W1, d.H2, d.W2, d.C) && df2_rows_per_wg(d, false) == 8) {
+    // (the table costs 25 to 35 us and the larger workgroups gain a fifth of the kernel's time: worth it from about
+    // 2^25 (pixel, position) pairs on; measured at B=2, 55x128 pixels: 0.61 -> 0.52 ms with fmap2 55x128, but
+    // 0.055 -> 0.087 ms with fmap2 13x32)
+    const bool large = (size_t)d.B * d.H1 * d.W1 * d.H2 * d.W2 >= ((size_t)1 << 25);
+    if (both && large && sepcorr_avg_table_v_eligible(d.B, d.H1, d.W1, d.H2, d.W2, d.C) && df2_rows_per_wg(d, false) == 8) {
         // eight rows per workgroup when the table's split sums fit into the region of d_f2's own (unused until the
         // kernel stores) and there are at least two splits
         Df2Plan p8 = df2_plan_rows(d, 8);
