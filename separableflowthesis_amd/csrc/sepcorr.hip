@@ -33,6 +33,7 @@
 #include <atomic>
 #include <mutex>
 #include <string>
+#include <type_traits>
 #include <vector>
 
 #include "sepcorr.h"
@@ -1380,6 +1381,7 @@ struct BwdArgs {
     int sk_total, sk_steps;          // steps (rows per wave) over all tiles, per tile; 0 = whole tiles
     float *sk_state;                 // [2 * grid.x * grid.y] slots of 32 x (128 * NCB) floats
     int *sk_count;                   // [tiles * grid.y], zero at launch
+    int flush_rows;                  // d_f1: rows of a wave whose products one register accumulator takes
 };
 }  // namespace sepcorr_impl
 namespace {
@@ -1603,6 +1605,55 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
         for (int t = 0; t < 4; ++t)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[cb][t][e] = 0.f;
+    // Short chains of additions: a register accumulator takes the products of FLUSH_ROWS (4) rows of this wave only
+    // (128 products at 32 columns per row), then it is added to a running sum in the wave's LDS region and starts
+    // again from zero.  One fp32 accumulator over all rows of a tile (1760 products at 55 x 128) lost the low bits
+    // of every product it added once the sum had grown; sums of short blocks keep them.  The order stays fixed.
+    // An accumulator joins the running sum just before the first product of the new block overwrites it; that
+    // product takes a zero addend, so nothing has to be cleared.  The additions are vector instructions, which take
+    // matrix time here: 2 per accumulator register and block (the LDS unit's own float addition, ds_add_f32, takes
+    // no vector instruction but handles about one lane in three cycles: tried, five times slower).
+    // Layout [group of 4 registers][lane][4]: 16-byte accesses without bank conflicts, wave-private, the same bytes
+    // the wave's [pixel][channel] partial is written to at the end.
+    const int FLUSH_ROWS = a.flush_rows;
+    v4f *const run = reinterpret_cast<v4f *>(smem + wave * (TP * RS)) + lane;
+    {
+        const v4f z4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int q = 0; q < NCB * 16; ++q) run[q * 64] = z4;
+    }
+    auto run_load = [&](int cbt, v4f (&x)[4]) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) x[q] = run[(cbt * 4 + q) * 64];
+    };
+    // With one wave per SIMD the accumulators live in the accumulation registers, which vector additions cannot
+    // read: each value is copied out first.  The copy is written as assembly so that it stays where the running sum
+    // is updated; left to the compiler, all 128 copies were hoisted to the top of every row.  The compiler keeps no
+    // wait states for assembly: matrix_results_settled() stands between the last matrix instruction and the first
+    // copy (a matrix result may be read 19 wait states after the instruction that wrote it).
+    auto acc_value = [&](int cbt, int e) {
+        if constexpr (MAXT > 256) {
+            return acc[cbt >> 2][cbt & 3][e];
+        } else {
+            float x;
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(x) : "a"(acc[cbt >> 2][cbt & 3][e]));
+            return x;
+        }
+    };
+    auto matrix_results_settled = [] {
+        if constexpr (MAXT <= 256) asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
+    };
+    auto run_add_store = [&](int cbt, v4f (&x)[4]) {
+        float y[16];   // all copies first: a copy followed at once by the addition that reads it waits for it
+#pragma unroll
+        for (int e = 0; e < 16; ++e) y[e] = acc_value(cbt, e);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[q][e] += y[4 * q + e];
+            run[(cbt * 4 + q) * 64] = x[q];
+        }
+    };
 
     // rows wider than 256 columns: passes of 256 columns accumulate into the same registers
     for (int vp = 0; vp < a.vpasses; ++vp) {
@@ -1711,16 +1762,34 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
         G[r] = gval<GMODE, KC>(wv[r], wu_n, ufirst, vmap(r, 0), true);
     }
     UW<GMODE, KC> wu_next = load_uw_row(min(ufirst + NUG, H2 - 1));
-    auto compute = [&](int u, int g, v4f(&buf)[GS][NCB]) {
+    auto compute = [&](int u, int g, v4f(&buf)[GS][NCB], auto fresh) {
         static_assert(GS == 2, "two G values are produced per group");
         if (g == 0) {
             wu_n = wu_next;                                                       // weights of row u + NUG
             wu_next = load_uw_row(min(u + 2 * NUG, H2 - 1));                      // and of the row after it
         }
+        if (g == 0 && decltype(fresh)::value) {
+            // first products of a new block: hand each accumulator to the running sum, then restart it from zero;
+            // the running sum of the next accumulator is fetched while the matrix instruction of this one runs
+            const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            v4f rs[2][4];
+            run_load(0, rs[0]);
+            matrix_results_settled();
 #pragma unroll
-        for (int cb = 0; cb < NCB; ++cb)
+            for (int cbt = 0; cbt < NCB * 4; ++cbt) {
+                if (cbt + 1 < NCB * 4) run_load(cbt + 1, rs[(cbt + 1) & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+                run_add_store(cbt, rs[cbt & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+                acc[cbt >> 2][cbt & 3] = mfma(buf[0][cbt >> 2][cbt & 3], G[0], zero);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
 #pragma unroll
-            for (int t = 0; t < 4; ++t) acc[cb][t] = mfma(buf[0][cb][t], G[g * GS], acc[cb][t]);
+            for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) acc[cb][t] = mfma(buf[0][cb][t], G[g * GS], acc[cb][t]);
+        }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int ss = 0; ss < GS; ++ss) {
@@ -1751,20 +1820,40 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
         issue(min(ufirst, H2 - 1), k, ring[k]);
         __builtin_amdgcn_sched_barrier(0);
     }
-    for (int u = ufirst; u < u_end; u += NUG) {
+    // (two copies of the row body, the first row of a block and the others: with one body and a branch around
+    // the block change the compiler copied all accumulators between the register files in every row)
+    auto sweep_row = [&](int u, auto fresh) {
 #pragma unroll
         for (int g = 0; g < NG; ++g) {
             constexpr int AHEAD = NB - 1;
+            // (no condition on the fetch ahead into the next row: behind a branch the compiler has to assume that
+            // the loads were not issued and waits for all but the last few at the end of every row; the last row of
+            // a piece fetches a valid row that nobody uses)
             if (g + AHEAD < NG) issue(u, g + AHEAD, ring[(g + AHEAD) % NB]);
-            else if (u + NUG < u_end) issue(u + NUG, g + AHEAD - NG, ring[(g + AHEAD) % NB]);
+            else issue(min(u + NUG, H2 - 1), g + AHEAD - NG, ring[(g + AHEAD) % NB]);
             __builtin_amdgcn_sched_barrier(0);
-            compute(u, g, ring[g % NB]);
+            compute(u, g, ring[g % NB], fresh);
             __builtin_amdgcn_sched_barrier(0);
         }
+    };
+    for (int u = ufirst; u < u_end;) {
+        sweep_row(u, std::true_type{});
+        u += NUG;
+        for (int j = 1; j < FLUSH_ROWS && u < u_end; ++j, u += NUG) sweep_row(u, std::false_type{});
     }
 
     }   // column passes
 
+    // the last block joins the running sum in the registers
+#pragma unroll
+    for (int cbt = 0; cbt < NCB * 4; ++cbt) {
+        v4f x[4];
+        run_load(cbt, x);
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[cbt >> 2][cbt & 3][4 * q + e] += x[q][e];
+    }
     // every wave leaves its partial [32][CB] in its own LDS region; they are added in wave order on the way out
     {
         float *mine = smem + wave * (TP * RS);
@@ -3261,6 +3350,10 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s
         const dim3 block(64 * nW);
         const size_t lds = (size_t)nW * TP * (128 * ncb + 4) * sizeof(float);   // one [32][channels] region per wave
         a.sk_total = 0;
+        // Rows per block of d_f1's register accumulation.  Measured at B=2, 55x128, C=256 (error against fp64 relative
+        // to the fp32 CPU path's / kernel time): whole tiles 2.45 / 0.422 ms, 12 rows 1.28, 8 rows 1.08 / 0.434,
+        // 6 rows 0.97, 4 rows 0.83 / 0.444, 2 rows 0.66 / 0.468, 1 row 0.517 ms.
+        a.flush_rows = 4;
 #define SEPCORR_DF1_K(...)                                                                         \
     do {                                                                                           \
         auto k = df1_kernel<__VA_ARGS__>;                                                          \

@@ -101,6 +101,12 @@ def test_fused_backward_at_headline_size_matches_the_oracle(device):
     # the two reference entry points at the same inputs, for the same comparison
     c1, c2, _, _ = ms.compression_backward(d(f1), d(f2), d(a_u), d(a_v), d(g_cu), d(g_cv))
     m1, m2 = ms.max_argmax_avg_backward(d(f1), d(f2), au, av, d(g_u), d(g_v))
+    # the same call through the two dense contractions (at this size the library takes the gather form by itself)
+    ms.set_max_avg_backward(ms.MAXAVG_DENSE)
+    try:
+        n1, n2 = ms.max_argmax_avg_backward(d(f1), d(f2), au, av, d(g_u), d(g_v))
+    finally:
+        ms.set_max_avg_backward(ms.MAXAVG_AUTO)
     for b in range(B):
         sl = slice(b, b + 1)
         ref = {}
@@ -110,13 +116,21 @@ def test_fused_backward_at_headline_size_matches_the_oracle(device):
             rm = O.max_argmax_avg_backward(x1, x2, au[sl].cpu(), av[sl].cpu(), g_u[sl].to(dt), g_v[sl].to(dt))
             ref[dt] = (rc[0] + rm[0], rc[1] + rm[1], rc[0], rc[1], rm[0], rm[1])
         r64, r32 = ref[torch.float64], ref[torch.float32]
-        # d_f1: a wave adds its 55 x 32 = 1760 products per output one after the other in the MFMA accumulator
-        # (4 such partial sums per output).  d_f2: the pixel range is cut into few long splits to keep the scratch
-        # small; a split adds up to 49 tiles of 32 pixels in one accumulator (the max/avg call gathers rows instead:
-        # sums of a few hundred).  chain_ratio turns these lengths into the expected ratio.
-        error_report(d1[sl], r64[0], r32[0], f"fused d_f1 [b={b}]", max_ratio=chain_ratio(1760))
+        # d_f1: a wave's register accumulator takes the products of two rows (64), then joins a running sum: the
+        # GPU's error has to stay within twice the fp32 CPU path's, and for the reference's two entry points no more
+        # elements may fall outside the plain rtol 1e-4 / atol 1e-5 than the CPU path leaves outside.
+        # d_f2: the pixel range is cut into few long splits to keep the scratch small; a split adds up to 49 tiles
+        # of 32 pixels in one accumulator (chain_ratio turns that length into the expected ratio); the max/avg
+        # call gathers rows instead: sums of a few hundred.
+        rep = error_report(d1[sl], r64[0], r32[0], f"fused d_f1 [b={b}]")
+        assert rep["gpu_outside_plain_tol"] <= rep["cpu32_outside_plain_tol"], rep
         error_report(d2[sl], r64[1], r32[1], f"fused d_f2 [b={b}]", max_ratio=chain_ratio(49 * 32))
-        error_report(c1[sl], r64[2], r32[2], f"compression d_f1 [b={b}]", max_ratio=chain_ratio(1760))
+        rep = error_report(c1[sl], r64[2], r32[2], f"compression d_f1 [b={b}]")
+        assert rep["gpu_outside_plain_tol"] <= rep["cpu32_outside_plain_tol"], rep
         error_report(c2[sl], r64[3], r32[3], f"compression d_f2 [b={b}]", max_ratio=chain_ratio(49 * 32))
-        error_report(m1[sl], r64[4], r32[4], f"max/avg d_f1 [b={b}]", max_ratio=chain_ratio(1760))
-        error_report(m2[sl], r64[5], r32[5], f"max/avg d_f2 [b={b}]", max_ratio=chain_ratio(49 * 32))
+        rep = error_report(m1[sl], r64[4], r32[4], f"max/avg d_f1 [b={b}]")
+        assert rep["gpu_outside_plain_tol"] <= rep["cpu32_outside_plain_tol"], rep
+        error_report(m2[sl], r64[5], r32[5], f"max/avg d_f2 [b={b}]")
+        rep = error_report(n1[sl], r64[4], r32[4], f"max/avg d_f1, dense [b={b}]")
+        assert rep["gpu_outside_plain_tol"] <= rep["cpu32_outside_plain_tol"], rep
+        error_report(n2[sl], r64[5], r32[5], f"max/avg d_f2, dense [b={b}]", max_ratio=chain_ratio(49 * 32))
