@@ -21,23 +21,34 @@ def _attention(K, seed):
     return torch.nn.Conv3d(2, K, 3, padding=1), torch.nn.Conv3d(2, K, 3, padding=1)
 
 
+# How the block runs its pyramid (fp32 contraction throughout): every level in shared launches ("all", the default),
+# level 0 in launches of its own and the others together ("first_alone"; with 2 levels "the others" is a single
+# level), one autograd node per level ("level"), and a block of one level, which always takes the per-level node.
+PYRAMID_CASES = [("all", 4), ("first_alone", 4), ("level", 4), ("all", 2), ("first_alone", 2), ("level", 2),
+                 ("all", 3), ("all", 1), ("level", 1)]
+
+
+@pytest.mark.parametrize("mode,levels", PYRAMID_CASES)
 @pytest.mark.parametrize("B,C,H,W,K,backward", [(1, 32, 16, 24, 2, True), (2, 64, 11, 20, 4, True), (1, 256, 24, 32, 0, False)])
-def test_corr_block_matches_full_4d_corr_block(device, B, C, H, W, K, backward):
+def test_corr_block_matches_full_4d_corr_block(device, B, C, H, W, K, backward, mode, levels):
     from separableflowthesis_amd import AlternateCorrBlockSepflow
+    if K == 0 and (mode, levels) not in (("all", 4), ("all", 1)):
+        pytest.skip("without attention modules the pyramid mode selects nothing")
     fmap1, fmap2, _, _ = O.make_inputs(B, H, W, C, seed=77)
     att = _attention(K, 5) if K else None
     # oracle: stored 4D volume, fp64
     r1 = fmap1.double().requires_grad_(backward)
     r2 = fmap2.double().requires_grad_(backward)
     ratt = tuple(copy.deepcopy(m).double() for m in att) if att else None
-    rc1, rc2 = O.CorrBlock4D(r1, r2, num_levels=4).separate(ratt)
+    rc1, rc2 = O.CorrBlock4D(r1, r2, num_levels=levels).separate(ratt)
     # operator on the GPU
     g1 = fmap1.to(device).requires_grad_(backward)
     g2 = fmap2.to(device).requires_grad_(backward)
     gatt = tuple(copy.deepcopy(m).to(device) for m in att) if att else None
-    blk = AlternateCorrBlockSepflow(g1, g2, None, num_levels=4, support_backward=backward)
+    blk = AlternateCorrBlockSepflow(g1, g2, None, num_levels=levels, support_backward=backward)
+    blk.pyramid_mode = mode
     c1, c2 = blk(None, sep=True, attention_weights=gatt)
-    nch = (2 + K) * 4
+    nch = (2 + K) * levels
     assert c1.shape == (B, nch, W, H, W) and c2.shape == (B, nch, H, H, W)
     assert_close(c1, rc1, "corr1")
     assert_close(c2, rc2, "corr2")

@@ -210,6 +210,42 @@ def test_fused_backward_is_the_sum_of_both_backwards(device, shape, K):
     assert_close(da_v, ra_v, "grad_attention_v", scale_atol=True)
 
 
+# From 2^25 (pixel, position) pairs on the library takes the combined d_f2 with 8-row workgroups, whose average term
+# of g_v comes from a table; sizes above that limit with one and two channel blocks, two and four weight channels,
+# rows that are no multiple of 32 columns and row counts that are no multiple of 8.
+@pytest.mark.parametrize("shape,K", [((2, 56, 100, 56, 100, 64), 2), ((1, 72, 120, 72, 120, 128), 4),
+                                     ((1, 78, 112, 78, 112, 128), 2), ((1, 64, 96, 64, 96, 256), 2)])
+def test_fused_backward_above_the_8_row_limit(device, shape, K):
+    B, H1, W1, H2, W2, C = shape
+    assert B * H1 * W1 * H2 * W2 >= 2 ** 25
+    f1, f2, g = op_inputs(B, H1, W1, H2, W2, C, seed=151 + K)
+    a_u = softmax_weights(B, H1, W1, K, W2, g)
+    a_v = softmax_weights(B, H1, W1, K, H2, g)
+    g_cu = torch.randn(B, H1, W1, K, H2, generator=g)
+    g_cv = torch.randn(B, H1, W1, K, W2, generator=g)
+    g_u = torch.randn(B, H1, W1, 2, H2, generator=g)
+    g_v = torch.randn(B, H1, W1, 2, W2, generator=g)
+    d = lambda t: t.to(device)
+    ms = _native()
+    _, _, au, av = ms.max_argmax_avg_forward(d(f1), d(f2))
+    d1, d2 = ms.fused_backward(d(f1), d(f2), au, av, d(g_u), d(g_v), d(a_u), d(a_v), d(g_cu), d(g_cv))
+    # the library's two separate backward calls
+    x1, x2, _, _ = ms.compression_backward(d(f1), d(f2), d(a_u), d(a_v), d(g_cu), d(g_cv))
+    y1, y2 = ms.max_argmax_avg_backward(d(f1), d(f2), au, av, d(g_u), d(g_v))
+    assert_close(d1, (x1 + y1).double(), "grad_fmap1_l0 against the two calls", scale_atol=True)
+    assert_close(d2, (x2 + y2).double(), "grad_fmap2_lk against the two calls", scale_atol=True)
+    # the fp64 oracle, one batch entry at a time (the 4D volume of these sizes is 0.3-0.6 GB in fp64)
+    for b in range(B):
+        sl = slice(b, b + 1)
+        m1, m2 = O.max_argmax_avg_backward(f1[sl].double(), f2[sl].double(), au[sl].cpu(), av[sl].cpu(),
+                                           g_u[sl].double(), g_v[sl].double())
+        c1, c2, _, _ = O.compression_backward(*(t[sl].double() for t in (f1, f2, a_u, a_v, g_cu, g_cv)))
+        assert_close(d1[sl], m1 + c1, "grad_fmap1_l0", scale_atol=True)
+        assert_close(d2[sl], m2 + c2, "grad_fmap2_lk", scale_atol=True)
+    e1, e2 = ms.fused_backward(d(f1), d(f2), au, av, d(g_u), d(g_v), d(a_u), d(a_v), d(g_cu), d(g_cv))
+    assert torch.equal(d1, e1) and torch.equal(d2, e2)
+
+
 def test_autograd_functions_match_autograd_through_4d(device):
     # mirrors overall_grad_test (scripts/test_maxavg_autograd.py:478-502, test_compression_autograd.py:442-484):
     # loss = sum of MSE(channel, 0) over all output channels, at a pooled level
