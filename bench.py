@@ -4,10 +4,11 @@
 A step is one pass of the hot path over one synthetic batch, called through the C ABI with every
 input already resident in HBM.  The headline workload is benchmark configuration 4 (B=2, C=256, 55x128,
 K'=4): max/argmax/avg forward, attention-compression forward, compression backward, max/avg backward.
-Prints ONE JSON line.  `value` is algorithmic TFLOP/s: (contraction passes x 2*B*N1*N2*C) / time,
-with passes = 7 for forward+backward with attention; epilogue flops are not counted.  Where the library runs
-the max/avg backward as gathers instead of its two contractions, the passes actually executed on the matrix
-cores and the timing of the all-dense step are reported beside it (`contraction_passes_executed`, `all_dense`).  The same line
+Prints ONE JSON line.  `value` is the MFMA TFLOP/s of the step: (contraction passes executed on the matrix cores x
+2*B*N1*N2*C) / time; epilogue flops are not counted.  The reference's formulation has 7 passes for forward+backward
+with attention; where the library runs the max/avg backward as gathers instead of its two contractions, 5 of them
+are executed and counted, and the algorithmic figure (7 passes over the same time) and the timing of the all-dense
+step stand beside it (`algorithmic_tflops`, `all_dense`).  `ms_per_step` is the figure to compare builds by.  The same line
 carries a `configs` table with all five benchmark configurations (ms/step, TFLOP/s, fraction of the
 fp32 MFMA peak, peak HBM allocated, dominant-kernel roofline), the CPU baseline (full-4D torch path on
 the host cores, one thread and all threads) and, as extras, the caller-level measurements.
@@ -123,28 +124,28 @@ def _cpu_step(name, torch, pixel_fraction=1):
     return once, sum(PASSES[o] for o in ops) * 2.0 * n1 * (H * W) * C
 
 
-def _time_cpu(fn, budget_s, max_reps, warm):
-    if warm:
-        fn()
+def _time_cpu(fn, budget_s, max_reps, min_reps=3):
+    """Mean of at least `min_reps` repeats after one warm-up call; more while the time budget lasts."""
+    fn()
     n, t0 = 0, time.perf_counter()
     while True:
         fn()
         n += 1
         dt = time.perf_counter() - t0
-        if dt >= budget_s or n >= max_reps:
+        if n >= min_reps and (dt >= budget_s or n >= max_reps):
             return dt / n * 1e3, n
 
 
 def cpu_baseline(torch, headline="cfg4"):
-    """Bounded sample of every workload at batch 1: the headline with all host threads (warm-up + repeats, ~10 s) and
-    with one thread (one repeat), the other configurations once each with all threads; config 5 on every 8th
-    image-1 pixel row (its whole 4D volume is 4.26 GB per copy)."""
+    """Bounded sample of every workload at batch 1, each figure the mean of at least 3 repeats after a warm-up call:
+    the headline with all host threads (~8 s) and with one thread, the other configurations with all threads;
+    config 5 on every 8th image-1 pixel row (its whole 4D volume is 4.26 GB per copy)."""
     threads = torch.get_num_threads()
     fn, flops = _cpu_step(headline, torch)
-    ms_all, n_all = _time_cpu(fn, 10.0, 12, warm=True)
+    ms_all, n_all = _time_cpu(fn, 8.0, 12)
     torch.set_num_threads(1)
     try:
-        ms_one, _ = _time_cpu(fn, 0.0, 1, warm=False)
+        ms_one, n_one = _time_cpu(fn, 0.0, 3)
     finally:
         torch.set_num_threads(threads)
     _, H, W, Kp, ops = WORKLOADS[headline]
@@ -155,7 +156,8 @@ def cpu_baseline(torch, headline="cfg4"):
         "host_cpus": os.cpu_count(),
         "sample": f"batch 1 of the workload (B=1, {H}x{W}, C={C}, K'={Kp}), full-4D torch path "
                   f"{'fwd+bwd via autograd' if 'C' in ops or 'F' in ops else 'fwd'}: {n_all} repeats after 1 warm-up with "
-                  f"{threads} threads, 1 repeat with 1 thread; same algorithmic flop count as the GPU step",
+                  f"{threads} threads, {n_one} repeats after 1 warm-up with 1 thread; the other configurations 3 repeats "
+                  f"after 1 warm-up each; same algorithmic flop count as the GPU step",
         "configs": {},
     }
     for name in sorted(WORKLOADS):
@@ -164,8 +166,9 @@ def cpu_baseline(torch, headline="cfg4"):
             continue
         frac = 8 if name == "cfg5" else 1
         fn, fl = _cpu_step(name, torch, frac)
-        ms, _ = _time_cpu(fn, 0.0, 1, warm=name != "cfg5")
-        ent = {"ms_per_step_b1": round(ms * frac, 1), "tflops": round(fl / (ms * 1e-3) / 1e12, 4), "cores": threads}
+        ms, nrep = _time_cpu(fn, 0.0, 3)
+        ent = {"ms_per_step_b1": round(ms * frac, 1), "tflops": round(fl / (ms * 1e-3) / 1e12, 4), "cores": threads,
+               "repeats": nrep}
         if frac > 1:
             ent["sample"] = f"every {frac}th image-1 pixel row, time scaled by {frac}"
         out["configs"][name] = ent
@@ -296,13 +299,14 @@ class Workload:
                   key=lambda k: kernels[k]["avg_ms"] * kernels[k]["launches_per_step"])
         ach = kernels[dom]["tflops"]
         passes = sum(PASSES[o] for o in ops)
-        value = passes * Wf / (ms * 1e-3) / 1e12
+        algorithmic = passes * Wf / (ms * 1e-3) / 1e12
         # The max/avg backward may run as gathers of feature rows instead of its two contractions (the library picks
-        # the faster way for the sizes): `value` keeps the algorithmic work of the step, 2*B*N1*N2*C per pass of the
-        # reference's formulation, and the passes that actually ran on the matrix cores are reported next to it,
-        # together with the same step timed with the dense max/avg backward.
+        # the faster way for the sizes): `tflops` counts the passes that actually ran on the matrix cores; the
+        # algorithmic work of the step, 2*B*N1*N2*C per pass of the reference's formulation, over the same time is
+        # reported next to it, together with the same step timed with the dense max/avg backward.
         gathered = any(k.endswith("_gather") for k in kernels)
         executed = passes - (PASSES["F"] if gathered else 0)
+        value = executed * Wf / (ms * 1e-3) / 1e12
         dense = None
         if gathered:
             prev_mode = self.lib.sepcorr_set_max_avg_backward(1)
@@ -323,12 +327,13 @@ class Workload:
             "frac_of_fp32_mfma_peak": round(value / PEAK_FP32_MFMA_TFLOPS, 4),
             "contraction_passes": passes, "gflop_per_step": round(passes * Wf / 1e9, 2),
             "contraction_passes_executed": executed,
-            "tflops_executed": round(executed * Wf / (ms * 1e-3) / 1e12, 3),
+            "algorithmic_tflops": round(algorithmic, 3),
             "max_avg_backward": ("gather" if gathered else "dense") if "F" in ops else None,
             "all_dense": dense,
-            "note": ("tflops / frac_of_fp32_mfma_peak count the algorithmic work of the step (contraction_passes x 2*B*N1*N2*C); "
-                     "the max/avg backward ran as gathers of feature rows, so contraction_passes_executed of them ran on the "
-                     "matrix cores (tflops_executed); all_dense is the same step with every pass a contraction")
+            "note": ("tflops / frac_of_fp32_mfma_peak count the contraction_passes_executed passes that ran on the matrix "
+                     "cores; the max/avg backward ran as gathers of feature rows instead of its two contractions; "
+                     "algorithmic_tflops counts all contraction_passes of the reference's formulation over the same time; "
+                     "all_dense is the same step with every pass a contraction")
                     if gathered else None,
             "peak_hbm_allocated_mib": round(peak / _MIB, 1),
             "backward_workspace_mib": round(self.workspace_bytes / _MIB, 1),
@@ -501,7 +506,7 @@ def main():
         "config": {"workload": head["workload"] + " " + OPS_TEXT,
                    "contraction_passes": head["contraction_passes"], "gflop_per_step": head["gflop_per_step"],
                    "contraction_passes_executed": head["contraction_passes_executed"],
-                   "tflops_executed": head["tflops_executed"], "max_avg_backward": head["max_avg_backward"],
+                   "algorithmic_tflops": head["algorithmic_tflops"], "max_avg_backward": head["max_avg_backward"],
                    "all_dense": head["all_dense"], "note": head["note"],
                    "frac_of_fp32_mfma_peak": head["frac_of_fp32_mfma_peak"],
                    "peak_hbm_allocated_mib": head["peak_hbm_allocated_mib"],

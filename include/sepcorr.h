@@ -160,6 +160,9 @@ int sepcorr_max_argmax_avg_backward(const float *f1, const float *f2,
  * counterpart in the reference.  The scratch memory is an array of SEPCORR_STATIC_SCRATCH_BYTES bytes inside the
  * library's device image (one copy per GPU, held until the process ends) instead of a workspace argument; the
  * call allocates nothing, creates no streams or events and runs all its kernels on `stream`.
+ *   - It always contracts in fp32: results are bit-equal to the workspace variant's under SEPCORR_CONTRACT_FP32 (the
+ *     default); with sepcorr_set_contraction(SEPCORR_CONTRACT_BF16X3) the workspace variant's dense d_f1 takes the
+ *     bf16-plane kernels (which allocate stream-ordered memory) and the two agree to rounding only.
  *   - Sizes that need more scratch than SEPCORR_STATIC_SCRATCH_BYTES are refused with SEPCORR_EWORKSPACE; use the
  *     workspace variant for them.  (Any size whose sepcorr_backward_workspace_bytes() fits is accepted; that figure
  *     also covers the other backward entry points, so somewhat larger sizes fit as well.)

@@ -3,8 +3,8 @@
 // one weight, so both feature gradients are sums of a few feature rows per output element.
 //
 // With S[p,(u,v)] = <f1[p,:], f2[(u,v),:]>, out_u[p,0,u] = max_v S, out_u[p,1,u] = mean_v S, out_v likewise over u
-// (max_avg_forward_kernel and its backward in libs/MemorySaver/MemorySaver_cuda_kernel.cu of the reference define
-// these outputs; the reference's backward visits every (p, u, v)):
+// (the reference defines these outputs in libs/MemorySaver/src/MemorySaver_kernel_forward.cu:328-533; its backward,
+// libs/MemorySaver/src/MemorySaver_kernel_max_avg_argmax_backward.cu:785-921, visits every (p, u, v)):
 //
 //   d_f1[p,:]     = sum_u g_u[p,0,u] f2[(u, am_u[p,u]),:] + sum_v g_v[p,0,v] f2[(am_v[p,v], v),:]           (gather)
 //                 + sum_u g_u[p,1,u] R[u,:] + sum_v g_v[p,1,v] Q[v,:]                                         (product)

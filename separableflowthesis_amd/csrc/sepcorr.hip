@@ -1615,6 +1615,11 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
     // no vector instruction but handles about one lane in three cycles: tried, five times slower).
     // Layout [group of 4 registers][lane][4]: 16-byte accesses without bank conflicts, wave-private, the same bytes
     // the wave's [pixel][channel] partial is written to at the end.
+    // Where registers allow, the first row of a block is a copy of the row body whose first products take the zero
+    // addend (PEEL).  The combined mode (both operators' dL/dS: 176 weight registers per lane) has no room for a
+    // second body (every form of it tried spilled hundreds of registers): there the accumulators are handed over and
+    // cleared in a branch ahead of the block's first row, 3 vector instructions per register and block.
+    constexpr bool PEEL = GMODE != GMODE_BOTH;
     const int FLUSH_ROWS = a.flush_rows;
     v4f *const run = reinterpret_cast<v4f *>(smem + wave * (TP * RS)) + lane;
     {
@@ -1644,14 +1649,17 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
         if constexpr (MAXT <= 256) asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
     };
     auto run_add_store = [&](int cbt, v4f (&x)[4]) {
-        float y[16];   // all copies first: a copy followed at once by the addition that reads it waits for it
 #pragma unroll
-        for (int e = 0; e < 16; ++e) y[e] = acc_value(cbt, e);
+        for (int half = 0; half < 2; ++half) {
+            float y[8];   // a batch of copies first: a copy followed at once by the addition that reads it waits for it
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
+            for (int e = 0; e < 8; ++e) y[e] = acc_value(cbt, 8 * half + e);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) x[q][e] += y[4 * q + e];
-            run[(cbt * 4 + q) * 64] = x[q];
+            for (int q = 0; q < 2; ++q) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) x[2 * half + q][e] += y[4 * q + e];
+                run[(cbt * 4 + 2 * half + q) * 64] = x[2 * half + q];
+            }
         }
     };
 
@@ -1762,6 +1770,7 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
         G[r] = gval<GMODE, KC>(wv[r], wu_n, ufirst, vmap(r, 0), true);
     }
     UW<GMODE, KC> wu_next = load_uw_row(min(ufirst + NUG, H2 - 1));
+    bool hand_over = false;   // the row that starts a block has a finished block in the accumulators
     auto compute = [&](int u, int g, v4f(&buf)[GS][NCB], auto fresh) {
         static_assert(GS == 2, "two G values are produced per group");
         if (g == 0) {
@@ -1771,15 +1780,23 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
         if (g == 0 && decltype(fresh)::value) {
             // first products of a new block: hand each accumulator to the running sum, then restart it from zero;
             // the running sum of the next accumulator is fetched while the matrix instruction of this one runs
+            // (one set of 16 registers: the running sum of the next accumulator is fetched into it once the additions
+            // of this one have read it, ahead of this one's matrix instruction, whose 64 cycles cover the fetch)
             const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            v4f rs[2][4];
-            run_load(0, rs[0]);
-            matrix_results_settled();
+            // (the first row of a piece has nothing to hand over: it only starts the accumulators.  The condition
+            // stands around the additions alone, the matrix instruction behind it is the same either way.)
+            v4f rs[4];
+            if (hand_over) {
+                run_load(0, rs);
+                matrix_results_settled();
+            }
 #pragma unroll
             for (int cbt = 0; cbt < NCB * 4; ++cbt) {
-                if (cbt + 1 < NCB * 4) run_load(cbt + 1, rs[(cbt + 1) & 1]);
-                __builtin_amdgcn_sched_barrier(0);
-                run_add_store(cbt, rs[cbt & 1]);
+                if (hand_over) {
+                    run_add_store(cbt, rs);
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (cbt + 1 < NCB * 4) run_load(cbt + 1, rs);
+                }
                 __builtin_amdgcn_sched_barrier(0);
                 acc[cbt >> 2][cbt & 3] = mfma(buf[0][cbt >> 2][cbt & 3], G[0], zero);
                 __builtin_amdgcn_sched_barrier(0);
@@ -1820,8 +1837,6 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
         issue(min(ufirst, H2 - 1), k, ring[k]);
         __builtin_amdgcn_sched_barrier(0);
     }
-    // (two copies of the row body, the first row of a block and the others: with one body and a branch around
-    // the block change the compiler copied all accumulators between the register files in every row)
     auto sweep_row = [&](int u, auto fresh) {
 #pragma unroll
         for (int g = 0; g < NG; ++g) {
@@ -1836,10 +1851,36 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    for (int u = ufirst; u < u_end;) {
-        sweep_row(u, std::true_type{});
-        u += NUG;
-        for (int j = 1; j < FLUSH_ROWS && u < u_end; ++j, u += NUG) sweep_row(u, std::false_type{});
+    if constexpr (PEEL) {
+        // two copies of the row body, the first row of a block and the others (with one body and a branch around the
+        // block change the compiler copied all accumulators between the register files in every row)
+        for (int u = ufirst; u < u_end;) {
+            hand_over = u != ufirst || vp > 0;   // (a later pass of 256 columns starts with the block of the pass before)
+            sweep_row(u, std::true_type{});
+            u += NUG;
+            for (int j = 1; j < FLUSH_ROWS && u < u_end; ++j, u += NUG) sweep_row(u, std::false_type{});
+        }
+    } else {
+        // one row body; between two blocks the accumulators join the running sum and are cleared
+        int rows_in_block = 0;
+        for (int u = ufirst; u < u_end; u += NUG) {
+            if (rows_in_block == FLUSH_ROWS) {
+                rows_in_block = 0;
+                __builtin_amdgcn_sched_barrier(0);
+                matrix_results_settled();
+#pragma unroll
+                for (int cbt = 0; cbt < NCB * 4; ++cbt) {
+                    v4f x[4];
+                    run_load(cbt, x);
+                    run_add_store(cbt, x);
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) acc[cbt >> 2][cbt & 3][e] = 0.f;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            ++rows_in_block;
+            sweep_row(u, std::false_type{});
+        }
     }
 
     }   // column passes
@@ -3352,7 +3393,8 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s
         a.sk_total = 0;
         // Rows per block of d_f1's register accumulation.  Measured at B=2, 55x128, C=256 (error against fp64 relative
         // to the fp32 CPU path's / kernel time): whole tiles 2.45 / 0.422 ms, 12 rows 1.28, 8 rows 1.08 / 0.434,
-        // 6 rows 0.97, 4 rows 0.83 / 0.444, 2 rows 0.66 / 0.468, 1 row 0.517 ms.
+        // 6 rows 0.97, 4 rows 0.83 / 0.444, 2 rows 0.66 / 0.468, 1 row 0.517 ms; the combined mode 0.546 ms for whole
+        // tiles, 0.553 for 12 rows, 0.575 for 4.
         a.flush_rows = 4;
 #define SEPCORR_DF1_K(...)                                                                         \
     do {                                                                                           \

@@ -116,9 +116,9 @@ def test_fused_backward_at_headline_size_matches_the_oracle(device):
             rm = O.max_argmax_avg_backward(x1, x2, au[sl].cpu(), av[sl].cpu(), g_u[sl].to(dt), g_v[sl].to(dt))
             ref[dt] = (rc[0] + rm[0], rc[1] + rm[1], rc[0], rc[1], rm[0], rm[1])
         r64, r32 = ref[torch.float64], ref[torch.float32]
-        # d_f1: a wave's register accumulator takes the products of two rows (64), then joins a running sum: the
-        # GPU's error has to stay within twice the fp32 CPU path's, and for the reference's two entry points no more
-        # elements may fall outside the plain rtol 1e-4 / atol 1e-5 than the CPU path leaves outside.
+        # d_f1: a wave's register accumulator takes the products of 4 rows (128), then
+        # joins a running sum: the GPU's error has to stay within twice the fp32 CPU path's, and for the reference's two
+        # entry points no more elements may fall outside the plain rtol 1e-4 / atol 1e-5 than the CPU path leaves outside.
         # d_f2: the pixel range is cut into few long splits to keep the scratch small; a split adds up to 49 tiles
         # of 32 pixels in one accumulator (chain_ratio turns that length into the expected ratio); the max/avg
         # call gathers rows instead: sums of a few hundred.
