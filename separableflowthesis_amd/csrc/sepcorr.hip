@@ -1330,6 +1330,14 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         int wlast = wfirst;                                              // the workgroup that holds step t1 - 1
         while (((long)(wlast + 1) * sk_total) / G < t1) ++wlast;
         const int npieces = wlast - wfirst + 1;
+        // Hand-over without a fence.  What it rests on: (1) the slot was written with sc0 sc1 stores, which are
+        // written through to device memory, and vmcnt counts such a store only when that write is acknowledged, so
+        // after vmcnt(0) in every wave and the barrier the whole piece is in memory; (2) the counter is a device-scope
+        // atomic, executed where all XCDs see one value, and it is issued after the barrier; (3) the piece that reads
+        // "I am the last" issues its slot reads after the atomic has returned (the flag goes through LDS and a
+        // barrier), and those reads carry sc0 sc1, which never take a line from this XCD's caches.  A release fence
+        // in front of the atomic (buffer_wbl2 sc1: write back every dirty line of this XCD's L2) adds nothing for
+        // these accesses and was measured to cost the forward sweeps 4-5 % at B=2, 55x128.
         __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave_e's words of the piece have arrived
         __syncthreads();
         int *flag = reinterpret_cast<int *>(smem);
