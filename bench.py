@@ -175,6 +175,48 @@ def cpu_baseline(torch, headline="cfg4"):
     return out
 
 
+def stored_volume_path_memory(torch, dev, names=("cfg3", "cfg4", "cfg5")):
+    """Part of the baseline leg: peak device memory of the stored-volume path (the oracle's CorrBlock4D: full 4D
+    volume, pooled pyramid, max / mean / einsum / Conv3d / interpolate through torch autograd) run on the GPU in fp32
+    at whole-batch size, forward and forward + backward (configuration 5 forward only), measured as the block's own
+    figures are: peak of torch's allocator above what is held before the call, dense upstream gradients.  This is the
+    second column of the both-models memory table of scripts/test_model.py:320-382."""
+    from oracle import oracle as O
+    out = {}
+    for name in names:
+        B, H, W, Kp, _ = WORKLOADS[name]
+        g = torch.Generator().manual_seed(1234)
+        fmap1 = torch.randn(B, C, H, W, generator=g).to(dev).requires_grad_()
+        fmap2 = torch.randn(B, C, H, W, generator=g).to(dev).requires_grad_()
+        torch.manual_seed(1234)
+        att = tuple(torch.nn.Conv3d(2, Kp, 3, padding=1).to(dev) for _ in range(2))
+        ups = None
+        ent = {}
+        for key, bw in (("forward", False), ("forward_backward", True)):
+            if bw and name == "cfg5":
+                continue
+            gc.collect()
+            torch.cuda.empty_cache()
+            torch.cuda.synchronize()
+            torch.cuda.reset_peak_memory_stats()
+            base = torch.cuda.memory_allocated()
+            with torch.set_grad_enabled(bw):
+                c1, c2 = O.CorrBlock4D(fmap1, fmap2, num_levels=4).separate(att)
+                if bw:
+                    if ups is None:
+                        ups = [torch.randn(c.shape, generator=g).to(dev) for c in (c1, c2)]
+                        base += sum(u.numel() * 4 for u in ups)   # held by the layers above, as in module_level()
+                    torch.autograd.backward([c1, c2], ups)
+            torch.cuda.synchronize()
+            ent[f"stored_4d_path_{key}_peak_allocated_mib"] = round((torch.cuda.max_memory_allocated() - base) / _MIB, 1)
+            del c1, c2
+        out[name] = ent
+        del fmap1, fmap2, att, ups
+        gc.collect()
+        torch.cuda.empty_cache()
+    return out
+
+
 # ------------------------------------------------------------------------------------------------
 # GPU: one workload through the C ABI
 # ------------------------------------------------------------------------------------------------
@@ -564,6 +606,14 @@ def main():
         out["lookup"] = lookup_level(B, H, W, torch, dev)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch, args.workload)
+        if "memory" in out:
+            # the stored-volume path beside the block, measured on this GPU (a baseline like the CPU timing above)
+            for name, ent in stored_volume_path_memory(torch, dev).items():
+                out["memory"][name].update(ent)
+            out["memory"]["what"] = ("peak of torch's allocator above what is held before the call: the block that never stores the "
+                                     "volume (forward_*, forward_backward_*) beside the stored-volume path (stored_4d_path_*: the "
+                                     "oracle's CorrBlock4D through torch autograd on this GPU); stored_4d_pyramid_would_take_mib is "
+                                     "the size of the 4D pyramid alone")
     print(json.dumps(out))
 
 
