@@ -291,7 +291,7 @@ struct FwdLevel {
     const float *st_wv, *st_wu, *z_ou, *st_ou, *dot_ou, *z_ov, *st_ov, *dot_ov;   // softmax inside (see FwdArgs)
     int H2, W2;
     int nvc;           // column chunks of 32 = waves side by side; the other waves of the workgroup form row groups
-    int steps, step0;  // steps of this level per tile, and of the levels before it
+    int steps, step0;  // units (steps, or half steps of two-row steps) of this level per tile, and of the levels before it
     int stage;
 };
 struct FwdArgs {
@@ -407,7 +407,12 @@ __device__ __attribute__((noinline)) void merge_pieces(KArgs ka_in, int lvl_in, 
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
-                        if (x[j][0][e] > acc4[0][e]) { acc4[0][e] = x[j][0][e]; acc4[1][e] = x[j][1][e]; }
+                        // (equal maxima keep the lower row: the rows of two neighbouring pieces may alternate)
+                        if (x[j][0][e] > acc4[0][e] ||
+                            (x[j][0][e] == acc4[0][e] && __float_as_int(x[j][1][e]) < __float_as_int(acc4[1][e]))) {
+                            acc4[0][e] = x[j][0][e];
+                            acc4[1][e] = x[j][1][e];
+                        }
                     acc4[2] += x[j][2];
                 }
             }
@@ -542,8 +547,18 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     if constexpr (SK) asm volatile("" : "+v"(tid));
     const int wave = tid >> 6, lane = tid & 63, pl = lane & 31, h = lane >> 5;
     const int tile = pb / S;
-    const int sa = pb - ubeg;                           // first step of this piece within its unit
-    const int sb = pe - ubeg;                           // one past its last step
+    // What is dealt out.  With one row per step and wave (UR == 1) it is steps.  With two (UR == 2) it is half steps:
+    // the first rows of all waves' steps, then their second rows.  Half step hs of a tile holds the rows
+    // ((hs / 2) NUG + ug) 2 + hs % 2 of the waves' row groups ug.  A piece [sa, sb) takes them two at a time, whatever
+    // the parity of sa, and when their number is odd its last step has one row per wave: that step's matrix
+    // instructions for the second row are left out, not masked.  (Whole steps cost the small grids a quarter of the
+    // chip: 2.25 steps of 8 rows per workgroup at B=1, 48x64 mean 3 for one workgroup in four.)  Only the form without
+    // row groups does this (rows of 97 to 256 columns): with row groups it measured slower (B=1, 48x64: 0.078 against
+    // 0.0745 ms; B=4, 48x64, where whole steps already divide evenly: 0.197 against 0.193 ms), without them faster
+    // (B=2, 55x128: 0.423 against 0.440 ms, of which 1.8 % is the 56th row that is no longer multiplied).
+    constexpr int HU = (SK && UR == 2 && WM == 0) ? 2 : 1;
+    const int sa = pb - ubeg;                           // first unit of this piece within its tile (and level)
+    const int sb = pe - ubeg;                           // one past its last unit
     const bool whole = !SK || !sk_total || (pb == ubeg && pe == uend);
     const int b = tile / a.tiles_per_batch;
     const int p0 = (tile % a.tiles_per_batch) * TP;
@@ -555,6 +570,16 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     const float *Lf2 = a.lev[lvl].f2, *Lwu = a.lev[lvl].wu;
     const int nvc = RG ? a.lev[lvl].nvc : nW, NUG = RG ? nW / nvc : 1;
     const int vcw = RG ? wave % nvc : wave, ug = RG ? wave / nvc : 0;
+    // row r of step `step` of the waves in row group g, and whether this piece owns it
+    auto row_of = [&](int step, int r, int g) {
+        if constexpr (HU == 2) {
+            const int hs = sa + 2 * step + r;
+            return ((hs >> 1) * NUG + g) * 2 + (hs & 1);
+        } else {
+            return ((sa + step) * NUG + g) * UR + r;
+        }
+    };
+    auto row_on = [&](int step, int r) { return HU == 1 || sa + 2 * step + r < sb; };
     if (seg_no > 0) __syncthreads();   // the previous piece has finished with LDS
     const KArgs kp = kernargs_now();
 
@@ -688,7 +713,8 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     }
     const int NJ = a.CP >> 3;
     const int NG = (NJ + GJ - 1) / GJ;
-    const int nsteps = sk_total ? sb - sa : ((H2 + UR - 1) / UR + NUG - 1) / NUG;   // steps per wave; rows past H2 are skipped
+    const int nsteps = sk_total ? (sb - sa + HU - 1) / HU : ((H2 + UR - 1) / UR + NUG - 1) / NUG;   // steps per wave; rows past H2 are skipped
+    const bool tail_single = HU == 2 && ((sb - sa) & 1);   // the last step has one row per wave
     const int T = nsteps * NG;
 
     v16f acc[UR];
@@ -702,7 +728,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     auto issue = [&](int step, int g, v4f(&buf)[UR][GJ]) {
 #pragma unroll
         for (int r = 0; r < UR; ++r) {
-            const int u = ((sa + step) * NUG + ug) * UR + r;
+            const int u = row_of(step, r, ug);
 #pragma unroll
             for (int jj = 0; jj < GJ; ++jj) {
                 const int j = g * GJ + jj;
@@ -720,8 +746,8 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         if constexpr (is_weighted(MODE)) {
             for (int idx = tid; idx < NUG * UR * KC * 32; idx += blockDim.x) {
                 const int p = idx & 31, k = (idx >> 5) % KC, ru = (idx / (32 * KC)) % UR, g2 = idx / (32 * KC * UR);
-                const int u = ((sa + step) * NUG + g2) * UR + ru;
-                if (u < H2 && p0 + p < N1) {
+                const int u = row_of(step, ru, g2);
+                if (u < H2 && row_on(step, ru) && p0 + p < N1) {
                     const float *src = pbr + (g2 * nvc) * WSTR + (ru * NPART + k) * 32 + p;
                     float x[8];   // all reads before the first addition
 #pragma unroll
@@ -753,8 +779,8 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         } else {
             for (int idx = tid; idx < NUG * UR * 32; idx += blockDim.x) {
                 const int p = idx & 31, ru = (idx >> 5) % UR, g2 = idx / (32 * UR);
-                const int u = ((sa + step) * NUG + g2) * UR + ru;
-                if (u < H2 && p0 + p < N1) {
+                const int u = row_of(step, ru, g2);
+                if (u < H2 && row_on(step, ru) && p0 + p < N1) {
                     const float *src = pbr + (g2 * nvc) * WSTR + (ru * NPART) * 32 + p;
                     float xm[8], xi[8], xs[8];
 #pragma unroll
@@ -812,8 +838,8 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         float *pb = part + (step & 1) * (UR * NPART * nW * 32) + wave * (UR * NPART * 32) + pl;
 #pragma unroll
         for (int ru = 0; ru < UR; ++ru) {
-            const int u = ((sa + step) * NUG + ug) * UR + ru;
-            if (u < H2) {
+            const int u = row_of(step, ru, ug);
+            if (u < H2 && row_on(step, ru)) {
                 if constexpr (is_weighted(MODE)) {
                     float sk[KC];
 #pragma unroll
@@ -884,7 +910,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
             if (g == 0) {
 #pragma unroll
                 for (int r = 0; r < UR; ++r) {
-                    const int u = ((sa + step) * NUG + ug) * UR + r;
+                    const int u = row_of(step, r, ug);
 #pragma unroll
                     for (int k = 0; k < KC; ++k)
                     {
@@ -920,7 +946,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         auto issueB = [&](int step, int J, v4f(&buf)[UR][6]) {
 #pragma unroll
             for (int r = 0; r < UR; ++r) {
-                const unsigned row = (unsigned)(((sa + step) * NUG + ug) * UR + r) * rowbytes;   // wave-uniform: travels in a scalar register
+                const unsigned row = (unsigned)row_of(step, r, ug) * rowbytes;   // wave-uniform: travels in a scalar register
 #pragma unroll
                 for (int i = 0; i < 6; ++i) buf[r][i] = buf_load4s(rsrc, lane_off, row + (unsigned)(J * 6 + i) * 1024u);   // i = 2 plane + k-step
             }
@@ -931,7 +957,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                 if (J == 0) {
 #pragma unroll
                     for (int r = 0; r < UR; ++r) {
-                        const int u = min(((sa + step) * NUG + ug) * UR + r, H2 - 1);
+                        const int u = min(row_of(step, r, ug), H2 - 1);
 #pragma unroll
                         for (int k = 0; k < KC; ++k) wur[r][k] = Lwu[(bp * a.KT + a.k0 + k) * H2 + u];
                     }
@@ -988,7 +1014,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         auto issueF = [&](int step, int J, v4f(&buf)[UR][4]) {
 #pragma unroll
             for (int r = 0; r < UR; ++r) {
-                const unsigned off = lane_off + (unsigned)(((sa + step) * NUG + ug) * UR + r) * rowbytes + (unsigned)J * 128u;
+                const unsigned off = lane_off + (unsigned)row_of(step, r, ug) * rowbytes + (unsigned)J * 128u;
 #pragma unroll
                 for (int tq = 0; tq < 4; ++tq) {
                     buf[r][tq] = buf_load4(rsrc, off + 16u * tq);
@@ -1003,14 +1029,15 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
             rsrc_wu = make_rsrc(Lwu + (size_t)b * N1 * a.KT * H2, (unsigned)N1 * a.KT * H2 * 4u);
             wu_lane = (unsigned)(((pok ? pix : 0) * a.KT + a.k0) * H2) * 4u;
         }
-        auto computeF = [&](int step, int J, v4f(&buf)[UR][4]) {
+        auto computeF = [&](int step, int J, v4f(&buf)[UR][4], auto single) {
+            constexpr int NR = decltype(single)::value ? 1 : UR;   // rows whose products are formed
             // the cross-wave sums of the step before (its partial results have been in LDS since that step's barrier)
             if (J == (NJB > 1 ? 1 : 0) && step > 0) combine(step - 1);
             if constexpr (is_weighted(MODE)) {
                 if (J == 0) {
 #pragma unroll
                     for (int r = 0; r < UR; ++r) {
-                        const int u = min(((sa + step) * NUG + ug) * UR + r, H2 - 1);
+                        const int u = min(row_of(step, r, ug), H2 - 1);
 #pragma unroll
                         for (int k = 0; k < KC; ++k) wur[r][k] = buf_load1s(rsrc_wu, wu_lane, (unsigned)(k * H2 + u) * 4u);
                     }
@@ -1039,7 +1066,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                         else acc[0] = mfma(buf[0][tq][t], bv[t], first && t == 0 ? zero16 : acc[0]);
                     } else {
 #pragma unroll
-                        for (int r = 0; r < UR; ++r) acc[r] = mfma(buf[r][tq][t], bv[t], first && t == 0 ? zero16 : acc[r]);
+                        for (int r = 0; r < NR; ++r) acc[r] = mfma(buf[r][tq][t], bv[t], first && t == 0 ? zero16 : acc[r]);
                     }
                 }
             };
@@ -1086,13 +1113,24 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
             v4f ring[NB][UR][4];
 #pragma unroll
             for (int k = 0; k < NB - 1; ++k) issueF(0, k, ring[k]);
-            for (int step = 0; step < nsteps; ++step) {
+            const int nfull = tail_single ? nsteps - 1 : nsteps;
+            for (int step = 0; step < nfull; ++step) {
 #pragma unroll
                 for (int J = 0; J < NJT; ++J) {
                     constexpr int AHEAD = NB - 1;
                     if (J + AHEAD < NJT) issueF(step, J + AHEAD, ring[(J + AHEAD) % NB]);
                     else if (step + 1 < nsteps) issueF(step + 1, J + AHEAD - NJT, ring[(J + AHEAD) % NB]);
-                    computeF(step, J, ring[J % NB]);
+                    computeF(step, J, ring[J % NB], std::false_type{});
+                }
+            }
+            if constexpr (HU == 2) {
+                if (tail_single) {   // one row per wave (the loads still fetch both)
+#pragma unroll
+                    for (int J = 0; J < NJT; ++J) {
+                        constexpr int AHEAD = NB - 1;
+                        if (J + AHEAD < NJT) issueF(nfull, J + AHEAD, ring[(J + AHEAD) % NB]);
+                        computeF(nfull, J, ring[J % NB], std::true_type{});
+                    }
                 }
             }
         } else {
@@ -1111,7 +1149,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                 for (int k = 0; k < NB; ++k) {
                     if (it + k < TF) {
                         if (it + k + NB - 1 < TF) { issueF(is, iJ, ring[(k + NB - 1) % NB]); advance(is, iJ); }
-                        computeF(cs, cJ, ring[k]);
+                        computeF(cs, cJ, ring[k], std::false_type{});
                         advance(cs, cJ);
                     }
                 }
@@ -1150,7 +1188,26 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     if (Lstage && vp == vpasses - 1) {
         __syncthreads();
         const int cht = (is_weighted(MODE)) ? a.KT : 2, ch0 = (is_weighted(MODE)) ? a.k0 : 0;
-        const int u0 = whole ? 0 : sa * NUG * UR, nu = (whole ? H2 : min(H2, sb * NUG * UR)) - u0;
+        // the piece's rows lie in [u0, u0 + nu); where half steps are dealt out, the rows of its first and last step
+        // alternate with those of its neighbours: row_mine() tells them apart
+        int u0 = 0, nu = H2;
+        if (!whole) {
+            if constexpr (HU == 2) {
+                u0 = ((sa >> 1) * NUG) * 2 + (sa & 1);
+                nu = min(H2, ((((sb - 1) >> 1) * NUG + NUG - 1) * 2 + ((sb - 1) & 1)) + 1) - u0;
+            } else {
+                u0 = sa * NUG * UR;
+                nu = min(H2, sb * NUG * UR) - u0;
+            }
+        }
+        auto row_mine = [&](int u) {
+            if constexpr (HU == 2) {
+                const int hs = 2 * ((u >> 1) / NUG) + (u & 1);
+                return whole || (hs >= sa && hs < sb);
+            } else {
+                return true;
+            }
+        };
         // A (pixel, channel) row of nu floats goes to 8, 16, 32 or 64 neighbouring lanes, so that several short rows
         // share a wave; the row index is the same for all lanes of a group (no division by nu anywhere).
         const int lsh = nu > 32 ? 6 : nu > 16 ? 5 : nu > 8 ? 4 : 3;
@@ -1166,7 +1223,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
                 for (int t = 0; t < UNR; ++t) {
                     const int r = r0 + t * nW * rpi;
                     const int p = r / NCHO, ch = r - p * NCHO, u = u0 + uu;
-                    const bool ok = r < TP * NCHO && p0 + p < N1;
+                    const bool ok = r < TP * NCHO && p0 + p < N1 && row_mine(u);
                     off[t] = ok ? ((((size_t)b * N1 + p0 + p) * cht + ch0 + ch) * H2 + u) : (size_t)-1;
                     lds_i[t] = r * H2 + u;
                     pk[t] = p * KC + ch;
@@ -1188,7 +1245,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         if constexpr (MODE == MODE_ARGMAX) {
             for (int p = wave_e * rpi + lr; p < TP; p += nW * rpi)
                 for (int uu = lu; uu < nu; uu += lpr)
-                    if (p0 + p < N1) ke->lev[lvl].am_u[((size_t)b * N1 + p0 + p) * H2 + u0 + uu] = ostage_am[p * H2 + u0 + uu];
+                    if (p0 + p < N1 && row_mine(u0 + uu)) ke->lev[lvl].am_u[((size_t)b * N1 + p0 + p) * H2 + u0 + uu] = ostage_am[p * H2 + u0 + uu];
         }
     }
     // merge the running state of the row groups into group 0, one group at a time, through the LDS
@@ -2870,14 +2927,21 @@ __global__ void __launch_bounds__(256) zero_ints_kernel(int *p, int n) {
 // steps of all tiles are dealt out evenly instead and pieces of a tile are combined by whichever finishes last.
 struct FwdSplit {
     bool on;
-    int G, S;          // workgroups, steps per tile
-    long T;            // steps in total
+    int G, S;          // workgroups, units per tile
+    long T;            // units in total
     size_t count_bytes, slot_floats, bytes;   // scratch: counters, one slot, everything
 };
 constexpr int kCUs = 256;
-FwdSplit fwd_split(int tiles, int H2, int W2, int rows_per_step, int nq, int wgs_per_cu) {
+// What a sweep deals out per tile: steps (ur rows per wave, nug row groups) where a wave takes one row per step, half
+// steps where it takes two (fwd_kernel: HU); the second half of the last step is left out when it holds no row.
+int fwd_units(int H2, int ur, int nug, int vpasses) {
+    const int steps = (H2 + ur * nug - 1) / (ur * nug);
+    if (ur != 2 || nug != 1 || vpasses != 1) return steps;   // (row groups, column passes: whole steps, as the kernel's HU says)
+    return 2 * steps - ((steps - 1) * 2 * nug + 1 >= H2 ? 1 : 0);
+}
+FwdSplit fwd_split(int tiles, int H2, int W2, int ur, int nug, int vpasses, int nq, int wgs_per_cu) {
     FwdSplit f;
-    f.S = (H2 + rows_per_step - 1) / rows_per_step;
+    f.S = fwd_units(H2, ur, nug, vpasses);
     f.T = (long)tiles * f.S;
     const long places = (long)kCUs * wgs_per_cu;
     const double plain = (double)tiles / (double)(((tiles + places - 1) / places) * places);
@@ -2898,7 +2962,7 @@ size_t fwd_split_bytes(int B, int H1, int W1, int H2, int W2, int K) {
     size_t best = 0;
     for (int ur = 1; ur <= 2; ++ur)
         for (int per = 1; per <= (nW <= 4 ? 2 : 1); ++per) {
-            const FwdSplit f = fwd_split(B * tpb, H2, W2, ur * wg.nug, nq, per);
+            const FwdSplit f = fwd_split(B * tpb, H2, W2, ur, wg.nug, wg.vpasses, nq, per);
             if (f.bytes > best) best = f.bytes;
         }
     return best;
@@ -2935,7 +2999,7 @@ int launch_fwd(FwdArgs a, int B, hipStream_t s) {
     const dim3 block(64 * nW);
     a.sk_total = 0;
     if (a.ws != nullptr && !a.f2_planes) {
-        const FwdSplit f = fwd_split(B * a.tiles_per_batch, a.H2, a.W2, UR * wg.nug, NPART, (nW <= 4 && lds <= 80 * 1024) ? 2 : 1);
+        const FwdSplit f = fwd_split(B * a.tiles_per_batch, a.H2, a.W2, UR, wg.nug, wg.vpasses, NPART, (nW <= 4 && lds <= 80 * 1024) ? 2 : 1);
         if (f.on && f.bytes <= a.ws_bytes) {
             a.sk_total = (int)f.T;
             a.sk_steps = f.S;
