@@ -55,6 +55,13 @@ def measured_traffic(workload):
             m = re.match(r"traffic\s+(\S+)\s+([\d.]+)\s+([\d.]+)\s+([\d.]+)\s*$", line)
             if m:
                 out[m.group(1)] = float(m.group(4)) * _MIB
+        return out
+    # the other configurations share one summary: `traffic <workload> <label> <fetch_KiB> <write_KiB> <MiB>`
+    for path in sorted(os.listdir(os.path.join(ROOT, "profiles"))):
+        for line in open(os.path.join(ROOT, "profiles", path)):
+            m = re.match(r"traffic\s+(\S+)\s+(\S+)\s+([\d.]+)\s+([\d.]+)\s+([\d.]+)\s*$", line)
+            if m and m.group(1) == workload:
+                out[m.group(2)] = float(m.group(5)) * _MIB
     return out
 
 
