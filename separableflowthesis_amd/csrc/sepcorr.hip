@@ -1001,7 +1001,8 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(Lf2 + (size_t)b * H2 * W2 * C, nbytes);
         const unsigned lane_off = vrow_ok ? ((unsigned)vrow * C + 16u * h) * 4u : nbytes;
         const int NJB = (CMODE == 3) ? 8 : (C >> 5);
-        constexpr bool BPIPE = !(is_weighted(MODE) && KC >= 3);   // needs 16 more registers
+        constexpr bool HEAVY = is_weighted(MODE) && KC >= 3;
+        constexpr bool BPIPE = true;   // needs 16 more registers
         constexpr bool DUAL = UR == 1 && !(is_weighted(MODE) && KC >= 3);
         v4f bcur[4];
         if constexpr (BPIPE) {
@@ -1109,7 +1110,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         // so NB-1 blocks of MFMA work cover the latency of an L2 miss.
         if constexpr (CMODE == 3) {
             constexpr int NJT = 8;
-            constexpr int NB = (UR == 1) ? 4 : 2;   // divides NJT: ring slots are static across steps
+            constexpr int NB = (UR == 1 && !HEAVY) ? 4 : 2;   // divides NJT: ring slots are static across steps
             v4f ring[NB][UR][4];
 #pragma unroll
             for (int k = 0; k < NB - 1; ++k) issueF(0, k, ring[k]);
