@@ -6,8 +6,11 @@
 // (core/sepflow.py:59-60, core/corr.py:437-446).  The convolution's depth axis is L, its height and
 // width are H1 and W1: weight[k][c][dl][di][dj].
 //
-// HBM-bound element-wise work (54 K multiply-adds per output): one wave per image-1 pixel, lanes along
-// L (rows of L contiguous floats: every access is coalesced), softmax statistics by wave reduction.
+// Vector-instruction work (54 K multiply-adds per output) with lanes along L (rows of L contiguous floats: every
+// access is coalesced), softmax statistics by wave reduction.  Rows of up to 256 entries run on the strip kernels: a
+// group of lanes takes a few neighbouring pixels, fetches the rows under them once and gets the neighbours along L
+// from the lanes beside it; anything else (longer rows, rows that are no multiple of the vector width they would
+// need, unaligned tensors) runs one wave per pixel.
 // The backward pass is three kernels: softmax backward -> dlogits (scratch), the transposed
 // convolution for d_sep, and the weight gradient as per-workgroup partial sums that a last kernel
 // adds in a fixed order (deterministic, no atomics).
@@ -205,6 +208,251 @@ __global__ void __launch_bounds__(64 * WPB) att_forward_long_kernel(const AttJob
     }
 }
 
+// ---- Strips ----------------------------------------------------------------------------------------------------
+// The kernels above give every pixel a wave (or a group of lanes) of its own, which fetches the rows of its nine
+// neighbours three times each (shifted by -1, 0, +1 along L): 54 loads per position for 54 K multiply-adds.  The strip
+// kernels give a group of lanes SP neighbouring pixels of one image row.  The group fetches the three image rows of
+// the SP + 2 columns under the strip once (6 (SP + 2) vector loads for 54 K SP NV multiply-adds per lane), and a
+// lane gets the neighbours along L from the lanes beside it (one data-parallel-primitive move each) instead of from
+// memory.  A lane holds NV consecutive positions l = NV * lane + e (rows of up to 64 NV entries; NV > 1 needs L to
+// be a multiple of NV and 4 NV-byte aligned tensors), so for e inside the vector the neighbour is the lane's own.
+// NV floats at p if ok, else zeros.  No branch: lanes that are not ok read `safe` (any readable, aligned address of
+// the same tensor) and discard it, so the loads of a window are issued back to back.
+template <int NV>
+__device__ __forceinline__ void load_vec(const float *p, const float *safe, bool ok, float (&x)[NV]) {
+    const float *q = ok ? p : safe;
+    if constexpr (NV == 1) {
+        const float v = *q;
+        x[0] = ok ? v : 0.f;
+    } else if constexpr (NV == 2) {
+        const float2 v = *reinterpret_cast<const float2 *>(q);
+        x[0] = ok ? v.x : 0.f; x[1] = ok ? v.y : 0.f;
+    } else {
+        const float4 v = *reinterpret_cast<const float4 *>(q);
+        x[0] = ok ? v.x : 0.f; x[1] = ok ? v.y : 0.f; x[2] = ok ? v.z : 0.f; x[3] = ok ? v.w : 0.f;
+    }
+}
+template <int NV>
+__device__ __forceinline__ void store_vec(float *p, const float (&x)[NV]) {
+    if constexpr (NV == 1) p[0] = x[0];
+    else if constexpr (NV == 2) *reinterpret_cast<float2 *>(p) = make_float2(x[0], x[1]);
+    else *reinterpret_cast<float4 *>(p) = make_float4(x[0], x[1], x[2], x[3]);
+}
+// a value that is the same in every lane, as a scalar
+__device__ __forceinline__ float uniform(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, x)));
+}
+// the value of the lane below / above (0 at the ends of the wave)
+__device__ __forceinline__ float lane_below(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x138, 0xf, 0xf, true));   // wave_shr:1
+}
+__device__ __forceinline__ float lane_above(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x130, 0xf, 0xf, true));   // wave_shl:1
+}
+// Sum or maximum over each aligned group of lw = 16, 32 or 64 lanes by data-parallel-primitive steps (no LDS round
+// trips: a chain of six dependent vector instructions instead of six permutes); the result stands in the highest lane
+// of the group.  Sums fill absent source lanes with 0; maxima keep the lane's own value there.
+template <bool MAX, int CTRL, int RM, int BM>
+__device__ __forceinline__ float reduce_step(float x) {
+    const int xi = __builtin_bit_cast(int, x);
+    if constexpr (MAX) return fmaxf(x, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(xi, xi, CTRL, RM, BM, false)));
+    else return x + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, xi, CTRL, RM, BM, true));
+}
+template <bool MAX>
+__device__ __forceinline__ float group_reduce_top(float x, int lw) {
+    x = reduce_step<MAX, 0x111, 0xf, 0xf>(x);                 // row_shr:1
+    x = reduce_step<MAX, 0x112, 0xf, 0xf>(x);                 // row_shr:2
+    x = reduce_step<MAX, 0x114, 0xf, 0xe>(x);                 // row_shr:4
+    x = reduce_step<MAX, 0x118, 0xf, 0xc>(x);                 // row_shr:8: lane 15 of every row holds the row's result
+    if (lw > 16) x = reduce_step<MAX, 0x142, 0xa, 0xf>(x);    // row_bcast:15 into rows 1 and 3
+    if (lw > 32) x = reduce_step<MAX, 0x143, 0xc, 0xf>(x);    // row_bcast:31 into rows 2 and 3
+    return x;
+}
+// the value of the group's highest lane in every lane of the group
+__device__ __forceinline__ float group_top(float x, int lw) {
+    if (lw == 64) return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 63));
+    return __shfl(x, (int)(threadIdx.x & 63) | (lw - 1));
+}
+// lanes per strip for rows of L entries held NV to a lane
+__host__ __device__ inline int strip_lanes(int L, int NV) {
+    const int n = (L + NV - 1) / NV;
+    return n <= 16 ? 16 : n <= 32 ? 32 : 64;
+}
+
+struct Strip {
+    bool active;     // the group has a strip (whole groups are idle past the end)
+    bool first, last;   // this lane is the lowest / highest of its group
+    int lw, lane;    // lanes of the group; this lane's number within it
+    int i, j0, n;    // image row, first column, pixels (1..SP)
+    long pix0;       // flattened (b, i, j0)
+};
+// the strip of this lane's group in wave-strip `wsidx` (a wave-strip = the 64 / lw strips a wave holds side by side)
+template <int SP>
+__device__ __forceinline__ Strip strip_at(const AttArgs &a, long wsidx, int lw) {
+    Strip t;
+    const int l64 = threadIdx.x & 63, sub = l64 / lw;
+    const int ns = (a.W1 + SP - 1) / SP;
+    const long s = wsidx * (64 / lw) + sub;
+    t.active = s < (long)a.B * a.H1 * ns;
+    const long row = s / ns;
+    t.i = (int)(row % a.H1);
+    t.j0 = (int)(s % ns) * SP;
+    t.n = a.W1 - t.j0 < SP ? a.W1 - t.j0 : SP;
+    t.pix0 = row * a.W1 + t.j0;
+    t.lw = lw;
+    t.lane = l64 & (lw - 1);
+    t.first = t.lane == 0;
+    t.last = t.lane == lw - 1;
+    return t;
+}
+template <int SP>
+__device__ __forceinline__ Strip strip_of(const AttArgs &a, int bx, int lw) {
+    return strip_at<SP>(a, (long)bx * WPB + (threadIdx.x >> 6), lw);
+}
+// wave-strips of a tensor; workgroups of a launch that gives every wave one
+static long wave_strips(int B, int H1, int W1, int L, int NV, int SP) {
+    const long per = 64 / strip_lanes(L, NV);
+    const long total = (long)B * H1 * ((W1 + SP - 1) / SP);
+    return (total + per - 1) / per;
+}
+template <int SP>
+static unsigned strip_groups(int B, int H1, int W1, int L, int NV) {
+    return (unsigned)((wave_strips(B, H1, W1, L, NV, SP) + WPB - 1) / WPB);
+}
+
+// The window of a strip: SP + 2 columns x 3 image rows x NCHAN channels of one tensor whose rows are (pixel, channel)
+// x L, with the values of the lanes beside (xm: position l - 1 of the lane's first entry, xp: l + 1 of its last).
+// fetch() issues the loads (tensors have fewer than 2^31 elements: 32-bit element offsets); finish() derives xm / xp.
+template <int NV, int SP, int NCHAN>
+struct Window {
+    float x[SP + 2][3][NCHAN][NV], xm[SP + 2][3][NCHAN], xp[SP + 2][3][NCHAN];
+    // chan0: first channel to fetch, nchan_total: channels per pixel in memory
+    __device__ __forceinline__ void fetch(const float *base, const Strip &t, int H1, int W1, int L, int nchan_total, int chan0) {
+        const bool lok = t.active && t.lane * NV < L;
+        const int p0 = (int)t.pix0;
+#pragma unroll
+        for (int col = 0; col < SP + 2; ++col) {
+            const int jj = t.j0 + col - 1;
+#pragma unroll
+            for (int r = 0; r < 3; ++r) {
+                const int ii = t.i + r - 1;
+                const bool ok = lok && ii >= 0 && ii < H1 && jj >= 0 && jj < W1 && col <= t.n + 1;
+                const int off = ((p0 + (r - 1) * W1 + (col - 1)) * nchan_total + chan0) * L + t.lane * NV;
+#pragma unroll
+                for (int c = 0; c < NCHAN; ++c) load_vec<NV>(base + (off + c * L), base, ok, x[col][r][c]);
+            }
+        }
+    }
+    __device__ __forceinline__ void finish(const Strip &t) {
+#pragma unroll
+        for (int col = 0; col < SP + 2; ++col)
+#pragma unroll
+            for (int r = 0; r < 3; ++r)
+#pragma unroll
+                for (int c = 0; c < NCHAN; ++c) {
+                    xm[col][r][c] = lane_below(x[col][r][c][NV - 1]);
+                    xp[col][r][c] = lane_above(x[col][r][c][0]);
+                }
+        if (t.lw < 64) {   // several strips in a wave: nothing crosses from one to the next
+#pragma unroll
+            for (int col = 0; col < SP + 2; ++col)
+#pragma unroll
+                for (int r = 0; r < 3; ++r)
+#pragma unroll
+                    for (int c = 0; c < NCHAN; ++c) {
+                        xm[col][r][c] = t.first ? 0.f : xm[col][r][c];
+                        xp[col][r][c] = t.last ? 0.f : xp[col][r][c];
+                    }
+        }
+    }
+    // entry e of the lane shifted by s = -1, 0, +1 along L
+    __device__ __forceinline__ float at(int col, int r, int c, int s, int e) const {
+        if (s == 0) return x[col][r][c][e];
+        if (s < 0) return e == 0 ? xm[col][r][c] : x[col][r][c][e - 1];
+        return e == NV - 1 ? xp[col][r][c] : x[col][r][c][e + 1];
+    }
+};
+
+// Forward over strips.  Filter by filter: the 54 weights of a filter go from LDS into registers once per strip and
+// serve its SP pixels.
+template <int NV, int SP>
+__global__ void __launch_bounds__(64 * WPB) att_forward_strip_kernel(const AttJobs m) {
+    ATT_JOB(m);
+    __shared__ __attribute__((aligned(16))) float ws[MAXK * 56 + MAXK];   // [k][56]: 54 weights (c, dl, di, dj) + 2 pad
+    const int K = a.K, L = a.L, H1 = a.H1, W1 = a.W1;
+    for (int t = threadIdx.x; t < K * 56; t += blockDim.x) ws[t] = t % 56 < 54 ? a.weight[(t / 56) * 54 + t % 56] : 0.f;
+    for (int t = threadIdx.x; t < K; t += blockDim.x) ws[MAXK * 56 + t] = a.bias ? a.bias[t] : 0.f;
+    __syncthreads();
+    const int lw = strip_lanes(L, NV);
+    const Strip st = strip_of<SP>(a, bx, lw);
+    if (!st.active) return;   // whole groups leave: the reductions below stay inside a group
+    Window<NV, SP, 2> win;
+    win.fetch(a.sep, st, H1, W1, L, 2, 0);
+    win.finish(st);
+    const bool lok = st.lane * NV < L;
+#pragma unroll 1
+    for (int k = 0; k < K; ++k) {
+        float w[56];   // the same in every lane: kept in scalar registers
+#pragma unroll
+        for (int q = 0; q < 14; ++q) {   // 14 reads of 16 bytes, the same address in every lane
+            const float4 w4 = *reinterpret_cast<const float4 *>(&ws[k * 56 + 4 * q]);
+            w[4 * q] = uniform(w4.x); w[4 * q + 1] = uniform(w4.y); w[4 * q + 2] = uniform(w4.z); w[4 * q + 3] = uniform(w4.w);
+        }
+        const float bias = uniform(ws[MAXK * 56 + k]);
+        float logit[SP][NV];
+#pragma unroll
+        for (int t = 0; t < SP; ++t)
+#pragma unroll
+            for (int e = 0; e < NV; ++e) {
+                float z = bias;
+#pragma unroll
+                for (int tap = 0; tap < 54; ++tap) {
+                    const int c = tap / 27, dl = (tap / 9) % 3, nb = tap % 9;
+                    z = fmaf(w[tap], win.at(t + nb % 3, nb / 3, c, dl - 1, e), z);
+                }
+                logit[t][e] = z;
+            }
+        // row statistics of the SP pixels side by side (independent chains)
+        float mx[SP], sum[SP], ex[SP][NV];
+#pragma unroll
+        for (int t = 0; t < SP; ++t) {
+            float v = logit[t][0];
+#pragma unroll
+            for (int e = 1; e < NV; ++e) v = fmaxf(v, logit[t][e]);
+            mx[t] = group_reduce_top<true>(lok ? v : -INFINITY, lw);
+        }
+#pragma unroll
+        for (int t = 0; t < SP; ++t) mx[t] = group_top(mx[t], lw);
+#pragma unroll
+        for (int t = 0; t < SP; ++t) {
+            float v = 0.f;
+#pragma unroll
+            for (int e = 0; e < NV; ++e) {
+                ex[t][e] = lok ? __expf(logit[t][e] - mx[t]) : 0.f;
+                v += ex[t][e];
+            }
+            sum[t] = group_reduce_top<false>(v, lw);
+        }
+#pragma unroll
+        for (int t = 0; t < SP; ++t) sum[t] = group_top(sum[t], lw);
+#pragma unroll
+        for (int t = 0; t < SP; ++t) {
+            const long pix = st.pix0 + t;
+            if (t < st.n && a.stats && st.lane == 0) {
+                a.stats[2 * (pix * K + k)] = mx[t];
+                a.stats[2 * (pix * K + k) + 1] = sum[t];
+            }
+            if (t < st.n && lok) {
+                const float inv = 1.f / sum[t];
+                float o[NV];
+#pragma unroll
+                for (int e = 0; e < NV; ++e) o[e] = a.logits_only ? logit[t][e] : ex[t][e] * inv;
+                store_vec<NV>(a.out + (pix * K + k) * L + st.lane * NV, o);
+            }
+        }
+    }
+}
+
 // dlogits = a * (grad_a - sum_l a * grad_a), one wave per pixel.
 __global__ void __launch_bounds__(64 * WPB) att_softmax_backward_kernel(const AttJobs m) {
     ATT_JOB(m);
@@ -396,6 +644,221 @@ __global__ void __launch_bounds__(256) att_weight_reduce_kernel(const float *par
     }
 }
 
+// d_sep over strips.  Filter by filter: a window of the filter's logit gradients (fetched while the previous filter is
+// applied), its 2 x 27 weights in scalar registers, 2 x NV accumulators per pixel of the strip.
+template <int NV, int SP>
+__global__ void __launch_bounds__(64 * WPB) att_input_backward_strip_kernel(const AttJobs m) {
+    ATT_JOB(m);
+    __shared__ __attribute__((aligned(16))) float ws[MAXK * 56];   // [k][c][28]: 27 weights (dl, di, dj) + 1 pad
+    const int K = a.K, L = a.L, H1 = a.H1, W1 = a.W1;
+    for (int t = threadIdx.x; t < K * 56; t += blockDim.x) ws[t] = t % 28 < 27 ? a.weight[(t / 28) * 27 + t % 28] : 0.f;
+    __syncthreads();
+    const int lw = strip_lanes(L, NV);
+    const Strip st = strip_of<SP>(a, bx, lw);
+    if (!st.active) return;
+    const bool lok = st.lane * NV < L;
+    float d[SP][2][NV];
+#pragma unroll
+    for (int t = 0; t < SP; ++t)
+#pragma unroll
+        for (int c = 0; c < 2; ++c)
+#pragma unroll
+            for (int e = 0; e < NV; ++e) d[t][c][e] = 0.f;
+    Window<NV, SP, 1> win, nxt;
+    nxt.fetch(a.dlogits, st, H1, W1, L, K, 0);
+#pragma unroll 1
+    for (int k = 0; k < K; ++k) {
+#pragma unroll
+        for (int col = 0; col < SP + 2; ++col)
+#pragma unroll
+            for (int r = 0; r < 3; ++r)
+#pragma unroll
+                for (int e = 0; e < NV; ++e) win.x[col][r][0][e] = nxt.x[col][r][0][e];
+        win.finish(st);
+        if (k + 1 < K) nxt.fetch(a.dlogits, st, H1, W1, L, K, k + 1);
+        float w[56];   // the same in every lane: kept in scalar registers
+#pragma unroll
+        for (int q = 0; q < 14; ++q) {
+            const float4 w4 = *reinterpret_cast<const float4 *>(&ws[k * 56 + 4 * q]);
+            w[4 * q] = uniform(w4.x); w[4 * q + 1] = uniform(w4.y); w[4 * q + 2] = uniform(w4.z); w[4 * q + 3] = uniform(w4.w);
+        }
+        // the gradient of pixel (i, j) takes tap (dl, di, dj) from pixel (i - di + 1, j - dj + 1) at l - dl + 1
+#pragma unroll
+        for (int t = 0; t < SP; ++t)
+#pragma unroll
+            for (int tap = 0; tap < 27; ++tap) {
+                const int dl = tap / 9, di = (tap % 9) / 3, dj = tap % 3;
+#pragma unroll
+                for (int e = 0; e < NV; ++e) {
+                    const float g = win.at(t + 2 - dj, 2 - di, 0, 1 - dl, e);
+                    d[t][0][e] = fmaf(w[tap], g, d[t][0][e]);
+                    d[t][1][e] = fmaf(w[28 + tap], g, d[t][1][e]);
+                }
+            }
+    }
+    if (lok) {
+#pragma unroll
+        for (int t = 0; t < SP; ++t) {
+            if (t >= st.n) break;
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                const long o = ((st.pix0 + t) * 2 + c) * L + st.lane * NV;
+                if (a.init) {
+                    float v[NV];
+                    load_vec<NV>(a.init + o, a.init, true, v);
+#pragma unroll
+                    for (int e = 0; e < NV; ++e) d[t][c][e] += v[e];
+                }
+                store_vec<NV>(a.out + o, d[t][c]);
+            }
+        }
+    }
+}
+
+// Weight and bias gradient over strips, stage 1.  Workgroup (x, y): wave-strips [x * DW_WS, ...), input channel
+// c = y % 2, weight channels [4 (y / 2), +4); a wave takes every 4th of them, SP = 4 / NV pixels per strip.  Per strip:
+// the window of channel c and the 4 logit gradients of its pixels (both fetched while the previous strip is worked on),
+// then 27 x 4 accumulators are updated per position; reduced over lanes and waves in a fixed order and written as
+// partial[x][...] like att_weight_backward_kernel's.
+constexpr int DW_WS = 32;
+template <int NV>
+__global__ void __launch_bounds__(256) att_weight_backward_strip_kernel(const AttJobs m) {
+    ATT_JOB(m);
+    constexpr int SP = 4 / NV;
+    __shared__ float red[4][27 * DW_KC + DW_KC];
+    const int K = a.K, L = a.L, H1 = a.H1, W1 = a.W1;
+    const int lw = strip_lanes(L, NV);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int c = blockIdx.y & 1, k0 = (blockIdx.y >> 1) * DW_KC;
+    const long nws = ((long)a.B * H1 * ((W1 + SP - 1) / SP) + 64 / lw - 1) / (64 / lw);
+    const long ws0 = (long)bx * DW_WS;
+    const int nmine = (int)(nws - ws0 < DW_WS ? nws - ws0 : DW_WS);   // wave-strips of this workgroup
+    const int nit = (nmine - wave + 3) / 4;
+    float acc[27][DW_KC], accb[DW_KC];
+#pragma unroll
+    for (int t = 0; t < 27; ++t)
+#pragma unroll
+        for (int k = 0; k < DW_KC; ++k) acc[t][k] = 0.f;
+#pragma unroll
+    for (int k = 0; k < DW_KC; ++k) accb[k] = 0.f;
+    Window<NV, SP, 1> win, nxt;
+    float g[SP][DW_KC][NV], gn[SP][DW_KC][NV];
+    Strip st = strip_at<SP>(a, ws0 + wave, lw);
+    auto fetch = [&](int it) {
+        st = strip_at<SP>(a, ws0 + wave + 4 * it, lw);
+        nxt.fetch(a.sep, st, H1, W1, L, 2, c);
+        const bool lok = st.active && st.lane * NV < L;
+        const int p0 = (int)st.pix0;
+#pragma unroll
+        for (int t = 0; t < SP; ++t)
+#pragma unroll
+            for (int k = 0; k < DW_KC; ++k)
+                load_vec<NV>(a.dlogits + (((p0 + t) * K + k0 + k) * L + st.lane * NV), a.dlogits, lok && t < st.n && k0 + k < K, gn[t][k]);
+    };
+    if (nit > 0) fetch(0);
+#pragma unroll 1
+    for (int it = 0; it < nit; ++it) {
+#pragma unroll
+        for (int col = 0; col < SP + 2; ++col)
+#pragma unroll
+            for (int r = 0; r < 3; ++r)
+#pragma unroll
+                for (int e = 0; e < NV; ++e) win.x[col][r][0][e] = nxt.x[col][r][0][e];
+#pragma unroll
+        for (int t = 0; t < SP; ++t)
+#pragma unroll
+            for (int k = 0; k < DW_KC; ++k)
+#pragma unroll
+                for (int e = 0; e < NV; ++e) g[t][k][e] = gn[t][k][e];
+        win.finish(st);   // first / last depend on the lane only
+        if (it + 1 < nit) fetch(it + 1);
+#pragma unroll
+        for (int t = 0; t < SP; ++t)
+#pragma unroll
+            for (int e = 0; e < NV; ++e) {
+#pragma unroll
+                for (int k = 0; k < DW_KC; ++k) accb[k] += g[t][k][e];
+#pragma unroll
+                for (int tap = 0; tap < 27; ++tap) {   // [dl][di][dj]: the order of the weights
+                    const float x = win.at(t + tap % 3, (tap % 9) / 3, 0, tap / 9 - 1, e);
+#pragma unroll
+                    for (int k = 0; k < DW_KC; ++k) acc[tap][k] = fmaf(g[t][k][e], x, acc[tap][k]);
+                }
+            }
+    }
+#pragma unroll
+    for (int t = 0; t < 27; ++t)
+#pragma unroll
+        for (int k = 0; k < DW_KC; ++k) {
+            const float r = wave_sum_dpp(acc[t][k]);
+            if (lane == 63) red[wave][t * DW_KC + k] = r;
+        }
+#pragma unroll
+    for (int k = 0; k < DW_KC; ++k) {
+        const float r = wave_sum_dpp(accb[k]);
+        if (lane == 63) red[wave][27 * DW_KC + k] = r;
+    }
+    __syncthreads();
+    float *dst = a.partial + (long)bx * (K * 54 + K);
+    for (int t = threadIdx.x; t < 27 * DW_KC; t += blockDim.x) {
+        const int k = t % DW_KC, tap = t / DW_KC;
+        if (k0 + k < K) dst[(k0 + k) * 54 + c * 27 + tap] = red[0][t] + red[1][t] + red[2][t] + red[3][t];
+    }
+    if (c == 0)   // the bias gradient is counted once
+        for (int t = threadIdx.x; t < DW_KC; t += blockDim.x)
+            if (k0 + t < K)
+                dst[K * 54 + k0 + t] = red[0][27 * DW_KC + t] + red[1][27 * DW_KC + t] + red[2][27 * DW_KC + t] + red[3][27 * DW_KC + t];
+}
+
+// pixels per strip for NV positions per lane (the window of a strip fills 108 to 144 registers)
+constexpr int strip_sp(int nv) { return nv == 4 ? 2 : 4; }
+static bool aligned_for(const void *p, int nv) { return !p || (reinterpret_cast<uintptr_t>(p) & (uintptr_t)(4 * nv - 1)) == 0; }
+// rows of L entries can be held nv to a lane
+static bool strip_fits(int L, int nv) { return L <= 64 * nv && L % nv == 0; }
+// The strip variant (positions per lane; 0: none, the job runs one wave per pixel) of every job of a call.  A job
+// takes the smallest that holds its rows with all its tensors (t0..t3, unused ones NULL) aligned for the vector
+// accesses; jobs that could also run with the largest variant among them are moved to it, so that they share its launch.
+template <typename Tensors>
+static void strip_variants(const AttArgs *jobs, int n, Tensors tensors, int (&var)[MAXJOBS]) {
+    auto ok = [&](int j, int nv) {
+        if (!strip_fits(jobs[j].L, nv)) return false;
+        const void *t[4];
+        tensors(jobs[j], t);
+        return aligned_for(t[0], nv) && aligned_for(t[1], nv) && aligned_for(t[2], nv) && aligned_for(t[3], nv);
+    };
+    int top = 0;
+    for (int j = 0; j < n; ++j) {
+        var[j] = ok(j, 1) ? 1 : ok(j, 2) ? 2 : ok(j, 4) ? 4 : 0;
+        if (var[j] > top) top = var[j];
+    }
+    for (int j = 0; j < n; ++j)
+        if (var[j] > 0 && var[j] < top && ok(j, top)) var[j] = top;
+}
+// workgroups (= partial sums) of the weight-gradient launch of one job, by kernel variant (nv = 0: one wave per pixel)
+static unsigned weight_groups(int B, int H1, int W1, int L, int nv) {
+    if (nv == 0) return (unsigned)(((long)B * H1 * W1 + DW_PIX - 1) / DW_PIX);
+    return (unsigned)((wave_strips(B, H1, W1, L, nv, 4 / nv) + DW_WS - 1) / DW_WS);
+}
+// the largest over the variants a job with rows of L entries can run with: which one it is depends on the alignment
+// of the tensors and on the other jobs of the call
+static size_t weight_groups_max(int B, int H1, int W1, int L) {
+    unsigned most = weight_groups(B, H1, W1, L, 0);
+    for (int nv = 1; nv <= 4; nv *= 2)
+        if (strip_fits(L, nv)) {
+            const unsigned g = weight_groups(B, H1, W1, L, nv);
+            if (g > most) most = g;
+        }
+    return most;
+}
+template <int NV>
+static void launch_backward_strip(const AttJobs &mi, unsigned gi, const AttJobs &mw, unsigned gw, int K, hipStream_t s) {
+    hipLaunchKernelGGL((att_input_backward_strip_kernel<NV, strip_sp(NV)>), dim3(gi), dim3(64 * WPB), 0, s, mi);
+    hipLaunchKernelGGL((att_weight_backward_strip_kernel<NV>), dim3(gw, 2 * ((K + DW_KC - 1) / DW_KC)), dim3(256), 0, s, mw);
+}
+template <int NV>
+static void launch_forward_strip(const AttJobs &m, unsigned nwg, hipStream_t s) {
+    hipLaunchKernelGGL((att_forward_strip_kernel<NV, strip_sp(NV)>), dim3(nwg), dim3(64 * WPB), 0, s, m);
+}
 int check(const void *p, const char *name) {
     if (p) return 0;
     char msg[128];
@@ -437,26 +900,42 @@ static unsigned pixel_groups(long npix, int L);
 static int attention_conv_backward_jobs(const AttArgs *jobs, int n, float *partial, float *d_weight, float *d_bias, void *stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int K = jobs[0].K;
-    AttJobs mi = {}, mw = {};
-    unsigned gi = 0, gw = 0;
-    for (int j = 0; j < n; ++j) {
-        const long npix = (long)jobs[j].B * jobs[j].H1 * jobs[j].W1;
-        mi.job[j] = jobs[j];
-        mi.first[j] = (int)gi;
-        gi += pixel_groups(npix, jobs[j].L);
-        mw.job[j] = jobs[j];
-        mw.job[j].partial = partial + (size_t)gw * (K * 54 + K);
-        mw.first[j] = (int)gw;
-        gw += (unsigned)((npix + DW_PIX - 1) / DW_PIX);
+    unsigned gw_all = 0;   // partial sums written so far: the launches below share `partial`
+    int vars[MAXJOBS];
+    strip_variants(jobs, n, [](const AttArgs &j, const void *(&t)[4]) { t[0] = j.sep; t[1] = j.dlogits; t[2] = j.out; t[3] = j.init; }, vars);
+    for (int var = 0; var <= 4; ++var) {   // one pair of launches per kernel variant among the jobs
+        if (var == 3) continue;
+        AttJobs mi = {}, mw = {};
+        unsigned gi = 0, gw = 0;
+        for (int j = 0; j < n; ++j) {
+            if (vars[j] != var) continue;
+            const long npix = (long)jobs[j].B * jobs[j].H1 * jobs[j].W1;
+            const int q = mi.njobs;
+            mi.job[q] = jobs[j];
+            mi.first[q] = (int)gi;
+            gi += var == 0 ? pixel_groups(npix, jobs[j].L)
+                : var == 4 ? strip_groups<strip_sp(4)>(jobs[j].B, jobs[j].H1, jobs[j].W1, jobs[j].L, var)
+                           : strip_groups<strip_sp(1)>(jobs[j].B, jobs[j].H1, jobs[j].W1, jobs[j].L, var);
+            mw.job[q] = jobs[j];
+            mw.job[q].partial = partial + (size_t)(gw_all + gw) * (K * 54 + K);
+            mw.first[q] = (int)gw;
+            gw += weight_groups(jobs[j].B, jobs[j].H1, jobs[j].W1, jobs[j].L, var);
+            mi.njobs = mw.njobs = q + 1;
+            mi.first[q + 1] = (int)gi; mw.first[q + 1] = (int)gw;
+        }
+        if (mi.njobs == 0) continue;
+        if (var == 0) {
+            hipLaunchKernelGGL(att_input_backward_kernel, dim3(gi), dim3(64 * WPB), 0, s, mi);
+            hipLaunchKernelGGL(att_weight_backward_kernel, dim3(gw, 2 * ((K + DW_KC - 1) / DW_KC)), dim3(256), 0, s, mw);
+        }
+        else if (var == 1) launch_backward_strip<1>(mi, gi, mw, gw, K, s);
+        else if (var == 2) launch_backward_strip<2>(mi, gi, mw, gw, K, s);
+        else launch_backward_strip<4>(mi, gi, mw, gw, K, s);
+        if (int rc = launched("attention input / weight gradient kernels")) return rc;
+        gw_all += gw;
     }
-    mi.first[n] = (int)gi; mw.first[n] = (int)gw;
-    mi.njobs = mw.njobs = n;
-    hipLaunchKernelGGL(att_input_backward_kernel, dim3(gi), dim3(64 * WPB), 0, s, mi);
-    if (int rc = launched("attention input gradient kernel")) return rc;
-    hipLaunchKernelGGL(att_weight_backward_kernel, dim3(gw, 2 * ((K + DW_KC - 1) / DW_KC)), dim3(256), 0, s, mw);
-    if (int rc = launched("attention weight gradient kernel")) return rc;
     const int nw = K * 54 + K;
-    hipLaunchKernelGGL(att_weight_reduce_kernel, dim3((nw + 3) / 4), dim3(256), 0, s, partial, d_weight, d_bias, (int)gw, K);
+    hipLaunchKernelGGL(att_weight_reduce_kernel, dim3((nw + 3) / 4), dim3(256), 0, s, partial, d_weight, d_bias, (int)gw_all, K);
     return launched("attention weight gradient reduction");
 }
 
@@ -467,11 +946,32 @@ static unsigned pixel_groups(long npix, int L) {
 }
 // kernel variant of the forward pass for rows of L entries: 1, 2, 4 chunks of 64, or 0 for the long-row kernel
 static int forward_variant(int L) { return L <= 64 ? 1 : L <= 128 ? 2 : L <= 256 ? 4 : 0; }
-
 // Forward pass of n jobs (levels) that share weight and bias: one launch per kernel variant among them.
 static int attention_forward_jobs(const AttArgs *jobs, int n, void *stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     bool done[MAXJOBS] = {};
+    int vars[MAXJOBS];
+    strip_variants(jobs, n, [](const AttArgs &j, const void *(&t)[4]) { t[0] = j.sep; t[1] = j.out; t[2] = t[3] = nullptr; }, vars);
+    for (int i = 0; i < n; ++i) {   // strips: one launch per variant among the jobs
+        if (done[i]) continue;
+        const int nv = vars[i];
+        if (nv == 0) continue;
+        AttJobs m = {};
+        unsigned nwg = 0;
+        for (int j = i; j < n; ++j) {
+            if (done[j] || vars[j] != nv) continue;
+            done[j] = true;
+            m.job[m.njobs] = jobs[j];
+            m.first[m.njobs] = (int)nwg;
+            nwg += nv == 4 ? strip_groups<strip_sp(4)>(jobs[j].B, jobs[j].H1, jobs[j].W1, jobs[j].L, nv)
+                           : strip_groups<strip_sp(1)>(jobs[j].B, jobs[j].H1, jobs[j].W1, jobs[j].L, nv);
+            m.first[++m.njobs] = (int)nwg;
+        }
+        if (nv == 1) launch_forward_strip<1>(m, nwg, s);
+        else if (nv == 2) launch_forward_strip<2>(m, nwg, s);
+        else launch_forward_strip<4>(m, nwg, s);
+        if (int rc = launched("attention forward kernel (strips)")) return rc;
+    }
     for (int i = 0; i < n; ++i) {
         if (done[i]) continue;
         const int var = forward_variant(jobs[i].L);
@@ -535,13 +1035,13 @@ int sepcorr_attention_logits_forward(const float *sep, const float *weight, cons
 size_t sepcorr_attention_workspace_bytes(int B, int H1, int W1, int L, int K) {
     if (B < 1 || H1 < 1 || W1 < 1 || L < 1 || K < 1 || K > MAXK) return 0;
     const size_t npix = (size_t)B * H1 * W1;
-    const size_t nwg = (npix + DW_PIX - 1) / DW_PIX;
+    const size_t nwg = weight_groups_max(B, H1, W1, L);
     return align256(npix * K * L * sizeof(float)) + align256(nwg * (K * 54 + K) * sizeof(float));
 }
 
 size_t sepcorr_attention_logits_workspace_bytes(int B, int H1, int W1, int L, int K) {
     if (B < 1 || H1 < 1 || W1 < 1 || L < 1 || K < 1 || K > MAXK) return 0;
-    const size_t nwg = ((size_t)B * H1 * W1 + DW_PIX - 1) / DW_PIX;
+    const size_t nwg = weight_groups_max(B, H1, W1, L);
     return align256(nwg * (K * 54 + K) * sizeof(float));
 }
 

@@ -101,7 +101,13 @@ def test_corr_block_other_paths(device, kind, backward):
 
 
 @pytest.mark.parametrize("B,H1,W1,L,K", [(1, 3, 4, 5, 1), (2, 9, 13, 70, 4), (1, 6, 10, 128, 4), (1, 4, 5, 200, 3),
-                                          (1, 3, 6, 300, 2), (1, 2, 3, 1, 8)])
+                                          (1, 3, 6, 300, 2), (1, 2, 3, 1, 8),
+                                          # strips of pixels: rows of 16 / 32 / 64 lanes (several strips per wave), 2 and 4
+                                          # positions per lane, image rows that end inside a strip, one-pixel images
+                                          (2, 5, 9, 16, 4), (1, 4, 7, 13, 2), (2, 3, 6, 27, 4), (1, 7, 5, 32, 3),
+                                          (1, 5, 11, 55, 4), (2, 4, 8, 64, 5), (1, 3, 5, 66, 4), (1, 4, 6, 127, 2),
+                                          (1, 3, 3, 136, 4), (1, 2, 7, 240, 4), (1, 3, 2, 256, 8), (1, 1, 1, 128, 4),
+                                          (1, 1, 9, 6, 4), (1, 6, 1, 64, 4)])
 def test_attention_producer_matches_conv3d_softmax(device, B, H1, W1, L, K):
     from separableflowthesis_amd import MemorySaver
     g = torch.Generator().manual_seed(11)
