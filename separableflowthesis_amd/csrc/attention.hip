@@ -216,20 +216,41 @@ __global__ void __launch_bounds__(64 * WPB) att_forward_long_kernel(const AttJob
 // lane gets the neighbours along L from the lanes beside it (one data-parallel-primitive move each) instead of from
 // memory.  A lane holds NV consecutive positions l = NV * lane + e (rows of up to 64 NV entries; NV > 1 needs L to
 // be a multiple of NV and 4 NV-byte aligned tensors), so for e inside the vector the neighbour is the lane's own.
-// NV floats at p if ok, else zeros.  No branch: lanes that are not ok read `safe` (any readable, aligned address of
-// the same tensor) and discard it, so the loads of a window are issued back to back.
+// Raw buffer resource over `bytes` bytes at p (wave-uniform): loads whose per-lane byte offset is >= bytes return 0,
+// which stands in for every bounds branch of a window (image borders, lanes past the end of a row).
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p, unsigned bytes) {
+    const uint64_t addr = reinterpret_cast<uint64_t>(p);
+    const uint64_t lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)addr);
+    const uint64_t hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(addr >> 32));
+    const int n = __builtin_amdgcn_readfirstlane((int)bytes);
+    return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void *>((hi << 32) | lo), 0, n, 0x00020000);
+}
+constexpr unsigned OOB = 0x80000000u;   // a byte offset above the size of every tensor the strip kernels take
+// NV floats at byte offset lane_off + uniform_off (the second the same in every lane; it takes no part in the bounds check)
 template <int NV>
-__device__ __forceinline__ void load_vec(const float *p, const float *safe, bool ok, float (&x)[NV]) {
-    const float *q = ok ? p : safe;
+__device__ __forceinline__ void buf_load_vec(__amdgpu_buffer_rsrc_t r, unsigned lane_off, unsigned uniform_off, float (&x)[NV]) {
     if constexpr (NV == 1) {
-        const float v = *q;
-        x[0] = ok ? v : 0.f;
+        x[0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, lane_off, uniform_off, 0));
     } else if constexpr (NV == 2) {
-        const float2 v = *reinterpret_cast<const float2 *>(q);
-        x[0] = ok ? v.x : 0.f; x[1] = ok ? v.y : 0.f;
+        const v2f v = __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(r, lane_off, uniform_off, 0));
+        x[0] = v.x; x[1] = v.y;
     } else {
-        const float4 v = *reinterpret_cast<const float4 *>(q);
-        x[0] = ok ? v.x : 0.f; x[1] = ok ? v.y : 0.f; x[2] = ok ? v.z : 0.f; x[3] = ok ? v.w : 0.f;
+        const v4f v = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r, lane_off, uniform_off, 0));
+        x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+    }
+}
+template <int NV>
+__device__ __forceinline__ void load_vec(const float *p, float (&x)[NV]) {
+    if constexpr (NV == 1) {
+        x[0] = *p;
+    } else if constexpr (NV == 2) {
+        const float2 v = *reinterpret_cast<const float2 *>(p);
+        x[0] = v.x; x[1] = v.y;
+    } else {
+        const float4 v = *reinterpret_cast<const float4 *>(p);
+        x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
     }
 }
 template <int NV>
@@ -322,24 +343,35 @@ static unsigned strip_groups(int B, int H1, int W1, int L, int NV) {
 
 // The window of a strip: SP + 2 columns x 3 image rows x NCHAN channels of one tensor whose rows are (pixel, channel)
 // x L, with the values of the lanes beside (xm: position l - 1 of the lane's first entry, xp: l + 1 of its last).
-// fetch() issues the loads (tensors have fewer than 2^31 elements: 32-bit element offsets); finish() derives xm / xp.
+// fetch() issues the loads (buffer loads: what lies outside the image or the row reads as 0); finish() derives xm / xp.
 template <int NV, int SP, int NCHAN>
 struct Window {
     float x[SP + 2][3][NCHAN][NV], xm[SP + 2][3][NCHAN], xp[SP + 2][3][NCHAN];
     // chan0: first channel to fetch, nchan_total: channels per pixel in memory
-    __device__ __forceinline__ void fetch(const float *base, const Strip &t, int H1, int W1, int L, int nchan_total, int chan0) {
+    __device__ __forceinline__ void fetch(__amdgpu_buffer_rsrc_t rs, const Strip &t, int H1, int W1, int L, int nchan_total, int chan0) {
         const bool lok = t.active && t.lane * NV < L;
         const int p0 = (int)t.pix0;
+        // byte offset of the lane's entries in channel chan0 of the strip's first pixel, rows i - 1 .. i + 1.  The
+        // per-lane offset must be in range by itself (the bounds check does not see the uniform part), so the column
+        // left of the strip gets an offset of its own instead of a negative uniform part.
+        unsigned rowoff[3];
+        const unsigned pixel = (unsigned)(nchan_total * L) * 4u;
+#pragma unroll
+        for (int r = 0; r < 3; ++r) {
+            const int ii = t.i + r - 1;
+            const unsigned off = (unsigned)(((p0 + (r - 1) * W1) * nchan_total + chan0) * L + t.lane * NV) * 4u;
+            rowoff[r] = (lok && ii >= 0 && ii < H1) ? off : OOB;
+        }
 #pragma unroll
         for (int col = 0; col < SP + 2; ++col) {
             const int jj = t.j0 + col - 1;
+            const bool okc = jj >= 0 && jj < W1 && col <= t.n + 1;
 #pragma unroll
             for (int r = 0; r < 3; ++r) {
-                const int ii = t.i + r - 1;
-                const bool ok = lok && ii >= 0 && ii < H1 && jj >= 0 && jj < W1 && col <= t.n + 1;
-                const int off = ((p0 + (r - 1) * W1 + (col - 1)) * nchan_total + chan0) * L + t.lane * NV;
+                const unsigned off = !okc || rowoff[r] == OOB ? OOB : col == 0 ? rowoff[r] - pixel : rowoff[r];
 #pragma unroll
-                for (int c = 0; c < NCHAN; ++c) load_vec<NV>(base + (off + c * L), base, ok, x[col][r][c]);
+                for (int c = 0; c < NCHAN; ++c)
+                    buf_load_vec<NV>(rs, off, (unsigned)(((col == 0 ? 0 : col - 1) * nchan_total + c) * L) * 4u, x[col][r][c]);
             }
         }
     }
@@ -387,7 +419,7 @@ __global__ void __launch_bounds__(64 * WPB) att_forward_strip_kernel(const AttJo
     const Strip st = strip_of<SP>(a, bx, lw);
     if (!st.active) return;   // whole groups leave: the reductions below stay inside a group
     Window<NV, SP, 2> win;
-    win.fetch(a.sep, st, H1, W1, L, 2, 0);
+    win.fetch(make_rsrc(a.sep, (unsigned)((long)a.B * H1 * W1 * 2 * L * 4)), st, H1, W1, L, 2, 0);
     win.finish(st);
     const bool lok = st.lane * NV < L;
 #pragma unroll 1
@@ -665,7 +697,8 @@ __global__ void __launch_bounds__(64 * WPB) att_input_backward_strip_kernel(cons
 #pragma unroll
             for (int e = 0; e < NV; ++e) d[t][c][e] = 0.f;
     Window<NV, SP, 1> win, nxt;
-    nxt.fetch(a.dlogits, st, H1, W1, L, K, 0);
+    const __amdgpu_buffer_rsrc_t rs = make_rsrc(a.dlogits, (unsigned)((long)a.B * H1 * W1 * K * L * 4));
+    nxt.fetch(rs, st, H1, W1, L, K, 0);
 #pragma unroll 1
     for (int k = 0; k < K; ++k) {
 #pragma unroll
@@ -675,7 +708,7 @@ __global__ void __launch_bounds__(64 * WPB) att_input_backward_strip_kernel(cons
 #pragma unroll
                 for (int e = 0; e < NV; ++e) win.x[col][r][0][e] = nxt.x[col][r][0][e];
         win.finish(st);
-        if (k + 1 < K) nxt.fetch(a.dlogits, st, H1, W1, L, K, k + 1);
+        if (k + 1 < K) nxt.fetch(rs, st, H1, W1, L, K, k + 1);
         float w[56];   // the same in every lane: kept in scalar registers
 #pragma unroll
         for (int q = 0; q < 14; ++q) {
@@ -705,7 +738,7 @@ __global__ void __launch_bounds__(64 * WPB) att_input_backward_strip_kernel(cons
                 const long o = ((st.pix0 + t) * 2 + c) * L + st.lane * NV;
                 if (a.init) {
                     float v[NV];
-                    load_vec<NV>(a.init + o, a.init, true, v);
+                    load_vec<NV>(a.init + o, v);
 #pragma unroll
                     for (int e = 0; e < NV; ++e) d[t][c][e] += v[e];
                 }
@@ -744,16 +777,24 @@ __global__ void __launch_bounds__(256) att_weight_backward_strip_kernel(const At
     Window<NV, SP, 1> win, nxt;
     float g[SP][DW_KC][NV], gn[SP][DW_KC][NV];
     Strip st = strip_at<SP>(a, ws0 + wave, lw);
+    const __amdgpu_buffer_rsrc_t rs_sep = make_rsrc(a.sep, (unsigned)((long)a.B * H1 * W1 * 2 * L * 4));
+    const __amdgpu_buffer_rsrc_t rs_g = make_rsrc(a.dlogits, (unsigned)((long)a.B * H1 * W1 * K * L * 4));
     auto fetch = [&](int it) {
         st = strip_at<SP>(a, ws0 + wave + 4 * it, lw);
-        nxt.fetch(a.sep, st, H1, W1, L, 2, c);
+        nxt.fetch(rs_sep, st, H1, W1, L, 2, c);
         const bool lok = st.active && st.lane * NV < L;
-        const int p0 = (int)st.pix0;
+        const unsigned goff = (unsigned)(((int)st.pix0 * K + k0) * L + st.lane * NV) * 4u;
 #pragma unroll
-        for (int t = 0; t < SP; ++t)
+        for (int t = 0; t < SP; ++t) {
+            const unsigned off = (lok && t < st.n) ? goff : OOB;
 #pragma unroll
-            for (int k = 0; k < DW_KC; ++k)
-                load_vec<NV>(a.dlogits + (((p0 + t) * K + k0 + k) * L + st.lane * NV), a.dlogits, lok && t < st.n && k0 + k < K, gn[t][k]);
+            for (int k = 0; k < DW_KC; ++k) {
+                if (k0 + k < K) buf_load_vec<NV>(rs_g, off, (unsigned)((t * K + k) * L) * 4u, gn[t][k]);
+                else
+#pragma unroll
+                    for (int e = 0; e < NV; ++e) gn[t][k][e] = 0.f;
+            }
+        }
     };
     if (nit > 0) fetch(0);
 #pragma unroll 1
@@ -822,6 +863,8 @@ template <typename Tensors>
 static void strip_variants(const AttArgs *jobs, int n, Tensors tensors, int (&var)[MAXJOBS]) {
     auto ok = [&](int j, int nv) {
         if (!strip_fits(jobs[j].L, nv)) return false;
+        const int ch = jobs[j].K > 2 ? jobs[j].K : 2;   // buffer loads address a tensor with 31-bit byte offsets
+        if ((double)jobs[j].B * jobs[j].H1 * jobs[j].W1 * ch * jobs[j].L * 4.0 >= 2147483648.0) return false;
         const void *t[4];
         tensors(jobs[j], t);
         return aligned_for(t[0], nv) && aligned_for(t[1], nv) && aligned_for(t[2], nv) && aligned_for(t[3], nv);
