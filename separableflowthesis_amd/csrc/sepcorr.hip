@@ -2881,43 +2881,84 @@ __global__ void __launch_bounds__(256) row_stats_kernel(const float *__restrict_
     sum = wave_sum64(sum);
     if (lane == 0) { st[2 * row] = m; st[2 * row + 1] = sum; }
 }
-// dot[row] = sum_l x[row,l] * y[row,l]
-__global__ void __launch_bounds__(256) row_dot_kernel(const float *__restrict__ x, const float *__restrict__ y, float *__restrict__ dot,
-                                                      long nrows, int L) {
-    const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+// Rows of L floats dealt to the waves of a workgroup with lanes along the row, VL entries per lane (4: 16-byte
+// accesses, for rows whose length is a multiple of 4 in 16-byte aligned tensors): lpr lanes per row (a power of two,
+// at least ceil(L / VL), at most 64), 64 / lpr rows side by side in a wave, ROWS_PER_WAVE rows per wave in all.
+constexpr int ROWS_PER_WAVE = 8;   // (a step's loads, arithmetic and store follow one another: 32 rows per wave measured slower)
+struct RowDeal {
+    int lpr, rpw, row, pos;   // lanes per row, rows per wave and step, this lane's row within the step, its place in the row
+};
+__device__ __forceinline__ RowDeal row_deal(int L, int VL) {
+    RowDeal r;
+    const int need = (L + VL - 1) / VL;
+    r.lpr = need <= 1 ? 1 : need >= 33 ? 64 : 1 << (32 - __builtin_clz(need - 1));
+    r.rpw = 64 / r.lpr;
     const int lane = threadIdx.x & 63;
-    if (row >= nrows) return;
-    float sum = 0.f;
-    for (int l = lane; l < L; l += 64) sum += x[row * L + l] * y[row * L + l];
-    sum = wave_sum64(sum);
-    if (lane == 0) dot[row] = sum;
+    r.row = lane / r.lpr;
+    r.pos = lane & (r.lpr - 1);
+    return r;
+}
+inline bool rows_vec4(const void *p, int L) { return L % 4 == 0 && (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+inline unsigned row_groups(size_t nrows) { return (unsigned)((nrows + 4 * ROWS_PER_WAVE - 1) / (4 * ROWS_PER_WAVE)); }
+
+// dot[row] = sum_l x[row,l] * y[row,l] of one pair of tensors; the sum over a row's lanes by a butterfly (fixed order)
+__device__ __forceinline__ void row_dots(const float *__restrict__ x, const float *__restrict__ y, float *__restrict__ dot, long nrows,
+                                         int L, bool vec4) {
+    const RowDeal rd = row_deal(L, vec4 ? 4 : 1);
+    const long r0 = ((long)blockIdx.x * 4 + (threadIdx.x >> 6)) * ROWS_PER_WAVE;
+    for (int i = rd.row; i < ROWS_PER_WAVE; i += rd.rpw) {
+        const long row = r0 + i;
+        float sum = 0.f;
+        if (row < nrows) {
+            const float *xr = x + row * L, *yr = y + row * L;
+            if (vec4) {
+                for (int l = 4 * rd.pos; l < L; l += 4 * rd.lpr) {
+                    const float4 a = *reinterpret_cast<const float4 *>(xr + l), b = *reinterpret_cast<const float4 *>(yr + l);
+                    sum += (a.x * b.x + a.y * b.y) + (a.z * b.z + a.w * b.w);
+                }
+            } else {
+                for (int l = rd.pos; l < L; l += rd.lpr) sum += xr[l] * yr[l];
+            }
+        }
+        for (int o = rd.lpr >> 1; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+        if (row < nrows && rd.pos == 0) dot[row] = sum;
+    }
+}
+__global__ void __launch_bounds__(256) row_dot_kernel(const float *__restrict__ x, const float *__restrict__ y, float *__restrict__ dot,
+                                                      long nrows, int L, int vec4) {
+    row_dots(x, y, dot, nrows, L, vec4 != 0);
 }
 // The same for up to 8 pairs of tensors with the same number of rows (the two outputs of every pyramid level) in one
 // launch: blockIdx.y picks the pair.
 struct RowDotJobs {
     const float *x[8], *y[8];
     float *dot[8];
-    int L[8];
+    int L[8], vec4[8];
 };
 __global__ void __launch_bounds__(256) row_dot_multi_kernel(const RowDotJobs j, long nrows) {
-    const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int lane = threadIdx.x & 63, job = blockIdx.y;
-    if (row >= nrows) return;
-    const int L = j.L[job];
-    const float *x = j.x[job] + row * L, *y = j.y[job] + row * L;
-    float sum = 0.f;
-    for (int l = lane; l < L; l += 64) sum += x[l] * y[l];
-    sum = wave_sum64(sum);
-    if (lane == 0) j.dot[job][row] = sum;
+    const int job = blockIdx.y;
+    row_dots(j.x[job], j.y[job], j.dot[job], nrows, j.L[job], j.vec4[job] != 0);
 }
 // a[row,l] = exp(z[row,l] - max) / sum
 __global__ void __launch_bounds__(256) softmax_apply_kernel(const float *__restrict__ z, const float *__restrict__ st, float *__restrict__ a,
-                                                            long nrows, int L) {
-    const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int lane = threadIdx.x & 63;
-    if (row >= nrows) return;
-    const float m = st[2 * row], il = 1.f / st[2 * row + 1];
-    for (int l = lane; l < L; l += 64) a[row * L + l] = __expf(z[row * L + l] - m) * il;
+                                                            long nrows, int L, int vec4) {
+    const RowDeal rd = row_deal(L, vec4 ? 4 : 1);
+    const long r0 = ((long)blockIdx.x * 4 + (threadIdx.x >> 6)) * ROWS_PER_WAVE;
+    for (int i = rd.row; i < ROWS_PER_WAVE; i += rd.rpw) {
+        const long row = r0 + i;
+        if (row >= nrows) break;
+        const float m = st[2 * row], il = 1.f / st[2 * row + 1];
+        const float *zr = z + row * L;
+        float *ar = a + row * L;
+        if (vec4) {
+            for (int l = 4 * rd.pos; l < L; l += 4 * rd.lpr) {
+                const float4 v = *reinterpret_cast<const float4 *>(zr + l);
+                *reinterpret_cast<float4 *>(ar + l) = make_float4(__expf(v.x - m) * il, __expf(v.y - m) * il, __expf(v.z - m) * il, __expf(v.w - m) * il);
+            }
+        } else {
+            for (int l = rd.pos; l < L; l += rd.lpr) ar[l] = __expf(zr[l] - m) * il;
+        }
+    }
 }
 
 __global__ void __launch_bounds__(256) zero_ints_kernel(int *p, int n) {
@@ -4064,7 +4105,8 @@ int sepcorr_softmax_rows(const float *logits, float *stats, int stats_given, flo
     hipStream_t s = static_cast<hipStream_t>(stream);
     const dim3 grid((unsigned)((nrows + 3) / 4)), block(256);
     if (!stats_given) hipLaunchKernelGGL(row_stats_kernel, grid, block, 0, s, logits, stats, nrows, L);
-    if (a) hipLaunchKernelGGL(softmax_apply_kernel, grid, block, 0, s, logits, stats, a, nrows, L);
+    if (a) hipLaunchKernelGGL(softmax_apply_kernel, dim3(row_groups((size_t)nrows)), block, 0, s, logits, stats, a, nrows, L,
+                              (int)(rows_vec4(logits, L) && rows_vec4(a, L)));
     return check_launch("softmax rows");
 }
 
@@ -4129,10 +4171,10 @@ int sepcorr_compression_backward_from_logits(const float *f1, const float *f2, c
     float *dot_u = reinterpret_cast<float *>(base + sweep_bytes);               // sum_u g_cu * comp_u = sum_v a_u * d_a_u
     float *dot_v = reinterpret_cast<float *>(base + sweep_bytes + dot_bytes);   // sum_v g_cv * comp_v = sum_u a_v * d_a_v
     {
-        const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+        const dim3 grid(row_groups(rows)), block(256);
         ProfScope ps("row_dots", s);
-        hipLaunchKernelGGL(row_dot_kernel, grid, block, 0, s, g_cu, comp_u, dot_u, (long)rows, H2);
-        hipLaunchKernelGGL(row_dot_kernel, grid, block, 0, s, g_cv, comp_v, dot_v, (long)rows, W2);
+        hipLaunchKernelGGL(row_dot_kernel, grid, block, 0, s, g_cu, comp_u, dot_u, (long)rows, H2, (int)(rows_vec4(g_cu, H2) && rows_vec4(comp_u, H2)));
+        hipLaunchKernelGGL(row_dot_kernel, grid, block, 0, s, g_cv, comp_v, dot_v, (long)rows, W2, (int)(rows_vec4(g_cv, W2) && rows_vec4(comp_v, W2)));
         if (int rc = check_launch("row dot products")) return rc;
     }
     // d_a_v[k,u] = sum_v S g_cv[k,v] and d_a_u[k,v] = sum_u S g_cu[k,u] as in sepcorr_compression_backward, turned into
@@ -4149,10 +4191,10 @@ int sepcorr_compression_backward_from_logits(const float *f1, const float *f2, c
     float *a_u = reinterpret_cast<float *>(base + sweep_bytes + 2 * dot_bytes);
     float *a_v = reinterpret_cast<float *>(base + sweep_bytes + 2 * dot_bytes + ((rows * W2 * sizeof(float) + 255) & ~(size_t)255));
     {
-        const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+        const dim3 grid(row_groups(rows)), block(256);
         ProfScope ps("softmax_apply", s);
-        hipLaunchKernelGGL(softmax_apply_kernel, grid, block, 0, s, logits_u, stats_u, a_u, (long)rows, W2);
-        hipLaunchKernelGGL(softmax_apply_kernel, grid, block, 0, s, logits_v, stats_v, a_v, (long)rows, H2);
+        hipLaunchKernelGGL(softmax_apply_kernel, grid, block, 0, s, logits_u, stats_u, a_u, (long)rows, W2, (int)(rows_vec4(logits_u, W2) && rows_vec4(a_u, W2)));
+        hipLaunchKernelGGL(softmax_apply_kernel, grid, block, 0, s, logits_v, stats_v, a_v, (long)rows, H2, (int)(rows_vec4(logits_v, H2) && rows_vec4(a_v, H2)));
         if (int rc2 = check_launch("softmax from statistics")) return rc2;
     }
     const BwdWs lay = bwd_ws(d);
@@ -4354,12 +4396,14 @@ int sepcorr_compression_backward_from_logits_levels(const float *f1, const float
             float *dot_v = reinterpret_cast<float *>(base + (2 * l + 1) * dot_bytes);   // sum_v g_cv comp_v
             jobs.x[2 * l] = g_cu[l]; jobs.y[2 * l] = comp_u[l]; jobs.dot[2 * l] = dot_u; jobs.L[2 * l] = h2[l];
             jobs.x[2 * l + 1] = g_cv[l]; jobs.y[2 * l + 1] = comp_v[l]; jobs.dot[2 * l + 1] = dot_v; jobs.L[2 * l + 1] = w2[l];
+            jobs.vec4[2 * l] = rows_vec4(g_cu[l], h2[l]) && rows_vec4(comp_u[l], h2[l]);
+            jobs.vec4[2 * l + 1] = rows_vec4(g_cv[l], w2[l]) && rows_vec4(comp_v[l], w2[l]);
             lev[l].wv = g_cv[l]; lev[l].wu = g_cu[l];
             lev[l].out_u = d_logits_v[l]; lev[l].out_v = d_logits_u[l];
             lev[l].z_ou = logits_v[l]; lev[l].st_ou = stats_v[l]; lev[l].dot_ou = dot_v;
             lev[l].z_ov = logits_u[l]; lev[l].st_ov = stats_u[l]; lev[l].dot_ov = dot_u;
         }
-        hipLaunchKernelGGL(row_dot_multi_kernel, dim3((unsigned)((rows + 3) / 4), 2 * nlev), dim3(256), 0, s, jobs, (long)rows);
+        hipLaunchKernelGGL(row_dot_multi_kernel, dim3(row_groups(rows), 2 * nlev), dim3(256), 0, s, jobs, (long)rows);
         if (int rc = check_launch("row dot products")) return rc;
     }
     return soft_levels(f1, f2_levels, h2, w2, nlev, lev, 1, B, H1, W1, C, K, workspace, sweep, s);
