@@ -2499,17 +2499,17 @@ __global__ void __launch_bounds__(256) transpose_uw_kernel(const BwdArgs a, int 
         src = reinterpret_cast<const float *>(a.am_u) + ((size_t)b * N1 + p0) * H2;
         pstride = (size_t)H2;
     }
+    // a wave takes every 4th pixel with lanes along u (two pixels at a time when a row has at most 32 entries), then
+    // every 4th row u with lanes along the pixels
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     for (int u0 = 0; u0 < H2; u0 += 64) {
         const int nu = min(64, H2 - u0);
-        for (int idx = threadIdx.x; idx < np * nu; idx += 256) {
-            const int p = idx / nu, u = idx - p * nu;
-            tile[p * 65 + u] = src[p * pstride + u0 + u];
-        }
+        const int lpr = nu <= 32 ? 32 : 64, sub = lane / lpr, u = lane & (lpr - 1);
+        if (u < nu)
+            for (int p = wave * (64 / lpr) + sub; p < np; p += 4 * (64 / lpr)) tile[p * 65 + u] = src[p * pstride + u0 + u];
         __syncthreads();
-        for (int idx = threadIdx.x; idx < nu * np; idx += 256) {
-            const int u = idx / np, p = idx - u * np;
-            out[(((size_t)b * H2 + u0 + u) * NF + f) * N1 + p0 + p] = tile[p * 65 + u];
-        }
+        if (lane < np)
+            for (int uu = wave; uu < nu; uu += 4) out[(((size_t)b * H2 + u0 + uu) * NF + f) * N1 + p0 + lane] = tile[lane * 65 + uu];
         __syncthreads();
     }
 }
