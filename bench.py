@@ -417,6 +417,10 @@ def module_level(name, torch, dev, reps=5, backward=True):
             if bw:
                 if not ups:
                     ups["g"] = [torch.randn(c.shape, generator=g).to(dev) for c in (c1, c2)]
+                # as a training step does before its backward pass (optimizer.zero_grad(), which drops the tensors):
+                # the gradients are then stored, not added to those of the previous repeat
+                for t in (fmap1, fmap2) + tuple(p for m in (att or ()) for p in m.parameters()):
+                    t.grad = None
                 torch.autograd.backward([c1, c2], ups["g"])
 
     out = {}

@@ -288,6 +288,15 @@ int sepcorr_fused_backward(const float *f1, const float *f2,
                            float *d_f1, float *d_f2,
                            int B, int H1, int W1, int H2, int W2, int C, int K,
                            void *workspace, size_t workspace_bytes, void *stream);
+/* The same, but d_f1 is added to what the buffer holds: fmap1 is shared by all pyramid levels (core/corr.py:419),
+ * so its gradient is the sum over the levels' calls; d_f2 (one tensor per level) is written as above. */
+int sepcorr_fused_backward_add(const float *f1, const float *f2,
+                               const int32_t *argmax_u, const int32_t *argmax_v,
+                               const float *grad_u, const float *grad_v,
+                               const float *a_u, const float *a_v, const float *g_cu, const float *g_cv,
+                               float *d_f1, float *d_f2,
+                               int B, int H1, int W1, int H2, int W2, int C, int K,
+                               void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * Attention-weight producer in the operator's layout.  Replaces, for one of the two volumes, the caller's

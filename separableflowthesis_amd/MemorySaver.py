@@ -468,9 +468,12 @@ def compression_logit_gradients_levels(img1_features_l0, img2_features_lvls, log
 
 
 def fused_backward(img1_features_l0, img2_features_lk, argmax_output_u, argmax_output_v, grad_MaxAvg_u, grad_MaxAvg_v,
-                   attention_weights_u, attention_weights_v, grad_compressed_output_u, grad_compressed_output_v):
+                   attention_weights_u, attention_weights_v, grad_compressed_output_u, grad_compressed_output_v,
+                   add_to_grad_fmap1=None):
     """-> [grad_fmap1_l0, grad_fmap2_lk]: the sum of what max_argmax_avg_backward and compression_backward return
-    for the features, from one contraction per output (dL/dS of both operators is added before it is used)."""
+    for the features, from one contraction per output (dL/dS of both operators is added before it is used).
+    add_to_grad_fmap1: a gradient of fmap1 from other pyramid levels; this level's is added to it in place and the
+    tensor returned as grad_fmap1_l0."""
     f1, f2 = img1_features_l0, img2_features_lk
     B, H1, W1, H2, W2, C = _dims(f1, f2)
     dev = f1.device
@@ -486,10 +489,12 @@ def fused_backward(img1_features_l0, img2_features_lk, argmax_output_u, argmax_o
     _expect("grad_compressed_output_v", grad_compressed_output_v, (B, H1, W1, K, W2), dev)
     lib = _lib.load()
     with torch.cuda.device(dev):
-        d1 = torch.empty_like(f1)
+        if add_to_grad_fmap1 is not None:
+            _expect("add_to_grad_fmap1", add_to_grad_fmap1, tuple(f1.shape), dev)
+        d1 = torch.empty_like(f1) if add_to_grad_fmap1 is None else add_to_grad_fmap1
         d2 = torch.empty_like(f2)
         ws, n = _workspace(lib, (B, H1, W1, H2, W2, C), dev)
-        _lib.check(lib.sepcorr_fused_backward(
+        _lib.check((lib.sepcorr_fused_backward if add_to_grad_fmap1 is None else lib.sepcorr_fused_backward_add)(
             f1.data_ptr(), f2.data_ptr(), argmax_output_u.data_ptr(), argmax_output_v.data_ptr(),
             grad_MaxAvg_u.data_ptr(), grad_MaxAvg_v.data_ptr(),
             attention_weights_u.data_ptr(), attention_weights_v.data_ptr(),

@@ -37,6 +37,7 @@ SIGNATURES = {
     "sepcorr_compression_backward_from_logits_levels": (_I, [_P] * 4 + [_I] + [_P] * 10 + [_I] * 5 + [_P, _SZ, _P]),
     "sepcorr_softmax_rows": (_I, [_P, _P, _I, _P, ctypes.c_long, _I, _P]),
     "sepcorr_fused_backward": (_I, [_P] * 12 + [_I] * 7 + [_P, _SZ, _P]),
+    "sepcorr_fused_backward_add": (_I, [_P] * 12 + [_I] * 7 + [_P, _SZ, _P]),
     "sepcorr_attention_logits_forward": (_I, [_P] * 5 + [_I] * 5 + [_P]),
     "sepcorr_attention_logits_workspace_bytes": (_SZ, [_I] * 5),
     "sepcorr_attention_logits_backward": (_I, [_P] * 6 + [_I] * 5 + [_P, _SZ, _P]),

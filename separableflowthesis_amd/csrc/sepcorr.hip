@@ -1441,6 +1441,7 @@ struct BwdArgs {
     int uneven, q_units;             // q_units = blocks of output rows (B x row groups x column chunks)
     int xl[9], xs[9];
     int accumulate;                  // add to the destination instead of overwriting
+    int add_d1;                      // d_f1 only: add to what the caller's buffer holds
     int xcd_order;                   // map workgroup ids so that each XCD gets a contiguous range
     // d_f1 dealt out in pieces of tiles, as the forward sweeps are (FwdArgs::sk_*): a piece leaves its partial
     // [32 pixels][channels] sum in a slot; whichever piece of a tile finishes last adds them up in row order.
@@ -2009,7 +2010,7 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
             const int idx = idx0 + i * (int)blockDim.x;
             const int row = idx / (CB / 4), c = (idx - row * (CB / 4)) * 4;
             if (idx < NIT && p0 + row < N1)
-                store4<CVEC>(a.d1 + ((size_t)b * N1 + p0 + row) * C, cb0 + c, C, x[i], a.accumulate != 0);
+                store4<CVEC>(a.d1 + ((size_t)b * N1 + p0 + row) * C, cb0 + c, C, x[i], (a.accumulate | a.add_d1) != 0);
         }
     };
     if (whole) {
@@ -2070,7 +2071,7 @@ __global__ void __launch_bounds__(MAXT) df1_kernel(const BwdArgs a) {
                     const int idx = idx0 + i * (int)blockDim.x;
                     const int row = idx / (CB / 4), c = (idx - row * (CB / 4)) * 4;
                     if (idx < NIT && p0 + row < N1)
-                        store4<CVEC>(a.d1 + ((size_t)b * N1 + p0 + row) * C, cb0 + c, C, x[i], a.accumulate != 0);
+                        store4<CVEC>(a.d1 + ((size_t)b * N1 + p0 + row) * C, cb0 + c, C, x[i], (a.accumulate | a.add_d1) != 0);
                 }
             }
         }
@@ -2697,7 +2698,7 @@ __global__ void __launch_bounds__(64 * NW) df1_bf_kernel(const BwdArgs a, const 
     // contiguous KB
     float *reg = smem + (wave & 3) * 32 * DF1BF_RS;
     float *out = dst + ((size_t)(nvc > 1 ? vc : 0) * a.B + b) * N1 * 256;
-    const bool accum = nvc == 1 && a.accumulate != 0;
+    const bool accum = nvc == 1 && (a.accumulate | a.add_d1) != 0;
 #pragma unroll
     for (int half = 0; half < NW / 4; ++half) {
         if (half > 0) __syncthreads();
@@ -3574,7 +3575,7 @@ int launch_bwd(BwdArgs a, const Dims &d, void *ws, hipStream_t s1, hipStream_t s
                 if (nvc > 1) {
                     const int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
                     ProfScope ps("df1_reduce_chunks", s1);
-                    hipLaunchKernelGGL(reduce_splits_kernel, dim3(blocks), dim3(256), 0, s1, part, a.d1, n, nvc, a.accumulate);
+                    hipLaunchKernelGGL(reduce_splits_kernel, dim3(blocks), dim3(256), 0, s1, part, a.d1, n, nvc, a.accumulate | a.add_d1);
                 }
                 rc = check_launch("d_f1 kernel (bf16 planes)");
             }
@@ -4409,10 +4410,10 @@ int sepcorr_compression_backward_from_logits_levels(const float *f1, const float
     return soft_levels(f1, f2_levels, h2, w2, nlev, lev, 1, B, H1, W1, C, K, workspace, sweep, s);
 }
 
-int sepcorr_fused_backward(const float *f1, const float *f2, const int32_t *argmax_u, const int32_t *argmax_v,
-                           const float *grad_u, const float *grad_v, const float *a_u, const float *a_v,
-                           const float *g_cu, const float *g_cv, float *d_f1, float *d_f2, int B, int H1, int W1, int H2,
-                           int W2, int C, int K, void *workspace, size_t workspace_bytes, void *stream) {
+static int fused_backward(const float *f1, const float *f2, const int32_t *argmax_u, const int32_t *argmax_v,
+                          const float *grad_u, const float *grad_v, const float *a_u, const float *a_v,
+                          const float *g_cu, const float *g_cv, float *d_f1, float *d_f2, int add_d_f1, int B, int H1, int W1, int H2,
+                          int W2, int C, int K, void *workspace, size_t workspace_bytes, void *stream) {
     api_enter();
     REQUIRE_PTR(f1); REQUIRE_PTR(f2); REQUIRE_PTR(argmax_u); REQUIRE_PTR(argmax_v); REQUIRE_PTR(grad_u); REQUIRE_PTR(grad_v);
     REQUIRE_PTR(a_u); REQUIRE_PTR(a_v); REQUIRE_PTR(g_cu); REQUIRE_PTR(g_cv); REQUIRE_PTR(d_f1); REQUIRE_PTR(d_f2);
@@ -4425,6 +4426,7 @@ int sepcorr_fused_backward(const float *f1, const float *f2, const int32_t *argm
     a.f1 = f1; a.f2 = f2; a.am_u = argmax_u; a.am_v = argmax_v; a.g_u = grad_u; a.g_v = grad_v;
     a.a_u = a_u; a.a_v = a_v; a.g_cu = g_cu; a.g_cv = g_cv;
     a.d1 = d_f1; a.d2 = d_f2;
+    a.add_d1 = add_d_f1 != 0;
     a.B = B; a.N1 = H1 * W1; a.H2 = H2; a.W2 = W2; a.C = C; a.KT = K;
     ForkJoin fj(static_cast<hipStream_t>(stream), !bwd_ws(d).aliased);
     const int kch = W2 > 128 ? 2 : KCH;
@@ -4456,6 +4458,22 @@ int sepcorr_fused_backward(const float *f1, const float *f2, const int32_t *argm
     }
     const int rj = fj.join();
     return rc ? rc : rj;
+}
+
+int sepcorr_fused_backward(const float *f1, const float *f2, const int32_t *argmax_u, const int32_t *argmax_v,
+                           const float *grad_u, const float *grad_v, const float *a_u, const float *a_v,
+                           const float *g_cu, const float *g_cv, float *d_f1, float *d_f2, int B, int H1, int W1, int H2,
+                           int W2, int C, int K, void *workspace, size_t workspace_bytes, void *stream) {
+    return fused_backward(f1, f2, argmax_u, argmax_v, grad_u, grad_v, a_u, a_v, g_cu, g_cv, d_f1, d_f2, 0, B, H1, W1, H2, W2, C, K,
+                          workspace, workspace_bytes, stream);
+}
+
+int sepcorr_fused_backward_add(const float *f1, const float *f2, const int32_t *argmax_u, const int32_t *argmax_v,
+                               const float *grad_u, const float *grad_v, const float *a_u, const float *a_v,
+                               const float *g_cu, const float *g_cv, float *d_f1, float *d_f2, int B, int H1, int W1, int H2,
+                               int W2, int C, int K, void *workspace, size_t workspace_bytes, void *stream) {
+    return fused_backward(f1, f2, argmax_u, argmax_v, grad_u, grad_v, a_u, a_v, g_cu, g_cv, d_f1, d_f2, 1, B, H1, W1, H2, W2, C, K,
+                          workspace, workspace_bytes, stream);
 }
 
 }  // extern "C"

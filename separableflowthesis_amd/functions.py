@@ -267,8 +267,9 @@ class SeparatePyramidFunction(Function):
             for l in range(n):
                 a_u = MemorySaver.softmax_from_stats(z_u[l], st_u[l])
                 a_v = MemorySaver.softmax_from_stats(z_v[l], st_v[l])
-                d1, d2 = MemorySaver.fused_backward(f1, lv[l], am_u[l], am_v[l], d_out_u[l], d_out_v[l], a_u, a_v, g_cu[l], g_cv[l])
-                d_f1 = d1 if d_f1 is None else d_f1 + d1
+                # (the gradient of fmap1 is the sum over the levels: every level after the first adds to the same tensor)
+                d_f1, d2 = MemorySaver.fused_backward(f1, lv[l], am_u[l], am_v[l], d_out_u[l], d_out_v[l], a_u, a_v, g_cu[l], g_cv[l],
+                                                      add_to_grad_fmap1=d_f1)
                 d_f2.append(d2)
         return (d_f1, d_w1, d_b1, d_w2, d_b2, None, *d_f2)
 

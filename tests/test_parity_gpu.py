@@ -204,6 +204,12 @@ def test_fused_backward_is_the_sum_of_both_backwards(device, shape, K):
     assert_close(d2, m2 + c2, "grad_fmap2_lk", scale_atol=True)
     e1, e2 = ms.fused_backward(d(f1), d(f2), au, av, d(g_u), d(g_v), d(a_u), d(a_v), d(g_cu), d(g_cv))
     assert torch.equal(d1, e1) and torch.equal(d2, e2)
+    # added to a gradient of fmap1 that other pyramid levels left (sepcorr_fused_backward_add): same d_f2, d_f1 on top
+    other = torch.randn(f1.shape, generator=g).to(device)
+    s1, s2 = ms.fused_backward(d(f1), d(f2), au, av, d(g_u), d(g_v), d(a_u), d(a_v), d(g_cu), d(g_cv), add_to_grad_fmap1=other.clone())
+    assert torch.equal(s2, d2)
+    err = float((s1 - (other + d1)).abs().max())   # one fp32 addition apart
+    assert err <= 1e-6 * max(1.0, float(d1.abs().max())), f"grad_fmap1_l0 added to another level's: differs by {err}"
     # the weight gradients alone (compression backward without feature gradients)
     da_u, da_v = ms.compression_weight_gradients(d(f1), d(f2), d(a_u), d(a_v), d(g_cu), d(g_cv))
     assert_close(da_u, ra_u, "grad_attention_u", scale_atol=True)
