@@ -198,6 +198,7 @@ __global__ void __launch_bounds__(256) avg_table_reduce_kernel(const GatherArgs 
 
 // d1[p][c] = sum_j g_avg[p,j] lines[j][c]: rows p, columns c, over the H2 + W2 lines two at a time.  grid
 // (ceil(N1/32), B); the tile of gradients goes through LDS, JCHUNK lines at a time.
+constexpr int ROWS_NS = 4;
 __global__ void __launch_bounds__(256) df1_avg_rows_kernel(const GatherArgs a) {
     __shared__ float gsm[32][JCHUNK + 1];
     const int p0 = blockIdx.x * 32, b = blockIdx.y;
@@ -214,30 +215,50 @@ __global__ void __launch_bounds__(256) df1_avg_rows_kernel(const GatherArgs a) {
     for (int jc = 0; jc < L; jc += JCHUNK) {
         const int nj = min(JCHUNK, L - jc);
         if (jc) __syncthreads();
-        for (int i = threadIdx.x; i < 32 * JCHUNK; i += 256) {
-            const int px = i / JCHUNK, jl = i - px * JCHUNK, p = p0 + px, j = jc + jl;
-            float g = 0.f;
-            if (p < N1 && jl < nj)
-                g = j < H2 ? a.g_u[(((size_t)b * N1 + p) * 2 + 1) * H2 + j] : a.g_v[(((size_t)b * N1 + p) * 2 + 1) * W2 + (j - H2)];
-            gsm[px][jl] = g;
+        {   // thread t holds line jc + t of all 32 pixels: the 32 loads are issued before the first is stored
+            // (one after the other, a load and its store per pixel, they took 11 of the kernel's 38 us)
+            static_assert(JCHUNK == 256, "one line per thread");
+            const int jl = threadIdx.x, j = jc + jl;
+            const bool ju = j < H2;
+            const float *gp = ju ? a.g_u + ((size_t)b * N1 * 2 + 1) * H2 + j : a.g_v + ((size_t)b * N1 * 2 + 1) * W2 + (j - H2);
+            const size_t gs = ju ? 2 * (size_t)H2 : 2 * (size_t)W2;
+            float g[32];
+#pragma unroll
+            for (int px = 0; px < 32; ++px) g[px] = (p0 + px < N1 && jl < nj) ? gp[(size_t)(p0 + px) * gs] : 0.f;
+#pragma unroll
+            for (int px = 0; px < 32; ++px) gsm[px][jl] = g[px];
         }
         __syncthreads();
-        if (wave_on) {
-            for (int j0 = 0; j0 < nj; j0 += 8) {
-                float ga[4], x0[4], x1[4];
+        if (wave_on) {   // a ring of ROWS_NS steps of eight lines: operands fetched ROWS_NS - 1 steps ahead of their products
+            struct Ops { float ga[4], x0[4], x1[4]; };
+            auto load = [&](int j0, Ops &o) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int jl = j0 + 2 * i + h;               // < JCHUNK; entries from nj on are zero
                     const int jr = jl < nj ? jc + jl : 0;
-                    ga[i] = gsm[l32][jl];
-                    x0[i] = rp0[(size_t)jr * C];
-                    x1[i] = rp1[(size_t)jr * C];
+                    o.ga[i] = gsm[l32][jl];
+                    o.x0[i] = rp0[(size_t)jr * C];
+                    o.x1[i] = rp1[(size_t)jr * C];
                 }
+            };
+            auto products = [&](const Ops &o) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(ga[i], x0[i], acc0, 0, 0, 0);
-                    acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(ga[i], x1[i], acc1, 0, 0, 0);
+                    acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(o.ga[i], o.x0[i], acc0, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(o.ga[i], o.x1[i], acc1, 0, 0, 0);
                 }
+            };
+            Ops ring[ROWS_NS];
+#pragma unroll
+            for (int st = 0; st < ROWS_NS; ++st)
+                if (8 * st < nj) load(8 * st, ring[st]);
+            for (int j0 = 0; j0 < nj; j0 += 8 * ROWS_NS) {
+#pragma unroll
+                for (int st = 0; st < ROWS_NS; ++st)
+                    if (j0 + 8 * st < nj) {
+                        products(ring[st]);
+                        if (j0 + 8 * (st + ROWS_NS) < nj) load(j0 + 8 * (st + ROWS_NS), ring[st]);
+                    }
             }
         }
     }
