@@ -396,7 +396,7 @@ class Workload:
 # caller level (extras, never `value`)
 # ------------------------------------------------------------------------------------------------
 
-def module_level(name, torch, dev, reps=5, backward=True):
+def module_level(name, torch, dev, reps=20, backward=True, warmup=5):
     """The caller's whole separate() over 4 pyramid levels through the drop-in classes: NHWC copies, both operators
     per level, the attention producer and volume assembly, torch autograd; with the peak memory it allocates next to
     what the stored 4D pyramid alone would take (the comparison of scripts/test_model.py:320-382 for this block)."""
@@ -427,7 +427,7 @@ def module_level(name, torch, dev, reps=5, backward=True):
     for key, bw in (("forward", False), ("forward_backward", True)):
         if bw and not backward:
             continue
-        for _ in range(2):
+        for _ in range(warmup):   # (enough passes for the clocks to settle: the timed loop is a few tens of milliseconds)
             run(bw)
         torch.cuda.synchronize()
         torch.cuda.reset_peak_memory_stats()
@@ -610,7 +610,7 @@ def main():
         # peak memory of the block that never stores the volume, next to the stored 4D pyramid, per configuration
         mem = {}
         for name in ("cfg3", "cfg4", "cfg5"):
-            m = out["module_level"] if name == args.workload else module_level(name, torch, dev, reps=2, backward=name != "cfg5")
+            m = out["module_level"] if name == args.workload else module_level(name, torch, dev, reps=2, backward=name != "cfg5", warmup=2)
             mem[name] = {k: v for k, v in m.items() if k.endswith("_mib")}
             torch.cuda.empty_cache()
         out["memory"] = mem
