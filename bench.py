@@ -506,8 +506,9 @@ def lookup_level(B, H, W, torch, dev, reps=20):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=20,
+                    help="untimed steps first: the clocks of an idle GPU take some tens of milliseconds to settle")
     ap.add_argument("--workload", default="cfg4", choices=sorted(WORKLOADS),
                     help="the workload `value` is quoted on (the headline metric is cfg4)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
