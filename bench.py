@@ -302,6 +302,14 @@ class Workload:
 
     def time(self, fn, steps, warmup):
         torch = self.torch
+        # The clocks of an idle GPU settle over some tens of milliseconds of load (the same build: 2.64 ms per step
+        # right after 3 steps, 2.59 after 20 and after 50).  Part of the set-up, like building the inputs: the step
+        # runs for about 0.1 s, whatever the number of warm-up steps asked for, so that the timed steps see the
+        # clocks a training loop sees.
+        t_end = time.perf_counter() + SETTLE_SECONDS
+        while time.perf_counter() < t_end:
+            fn()
+            torch.cuda.synchronize()
         for _ in range(warmup):
             fn()
         torch.cuda.synchronize()
@@ -396,6 +404,9 @@ class Workload:
 # caller level (extras, never `value`)
 # ------------------------------------------------------------------------------------------------
 
+SETTLE_SECONDS = 0.1   # untimed load before every timed loop (see Workload.time)
+
+
 def module_level(name, torch, dev, reps=20, backward=True, warmup=5):
     """The caller's whole separate() over 4 pyramid levels through the drop-in classes: NHWC copies, both operators
     per level, the attention producer and volume assembly, torch autograd; with the peak memory it allocates next to
@@ -427,7 +438,11 @@ def module_level(name, torch, dev, reps=20, backward=True, warmup=5):
     for key, bw in (("forward", False), ("forward_backward", True)):
         if bw and not backward:
             continue
-        for _ in range(warmup):   # (enough passes for the clocks to settle: the timed loop is a few tens of milliseconds)
+        t_end = time.perf_counter() + SETTLE_SECONDS   # (clocks of an idle GPU: see Workload.time)
+        while time.perf_counter() < t_end:
+            run(bw)
+            torch.cuda.synchronize()
+        for _ in range(warmup):
             run(bw)
         torch.cuda.synchronize()
         torch.cuda.reset_peak_memory_stats()
@@ -555,7 +570,8 @@ def main():
     head = wl.report(args.steps, args.warmup, args.profile_steps)
     out = {
         "metric": METRIC, "value": head["tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "warmup": args.warmup, "settle_seconds_before_warmup": SETTLE_SECONDS,
+        "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": head["workload"] + " " + OPS_TEXT,
                    "contraction_passes": head["contraction_passes"], "gflop_per_step": head["gflop_per_step"],
