@@ -336,8 +336,7 @@ static long wave_strips(int B, int H1, int W1, int L, int NV, int SP) {
     const long total = (long)B * H1 * ((W1 + SP - 1) / SP);
     return (total + per - 1) / per;
 }
-template <int SP>
-static unsigned strip_groups(int B, int H1, int W1, int L, int NV) {
+static unsigned strip_groups(int B, int H1, int W1, int L, int NV, int SP) {
     return (unsigned)((wave_strips(B, H1, W1, L, NV, SP) + WPB - 1) / WPB);
 }
 
@@ -851,8 +850,12 @@ __global__ void __launch_bounds__(256) att_weight_backward_strip_kernel(const At
                 dst[K * 54 + k0 + t] = red[0][27 * DW_KC + t] + red[1][27 * DW_KC + t] + red[2][27 * DW_KC + t] + red[3][27 * DW_KC + t];
 }
 
-// pixels per strip for NV positions per lane (the window of a strip fills 108 to 144 registers)
-constexpr int strip_sp(int nv) { return nv == 4 ? 2 : 4; }
+// pixels per strip for nv positions per lane
+// the forward kernel with two positions per lane: strips of 2 (126 registers, four waves per SIMD; 52 us for attention 1
+// over four levels at B=2, 55x128) are faster than strips of 4 (62 us) or 1 (56 us)
+constexpr int fwd_sp(int nv) { return nv == 1 ? 4 : 2; }
+// the input gradient: strips of 4 and of 2 measure the same with two positions per lane (48 us)
+constexpr int bwd_sp(int nv) { return nv == 4 ? 2 : 4; }
 static bool aligned_for(const void *p, int nv) { return !p || (reinterpret_cast<uintptr_t>(p) & (uintptr_t)(4 * nv - 1)) == 0; }
 // rows of L entries can be held nv to a lane
 static bool strip_fits(int L, int nv) { return L <= 64 * nv && L % nv == 0; }
@@ -895,12 +898,12 @@ static size_t weight_groups_max(int B, int H1, int W1, int L) {
 }
 template <int NV>
 static void launch_backward_strip(const AttJobs &mi, unsigned gi, const AttJobs &mw, unsigned gw, int K, hipStream_t s) {
-    hipLaunchKernelGGL((att_input_backward_strip_kernel<NV, strip_sp(NV)>), dim3(gi), dim3(64 * WPB), 0, s, mi);
+    hipLaunchKernelGGL((att_input_backward_strip_kernel<NV, bwd_sp(NV)>), dim3(gi), dim3(64 * WPB), 0, s, mi);
     hipLaunchKernelGGL((att_weight_backward_strip_kernel<NV>), dim3(gw, 2 * ((K + DW_KC - 1) / DW_KC)), dim3(256), 0, s, mw);
 }
 template <int NV>
 static void launch_forward_strip(const AttJobs &m, unsigned nwg, hipStream_t s) {
-    hipLaunchKernelGGL((att_forward_strip_kernel<NV, strip_sp(NV)>), dim3(nwg), dim3(64 * WPB), 0, s, m);
+    hipLaunchKernelGGL((att_forward_strip_kernel<NV, fwd_sp(NV)>), dim3(nwg), dim3(64 * WPB), 0, s, m);
 }
 int check(const void *p, const char *name) {
     if (p) return 0;
@@ -957,8 +960,7 @@ static int attention_conv_backward_jobs(const AttArgs *jobs, int n, float *parti
             mi.job[q] = jobs[j];
             mi.first[q] = (int)gi;
             gi += var == 0 ? pixel_groups(npix, jobs[j].L)
-                : var == 4 ? strip_groups<strip_sp(4)>(jobs[j].B, jobs[j].H1, jobs[j].W1, jobs[j].L, var)
-                           : strip_groups<strip_sp(1)>(jobs[j].B, jobs[j].H1, jobs[j].W1, jobs[j].L, var);
+                           : strip_groups(jobs[j].B, jobs[j].H1, jobs[j].W1, jobs[j].L, var, bwd_sp(var));
             mw.job[q] = jobs[j];
             mw.job[q].partial = partial + (size_t)(gw_all + gw) * (K * 54 + K);
             mw.first[q] = (int)gw;
@@ -1006,8 +1008,7 @@ static int attention_forward_jobs(const AttArgs *jobs, int n, void *stream) {
             done[j] = true;
             m.job[m.njobs] = jobs[j];
             m.first[m.njobs] = (int)nwg;
-            nwg += nv == 4 ? strip_groups<strip_sp(4)>(jobs[j].B, jobs[j].H1, jobs[j].W1, jobs[j].L, nv)
-                           : strip_groups<strip_sp(1)>(jobs[j].B, jobs[j].H1, jobs[j].W1, jobs[j].L, nv);
+            nwg += strip_groups(jobs[j].B, jobs[j].H1, jobs[j].W1, jobs[j].L, nv, fwd_sp(nv));
             m.first[++m.njobs] = (int)nwg;
         }
         if (nv == 1) launch_forward_strip<1>(m, nwg, s);
