@@ -114,3 +114,38 @@ def test_split_d_f1_agrees_with_itself_under_memory_traffic(device):
         for x, y, name in zip(got, ref, ("d_f1", "d_f2", "d_a_u", "d_a_v")):
             assert torch.equal(x, y), f"launch {n}: {name} differs from the first call's"
     side.synchronize()
+
+
+@pytest.mark.parametrize("dims", [(1, 55, 128, 55, 128, 256), (1, 48, 64, 48, 64, 256)], ids=["cfg3", "cfg1"])
+def test_sweep_with_and_without_scratch(device, dims):
+    """The shape of the workgroups depends on whether the steps are dealt out (scratch given: two 4-wave workgroups per
+    CU) or whole tiles are swept (no scratch: 8 waves): same maxima and argmax, sums to rounding.  A buffer smaller
+    than sepcorr_forward_workspace_bytes() is refused, not silently ignored."""
+    lib = _lib.load()
+    B, H1, W1, H2, W2, C = dims
+    f1, f2, g = op_inputs(*dims, seed=33)
+    f1, f2 = f1.to(device), f2.to(device)
+    P = lambda t: t.data_ptr()
+    E = lambda *s, dt=torch.float32: torch.empty(*s, dtype=dt, device=device)
+    nws = lib.sepcorr_forward_workspace_bytes(*dims, 2)
+    assert nws > 0
+    ws = torch.empty(nws, dtype=torch.uint8, device=device)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def run(n):
+        ou, ov = E(B, H1, W1, 2, H2), E(B, H1, W1, 2, W2)
+        au, av = E(B, H1, W1, 1, H2, dt=torch.int32), E(B, H1, W1, 1, W2, dt=torch.int32)
+        rc = lib.sepcorr_max_argmax_avg_forward(P(f1), P(f2), P(ou), P(ov), P(au), P(av), *dims, P(ws) if n else None, n, stream)
+        torch.cuda.synchronize()
+        return rc, (ou, ov, au, av)
+
+    rc, ref = run(nws)
+    assert rc == 0
+    rc, got = run(0)
+    assert rc == 0
+    assert torch.equal(got[0][:, :, :, 0], ref[0][:, :, :, 0]) and torch.equal(got[1][:, :, :, 0], ref[1][:, :, :, 0]), "maxima differ"
+    assert torch.equal(got[2], ref[2]) and torch.equal(got[3], ref[3]), "argmax differs"
+    for x, y in ((got[0][:, :, :, 1], ref[0][:, :, :, 1]), (got[1][:, :, :, 1], ref[1][:, :, :, 1])):
+        assert float((x - y).abs().max()) <= 2e-6 * max(1.0, float(y.abs().max())), "averages differ"
+    rc, _ = run((nws // 2) & ~255)
+    assert rc != 0 and b"workspace" in lib.sepcorr_last_error()
