@@ -355,6 +355,16 @@ __device__ __forceinline__ KArgs kernargs_now() {
     return p;
 }
 
+// The workgroups wfirst .. wlast that hold the steps [t0, t1) of a tile when sk_total steps are dealt out evenly to G
+// workgroups (workgroup w holds the steps [w sk_total / G, (w + 1) sk_total / G)).
+__device__ __forceinline__ void pieces_of(long t0, long t1, int G, int sk_total, int &wfirst, int &wlast) {
+    wfirst = (int)((t0 * G) / sk_total);                           // the workgroup that holds step t0
+    while (wfirst > 0 && ((long)wfirst * sk_total) / G > t0) --wfirst;
+    while (((long)(wfirst + 1) * sk_total) / G <= t0) ++wfirst;
+    wlast = wfirst;                                                  // the workgroup that holds step t1 - 1
+    while (((long)(wlast + 1) * sk_total) / G < t1) ++wlast;
+}
+
 // The last piece of a tile to finish adds up the column state of all its pieces in row order (equal maxima keep the
 // lower row) and writes the finished out_v columns.  A function of its own: its registers (the pieces of a batch are
 // fetched together) are then allotted apart from those of the sweep.  Arguments are the same in every lane.
@@ -650,6 +660,9 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     const size_t bp = (size_t)b * N1 + (pok ? pix : 0);
     // Rows wider than 256 columns are swept in passes of 256 columns; a pass merges its out_u rows with
     // what the earlier passes left (same thread, same address), the out_v columns of a pass are its own.
+    // Whether this piece, finding every other piece of its tile already in its slot, took them into its own registers
+    // and finished the tile itself (below).
+    bool merged_here = false;
     for (int vp = 0; vp < vpasses; ++vp) {
     if (vp > 0) __syncthreads();   // the previous pass has finished with the LDS partial buffers
     const int vbase = (WM == 2) ? vp * 256 : 0;
@@ -1287,9 +1300,62 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
         }
     }
 
+    // The piece that comes last does not need a slot.  Pieces publish themselves by adding one to the tile's counter
+    // after their slot is in memory (below); a piece that reads "all the others are there" before it has written
+    // anything takes their column state into its own registers instead -- a slot holds it in the very order a wave
+    // keeps it in: wave (column chunk) and lane of the reader are those of the writer -- and then finishes the tile as
+    // a whole tile does, from registers.  Only tiles of two pieces are finished this way (nearly all are): the sum of
+    // two numbers does not depend on which is added to which, so the result is the one merge_pieces gives, whichever
+    // piece came last and whichever path it took; maxima keep the lower row on ties either way.  Of a tile's two pieces the one
+    // with the tile's first rows is the end of its workgroup's share and nearly always the late one: its slot
+    // (written and read back: a third of a sweep's HBM traffic at B=2, 55x128) and the separate merge pass go away.
+    // Only for one pass of columns (with several, the registers hold the state of the last pass only).
+    if (SK && !whole && vpasses == 1) {
+        const int G = (int)gridDim.x;
+        int wfirst, wlast;
+        pieces_of(ubeg, uend, G, sk_total, wfirst, wlast);
+        __syncthreads();   // (LDS word 0 is free: the row groups are merged)
+        int *flag = reinterpret_cast<int *>(smem);
+        if (tide == 0)
+            *flag = __hip_atomic_fetch_add(ke->sk_count + (multi ? tile * a.nlev + lvl : tile), 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        merged_here = wlast == wfirst + 1 && *flag == 1;   // a tile of two pieces, and the other one is there
+        __syncthreads();
+        if (merged_here && ug_e == 0 && vbase + 32 * vcw_e < W2) {
+            constexpr int NQ = (is_weighted(MODE)) ? KC : 3;
+            const __amdgpu_buffer_rsrc_t rs_sk = make_rsrc(ke->sk_state, 2u * gridDim.x * (unsigned)a.sk_slot * 4u);
+            const unsigned mine = (unsigned)((vbase >> 5) + vcw_e) * (NQ * 1024u) + 4u * lane_e;
+            auto fetch = [&](int w, v4f (&x)[NQ][4]) {
+                const bool first_piece = ((long)w * sk_total) / G >= ubeg;   // w's share starts inside this tile: its slot 0
+                const unsigned base = ((unsigned)(2 * w + (first_piece ? 0 : 1)) * (unsigned)a.sk_slot + mine) * 4u;
+#pragma unroll
+                for (int q = 0; q < NQ; ++q)
+#pragma unroll
+                    for (int g4 = 0; g4 < 4; ++g4) x[q][g4] = load_shared4(rs_sk, base + (unsigned)(q * 4 + g4) * 1024u);
+            };
+            // (two pieces: the sum of the two is the same whichever is added to which)
+            const int w = wg == wfirst ? wlast : wfirst;
+            v4f x[NQ][4];
+            fetch(w, x);
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if constexpr (is_weighted(MODE)) {
+#pragma unroll
+                        for (int q = 0; q < NQ; ++q) rv[q][4 * g4 + e] += x[q][g4][e];
+                    } else {
+                        const float m2 = x[0][g4][e];
+                        const int i2 = __float_as_int(x[1][g4][e]);
+                        if (m2 > vmax[4 * g4 + e] || (m2 == vmax[4 * g4 + e] && i2 < vidx[4 * g4 + e])) { vmax[4 * g4 + e] = m2; vidx[4 * g4 + e] = i2; }
+                        vsum[4 * g4 + e] += x[2][g4][e];
+                    }
+                }
+        }
+    }
     // A piece of a tile leaves its column state in this workgroup's slot in register order, sums undivided:
     // [column chunk][quantity][register group g4][lane_e][4]: every store of a wave_e is one contiguous KB
-    if (!whole) {
+    if (!whole && !merged_here) {
         if (ug_e == 0 && vbase + 32 * vcw_e < W2) {
             constexpr int NQ = (is_weighted(MODE)) ? KC : 3;
             const __amdgpu_buffer_rsrc_t rs_sk = make_rsrc(ke->sk_state, 2u * gridDim.x * (unsigned)a.sk_slot * 4u);
@@ -1375,18 +1441,15 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     const size_t bp_e = (size_t)b * N1 + (pok_e ? pix_e : 0);
     (void)lane_e; (void)h_e; (void)vcw_e; (void)ug_e; (void)bp_e;
 
-    if (!whole) {
+    if (!whole && !merged_here) {
         const KArgs ke = kernargs_now();
         // Publish this piece and find out whether it completes the tile.  The pieces of a tile belong to consecutive
         // workgroups; a workgroup keeps the first piece of its share in its slot 0 and a later one (which can only be
         // its last: the tiles between are whole) in its slot 1.
         const int G = (int)gridDim.x;
-        const long t0 = ubeg, t1 = uend;
-        int wfirst = (int)((t0 * G) / sk_total);                       // the workgroup that holds step t0
-        while (wfirst > 0 && ((long)wfirst * sk_total) / G > t0) --wfirst;
-        while (((long)(wfirst + 1) * sk_total) / G <= t0) ++wfirst;
-        int wlast = wfirst;                                              // the workgroup that holds step t1 - 1
-        while (((long)(wlast + 1) * sk_total) / G < t1) ++wlast;
+        const long t0 = ubeg;
+        int wfirst, wlast;
+        pieces_of(ubeg, uend, G, sk_total, wfirst, wlast);
         const int npieces = wlast - wfirst + 1;
         // Hand-over without a fence.  What it rests on: (1) the slot was written with sc0 sc1 stores, which are
         // written through to device memory, and vmcnt counts such a store only when that write is acknowledged, so
