@@ -280,6 +280,16 @@ __device__ __forceinline__ int xcd_contiguous(int bid, int n) {
     const int c = bid & 7, slot = bid >> 3, q = n >> 3, r = n & 7;
     return c * q + (c < r ? c : r) + slot;
 }
+// The same for a grid of 512 workgroups that are resident two to a compute unit: an XCD hands its workgroups
+// 0 .. 31 to its 32 compute units in turn and 32 .. 63 to the same units again, so the units hold the pairs
+// (slot, slot + 32).  Here such a pair gets two neighbouring logical ids.  Shares of steps that are dealt out by
+// logical id differ by one step in a fixed rhythm (2 2 2 3 ...): with neighbours on a unit every unit gets two
+// steps more or less the same sum, where the plain order gave some units two long shares.  (Where the hardware
+// places workgroups differently this costs nothing but the balance.)
+__device__ __forceinline__ int xcd_paired(int bid) {
+    const int c = bid & 7, slot = bid >> 3;
+    return c * 64 + (slot < 32 ? 2 * slot : 2 * (slot - 32) + 1);
+}
 
 }  // namespace
 namespace sepcorr_impl {
@@ -310,6 +320,7 @@ struct FwdArgs {
     int vpasses;       // passes of 256 columns = ceil(W2 / 256)
     int stage;         // collect the rows of out_u in LDS and store them coalesced at the end
     int xcd_order;     // map workgroup ids so that each XCD gets a contiguous range
+    int pair_shares;   // dealt-out sweeps on 512 workgroups: the two workgroups of a compute unit get neighbouring shares
     // Work split finer than a pixel tile.  A tile's sweep is a sequence of steps (one step = the rows all waves of a
     // workgroup take in at once); the steps of all tiles, laid end to end, are dealt out evenly to the workgroups of
     // the grid.  A workgroup whose share ends inside a tile leaves the column state of its piece (max / argmax / sum
@@ -494,7 +505,8 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     constexpr bool ML = SK && WM == 1;   // may cover several pyramid levels
     const bool multi = ML && a.nlev > 1;
     const int vpasses = (WM == 2) ? a.vpasses : 1;
-    const int wg = a.xcd_order ? xcd_contiguous(blockIdx.x, gridDim.x) : (int)blockIdx.x;
+    const int wg = !a.xcd_order ? (int)blockIdx.x
+                   : (SK && a.pair_shares) ? xcd_paired(blockIdx.x) : xcd_contiguous(blockIdx.x, gridDim.x);
     const int N1 = a.N1, C = a.C;
     const int LS = BF ? BF_LS : a.CP + 4;
     float *f1s = smem;
@@ -2912,7 +2924,7 @@ WaveGrid wave_grid(int B, int tiles_per_batch, int W2, int H2, bool dealt = fals
     g.nug = 1;
     if (g.nvc <= 2) {
         g.nug = 4 / g.nvc;                                        // 4 waves
-        if ((long)B * tiles_per_batch * 4 < 1536) g.nug *= 2;     // small problem: 8 waves fill more SIMDs
+        if (!dealt && (long)B * tiles_per_batch * 4 < 1536) g.nug *= 2;     // small problem: 8 waves fill more SIMDs
         while (g.nug > 1 && g.nug > H2) g.nug /= 2;
     } else if (!dealt && g.nvc <= 4 && (long)B * tiles_per_batch <= 256 && H2 >= 8) {
         g.nug = 2;   // at most one workgroup per CU: two row groups give every SIMD a second wave
@@ -3127,6 +3139,7 @@ int launch_fwd(FwdArgs a, int B, hipStream_t s) {
         a.sk_state = reinterpret_cast<float *>(static_cast<char *>(a.ws) + f.count_bytes);
         a.sk_slot = (int)f.slot_floats;
         grid = dim3(f.G);
+        a.pair_shares = f.G == 2 * kCUs;
         const int n = B * a.tiles_per_batch;
         hipLaunchKernelGGL(zero_ints_kernel, dim3((n + 255) / 256), dim3(256), 0, s, a.sk_count, n);
     }
@@ -3218,6 +3231,7 @@ int launch_fwd_levels(FwdArgs a, int B, hipStream_t s) {
     a.sk_count = static_cast<int *>(a.ws);
     a.sk_state = reinterpret_cast<float *>(static_cast<char *>(a.ws) + count_bytes);
     a.sk_slot = (int)slot_floats;
+    a.pair_shares = G == 2 * kCUs;
     const int n = tiles * a.nlev;
     hipLaunchKernelGGL(zero_ints_kernel, dim3((n + 255) / 256), dim3(256), 0, s, a.sk_count, n);
     const dim3 grid(G), block(64 * nW);
