@@ -398,88 +398,119 @@ __device__ __attribute__((noinline)) void merge_pieces(KArgs ka_in, int lvl_in, 
     constexpr int NQ = (is_weighted(MODE)) ? KC : 3;
     const __amdgpu_buffer_rsrc_t rs_sk = make_rsrc(ka->sk_state, 2u * gridDim.x * (unsigned)ka->sk_slot * 4u);
     const int nchunks = (W2 + 31) >> 5;
-    for (int it = tid; it < nchunks * 256; it += blockDim.x) {
-        const int ln = it & 63, g4 = (it >> 6) & 3, chunk = it >> 8;
-        const int p = ln & 31, v = 32 * chunk + vmap(4 * g4, ln >> 5);
-        v4f acc4[NQ];
+    const int total = nchunks * 256;
+    constexpr int PB = 4;   // pieces fetched together (a tile rarely has more)
+    // items of a thread in flight together, their slot reads waiting side by side (one where four quantities per
+    // piece would take the registers of the sweep)
+    constexpr int IU = NQ <= 3 ? 2 : 1;
+    for (int it0 = tid; it0 < total; it0 += IU * (int)blockDim.x) {
+        v4f acc4[IU][NQ];
 #pragma unroll
-        for (int q = 0; q < NQ; ++q) acc4[q] = v4f{0.f, 0.f, 0.f, 0.f};
-        if constexpr (!is_weighted(MODE)) acc4[0] = v4f{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
-        constexpr int PB = 4;   // pieces fetched together (a tile rarely has more)
+        for (int i = 0; i < IU; ++i) {
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) acc4[i][q] = v4f{0.f, 0.f, 0.f, 0.f};
+            if constexpr (!is_weighted(MODE)) acc4[i][0] = v4f{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+        }
         for (int w0 = wfirst; w0 <= wlast; w0 += PB) {
-            v4f x[PB][NQ];
+            v4f x[IU][PB][NQ];
+            unsigned slot[PB];
 #pragma unroll
             for (int j = 0; j < PB; ++j) {
                 const int w = w0 + j;
                 const bool first_piece = ((long)w * sk_total) / G >= t0;   // w's share starts inside this tile
-                const unsigned base = ((unsigned)(2 * w + (first_piece ? 0 : 1)) * (unsigned)ka->sk_slot +
-                                       (unsigned)chunk * (NQ * 1024u) + 4u * ln) * 4u;
-                if (w <= wlast) {
-#pragma unroll
-                    for (int q = 0; q < NQ; ++q) x[j][q] = load_shared4(rs_sk, base + (unsigned)(q * 4 + g4) * 1024u);
-                }
+                slot[j] = (unsigned)(2 * w + (first_piece ? 0 : 1)) * (unsigned)ka->sk_slot;
             }
 #pragma unroll
-            for (int j = 0; j < PB; ++j) {
-                if (w0 + j > wlast) break;
-                if constexpr (is_weighted(MODE)) {
+            for (int i = 0; i < IU; ++i) {
+                const int it = it0 + i * (int)blockDim.x;
+                const int ln = it & 63, g4 = (it >> 6) & 3, chunk = it >> 8;
+                if (it < total) {
 #pragma unroll
-                    for (int q = 0; q < NQ; ++q) acc4[q] += x[j][q];
-                } else {
+                    for (int j = 0; j < PB; ++j) {
+                        const unsigned base = (slot[j] + (unsigned)chunk * (NQ * 1024u) + 4u * ln) * 4u;
+                        if (w0 + j <= wlast) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        // (equal maxima keep the lower row: the rows of two neighbouring pieces may alternate)
-                        if (x[j][0][e] > acc4[0][e] ||
-                            (x[j][0][e] == acc4[0][e] && __float_as_int(x[j][1][e]) < __float_as_int(acc4[1][e]))) {
-                            acc4[0][e] = x[j][0][e];
-                            acc4[1][e] = x[j][1][e];
+                            for (int q = 0; q < NQ; ++q) x[i][j][q] = load_shared4(rs_sk, base + (unsigned)(q * 4 + g4) * 1024u);
                         }
-                    acc4[2] += x[j][2];
+                    }
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < IU; ++i) {
+                if (it0 + i * (int)blockDim.x >= total) break;
+#pragma unroll
+                for (int j = 0; j < PB; ++j) {
+                    if (w0 + j > wlast) break;
+                    if constexpr (is_weighted(MODE)) {
+#pragma unroll
+                        for (int q = 0; q < NQ; ++q) acc4[i][q] += x[i][j][q];
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            // (equal maxima keep the lower row: the rows of two neighbouring pieces may alternate)
+                            if (x[i][j][0][e] > acc4[i][0][e] ||
+                                (x[i][j][0][e] == acc4[i][0][e] && __float_as_int(x[i][j][1][e]) < __float_as_int(acc4[i][1][e]))) {
+                                acc4[i][0][e] = x[i][j][0][e];
+                                acc4[i][1][e] = x[i][j][1][e];
+                            }
+                        acc4[i][2] += x[i][j][2];
+                    }
                 }
             }
         }
-        if (p0 + p >= N1) continue;
-        const size_t o = (size_t)b * N1 + p0 + p;
-        if constexpr (is_weighted(MODE)) {
-            if (soft_dlog) {   // sums of softmax-output gradients -> gradients of the logits
-                float r3[NQ][3], z[NQ][4];
 #pragma unroll
-                for (int q = 0; q < NQ; ++q) {
-                    const size_t row = o * ka->KT + ka->k0 + q;
-                    r3[q][0] = ka->lev[lvl].st_ov[2 * row]; r3[q][1] = ka->lev[lvl].st_ov[2 * row + 1]; r3[q][2] = ka->lev[lvl].dot_ov[row];
+        for (int i = 0; i < IU; ++i) {
+            const int it = it0 + i * (int)blockDim.x;
+            if (it >= total) break;
+            const int ln = it & 63, g4 = (it >> 6) & 3, chunk = it >> 8;
+            const int p = ln & 31, v = 32 * chunk + vmap(4 * g4, ln >> 5);
+            if (p0 + p >= N1) continue;
+            const size_t o = (size_t)b * N1 + p0 + p;
+            if constexpr (is_weighted(MODE)) {
+                if (soft_dlog) {   // sums of softmax-output gradients -> gradients of the logits
+                    float r3[NQ][3], z[NQ][4];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) z[q][e] = v + e < W2 ? ka->lev[lvl].z_ov[row * W2 + v + e] : 0.f;
-                }
+                    for (int q = 0; q < NQ; ++q) {
+                        const size_t row = o * ka->KT + ka->k0 + q;
+                        r3[q][0] = ka->lev[lvl].st_ov[2 * row]; r3[q][1] = ka->lev[lvl].st_ov[2 * row + 1]; r3[q][2] = ka->lev[lvl].dot_ov[row];
 #pragma unroll
-                for (int q = 0; q < NQ; ++q) {
-                    r3[q][1] = 1.f / r3[q][1];
+                        for (int e = 0; e < 4; ++e) z[q][e] = v + e < W2 ? ka->lev[lvl].z_ov[row * W2 + v + e] : 0.f;
+                    }
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) acc4[q][e] = dlogit3(z[q][e], r3[q], acc4[q][e]);
+                    for (int q = 0; q < NQ; ++q) {
+                        r3[q][1] = 1.f / r3[q][1];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc4[i][q][e] = dlogit3(z[q][e], r3[q], acc4[i][q][e]);
+                    }
                 }
             }
-        }
-        if ((W2 & 3) == 0 && (reinterpret_cast<uintptr_t>(ka->lev[lvl].out_v) & 15) == 0 && MODE != MODE_ARGMAX) {
-            if (v < W2) {
+            bool vec = (W2 & 3) == 0 && (reinterpret_cast<uintptr_t>(ka->lev[lvl].out_v) & 15) == 0;
+            if constexpr (MODE == MODE_ARGMAX) vec = vec && (reinterpret_cast<uintptr_t>(ka->lev[lvl].am_v) & 15) == 0;
+            if (vec) {
+                if (v < W2) {
+                    if constexpr (is_weighted(MODE)) {
+#pragma unroll
+                        for (int q = 0; q < NQ; ++q) *reinterpret_cast<v4f *>(ka->lev[lvl].out_v + (o * ka->KT + ka->k0 + q) * W2 + v) = acc4[i][q];
+                    } else {
+                        *reinterpret_cast<v4f *>(ka->lev[lvl].out_v + (o * 2 + 0) * W2 + v) = acc4[i][0];
+                        *reinterpret_cast<v4f *>(ka->lev[lvl].out_v + (o * 2 + 1) * W2 + v) = acc4[i][2] / (float)H2;
+                        if constexpr (MODE == MODE_ARGMAX)   // (the indices travel as the bit patterns of floats)
+                            *reinterpret_cast<v4f *>(ka->lev[lvl].am_v + o * W2 + v) = acc4[i][1];
+                    }
+                }
+                continue;
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (v + e >= W2) break;
                 if constexpr (is_weighted(MODE)) {
 #pragma unroll
-                    for (int q = 0; q < NQ; ++q) *reinterpret_cast<v4f *>(ka->lev[lvl].out_v + (o * ka->KT + ka->k0 + q) * W2 + v) = acc4[q];
+                    for (int q = 0; q < NQ; ++q) ka->lev[lvl].out_v[(o * ka->KT + ka->k0 + q) * W2 + v + e] = acc4[i][q][e];
                 } else {
-                    *reinterpret_cast<v4f *>(ka->lev[lvl].out_v + (o * 2 + 0) * W2 + v) = acc4[0];
-                    *reinterpret_cast<v4f *>(ka->lev[lvl].out_v + (o * 2 + 1) * W2 + v) = acc4[2] / (float)H2;
+                    ka->lev[lvl].out_v[(o * 2 + 0) * W2 + v + e] = acc4[i][0][e];
+                    ka->lev[lvl].out_v[(o * 2 + 1) * W2 + v + e] = acc4[i][2][e] / (float)H2;
+                    if constexpr (MODE == MODE_ARGMAX) ka->lev[lvl].am_v[o * W2 + v + e] = __float_as_int(acc4[i][1][e]);
                 }
-            }
-            continue;
-        }
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            if (v + e >= W2) break;
-            if constexpr (is_weighted(MODE)) {
-#pragma unroll
-                for (int q = 0; q < NQ; ++q) ka->lev[lvl].out_v[(o * ka->KT + ka->k0 + q) * W2 + v + e] = acc4[q][e];
-            } else {
-                ka->lev[lvl].out_v[(o * 2 + 0) * W2 + v + e] = acc4[0][e];
-                ka->lev[lvl].out_v[(o * 2 + 1) * W2 + v + e] = acc4[2][e] / (float)H2;
-                if constexpr (MODE == MODE_ARGMAX) ka->lev[lvl].am_v[o * W2 + v + e] = __float_as_int(acc4[1][e]);
             }
         }
     }
