@@ -1353,7 +1353,9 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdArgs a) {
     // with the tile's first rows is the end of its workgroup's share and nearly always the late one: its slot
     // (written and read back: a third of a sweep's HBM traffic at B=2, 55x128) and the separate merge pass go away.
     // Only for one pass of columns (with several, the registers hold the state of the last pass only).
-    if (SK && !whole && vpasses == 1) {
+    // (The piece at the end of a share is done first and holds its tile's first rows: the other pieces of that tile
+    // are the last thing their workgroups do, so it has nothing to look for and goes straight to its slot.)
+    if (SK && !whole && vpasses == 1 && !(seg_no == 0 && head)) {
         const int G = (int)gridDim.x;
         int wfirst, wlast;
         pieces_of(ubeg, uend, G, sk_total, wfirst, wlast);
